@@ -1,0 +1,214 @@
+/*
+ * yscv_hip.h -- C ABI of the MI355X (gfx950) backend for YSCV's quantized-matmul path.
+ *
+ * The Rust reference exposes this path as plain `pub fn`s over slices
+ * (crates/yscv-kernels/src/core.rs:173-186) and has no plugin registry for it, so
+ * the drop-in boundary is this function set.  Conventions, modelled on the two
+ * native-code precedents in the reference (the `.S` SGEMM kernels declared in
+ * crates/yscv-kernels/src/ops/matmul/asm.rs:44-152 and the RKNN matmul context in
+ * crates/yscv-kernels/src/rknn/backend.rs:1657-2077):
+ *
+ *   - every entry point returns an int32 status: 0 = ok, negative = error; the
+ *     message of the calling thread's last error is yscv_hip_last_error();
+ *   - raw pointers and size_t only, symbol prefix `yscv_hip_`;
+ *   - weights live in opaque handles that own device memory and are immutable
+ *     after creation, so any number of threads may use one handle concurrently;
+ *   - `*_dev` pointers are device addresses and the call is asynchronous on
+ *     `stream` (a hipStream_t passed as void*, NULL = the default stream);
+ *   - entry points whose names end in `_dispatch`, and every entry point that
+ *     takes `_host` pointers, borrow host memory for the duration of the call,
+ *     copy in and out themselves and return after the result is in host memory:
+ *     these have the exact argument lists of the Rust functions they replace;
+ *   - nothing here falls back to CPU arithmetic: a shape a kernel cannot run
+ *     is an error (YSCV_HIP_ERR_UNSUPPORTED), never a silent slow path.
+ */
+#ifndef YSCV_HIP_H
+#define YSCV_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
+
+#define YSCV_HIP_ABI_VERSION 1u
+
+/* status codes */
+#define YSCV_HIP_OK 0
+#define YSCV_HIP_ERR_INVALID_ARG (-1) /* shape/pointer contract violated (Rust: debug_assert!) */
+#define YSCV_HIP_ERR_DEVICE (-2)      /* a HIP runtime call failed */
+#define YSCV_HIP_ERR_OOM (-3)         /* device allocation failed */
+#define YSCV_HIP_ERR_UNSUPPORTED (-4) /* valid request this build has no kernel for */
+#define YSCV_HIP_ERR_NO_DEVICE (-5)   /* no gfx950 device visible */
+
+/* element types of activations, outputs and scales */
+#define YSCV_HIP_F32 0
+#define YSCV_HIP_F16 1
+#define YSCV_HIP_BF16 2
+
+/* nibble encodings accepted by yscv_hip_int4_weight_create */
+#define YSCV_HIP_NIBBLE_SIGNED 0   /* two's complement [-8,7], no zero point: int4_matmul.rs:10-25 */
+#define YSCV_HIP_NIBBLE_UNSIGNED 1 /* [0,15] with zero point (default 8): ONNX MatMulNBits */
+
+/* rounding rules of the requantize epilogue */
+#define YSCV_HIP_ROUND_HALF_AWAY 0 /* f32::round -- QLinearMatMul, linear.rs:481-485 */
+#define YSCV_HIP_ROUND_TIES_EVEN 1 /* round_ties_even -- int8_requant.rs:161-162,550-552 */
+
+/* ---- lifecycle -------------------------------------------------------------- */
+
+/* Select the device (index into the visible HIP devices) and create the
+ * library's context.  Idempotent; every other entry point calls it with device 0
+ * on first use.  No counterpart in the reference (host_cpu() feature probe,
+ * crates/yscv-cpu/src/lib.rs:74-119, plays the same once-per-process role). */
+int32_t yscv_hip_init(int32_t device_index);
+int32_t yscv_hip_shutdown(void);
+uint32_t yscv_hip_abi_version(void);
+/* Message of the last error raised on the calling thread ("" if none). */
+const char *yscv_hip_last_error(void);
+/* Human-readable device / kernel-selection report, like dispatch_report()
+ * (crates/yscv-kernels/src/core.rs:79-121).  Writes a NUL-terminated string. */
+int32_t yscv_hip_device_info(char *buf, size_t buf_len);
+
+/* Device memory helpers for hosts without their own HIP binding. */
+int32_t yscv_hip_malloc(void **dev_ptr, size_t bytes);
+int32_t yscv_hip_free(void *dev_ptr);
+int32_t yscv_hip_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes, void *stream);
+int32_t yscv_hip_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes, void *stream);
+int32_t yscv_hip_stream_synchronize(void *stream);
+
+/* ---- packed int4 weights ------------------------------------------------------ */
+
+/* Device-resident form of PackedInt4Weight
+ * (crates/yscv-onnx/src/quantize/packed_int4.rs:29-39). */
+typedef struct yscv_hip_int4_weight yscv_hip_int4_weight;
+
+/* Upload and re-tile a packed int4 weight.  Host inputs, borrowed:
+ *   packed       [n][k/2] bytes, element 2i in the low nibble (int4_matmul.rs:12-14)
+ *   scales       [n][k/group_size], scale_dtype F32 or F16
+ *   zero_points  NULL, or [n][ceil((k/group_size)/2)] bytes of uint4 (group 2j in the
+ *                low nibble) -- only with YSCV_HIP_NIBBLE_UNSIGNED
+ * group_size must be even and divide k (int4_matmul.rs:53-54). */
+int32_t yscv_hip_int4_weight_create(const uint8_t *packed, const void *scales, int32_t scale_dtype,
+                                    const uint8_t *zero_points, int32_t nibble_format, size_t n,
+                                    size_t k, size_t group_size, yscv_hip_int4_weight **out);
+int32_t yscv_hip_int4_weight_destroy(yscv_hip_int4_weight *w);
+int32_t yscv_hip_int4_weight_dims(const yscv_hip_int4_weight *w, size_t *n, size_t *k,
+                                  size_t *group_size, size_t *device_bytes);
+
+/* y[m][n] = sum_k x[m][k] * W[n][k]; x_dev is [m][k] row-major of x_dtype, y_dev is
+ * [m][n] of y_dtype.  `yscv_hip_int4_matmul` picks the kernel from m the way
+ * exec_matmul does (crates/yscv-onnx/src/runner/linear.rs:228-278: per-row GEMV
+ * below a threshold, GEMM above); `_gemv` forces the skinny kernel (m <= 16,
+ * replaces packed_int4_gemv_dispatch, int4_matmul.rs:310-377, called once per row)
+ * and `_gemm` the tiled MFMA kernel (replaces packed_int4_gemm_dispatch,
+ * int4_matmul.rs:548-605). */
+int32_t yscv_hip_int4_matmul(const yscv_hip_int4_weight *w, const void *x_dev, int32_t x_dtype,
+                             void *y_dev, int32_t y_dtype, size_t m, void *stream);
+int32_t yscv_hip_int4_gemv(const yscv_hip_int4_weight *w, const void *x_dev, int32_t x_dtype,
+                           void *y_dev, int32_t y_dtype, size_t m, void *stream);
+int32_t yscv_hip_int4_gemm(const yscv_hip_int4_weight *w, const void *x_dev, int32_t x_dtype,
+                           void *y_dev, int32_t y_dtype, size_t m, void *stream);
+
+/* Exact argument lists of the Rust functions (host slices -> host pointers):
+ * packed_int4_gemv_dispatch  int4_matmul.rs:310-318
+ * packed_int4_gemm_dispatch  int4_matmul.rs:548-557
+ * pack_int4_symmetric_per_group  int4_matmul.rs:611-616 (returns into caller buffers
+ *   packed_out[m_w*k/2], scales_out[m_w*k/group_size])
+ * dequantize_int4_to_f32     ops/quantize.rs:18 (output[2*n_bytes]) */
+int32_t yscv_hip_packed_int4_gemv_dispatch(const uint8_t *weight_packed, const float *scales,
+                                           const float *activation, float *output, size_t m_w,
+                                           size_t k, size_t group_size);
+int32_t yscv_hip_packed_int4_gemm_dispatch(const uint8_t *weight_packed, const float *scales,
+                                           const float *activation, float *output, size_t m,
+                                           size_t n, size_t k, size_t group_size);
+int32_t yscv_hip_pack_int4_symmetric_per_group(const float *weights, size_t m_w, size_t k,
+                                               size_t group_size, uint8_t *packed_out,
+                                               float *scales_out);
+int32_t yscv_hip_dequantize_int4_to_f32(const uint8_t *packed, size_t n_bytes, float scale,
+                                        int8_t zero_point, float *output);
+
+/* ---- int8 GEMM ------------------------------------------------------------------ */
+
+/* Device-resident form of PackedI8B (crates/yscv-kernels/src/ops/int8_matmul.rs:128-160):
+ * B re-tiled for the MFMA kernel plus its per-column sums. */
+typedef struct yscv_hip_i8_weight yscv_hip_i8_weight;
+
+/* pack_i8_b_for_matmul (int8_matmul.rs:163): b_host is row-major [k][n]. */
+int32_t yscv_hip_pack_i8_b_for_matmul(const int8_t *b_host, size_t k, size_t n,
+                                      yscv_hip_i8_weight **out);
+int32_t yscv_hip_i8_weight_destroy(yscv_hip_i8_weight *b);
+int32_t yscv_hip_i8_weight_dims(const yscv_hip_i8_weight *b, size_t *k, size_t *n);
+
+/* out[i][j] = sum_k (a[i][k] - a_zp) * b[k][j] in exact int32.
+ * a_dev is [m][k]; a_is_u8 = 0: int8 activations (then a_zp is usually 0, the
+ * int8_matmul_prepacked_dispatch contract, int8_matmul.rs:2420); a_is_u8 = 1: uint8
+ * activations with zero point a_zp (MatMulInteger, ONNX).  The zero point is folded as
+ * acc - a_zp * colsum(b), the algebra of
+ * crates/yscv-onnx/src/runner/conv/quantized.rs:119-147. */
+int32_t yscv_hip_int8_matmul(const void *a_dev, int32_t a_is_u8, int32_t a_zp,
+                             const yscv_hip_i8_weight *b, size_t m, int32_t *out_dev, void *stream);
+
+/* Same GEMM with the requantize epilogue fused (no int32 round trip through HBM):
+ *   q = clamp(round(f32(acc + corr[j]) * composite[j] + y_zp), clamp_lo, clamp_hi)
+ * corr_dev / composite_dev are per-column device arrays or NULL (then corr = 0 and
+ * the scalar `composite` is used).  round_mode HALF_AWAY with [-128,127] is the
+ * QLinearMatMul fast path (linear.rs:481-485); TIES_EVEN is
+ * requant_i8_per_channel_dispatch (int8_requant.rs:401-429).  out_dev is [m][n] bytes:
+ * int8 when clamp_lo < 0, otherwise uint8 (range [0,255] is an extension: the
+ * reference always clamps to [-128,127], linear.rs:484). */
+int32_t yscv_hip_int8_matmul_requant(const void *a_dev, int32_t a_is_u8, int32_t a_zp,
+                                     const yscv_hip_i8_weight *b, size_t m,
+                                     const int32_t *corr_dev, const float *composite_dev,
+                                     float composite, float y_zp, int32_t round_mode,
+                                     int32_t clamp_lo, int32_t clamp_hi, void *out_dev,
+                                     void *stream);
+
+/* Exact argument lists of int8_matmul_dispatch (int8_matmul.rs:2407; b is [k][n]) and
+ * int8_matmul_prepacked_dispatch (int8_matmul.rs:2420), host pointers. */
+int32_t yscv_hip_int8_matmul_dispatch(const int8_t *a, const int8_t *b, size_t m, size_t k,
+                                      size_t n, int32_t *out);
+int32_t yscv_hip_int8_matmul_prepacked_dispatch(const int8_t *a, const yscv_hip_i8_weight *b,
+                                                size_t m, int32_t *out);
+
+/* ---- quantize / requantize / DynamicQuantizeLinear (device pointers) -------------- */
+
+/* quantize_linear_f32_to_i8_dispatch (ops/quantize.rs:154):
+ * q = clamp(round_ties_even(v / scale + zero_point), -128, 127). */
+int32_t yscv_hip_quantize_linear_f32_to_i8(const float *data_dev, size_t len, float scale,
+                                           float zero_point, int8_t *out_dev, void *stream);
+/* requant_i8_per_channel_dispatch (ops/int8_requant.rs:401): acc is [len/c][c]. */
+int32_t yscv_hip_requant_i8_per_channel(const int32_t *acc_dev, size_t len,
+                                        const int32_t *corr_dev, const float *composite_dev,
+                                        float y_zp, int8_t *out_dev, size_t c, void *stream);
+/* requant_i32_row_to_i8_dispatch (ops/int8_requant.rs:81): bias_dev may be NULL. */
+int32_t yscv_hip_requant_i32_row_to_i8(const int32_t *acc_dev, size_t len, const int32_t *bias_dev,
+                                       float composite, float y_zp, int32_t relu, int8_t *out_dev,
+                                       size_t c, void *stream);
+/* exec_dynamic_quantize_linear (crates/yscv-onnx/src/runner/misc.rs:241-289):
+ * y_dev[len] uint8, scale_zp_dev[0] = scale, scale_zp_dev[1] = zero point (as f32). */
+int32_t yscv_hip_dynamic_quantize_linear(const float *x_dev, size_t len, uint8_t *y_dev,
+                                         float *scale_zp_dev, void *stream);
+
+/* Host-pointer forms with the Rust argument lists. */
+int32_t yscv_hip_quantize_linear_f32_to_i8_dispatch(const float *data, size_t len, float scale,
+                                                    float zero_point, int8_t *output);
+int32_t yscv_hip_requant_i8_per_channel_dispatch(const int32_t *acc, size_t len,
+                                                 const int32_t *corr, const float *composite,
+                                                 float y_zp, int8_t *out, size_t c);
+int32_t yscv_hip_requant_i32_row_to_i8_dispatch(const int32_t *acc, size_t len,
+                                                const int32_t *bias, float composite, float y_zp,
+                                                int32_t relu, int8_t *out, size_t c);
+int32_t yscv_hip_dynamic_quantize_linear_host(const float *x, size_t len, uint8_t *y,
+                                              float *scale, float *zero_point);
+
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
+#ifdef __cplusplus
+}
+#endif
+#endif /* YSCV_HIP_H */

@@ -1,0 +1,277 @@
+"""GPU parity of the packed-int4 matmul kernels against the CPU restatement of the reference,
+through the C ABI.  Float parity bar: see gpu_util.int4_tolerances."""
+import numpy as np
+import pytest
+
+from gpu_util import bf16_round, int4_tolerances, pack_zero_points
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return torch
+
+
+@pytest.fixture(scope="module")
+def K():
+    from yscv_amd import kernels
+
+    return kernels
+
+
+def _rand_packed(rng, n, k):
+    return rng.integers(0, 256, n * k // 2, dtype=np.uint8)
+
+
+# ---- the reference's own unit-test shapes, through the exact-signature entry points -----------
+
+@pytest.mark.parametrize("m_w,k,g,sw,sx", [(4, 128, 32, 0xCAFEBABE, 0xF00DBA12), (8, 256, 32, 0x12345678, 0x9ABCDEF0),
+                                           (2, 32, 16, 0xDEADBEEF, 7), (3, 96, 6, 1, 2), (4, 64, 32, 0xAA, 0xBB)])
+def test_gemv_dispatch_reference_shapes(oracle, K, m_w, k, g, sw, sx):
+    # int4_matmul.rs:720-758, :857-900 (reference tolerance between its own kernels: 1e-4)
+    packed, scales = oracle.pack_int4_symmetric_per_group(oracle.lcg_f32(sw, m_w * k), m_w, k, g)
+    x = oracle.lcg_f32(sx, k)
+    ref = oracle.packed_int4_gemv_scalar(packed, scales, x, m_w, k, g)
+    out = np.full(m_w, 999.0, np.float32)
+    K.packed_int4_gemv_dispatch(packed, scales, x, out, m_w, k, g)
+    assert np.abs(out - ref).max() <= 1e-4
+    int4_tolerances(out, ref, k, x)
+
+
+def test_gemv_zero_weights_emit_exact_zeros(oracle, K):
+    # int4_matmul.rs:761-773
+    m_w, k, g = 3, 32, 16
+    packed, scales = oracle.pack_int4_symmetric_per_group(np.zeros(m_w * k, np.float32), m_w, k, g)
+    out = np.full(m_w, 999.0, np.float32)
+    K.packed_int4_gemv_dispatch(packed, scales, np.full(k, 1.5, np.float32), out, m_w, k, g)
+    assert (out == 0).all()
+    m_w, k, g = 20, 256, 32  # tiled path
+    packed, scales = oracle.pack_int4_symmetric_per_group(np.zeros(m_w * k, np.float32), m_w, k, g)
+    out = np.full(m_w, 999.0, np.float32)
+    K.packed_int4_gemv_dispatch(packed, scales, np.full(k, 1.5, np.float32), out, m_w, k, g)
+    assert (out == 0).all()
+
+
+@pytest.mark.parametrize("m", [1, 4, 16, 32])
+def test_gemm_dispatch_reference_shapes(oracle, K, m):
+    # int4_matmul.rs:816-855 (reference tolerance 1e-3)
+    n, k, g = 8, 64, 32
+    packed, scales = oracle.pack_int4_symmetric_per_group(oracle.lcg_f32(0x100, n * k), n, k, g)
+    x = oracle.lcg_f32(0x200 + m, m * k)
+    ref = oracle.packed_int4_gemm_scalar(packed, scales, x, m, n, k, g)
+    out = np.full((m, n), 999.0, np.float32)
+    K.packed_int4_gemm_dispatch(packed, scales, x, out, m, n, k, g)
+    assert np.abs(out - ref).max() <= 1e-3
+    int4_tolerances(out, ref, k, x)
+
+
+def test_hand_kat(K):
+    # nibbles (1,2),(-8,-1), groups of 2, scales .5/.25, x = 1..4 -> -4.5 (generic kernel, g = 2)
+    out = np.zeros(1, np.float32)
+    K.packed_int4_gemv_dispatch(np.array([0x21, 0xF8], np.uint8), np.array([0.5, 0.25], np.float32),
+                                np.array([1, 2, 3, 4], np.float32), out, 1, 4, 2)
+    assert out.tolist() == [-4.5]
+
+
+def test_pack_int4_bit_exact(oracle, K):
+    rng = np.random.default_rng(31)
+    for (m_w, k, g) in [(4, 64, 16), (7, 256, 32), (3, 384, 128), (2, 12, 6)]:
+        w = rng.standard_normal(m_w * k).astype(np.float32)
+        w[: g] = 0  # an all-zero group -> scale 1.0
+        w[g] = np.float32(0.5) * np.float32(1e-3)
+        p_ref, s_ref = oracle.pack_int4_symmetric_per_group(w, m_w, k, g)
+        p, s = K.pack_int4_symmetric_per_group(w, m_w, k, g)
+        assert np.array_equal(s, s_ref) and np.array_equal(p, p_ref)
+
+
+def test_dequantize_int4_bit_exact(oracle, K):
+    rng = np.random.default_rng(32)
+    packed = rng.integers(0, 256, 777, dtype=np.uint8)
+    for scale, zp in [(0.5, 0), (0.1, 2), (0.25, 1), (0.1, -3)]:
+        out = np.empty(2 * packed.size, np.float32)
+        K.dequantize_int4_to_f32(packed, scale, zp, out)
+        assert np.array_equal(out, oracle.dequantize_int4_to_f32(packed, scale, zp))
+    out = np.empty(2, np.float32)
+    K.dequantize_int4_to_f32(np.array([0xE3], np.uint8), 0.5, 0, out)  # quantize.rs:681-688
+    assert out.tolist() == [1.5, -1.0]
+
+
+# ---- device handles: BASELINE config shapes -----------------------------------------------------
+
+def test_config1_gemv_4096(oracle, K, torch_cuda):
+    """BASELINE config 1: M=1 K=4096 N=4096, uint4 weights (zero point 8), g=32, f32 scales
+    U(0.005,0.02), f32 activations N(0,1)."""
+    torch = torch_cuda
+    rng = np.random.default_rng(1000)
+    n = k = 4096
+    g = 32
+    b = _rand_packed(rng, n, k)
+    scales = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float32)
+    x = rng.standard_normal(k).astype(np.float32)
+    ref = oracle.packed_int4_gemv_scalar(b ^ 0x88, scales, x, n, k, g)
+    w = K.PackedInt4Weight(b, scales, g, n, k, nibble_format=K.NIBBLE_UNSIGNED)
+    y = w.matmul(torch.from_numpy(x).cuda().reshape(1, k)).cpu().numpy().ravel()
+    d, rel = int4_tolerances(y, ref, k, x)
+    assert rel < 2e-5, rel  # what hi+lo fp16 activations and fp32 group accumulation deliver
+    # the same weight given in the reference's signed format is the same numbers
+    w2 = K.PackedInt4Weight(b ^ 0x88, scales, g, n, k)
+    y2 = w2.matmul(torch.from_numpy(x).cuda().reshape(1, k)).cpu().numpy().ravel()
+    assert np.array_equal(y, y2)
+    # explicit zero points that are all 8 take the same path
+    zp8 = np.full((n, (k // g + 1) // 2), 0x88, np.uint8)
+    w3 = K.PackedInt4Weight(b, scales, g, n, k, zero_points=zp8, nibble_format=K.NIBBLE_UNSIGNED)
+    y3 = w3.matmul(torch.from_numpy(x).cuda().reshape(1, k)).cpu().numpy().ravel()
+    assert np.array_equal(y, y3)
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8, 11, 16])
+@pytest.mark.parametrize("xdt", ["f32", "f16", "bf16"])
+def test_skinny_all_m_and_dtypes(oracle, K, torch_cuda, m, xdt):
+    torch = torch_cuda
+    rng = np.random.default_rng(2000 + m)
+    n, k, g = 528, 1024, 32
+    b = _rand_packed(rng, n, k)
+    scales16 = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float16)
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[xdt]
+    xt = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).to(tdt)
+    x = xt.float().numpy()  # exact widening of what the kernel sees
+    ref = oracle.packed_int4_gemm_scalar(b ^ 0x88, scales16.astype(np.float32), x, m, n, k, g)
+    w = K.PackedInt4Weight(b, scales16, g, n, k, nibble_format=K.NIBBLE_UNSIGNED)
+    y = w.matmul(xt.cuda(), out_dtype=torch.float32, mode="gemv").cpu().numpy()
+    d, rel = int4_tolerances(y, ref, k, x)
+    assert rel < 2e-5, rel
+    # GEMM kernel on the same data agrees with the skinny kernel to fp32 rounding
+    y2 = w.matmul(xt.cuda(), out_dtype=torch.float32, mode="gemm").cpu().numpy()
+    int4_tolerances(y2, ref, k, x)
+    assert np.abs(y2 - y).max() <= 1e-4 * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("m", [1, 16])
+def test_skinny_long_k_grid_split(oracle, K, torch_cuda, m):
+    """K = 14336 (Llama down projection) needs the grid-level K split + fixed-order reduction."""
+    torch = torch_cuda
+    rng = np.random.default_rng(2100 + m)
+    n, k, g = 272, 14336, 32
+    b = _rand_packed(rng, n, k)
+    scales16 = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float16)
+    xt = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).half()
+    x = xt.float().numpy()
+    ref = oracle.packed_int4_gemm_scalar(b ^ 0x88, scales16.astype(np.float32), x, m, n, k, g)
+    w = K.PackedInt4Weight(b, scales16, g, n, k, nibble_format=K.NIBBLE_UNSIGNED)
+    y = w.matmul(xt.cuda(), out_dtype=torch.float32).cpu().numpy()
+    d, rel = int4_tolerances(y, ref, k, x)
+    assert rel < 5e-5, rel
+    y_again = w.matmul(xt.cuda(), out_dtype=torch.float32).cpu().numpy()
+    assert np.array_equal(y, y_again)  # no atomics: bitwise reproducible
+
+
+@pytest.mark.parametrize("g", [64, 128, 256])
+@pytest.mark.parametrize("m", [3, 40])
+def test_group_sizes_and_zero_points(oracle, K, torch_cuda, g, m):
+    """Config-3 style weights: uint4 with zero points 6..10, fp16 scales, bf16 in / bf16 out."""
+    torch = torch_cuda
+    rng = np.random.default_rng(3000 + g + m)
+    n, k = 200, 1024
+    groups = k // g
+    b = _rand_packed(rng, n, k)
+    scales16 = rng.uniform(0.005, 0.02, n * groups).astype(np.float16)
+    zq = rng.integers(6, 11, (n, groups))
+    zps = pack_zero_points(zq)
+    xt = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).bfloat16()
+    x = xt.float().numpy()
+    ref = oracle.matmul_nbits(b, scales16.astype(np.float32), zps, x, m, n, k, g)
+    w = K.PackedInt4Weight(b, scales16, g, n, k, zero_points=zps, nibble_format=K.NIBBLE_UNSIGNED)
+    y32 = w.matmul(xt.cuda(), out_dtype=torch.float32).cpu().numpy()
+    d, rel = int4_tolerances(y32, ref, k, x)
+    assert rel < 5e-5, rel
+    # bf16 output = RNE narrowing of the f32 result (crates/yscv-tensor/src/tensor.rs:764-769)
+    ybf = w.matmul(xt.cuda()).float().cpu().numpy()
+    assert np.array_equal(ybf, bf16_round(y32))
+    int4_tolerances(ybf, bf16_round(ref), k, x)
+
+
+@pytest.mark.parametrize("n,k,g", [(37, 160, 32), (1, 32, 32), (17, 96, 32), (33, 192, 64)])
+def test_ragged_shapes(oracle, K, torch_cuda, n, k, g):
+    """N not a multiple of 16, K not a multiple of 128: padding must not leak into results."""
+    torch = torch_cuda
+    rng = np.random.default_rng(n * 1000 + k)
+    b = _rand_packed(rng, n, k)
+    scales = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float32)
+    for m in (1, 7, 20):
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        ref = oracle.packed_int4_gemm_scalar(b ^ 0x88, scales, x, m, n, k, g)
+        w = K.PackedInt4Weight(b, scales, g, n, k, nibble_format=K.NIBBLE_UNSIGNED)
+        canary = torch.full((m + 1, n), 777.0, device="cuda")
+        w.matmul(torch.from_numpy(x).cuda(), out=canary[:m])
+        y = canary.cpu().numpy()
+        assert (y[m] == 777.0).all()  # nothing written past the m rows
+        d, rel = int4_tolerances(y[:m], ref, k, x)
+        assert rel < 2e-5, rel
+
+
+def test_activation_range_is_normalised(oracle, K, torch_cuda):
+    """Huge and tiny activation rows go through the power-of-two normalisation unharmed."""
+    torch = torch_cuda
+    rng = np.random.default_rng(77)
+    n, k, g = 64, 512, 32
+    b = _rand_packed(rng, n, k)
+    scales = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float32)
+    x = rng.standard_normal((4, k)).astype(np.float32)
+    x[0] *= 1e6
+    x[1] *= 1e-6
+    x[2] = 0
+    ref = oracle.packed_int4_gemm_scalar(b ^ 0x88, scales, x, 4, n, k, g)
+    w = K.PackedInt4Weight(b, scales, g, n, k, nibble_format=K.NIBBLE_UNSIGNED)
+    y = w.matmul(torch.from_numpy(x).cuda()).cpu().numpy()
+    for i in range(4):
+        if i == 2:
+            assert (y[i] == 0).all()
+        else:
+            int4_tolerances(y[i], ref[i], k, x[i])
+            assert np.abs(y[i] - ref[i]).max() <= 2e-5 * np.abs(ref[i]).max()
+
+
+def test_invalid_arguments_are_rejected(K, torch_cuda):
+    import yscv_amd
+
+    with pytest.raises(yscv_amd.YscvHipError) as ei:
+        K.PackedInt4Weight(np.zeros(8, np.uint8), np.zeros(2, np.float32), 3, 2, 6 + 2)  # odd group size
+    assert ei.value.code == -1
+    with pytest.raises(yscv_amd.YscvHipError):
+        K.PackedInt4Weight(np.zeros(10, np.uint8), np.zeros(2, np.float32), 6, 2, 10)  # g does not divide k
+    w = K.PackedInt4Weight(np.zeros(32 * 16, np.uint8), np.ones(32, np.float32), 32, 32, 32)
+    x = torch_cuda.zeros(17, 32, device="cuda")
+    with pytest.raises(yscv_amd.YscvHipError):
+        w.matmul(x, mode="gemv")  # skinny kernel is m <= 16
+
+
+def test_prefill_gemm_sampled_at_full_size(oracle, K, torch_cuda):
+    """BASELINE config 3 at full size (M=2048 K=4096 N=14336, g=128, fp16 scales, zero points 6..10,
+    bf16 in/out); the oracle is evaluated on a sample of rows and columns."""
+    torch = torch_cuda
+    rng = np.random.default_rng(3)
+    m, k, n, g = 2048, 4096, 14336, 128
+    groups = k // g
+    b = _rand_packed(rng, n, k)
+    scales16 = rng.uniform(0.005, 0.02, n * groups).astype(np.float16)
+    zq = rng.integers(6, 11, (n, groups))
+    zps = pack_zero_points(zq)
+    xt = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).bfloat16()
+    w = K.PackedInt4Weight(b, scales16, g, n, k, zero_points=zps, nibble_format=K.NIBBLE_UNSIGNED)
+    y = w.matmul(xt.cuda())
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (m, n)
+    rows = np.sort(rng.choice(m, 24, replace=False))
+    cols = np.sort(rng.choice(n, 96, replace=False))
+    xs = xt.float().numpy()[rows]
+    bs = b.reshape(n, k // 2)[cols]
+    ss = scales16.reshape(n, groups)[cols].astype(np.float32)
+    zs = pack_zero_points(zq[cols])
+    ref = oracle.matmul_nbits(bs, ss, zs, xs, len(rows), len(cols), k, g)
+    got = y.float().cpu().numpy()[np.ix_(rows, cols)]
+    int4_tolerances(got, bf16_round(ref), k, xs)
+    # bf16 output: at most one bf16 ulp away from the rounded oracle
+    assert np.abs(got - bf16_round(ref)).max() <= np.abs(ref).max() * 2.0 ** -7

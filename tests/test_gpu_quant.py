@@ -1,0 +1,81 @@
+"""GPU parity (bit-exact) of the elementwise quantisation kernels, through the C ABI."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def K():
+    import torch
+
+    assert torch.cuda.is_available()
+    from yscv_amd import kernels
+
+    return kernels
+
+
+def test_quantize_linear_goldens_and_random(oracle, K):
+    data = np.array([-1000.0, -1.5, -0.5, 0.49, 0.5, 1.5, 1000.0], np.float32)
+    out = np.zeros(7, np.int8)
+    K.quantize_linear_f32_to_i8_dispatch(data, 1.0, 0.0, out)  # quantize.rs:826-832
+    assert out.tolist() == [-128, -2, 0, 0, 0, 2, 127]
+    # quantize.rs:803-814 inputs
+    i = np.arange(257, dtype=np.float32)
+    data = (np.sin(i * np.float32(0.37)) * 40.0 + (np.arange(257) % 7) * np.float32(0.11)).astype(np.float32)
+    out = np.zeros(257, np.int8)
+    K.quantize_linear_f32_to_i8_dispatch(data, 3.25, -2.0, out)
+    assert np.array_equal(out, oracle.quantize_linear_f32_to_i8(data, 3.25, -2.0))
+    rng = np.random.default_rng(41)
+    v = np.concatenate([rng.uniform(-60, 60, 100000), [np.nan, np.inf, -np.inf, 0.0, -0.0]]).astype(np.float32)
+    for scale, zp in [(0.3, -2.0), (0.007, 5.0), (1.0, 0.5)]:
+        out = np.zeros(v.size, np.int8)
+        K.quantize_linear_f32_to_i8_dispatch(v, scale, zp, out)
+        assert np.array_equal(out, oracle.quantize_linear_f32_to_i8(v, scale, zp))
+
+
+def test_requant_goldens_and_random(oracle, K):
+    out = np.zeros(8, np.int8)
+    K.requant_i32_row_to_i8_dispatch([1, -1, 3, -3, 5, -5, 7, -7], None, 0.5, 0.0, False, out, 8)  # int8_requant.rs:1217-1226
+    assert out.tolist() == [0, 0, 2, -2, 2, -2, 4, -4]
+    acc = np.array([1_000_000] * 8 + [-1_000_000] * 8, np.int32)
+    out = np.zeros(16, np.int8)
+    K.requant_i32_row_to_i8_dispatch(acc, None, 0.001, 0.0, False, out, 16)  # :1197-1214
+    assert out.tolist() == [127] * 8 + [-128] * 8
+    out = np.ones(24, np.int8)
+    K.requant_i32_row_to_i8_dispatch(np.full(24, -100, np.int32), None, 1.0, 0.0, True, out, 8)  # :1187-1194
+    assert (out == 0).all()
+    rng = np.random.default_rng(42)
+    for c in (4, 5, 16, 17, 24, 40, 72):  # int8_requant.rs:1045-1075
+        pixels = 37
+        acc = rng.integers(-2**20, 2**20, pixels * c, dtype=np.int32)
+        acc[:3] = [2**31 - 1, -2**31, 0]
+        corr = rng.integers(-2**16, 2**16, c, dtype=np.int32)
+        comp = rng.uniform(1e-5, 1e-3, c).astype(np.float32)
+        out = np.zeros(acc.size, np.int8)
+        K.requant_i8_per_channel_dispatch(acc, corr, comp, -3.0, out, c)
+        assert np.array_equal(out, oracle.requant_i8_per_channel(acc, corr, comp, -3.0, c))
+        out2 = np.zeros(acc.size, np.int8)
+        K.requant_i32_row_to_i8_dispatch(acc, corr, 0.00037, 2.0, True, out2, c)
+        assert np.array_equal(out2, oracle.requant_i32_row_to_i8(acc, corr, 0.00037, 2.0, True, c))
+    # exact ties under both signs: composite 0.5
+    acc = np.arange(-41, 42, dtype=np.int32)
+    out = np.zeros(acc.size, np.int8)
+    K.requant_i32_row_to_i8_dispatch(acc, None, 0.5, 0.0, False, out, 1)
+    assert np.array_equal(out, oracle.requant_i32_row_to_i8(acc, None, 0.5, 0.0, False, 1))
+
+
+def test_dynamic_quantize_linear(oracle, K):
+    y, s, z = K.dynamic_quantize_linear(np.array([-2.0, -1.0, 0.0, 1.0], np.float32))  # coverage.rs:210-249
+    assert abs(s - 3.0 / 255.0) < 1e-6 and z == 170.0 and y.tolist() == [0, 85, 170, 255]
+    rng = np.random.default_rng(43)
+    cases = [rng.standard_normal(5000).astype(np.float32) * 3, np.array([2.0, 4.0], np.float32),
+             np.zeros(3, np.float32), rng.uniform(1, 2, (512, 4096)).astype(np.float32),
+             np.array([-5.0], np.float32), np.concatenate([rng.standard_normal(100), [np.nan]]).astype(np.float32)]
+    for x in cases:
+        y, s, z = K.dynamic_quantize_linear(x)
+        ye, se, ze = oracle.dynamic_quantize_linear(x)
+        assert s == se and z == ze
+        assert np.array_equal(y.astype(np.float32), ye)
+    y, s, z = K.dynamic_quantize_linear(np.zeros(0, np.float32))
+    assert y.size == 0 and s == 1.0 and z == 0.0

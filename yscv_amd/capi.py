@@ -1,0 +1,113 @@
+"""ctypes binding of include/yscv_hip.h.  Loading fails loudly when the library is missing."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+F32, F16, BF16 = 0, 1, 2
+NIBBLE_SIGNED, NIBBLE_UNSIGNED = 0, 1
+ROUND_HALF_AWAY, ROUND_TIES_EVEN = 0, 1
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "lib", "libyscv_hip.so")
+
+STATUS_NAMES = {0: "OK", -1: "INVALID_ARG", -2: "DEVICE", -3: "OOM", -4: "UNSUPPORTED", -5: "NO_DEVICE"}
+
+
+class YscvHipError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"yscv_hip status {code} ({STATUS_NAMES.get(code, '?')}): {message}")
+        self.code = code
+        self.message = message
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+_sz, _vp, _i32, _f32 = C.c_size_t, C.c_void_p, C.c_int32, C.c_float
+
+# name -> argtypes; every function returns int32 status unless listed in _SPECIAL
+_SIGNATURES = {
+    "yscv_hip_init": [_i32],
+    "yscv_hip_shutdown": [],
+    "yscv_hip_device_info": [C.c_char_p, _sz],
+    "yscv_hip_malloc": [C.POINTER(_vp), _sz],
+    "yscv_hip_free": [_vp],
+    "yscv_hip_memcpy_h2d": [_vp, _vp, _sz, _vp],
+    "yscv_hip_memcpy_d2h": [_vp, _vp, _sz, _vp],
+    "yscv_hip_stream_synchronize": [_vp],
+    "yscv_hip_int4_weight_create": [_vp, _vp, _i32, _vp, _i32, _sz, _sz, _sz, C.POINTER(_vp)],
+    "yscv_hip_int4_weight_destroy": [_vp],
+    "yscv_hip_int4_weight_dims": [_vp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)],
+    "yscv_hip_int4_matmul": [_vp, _vp, _i32, _vp, _i32, _sz, _vp],
+    "yscv_hip_int4_gemv": [_vp, _vp, _i32, _vp, _i32, _sz, _vp],
+    "yscv_hip_int4_gemm": [_vp, _vp, _i32, _vp, _i32, _sz, _vp],
+    "yscv_hip_packed_int4_gemv_dispatch": [_vp, _vp, _vp, _vp, _sz, _sz, _sz],
+    "yscv_hip_packed_int4_gemm_dispatch": [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz],
+    "yscv_hip_pack_int4_symmetric_per_group": [_vp, _sz, _sz, _sz, _vp, _vp],
+    "yscv_hip_dequantize_int4_to_f32": [_vp, _sz, _f32, C.c_int8, _vp],
+    "yscv_hip_pack_i8_b_for_matmul": [_vp, _sz, _sz, C.POINTER(_vp)],
+    "yscv_hip_i8_weight_destroy": [_vp],
+    "yscv_hip_i8_weight_dims": [_vp, C.POINTER(_sz), C.POINTER(_sz)],
+    "yscv_hip_int8_matmul": [_vp, _i32, _i32, _vp, _sz, _vp, _vp],
+    "yscv_hip_int8_matmul_requant": [_vp, _i32, _i32, _vp, _sz, _vp, _vp, _f32, _f32, _i32, _i32, _i32, _vp, _vp],
+    "yscv_hip_int8_matmul_dispatch": [_vp, _vp, _sz, _sz, _sz, _vp],
+    "yscv_hip_int8_matmul_prepacked_dispatch": [_vp, _vp, _sz, _vp],
+    "yscv_hip_quantize_linear_f32_to_i8": [_vp, _sz, _f32, _f32, _vp, _vp],
+    "yscv_hip_requant_i8_per_channel": [_vp, _sz, _vp, _vp, _f32, _vp, _sz, _vp],
+    "yscv_hip_requant_i32_row_to_i8": [_vp, _sz, _vp, _f32, _f32, _i32, _vp, _sz, _vp],
+    "yscv_hip_dynamic_quantize_linear": [_vp, _sz, _vp, _vp, _vp],
+    "yscv_hip_quantize_linear_f32_to_i8_dispatch": [_vp, _sz, _f32, _f32, _vp],
+    "yscv_hip_requant_i8_per_channel_dispatch": [_vp, _sz, _vp, _vp, _f32, _vp, _sz],
+    "yscv_hip_requant_i32_row_to_i8_dispatch": [_vp, _sz, _vp, _f32, _f32, _i32, _vp, _sz],
+    "yscv_hip_dynamic_quantize_linear_host": [_vp, _sz, _vp, C.POINTER(_f32), C.POINTER(_f32)],
+}
+_SPECIAL = {
+    "yscv_hip_abi_version": ([], C.c_uint32),
+    "yscv_hip_last_error": ([], C.c_char_p),
+}
+
+EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + list(_SPECIAL))
+
+_lib = None
+
+
+class _Checked:
+    """Wraps the CDLL so that every status-returning call raises YscvHipError on failure."""
+
+    def __init__(self, cdll: C.CDLL):
+        self._cdll = cdll
+        for name, argtypes in _SIGNATURES.items():
+            fn = getattr(cdll, name)
+            fn.argtypes = argtypes
+            fn.restype = _i32
+            setattr(self, name[len("yscv_hip_"):], self._wrap(fn))
+        for name, (argtypes, restype) in _SPECIAL.items():
+            fn = getattr(cdll, name)
+            fn.argtypes = argtypes
+            fn.restype = restype
+            setattr(self, name[len("yscv_hip_"):], fn)
+
+    def _wrap(self, fn):
+        def call(*args):
+            st = fn(*args)
+            if st != 0:
+                msg = self._cdll.yscv_hip_last_error()
+                raise YscvHipError(st, msg.decode() if msg else "")
+            return st
+
+        call.raw = fn
+        return call
+
+
+def lib() -> _Checked:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise ImportError(
+                f"{_LIB_PATH} is missing: build it with `make -C yscv_amd/csrc -j8` "
+                "(or __graft_entry__.build()); there is no fallback path"
+            )
+        _lib = _Checked(C.CDLL(_LIB_PATH))
+    return _lib

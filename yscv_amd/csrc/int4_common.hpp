@@ -1,0 +1,109 @@
+// Device-side pieces shared by the int4 kernels: the tiled weight layout, the
+// nibble -> fp16 decode and the vector types the gfx950 MFMA builtins take.
+//
+// Tiled layout of a packed-int4 weight W[n][k] (n = output row, k = input channel)
+// ---------------------------------------------------------------------------------
+// The weight is cut into tiles of 16 rows x 128 k.  Tile (nt, kt) is one contiguous
+// 1 KiB block at ((nt * KT + kt) * 1024) bytes; inside it lane L = 16*c + r of a
+// wavefront owns 16 bytes = four 32-bit words j = 0..3, and word j holds the eight
+// weights W[16*nt + r][128*kt + 32*j + 8*c + 0..7].  That is exactly the B operand of
+// v_mfma_f32_16x16x32_f16 for the k-block [128*kt + 32*j, +32): one 128-bit coalesced
+// load per lane feeds four MFMAs, and each MFMA covers one quantisation group when
+// group_size == 32.
+// Nibbles are stored unsigned (q in [0,15], value q - zp) and permuted inside the
+// word: bits [4i,4i+4) for i = 0..3 hold elements 0,2,4,6 and for i = 4..7 elements
+// 1,3,5,7, so that masking with 0x000F000F yields two consecutive k in one register.
+// Rows >= n and k >= k are padded with nibble 8 and scale 0.
+//
+// Scales (and zero points, one byte each) are re-tiled as [nt][chunk][16 rows][SPT]:
+// for group_size <= 128 a chunk is one 128-k tile holding SPT = 128/group_size
+// values per row; for larger groups a chunk is one group (SPT = 1).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/yscv_hip.h"
+
+namespace yscv {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef int int4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int uint4_t __attribute__((ext_vector_type(4)));
+typedef int int16_t_v __attribute__((ext_vector_type(16)));
+
+constexpr int kTileRows = 16;
+constexpr int kTileK = 128;
+constexpr int kTileBytes = 1024;
+
+// group mode of a tiled weight
+enum : int { GM32 = 0, GM64 = 1, GM128 = 2 };
+
+__host__ __device__ inline int scales_per_chunk(int gm) { return gm == GM32 ? 4 : (gm == GM64 ? 2 : 1); }
+
+union U32H2 {
+  uint32_t u;
+  half2_t h;
+};
+
+// Decode one tiled word (8 weights) to fp16 (q - zp), in k order.
+// c1 = -(1024 + zp), c2 = -(64 + zp), both splat.  Every step is exact in fp16:
+// 0x6400 | q is 1024 + q, 0x6400 | (q << 4) is 1024 + 16 q.
+__device__ __forceinline__ half8_t decode8(uint32_t s, half2_t c1, half2_t c2) {
+  const uint32_t magic = 0x64006400u;
+  U32H2 r0, r1, r2, r3;
+  r0.u = (s & 0x000F000Fu) | magic;
+  r1.u = (s & 0x00F000F0u) | magic;
+  uint32_t s2 = s >> 8;
+  r2.u = (s2 & 0x000F000Fu) | magic;
+  r3.u = (s2 & 0x00F000F0u) | magic;
+  const half2_t sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+  half2_t h0 = r0.h + c1;
+  half2_t h1 = r1.h * sixteenth + c2;
+  half2_t h2 = r2.h + c1;
+  half2_t h3 = r3.h * sixteenth + c2;
+  half8_t out;
+  out[0] = h0[0];
+  out[1] = h0[1];
+  out[2] = h1[0];
+  out[3] = h1[1];
+  out[4] = h2[0];
+  out[5] = h2[1];
+  out[6] = h3[0];
+  out[7] = h3[1];
+  return out;
+}
+
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t b) {
+  return __uint_as_float(((uint32_t)b) << 16);
+}
+// round to nearest even, the rule of the reference's f32 -> bf16 narrowing
+// (crates/yscv-tensor/src/tensor.rs:764-769)
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  uint32_t bits = __float_as_uint(f);
+  uint32_t bias = 0x7FFFu + ((bits >> 16) & 1u);
+  return (uint16_t)((bits + bias) >> 16);
+}
+
+// store one result element as f32 / f16 / bf16
+__device__ __forceinline__ void store_out(void *y, size_t idx, float v, int dtype) {
+  if (dtype == YSCV_HIP_F32) {
+    reinterpret_cast<float *>(y)[idx] = v;
+  } else if (dtype == YSCV_HIP_F16) {
+    reinterpret_cast<_Float16 *>(y)[idx] = (_Float16)v;
+  } else {
+    reinterpret_cast<uint16_t *>(y)[idx] = float_to_bf16_bits(v);
+  }
+}
+
+__device__ __forceinline__ float load_in(const void *x, size_t idx, int dtype) {
+  if (dtype == YSCV_HIP_F32) return reinterpret_cast<const float *>(x)[idx];
+  if (dtype == YSCV_HIP_F16) return (float)reinterpret_cast<const _Float16 *>(x)[idx];
+  return bf16_bits_to_float(reinterpret_cast<const uint16_t *>(x)[idx]);
+}
+
+}  // namespace yscv

@@ -1,0 +1,250 @@
+// Load-time and per-call layout kernels of the int4 path: weight re-tiling, scale /
+// zero-point re-tiling, activation preparation, and the GPU forms of
+// pack_int4_symmetric_per_group and dequantize_int4_to_f32.
+#include "int4_common.hpp"
+#include "kernels.hpp"
+
+namespace yscv {
+
+// ---- weight re-tiling ----------------------------------------------------------------
+// One thread per output word.  Source: caller's [n][k/2] bytes (element 2i in the low
+// nibble, int4_matmul.rs:12-14).  See int4_common.hpp for the destination layout.
+__global__ void int4_retile_kernel(const uint8_t *__restrict__ raw, int is_signed, size_t n, size_t k,
+                                   size_t nt_count, size_t kt_count, uint32_t *__restrict__ tiles) {
+  size_t total = nt_count * kt_count * 256;  // words
+  for (size_t w = blockIdx.x * (size_t)blockDim.x + threadIdx.x; w < total;
+       w += (size_t)gridDim.x * blockDim.x) {
+    size_t j = w & 3;
+    size_t lane = (w >> 2) & 63;
+    size_t tile = w >> 8;
+    size_t kt = tile % kt_count, nt = tile / kt_count;
+    size_t r = lane & 15, c = lane >> 4;
+    size_t row = nt * 16 + r;
+    size_t k0 = kt * 128 + j * 32 + c * 8;
+    uint32_t e[8];
+    for (int i = 0; i < 8; i++) {
+      size_t kk = k0 + i;
+      uint32_t q = 8;  // padding: value 0 under the implicit zero point 8
+      if (row < n && kk < k) {
+        uint8_t byte = raw[row * (k / 2) + kk / 2];
+        q = (kk & 1) ? (byte >> 4) : (byte & 15);
+        if (is_signed) q ^= 8;  // two's complement nibble s -> s + 8
+      }
+      e[i] = q;
+    }
+    uint32_t word = e[0] | (e[2] << 4) | (e[4] << 8) | (e[6] << 12) | (e[1] << 16) | (e[3] << 20) |
+                    (e[5] << 24) | (e[7] << 28);
+    tiles[w] = word;
+  }
+}
+
+int32_t launch_int4_retile(const uint8_t *raw_in, int nibble_format, size_t n, size_t k, size_t nt,
+                           size_t kt, uint8_t *tiles, hipStream_t s) {
+  size_t total = nt * kt * 256;
+  int blocks = (int)((total + 255) / 256 < 65535 * 4 ? (total + 255) / 256 : 65535 * 4);
+  hipLaunchKernelGGL(int4_retile_kernel, dim3(blocks), dim3(256), 0, s, raw_in,
+                     nibble_format == YSCV_HIP_NIBBLE_SIGNED ? 1 : 0, n, k, nt, kt,
+                     reinterpret_cast<uint32_t *>(tiles));
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+template <typename T>
+__global__ void int4_retile_scales_kernel(const T *__restrict__ scales, const uint8_t *__restrict__ zps,
+                                          size_t n, size_t groups, size_t g, int spt, size_t nt_count,
+                                          size_t chunks, T *__restrict__ tscales,
+                                          uint8_t *__restrict__ tzps) {
+  size_t total = nt_count * chunks * 16 * (size_t)spt;
+  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * blockDim.x) {
+    size_t sj = idx % spt;
+    size_t r = (idx / spt) % 16;
+    size_t ch = (idx / spt / 16) % chunks;
+    size_t nt = idx / spt / 16 / chunks;
+    size_t row = nt * 16 + r;
+    size_t grp = ch * spt + sj;  // spt > 1: chunk = 128-k tile; spt == 1: chunk = group
+    T sv = (T)0;
+    uint8_t zv = 8;
+    if (row < n && grp < groups) {
+      sv = scales[row * groups + grp];
+      if (zps) zv = zps[row * groups + grp];
+    }
+    tscales[idx] = sv;
+    if (tzps) tzps[idx] = zv;
+  }
+  (void)g;
+}
+
+int32_t launch_int4_retile_scales(const void *scales_in, int scale_dtype, const uint8_t *zps_in,
+                                  size_t n, size_t k, size_t g, int gm, size_t nt, size_t chunks,
+                                  void *tscales, uint8_t *tzps, hipStream_t s) {
+  int spt = scales_per_chunk(gm);
+  size_t groups = k / g;
+  size_t total = nt * chunks * 16 * (size_t)spt;
+  int blocks = (int)((total + 255) / 256 < 262140 ? (total + 255) / 256 : 262140);
+  if (blocks < 1) blocks = 1;
+  if (scale_dtype == YSCV_HIP_F32) {
+    hipLaunchKernelGGL(int4_retile_scales_kernel<float>, dim3(blocks), dim3(256), 0, s,
+                       static_cast<const float *>(scales_in), zps_in, n, groups, g, spt, nt, chunks,
+                       static_cast<float *>(tscales), tzps);
+  } else {
+    hipLaunchKernelGGL(int4_retile_scales_kernel<_Float16>, dim3(blocks), dim3(256), 0, s,
+                       static_cast<const _Float16 *>(scales_in), zps_in, n, groups, g, spt, nt,
+                       chunks, static_cast<_Float16 *>(tscales), tzps);
+  }
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+__global__ void unpack_zps_kernel(const uint8_t *__restrict__ packed, size_t n, size_t groups,
+                                  uint8_t *__restrict__ out) {
+  size_t row_bytes = (groups + 1) / 2;
+  size_t total = n * groups;
+  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * blockDim.x) {
+    size_t row = idx / groups, grp = idx % groups;
+    uint8_t b = packed[row * row_bytes + grp / 2];
+    out[idx] = (grp & 1) ? (b >> 4) : (b & 15);
+  }
+}
+
+int32_t launch_unpack_zps(const uint8_t *zps_packed, size_t n, size_t groups, uint8_t *out,
+                          hipStream_t s) {
+  size_t total = n * groups;
+  int blocks = (int)((total + 255) / 256 < 262140 ? (total + 255) / 256 : 262140);
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(unpack_zps_kernel, dim3(blocks), dim3(256), 0, s, zps_packed, n, groups, out);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+__global__ void xor88_kernel(uint8_t *buf, size_t bytes) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < bytes;
+       i += (size_t)gridDim.x * blockDim.x)
+    buf[i] ^= 0x88;
+}
+int32_t launch_xor88(uint8_t *buf, size_t bytes, hipStream_t s) {
+  int blocks = (int)((bytes + 255) / 256 < 262140 ? (bytes + 255) / 256 : 262140);
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(xor88_kernel, dim3(blocks), dim3(256), 0, s, buf, bytes);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+// ---- activation preparation -------------------------------------------------------------
+// One workgroup per activation row.  The row is divided by a power of two so that its
+// largest magnitude lands in [2^14, 2^15) -- the top of the fp16 range -- then written as
+// fp16 `hi` and, for f32 input, a second fp16 `lo` = x' - hi.  hi + lo carries ~22
+// significant bits, f16/bf16 inputs are represented exactly by hi alone.  The power of
+// two is returned so the GEMV/GEMM epilogue can multiply it back (exactly).
+__global__ void __launch_bounds__(256) x_prep_kernel(const void *__restrict__ x, int x_dtype, size_t k,
+                                                     size_t k_pad, int split, _Float16 *__restrict__ xh,
+                                                     _Float16 *__restrict__ xl,
+                                                     float *__restrict__ row_scale) {
+  __shared__ float red[4];
+  size_t row = blockIdx.x;
+  size_t base = row * k;
+  float amax = 0.0f;
+  for (size_t i = threadIdx.x; i < k; i += blockDim.x) {
+    float v = fabsf(load_in(x, base + i, x_dtype));
+    amax = fmaxf(amax, v);  // NaN is ignored here; it still propagates through the values
+  }
+  for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  int e = 0;
+  if (amax > 0.0f && amax < 3.0e38f) {
+    (void)frexpf(amax, &e);  // amax = f * 2^e, f in [0.5, 1)
+    e -= 1;                  // amax in [2^e, 2^(e+1))
+  } else {
+    e = 14;  // all-zero or non-finite row: leave the values alone
+  }
+  int shift = 14 - e;
+  shift = shift > 100 ? 100 : (shift < -100 ? -100 : shift);
+  float up = ldexpf(1.0f, shift);
+  if (threadIdx.x == 0) row_scale[row] = ldexpf(1.0f, -shift);
+  size_t obase = row * k_pad;
+  for (size_t i = threadIdx.x; i < k_pad; i += blockDim.x) {
+    float v = (i < k) ? load_in(x, base + i, x_dtype) * up : 0.0f;
+    _Float16 h = (_Float16)v;
+    xh[obase + i] = h;
+    if (split == 2) xl[obase + i] = (_Float16)(v - (float)h);
+  }
+}
+
+int32_t launch_x_prep(const void *x, int x_dtype, size_t m, size_t k, size_t k_pad, int split,
+                      _Float16 *xh, _Float16 *xl, float *row_scale, hipStream_t s) {
+  hipLaunchKernelGGL(x_prep_kernel, dim3((unsigned)m), dim3(256), 0, s, x, x_dtype, k, k_pad, split,
+                     xh, xl, row_scale);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+// ---- pack_int4_symmetric_per_group (int4_matmul.rs:611-646) ---------------------------------
+// One wavefront per (row, group): abs-max, scale = absmax / 7 (1.0 when absmax <= EPSILON),
+// q = clamp(round_ties_even(w * (1/scale)), -8, 7), low nibble = even element.
+__global__ void __launch_bounds__(256) pack_int4_kernel(const float *__restrict__ w, size_t rows,
+                                                        size_t k, size_t g, uint8_t *__restrict__ packed,
+                                                        float *__restrict__ scales) {
+  size_t groups = k / g;
+  size_t wave = (blockIdx.x * (size_t)blockDim.x + threadIdx.x) >> 6;
+  int lane = threadIdx.x & 63;
+  size_t total = rows * groups;
+  size_t nwaves = ((size_t)gridDim.x * blockDim.x) >> 6;
+  for (size_t item = wave; item < total; item += nwaves) {
+    size_t row = item / groups, grp = item % groups;
+    const float *src = w + row * k + grp * g;
+    float amax = 0.0f;
+    for (size_t i = lane; i < g; i += 64) amax = fmaxf(amax, fabsf(src[i]));
+    for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    float scale = (amax <= 1.1920929e-7f) ? 1.0f : __fdiv_rn(amax, 7.0f);
+    float inv = __fdiv_rn(1.0f, scale);
+    if (lane == 0) scales[item] = scale;
+    for (size_t b = lane; b < g / 2; b += 64) {
+      float v0 = rintf(__fmul_rn(src[2 * b], inv));
+      float v1 = rintf(__fmul_rn(src[2 * b + 1], inv));
+      // clamp keeps NaN and `as i8` maps it to 0 (Rust semantics)
+      int q0 = (v0 != v0) ? 0 : (int)fminf(fmaxf(v0, -8.0f), 7.0f);
+      int q1 = (v1 != v1) ? 0 : (int)fminf(fmaxf(v1, -8.0f), 7.0f);
+      packed[row * (k / 2) + grp * (g / 2) + b] = (uint8_t)((q0 & 15) | ((q1 & 15) << 4));
+    }
+  }
+}
+
+int32_t launch_pack_int4_symmetric(const float *w, size_t m_w, size_t k, size_t g, uint8_t *packed,
+                                   float *scales, hipStream_t s) {
+  size_t items = m_w * (k / g);
+  size_t blocks = (items + 3) / 4;
+  if (blocks > 65535 * 8) blocks = 65535 * 8;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(pack_int4_kernel, dim3((unsigned)blocks), dim3(256), 0, s, w, m_w, k, g, packed,
+                     scales);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+// ---- dequantize_int4_to_f32 (ops/quantize.rs:215-222) ----------------------------------------
+__global__ void dequant_int4_kernel(const uint8_t *__restrict__ packed, size_t n_bytes, float scale,
+                                    float zp, float *__restrict__ out) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n_bytes;
+       i += (size_t)gridDim.x * blockDim.x) {
+    int b = packed[i];
+    int lo = ((b & 15) ^ 8) - 8, hi = ((b >> 4) ^ 8) - 8;
+    out[2 * i] = __fmul_rn(__fsub_rn((float)lo, zp), scale);
+    out[2 * i + 1] = __fmul_rn(__fsub_rn((float)hi, zp), scale);
+  }
+}
+
+int32_t launch_dequantize_int4(const uint8_t *packed, size_t n_bytes, float scale, int zp, float *out,
+                               hipStream_t s) {
+  size_t blocks = (n_bytes + 255) / 256;
+  if (blocks > 262140) blocks = 262140;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(dequant_int4_kernel, dim3((unsigned)blocks), dim3(256), 0, s, packed, n_bytes,
+                     scale, (float)zp, out);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+}  // namespace yscv

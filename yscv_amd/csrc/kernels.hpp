@@ -1,0 +1,102 @@
+// Internal interface between the C ABI (api.hip) and the kernel files.
+#pragma once
+
+#include "common.hpp"
+
+// Device-resident packed-int4 weight (see int4_common.hpp for the tiled layout).
+struct yscv_hip_int4_weight {
+  size_t n = 0, k = 0, g = 0;
+  int scale_dtype = YSCV_HIP_F32;  // storage type of the scales on the device
+  bool has_zp = false;             // false: every zero point is 8
+  bool tiled = false;              // fast layout built (g in {32,64} or g % 128 == 0)
+  int gm = 0;                      // group mode of the tiled layout
+  size_t nt = 0, kt = 0;           // tile counts: ceil(n/16), ceil(k/128)
+  size_t chunks = 0;               // scale chunks per n-tile
+  uint8_t *tiles = nullptr;        // [nt][kt][1 KiB]
+  void *tscales = nullptr;         // [nt][chunks][16][spt]
+  uint8_t *tzps = nullptr;         // same shape, one byte each; null when !has_zp
+  // generic layout, kept only when the tiled one cannot be built
+  uint8_t *raw = nullptr;    // [n][k/2], unsigned nibbles, natural order
+  void *rscales = nullptr;   // [n][k/g]
+  uint8_t *rzps = nullptr;   // [n][k/g] bytes; null when !has_zp
+  size_t device_bytes = 0;
+};
+
+// Device-resident int8 B matrix: transposed [n][k] fragments for the MFMA kernel + column sums.
+struct yscv_hip_i8_weight {
+  size_t k = 0, n = 0;
+  size_t kp = 0, np = 0;        // padded extents (k to 64, n to 16)
+  int8_t *frag = nullptr;       // [np/16][kp/64][64 lanes][16 B]
+  int32_t *col_sum = nullptr;   // [np], sum over k of b[k][j]
+  size_t device_bytes = 0;
+};
+
+namespace yscv {
+
+// ---- int4 ------------------------------------------------------------------------
+// raw_in: device copy of the caller's [n][k/2] bytes in its own nibble format.
+int32_t launch_int4_retile(const uint8_t *raw_in, int nibble_format, size_t n, size_t k,
+                           size_t nt, size_t kt, uint8_t *tiles, hipStream_t s);
+// scales_in [n][k/g] (f32 or f16) -> [nt][chunks][16][spt], same element type; zps likewise from
+// one byte per group.  Padded entries get scale 0 / zp 8.
+int32_t launch_int4_retile_scales(const void *scales_in, int scale_dtype, const uint8_t *zps_in,
+                                  size_t n, size_t k, size_t g, int gm, size_t nt, size_t chunks,
+                                  void *tscales, uint8_t *tzps, hipStream_t s);
+// unpack packed uint4 zero points [n][ceil(G/2)] -> one byte per group [n][G]
+int32_t launch_unpack_zps(const uint8_t *zps_packed, size_t n, size_t groups, uint8_t *out,
+                          hipStream_t s);
+// signed nibbles -> unsigned (byte ^ 0x88), natural order (generic layout)
+int32_t launch_xor88(uint8_t *buf, size_t bytes, hipStream_t s);
+
+// x [m][k] (f32/f16/bf16) -> fp16 hi (and lo when split == 2) [m][k_pad], plus the
+// power-of-two factor each row was divided by.
+int32_t launch_x_prep(const void *x, int x_dtype, size_t m, size_t k, size_t k_pad, int split,
+                      _Float16 *xh, _Float16 *xl, float *row_scale, hipStream_t s);
+
+struct SkinnyPlan {
+  int tpw;     // 128-k tiles per wave
+  int waves;   // wavefronts per workgroup (= k-slices per workgroup)
+  int ksg;     // grid-level k split (partials reduced by a second kernel when > 1)
+  int grid_x;  // workgroups along n
+  size_t partial_bytes;
+};
+SkinnyPlan plan_int4_skinny(const yscv_hip_int4_weight *w, size_t m, int split, int num_cus);
+int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan, const _Float16 *xh,
+                           const _Float16 *xl, const float *row_scale, size_t k_pad, int split,
+                           void *y, int y_dtype, size_t m, float *partial, hipStream_t s);
+int32_t launch_int4_generic(const yscv_hip_int4_weight *w, const void *x, int x_dtype, void *y,
+                            int y_dtype, size_t m, hipStream_t s);
+int32_t launch_int4_gemm(const yscv_hip_int4_weight *w, const _Float16 *xh, const _Float16 *xl,
+                         const float *row_scale, size_t k_pad, int split, void *y, int y_dtype,
+                         size_t m, hipStream_t s);
+
+int32_t launch_pack_int4_symmetric(const float *w, size_t m_w, size_t k, size_t g, uint8_t *packed,
+                                   float *scales, hipStream_t s);
+int32_t launch_dequantize_int4(const uint8_t *packed, size_t n_bytes, float scale, int zp,
+                               float *out, hipStream_t s);
+
+// ---- int8 --------------------------------------------------------------------------
+int32_t launch_i8_pack_b(const int8_t *b_kn, size_t k, size_t n, size_t kp, size_t np,
+                         int8_t *frag, int32_t *col_sum, hipStream_t s);
+struct I8Epilogue {
+  int mode;  // 0: int32 out, 1: requantize to bytes
+  const int32_t *corr;
+  const float *composite_v;
+  float composite;
+  float y_zp;
+  int round_mode;
+  int lo, hi;
+};
+int32_t launch_i8_gemm(const void *a, int a_is_u8, int a_zp, const yscv_hip_i8_weight *b, size_t m,
+                       void *out, const I8Epilogue &ep, hipStream_t s);
+
+// ---- elementwise ---------------------------------------------------------------------
+int32_t launch_quantize_linear_i8(const float *x, size_t len, float scale, float zp, int8_t *out,
+                                  hipStream_t s);
+int32_t launch_requant(const int32_t *acc, size_t len, size_t c, const int32_t *corr,
+                       const float *composite_v, float composite, float y_zp, int round_mode,
+                       int lo, int hi, int relu, void *out, hipStream_t s);
+int32_t launch_dynamic_quantize_linear(const float *x, size_t len, uint8_t *y, float *scale_zp,
+                                       hipStream_t s);
+
+}  // namespace yscv

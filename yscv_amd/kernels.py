@@ -1,0 +1,257 @@
+"""Host-side mirror of the yscv-kernels entry points for this path, over the C ABI.
+
+Names and argument order follow crates/yscv-kernels/src/core.rs:173-186.  The host-slice
+functions take numpy arrays (the Rust ``&[T]`` / ``&mut [T]`` slices); the handle classes own
+device memory and take torch CUDA tensors, which are used only as device buffers -- every
+computation happens inside libyscv_hip.so.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import capi
+from .capi import BF16, F16, F32, NIBBLE_SIGNED, NIBBLE_UNSIGNED, ROUND_HALF_AWAY, ROUND_TIES_EVEN, lib
+
+_sz = C.c_size_t
+
+
+def _np(a, dtype) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def _ptr(a: np.ndarray):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _torch_dtype_code(t) -> int:
+    import torch
+
+    return {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}[t.dtype]
+
+
+def _stream_ptr():
+    import torch
+
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+# ---- host-slice entry points (exact Rust argument lists) ---------------------------------
+
+def packed_int4_gemv_dispatch(weight_packed, scales, activation, output, m_w, k, group_size) -> None:
+    """int4_matmul.rs:310 -- output[m_w] = W[m_w][k] . activation[k]."""
+    w, s, x = _np(weight_packed, np.uint8), _np(scales, np.float32), _np(activation, np.float32)
+    assert isinstance(output, np.ndarray) and output.dtype == np.float32 and output.flags.c_contiguous
+    if w.size != m_w * k // 2 or s.size != m_w * (k // max(group_size, 1)) or x.size != k or output.size != m_w:
+        raise ValueError("slice lengths do not match m_w, k, group_size")
+    lib().packed_int4_gemv_dispatch(_ptr(w), _ptr(s), _ptr(x), _ptr(output), _sz(m_w), _sz(k), _sz(group_size))
+
+
+def packed_int4_gemm_dispatch(weight_packed, scales, activation, output, m, n, k, group_size) -> None:
+    """int4_matmul.rs:548 -- output[m][n] = activation[m][k] . W[n][k]^T."""
+    w, s, x = _np(weight_packed, np.uint8), _np(scales, np.float32), _np(activation, np.float32)
+    assert isinstance(output, np.ndarray) and output.dtype == np.float32 and output.flags.c_contiguous
+    if w.size != n * k // 2 or s.size != n * (k // max(group_size, 1)) or x.size != m * k or output.size != m * n:
+        raise ValueError("slice lengths do not match m, n, k, group_size")
+    lib().packed_int4_gemm_dispatch(_ptr(w), _ptr(s), _ptr(x), _ptr(output), _sz(m), _sz(n), _sz(k), _sz(group_size))
+
+
+def pack_int4_symmetric_per_group(weights, m_w, k, group_size):
+    """int4_matmul.rs:611 -- returns (packed u8[m_w*k/2], scales f32[m_w*k/group_size])."""
+    w = _np(weights, np.float32)
+    if w.size != m_w * k:
+        raise ValueError("weights length != m_w * k")
+    packed = np.empty(m_w * k // 2, np.uint8)
+    scales = np.empty(m_w * (k // group_size), np.float32)
+    lib().pack_int4_symmetric_per_group(_ptr(w), _sz(m_w), _sz(k), _sz(group_size), _ptr(packed), _ptr(scales))
+    return packed, scales
+
+
+def dequantize_int4_to_f32(packed, scale, zero_point, output) -> None:
+    """ops/quantize.rs:18."""
+    p = _np(packed, np.uint8)
+    assert output.dtype == np.float32 and output.size >= 2 * p.size
+    lib().dequantize_int4_to_f32(_ptr(p), _sz(p.size), C.c_float(scale), C.c_int8(zero_point), _ptr(output))
+
+
+def int8_matmul_dispatch(a, b, m, k, n, out) -> None:
+    """int8_matmul.rs:2407 -- b is row-major [k][n]."""
+    aa, bb = _np(a, np.int8), _np(b, np.int8)
+    assert out.dtype == np.int32 and out.flags.c_contiguous
+    if aa.size != m * k or bb.size != k * n or out.size != m * n:
+        raise ValueError("slice lengths do not match m, k, n")
+    lib().int8_matmul_dispatch(_ptr(aa), _ptr(bb), _sz(m), _sz(k), _sz(n), _ptr(out))
+
+
+def quantize_linear_f32_to_i8_dispatch(data, scale, zero_point, output) -> None:
+    """ops/quantize.rs:154."""
+    d = _np(data, np.float32)
+    assert output.dtype == np.int8 and output.size == d.size
+    lib().quantize_linear_f32_to_i8_dispatch(_ptr(d), _sz(d.size), C.c_float(scale), C.c_float(zero_point), _ptr(output))
+
+
+def requant_i8_per_channel_dispatch(acc, corr, composite, y_zp, out, c) -> None:
+    """ops/int8_requant.rs:401."""
+    a, co, cp = _np(acc, np.int32), _np(corr, np.int32), _np(composite, np.float32)
+    assert out.dtype == np.int8 and out.size == a.size
+    lib().requant_i8_per_channel_dispatch(_ptr(a), _sz(a.size), _ptr(co), _ptr(cp), C.c_float(y_zp), _ptr(out), _sz(c))
+
+
+def requant_i32_row_to_i8_dispatch(acc, bias, composite, y_zp, relu, out, c) -> None:
+    """ops/int8_requant.rs:81 -- bias may be None."""
+    a = _np(acc, np.int32)
+    b = None if bias is None else _np(bias, np.int32)
+    assert out.dtype == np.int8 and out.size == a.size
+    lib().requant_i32_row_to_i8_dispatch(_ptr(a), _sz(a.size), _ptr(b) if b is not None else None,
+                                         C.c_float(composite), C.c_float(y_zp), C.c_int32(int(bool(relu))), _ptr(out), _sz(c))
+
+
+def dynamic_quantize_linear(x):
+    """runner/misc.rs:241 -- returns (y uint8, scale f32, zero_point f32)."""
+    d = _np(x, np.float32)
+    y = np.empty(d.shape, np.uint8)
+    s, z = C.c_float(), C.c_float()
+    lib().dynamic_quantize_linear_host(_ptr(d), _sz(d.size), _ptr(y), C.byref(s), C.byref(z))
+    return y, np.float32(s.value), np.float32(z.value)
+
+
+# ---- device handles ---------------------------------------------------------------------------
+
+class PackedInt4Weight:
+    """Device-resident PackedInt4Weight (quantize/packed_int4.rs:29-39): packed nibbles + scales
+    (+ optional uint4 zero points for the MatMulNBits form), re-tiled for the MFMA kernels."""
+
+    def __init__(self, packed, scales, group_size, m_w, k, zero_points=None, nibble_format=NIBBLE_SIGNED):
+        p = _np(packed, np.uint8)
+        s = np.ascontiguousarray(scales)
+        if s.dtype == np.float32:
+            sd = F32
+        elif s.dtype == np.float16:
+            sd = F16
+        else:
+            raise TypeError("scales must be float32 or float16")
+        zp = None if zero_points is None else _np(zero_points, np.uint8)
+        if group_size <= 0 or p.size != m_w * k // 2 or s.size != m_w * (k // group_size):
+            raise ValueError("slice lengths do not match m_w, k, group_size")
+        h = C.c_void_p()
+        lib().int4_weight_create(_ptr(p), _ptr(s), sd, _ptr(zp) if zp is not None else None, nibble_format,
+                                 _sz(m_w), _sz(k), _sz(group_size), C.byref(h))
+        self._h = h
+        self.m_w, self.k, self.group_size = m_w, k, group_size
+
+    @property
+    def handle(self):
+        return self._h
+
+    def device_bytes(self) -> int:
+        n, k, g, b = _sz(), _sz(), _sz(), _sz()
+        lib().int4_weight_dims(self._h, C.byref(n), C.byref(k), C.byref(g), C.byref(b))
+        return b.value
+
+    def matmul(self, x, out=None, out_dtype=None, mode: str = "auto"):
+        """x: CUDA tensor [..., k] (f32/f16/bf16).  mode: auto | gemv | gemm.  Output shape is
+        x.shape[:-1] + [m_w], like exec_matmul's int4 branch (runner/linear.rs:269-270)."""
+        import torch
+
+        assert x.is_cuda and x.shape[-1] == self.k
+        x = x.contiguous()
+        m = x.numel() // self.k
+        odt = out_dtype or x.dtype
+        if out is None:
+            out = torch.empty(*x.shape[:-1], self.m_w, device=x.device, dtype=odt)
+        fn = {"auto": lib().int4_matmul, "gemv": lib().int4_gemv, "gemm": lib().int4_gemm}[mode]
+        fn(self._h, C.c_void_p(x.data_ptr()), _torch_dtype_code(x), C.c_void_p(out.data_ptr()),
+           _torch_dtype_code(out), _sz(m), _stream_ptr())
+        return out
+
+    def close(self):
+        if self._h:
+            lib().int4_weight_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class PackedI8B:
+    """Device-resident PackedI8B (int8_matmul.rs:128-160)."""
+
+    def __init__(self, b, k, n):
+        bb = _np(b, np.int8)
+        if bb.size != k * n:
+            raise ValueError("b length != k * n")
+        h = C.c_void_p()
+        lib().pack_i8_b_for_matmul(_ptr(bb), _sz(k), _sz(n), C.byref(h))
+        self._h = h
+        self._k, self._n = k, n
+
+    def k(self) -> int:
+        return self._k
+
+    def n(self) -> int:
+        return self._n
+
+    @property
+    def handle(self):
+        return self._h
+
+    def matmul_host(self, a, m, out) -> None:
+        """int8_matmul_prepacked_dispatch (int8_matmul.rs:2420), host slices."""
+        aa = _np(a, np.int8)
+        assert out.dtype == np.int32 and out.size == m * self._n and aa.size == m * self._k
+        lib().int8_matmul_prepacked_dispatch(_ptr(aa), self._h, _sz(m), _ptr(out))
+
+    def matmul(self, a, a_zp: int = 0, out=None):
+        """a: CUDA tensor [m][k] int8 or uint8 -> int32 [m][n] (exact)."""
+        import torch
+
+        assert a.is_cuda and a.dim() == 2 and a.shape[1] == self._k and a.dtype in (torch.int8, torch.uint8)
+        a = a.contiguous()
+        m = a.shape[0]
+        if out is None:
+            out = torch.empty(m, self._n, device=a.device, dtype=torch.int32)
+        lib().int8_matmul(C.c_void_p(a.data_ptr()), int(a.dtype == torch.uint8), int(a_zp), self._h, _sz(m),
+                          C.c_void_p(out.data_ptr()), _stream_ptr())
+        return out
+
+    def matmul_requant(self, a, a_zp, composite, y_zp, round_mode, clamp_lo, clamp_hi, corr=None, out=None):
+        """Fused GEMM + requantize.  composite: float or CUDA f32 tensor [n]; corr: CUDA i32 [n] or None."""
+        import torch
+
+        assert a.is_cuda and a.dim() == 2 and a.shape[1] == self._k and a.dtype in (torch.int8, torch.uint8)
+        a = a.contiguous()
+        m = a.shape[0]
+        if out is None:
+            out = torch.empty(m, self._n, device=a.device, dtype=torch.int8 if clamp_lo < 0 else torch.uint8)
+        comp_v, comp_s = (None, float(composite)) if not hasattr(composite, "data_ptr") else (composite, 0.0)
+        lib().int8_matmul_requant(C.c_void_p(a.data_ptr()), int(a.dtype == torch.uint8), int(a_zp), self._h, _sz(m),
+                                  C.c_void_p(corr.data_ptr()) if corr is not None else None,
+                                  C.c_void_p(comp_v.data_ptr()) if comp_v is not None else None,
+                                  C.c_float(comp_s), C.c_float(y_zp), int(round_mode), int(clamp_lo), int(clamp_hi),
+                                  C.c_void_p(out.data_ptr()), _stream_ptr())
+        return out
+
+    def close(self):
+        if self._h:
+            lib().i8_weight_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def pack_i8_b_for_matmul(b, k, n) -> PackedI8B:
+    """int8_matmul.rs:163."""
+    return PackedI8B(b, k, n)
+
+
+def int8_matmul_prepacked_dispatch(a, b: PackedI8B, m, out) -> None:
+    """int8_matmul.rs:2420."""
+    b.matmul_host(a, m, out)
