@@ -113,6 +113,17 @@ int32_t yscv_hip_int4_gemv(const yscv_hip_int4_weight *w, const void *x_dev, int
 int32_t yscv_hip_int4_gemm(const yscv_hip_int4_weight *w, const void *x_dev, int32_t x_dtype,
                            void *y_dev, int32_t y_dtype, size_t m, void *stream);
 
+/* Same as yscv_hip_int4_matmul, but every byte of device scratch comes from the caller, so
+ * the call allocates nothing (the reference allocates its output per call,
+ * linear.rs:237; there is no scratch to compare with).  workspace_dev must be 256-byte
+ * aligned and at least yscv_hip_int4_workspace_bytes(w, m, x_dtype) long (0 for fp16
+ * activations whose K is a multiple of 128 and fits one workgroup's K range). */
+int32_t yscv_hip_int4_workspace_bytes(const yscv_hip_int4_weight *w, size_t m, int32_t x_dtype,
+                                      size_t *bytes);
+int32_t yscv_hip_int4_matmul_ws(const yscv_hip_int4_weight *w, const void *x_dev, int32_t x_dtype,
+                                void *y_dev, int32_t y_dtype, size_t m, void *workspace_dev,
+                                size_t workspace_bytes, void *stream);
+
 /* Exact argument lists of the Rust functions (host slices -> host pointers):
  * packed_int4_gemv_dispatch  int4_matmul.rs:310-318
  * packed_int4_gemm_dispatch  int4_matmul.rs:548-557
@@ -204,6 +215,81 @@ int32_t yscv_hip_requant_i32_row_to_i8_dispatch(const int32_t *acc, size_t len,
                                                 int32_t relu, int8_t *out, size_t c);
 int32_t yscv_hip_dynamic_quantize_linear_host(const float *x, size_t len, uint8_t *y,
                                               float *scale, float *zero_point);
+
+/* ---- decode loop (Llama-style decoder, int4 projections, fp16 KV cache) ----------------- */
+
+/* GPU-resident counterpart of the llm-bench decode loop (apps/llm-bench/src/main.rs:403-561:
+ * feed the last token and the KV cache, greedy pick, repeat), of KvCache
+ * (crates/yscv-onnx/src/runner/kv_cache.rs:14-254) and of greedy generate()
+ * (crates/yscv-onnx/src/generate.rs:58-208, top_k = 1).  Every linear layer goes through the
+ * skinny int4 kernel; q/k/v and gate/up are fused into one weight each at finalize time. */
+typedef struct yscv_hip_decoder yscv_hip_decoder;
+
+typedef struct yscv_hip_decoder_config {
+  int32_t n_layers;
+  int32_t d_model;
+  int32_t n_heads;    /* query heads */
+  int32_t n_kv_heads; /* n_heads / n_kv_heads must be 1..4 */
+  int32_t head_dim;   /* 128 */
+  int32_t d_ff;
+  int32_t vocab;
+  int32_t group_size; /* int4 group size of every projection: 32, 64 or a multiple of 128 */
+  int32_t max_batch;  /* 1..16 */
+  int32_t max_ctx;    /* KV cache capacity in positions, multiple of 128 */
+  int32_t max_steps;  /* capacity of the generated-token history */
+  float rope_theta;
+  float rms_eps;
+} yscv_hip_decoder_config;
+
+/* projection kinds for yscv_hip_decoder_set_linear */
+#define YSCV_HIP_DEC_Q 0
+#define YSCV_HIP_DEC_K 1
+#define YSCV_HIP_DEC_V 2
+#define YSCV_HIP_DEC_O 3
+#define YSCV_HIP_DEC_GATE 4
+#define YSCV_HIP_DEC_UP 5
+#define YSCV_HIP_DEC_DOWN 6
+#define YSCV_HIP_DEC_LM_HEAD 7
+/* norm kinds for yscv_hip_decoder_set_norm */
+#define YSCV_HIP_DEC_ATTN_NORM 0
+#define YSCV_HIP_DEC_FFN_NORM 1
+#define YSCV_HIP_DEC_FINAL_NORM 2
+
+int32_t yscv_hip_decoder_create(const yscv_hip_decoder_config *cfg, yscv_hip_decoder **out);
+int32_t yscv_hip_decoder_destroy(yscv_hip_decoder *d);
+/* Host inputs, borrowed: packed [n][k/2] uint4 nibbles (zero point 8, MatMulNBits order),
+ * scales_f16 [n][k/group_size] fp16 bit patterns.  `layer` is ignored for LM_HEAD. */
+int32_t yscv_hip_decoder_set_linear(yscv_hip_decoder *d, int32_t layer, int32_t kind,
+                                    const uint8_t *packed, const uint16_t *scales_f16, size_t n,
+                                    size_t k);
+int32_t yscv_hip_decoder_set_norm(yscv_hip_decoder *d, int32_t layer, int32_t kind,
+                                  const float *gamma);
+int32_t yscv_hip_decoder_set_embedding(yscv_hip_decoder *d, const uint16_t *table_f16);
+/* Build the fused device weights from what was set; required before run. */
+int32_t yscv_hip_decoder_finalize(yscv_hip_decoder *d);
+/* Benchmark setup: random-initialised weights of the configured architecture generated on the
+ * device (uniform nibbles, scales ~U(0.005,0.02), embedding ~N(0,1)), and a KV cache filled with
+ * ~N(0,1) values.  No reference counterpart (llm-bench loads an ONNX file). */
+int32_t yscv_hip_decoder_init_random(yscv_hip_decoder *d, uint64_t seed);
+int32_t yscv_hip_decoder_fill_kv_random(yscv_hip_decoder *d, uint64_t seed);
+/* Load cache positions [0, n_positions) of one layer from host arrays laid out
+ * [batch][position][kv_head][head_dim] fp16 (keys already rotated). */
+int32_t yscv_hip_decoder_set_kv(yscv_hip_decoder *d, int32_t layer, const uint16_t *k_f16,
+                                const uint16_t *v_f16, int32_t batch, int32_t n_positions);
+/* Start a generation: batch rows, the position the next token is written at, one input token per row. */
+int32_t yscv_hip_decoder_reset(yscv_hip_decoder *d, int32_t batch, int32_t start_pos,
+                               const int32_t *tokens_host);
+/* Run n_steps decode steps (asynchronously on `stream`).  use_graph != 0 replays one captured HIP
+ * graph per step.  Fails if the KV cache or the token history would overflow (KvCache::append
+ * returns an error in the same situation, kv_cache.rs:160-185). */
+int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_graph, void *stream);
+/* Generated tokens of steps [first_step, first_step + n_steps), laid out [step][batch]. */
+int32_t yscv_hip_decoder_read_tokens(yscv_hip_decoder *d, int32_t first_step, int32_t n_steps,
+                                     int32_t *out_host);
+/* Logits of the last step, [batch][vocab] f32. */
+int32_t yscv_hip_decoder_read_logits(yscv_hip_decoder *d, float *out_host);
+/* Bytes of packed weights + scales one decode step streams through the projections. */
+int32_t yscv_hip_decoder_weight_bytes(const yscv_hip_decoder *d, size_t *bytes);
 
 #if defined(__GNUC__)
 #pragma GCC visibility pop

@@ -1,0 +1,101 @@
+"""TEST INFRASTRUCTURE ONLY -- numpy restatement of one Llama-style decode step.
+
+Tolerance-checked glue (libm-dependent, not bit-pinned), following the reference semantics of
+  RMSNorm   crates/yscv-kernels/src/ops/norm.rs:1497-1518
+  RoPE      crates/yscv-kernels/src/ops/rope.rs:24-117   (rotate-half pairs (i, i + d/2))
+  GQA       crates/yscv-onnx/src/runner/linear.rs:552-646 (kv_h = q_h / groups, scale 1/sqrt(d),
+            max-subtracted softmax) applied to every cached position up to the current token
+  greedy    apps/llm-bench/src/main.rs:538-543 (last index among equal maxima)
+and the int4 projection definition of packed_int4_gemm_scalar (int4_matmul.rs:387-435) through
+dequantised weights.  Activations are rounded to fp16 where the GPU decoder stores fp16.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+
+def f16(x):
+    return np.asarray(x, np.float32).astype(np.float16).astype(np.float32)
+
+
+def dequant_uint4(packed, scales16, n, k, g):
+    """[n][k/2] uint4 nibbles (zero point 8) + fp16 scales -> f32 [n][k]."""
+    pb = np.asarray(packed, np.uint8).reshape(n, k // 2)
+    q = np.empty((n, k), np.float32)
+    q[:, 0::2] = (pb & 15).astype(np.float32) - 8.0
+    q[:, 1::2] = (pb >> 4).astype(np.float32) - 8.0
+    s = np.asarray(scales16).reshape(n, k // g).astype(np.float32)
+    return q * np.repeat(s, g, axis=1)
+
+
+class RefDecoder:
+    def __init__(self, cfg: dict, linears: dict, norms: dict, emb16):
+        """linears[(layer, kind)] = (packed, scales16) with kind in q k v o gate up down, and
+        linears[('lm_head',)]; norms[(layer, 'attn'|'ffn')], norms[('final',)] f32 gamma."""
+        self.c = cfg
+        g = cfg["group_size"]
+        D, hd = cfg["d_model"], cfg["head_dim"]
+        hq, hkv, ff = cfg["n_heads"] * hd, cfg["n_kv_heads"] * hd, cfg["d_ff"]
+        shapes = {"q": (hq, D), "k": (hkv, D), "v": (hkv, D), "o": (D, hq), "gate": (ff, D), "up": (ff, D), "down": (D, ff)}
+        self.w = {}
+        for key, (p, s) in linears.items():
+            n, k = (cfg["vocab"], D) if key == ("lm_head",) else shapes[key[1]]
+            self.w[key] = dequant_uint4(p, s, n, k, g)
+        self.norms = norms
+        self.emb = np.asarray(emb16).view(np.float16).astype(np.float32).reshape(cfg["vocab"], D)
+        L, B = cfg["n_layers"], cfg["max_batch"]
+        self.kc = [[np.zeros((0, cfg["n_kv_heads"], hd), np.float32) for _ in range(B)] for _ in range(L)]
+        self.vc = [[np.zeros((0, cfg["n_kv_heads"], hd), np.float32) for _ in range(B)] for _ in range(L)]
+
+    def set_kv(self, layer, k_nat, v_nat):
+        """k_nat / v_nat: f32 [batch][pos][kv_head][d] (keys already rotated)."""
+        for b in range(k_nat.shape[0]):
+            self.kc[layer][b] = np.array(k_nat[b], np.float32)
+            self.vc[layer][b] = np.array(v_nat[b], np.float32)
+
+    def _rmsnorm(self, h, gamma):
+        inv = 1.0 / np.sqrt((h.astype(np.float32) ** 2).mean(-1, keepdims=True) + np.float32(self.c["rms_eps"]))
+        return f16(h * inv.astype(np.float32) * gamma)
+
+    def _rope(self, x, pos):
+        """x: [heads][d]."""
+        d = x.shape[-1]
+        i = np.arange(d // 2, dtype=np.float32)
+        inv_freq = (1.0 / np.power(np.float32(self.c["rope_theta"]), 2 * i / np.float32(d))).astype(np.float32)
+        ang = inv_freq * np.float32(pos)
+        cs, sn = np.cos(ang), np.sin(ang)
+        x0, x1 = x[..., : d // 2], x[..., d // 2:]
+        return f16(np.concatenate([x0 * cs - x1 * sn, x0 * sn + x1 * cs], -1))
+
+    def step(self, tokens, pos):
+        """tokens: int [batch]; pos: position the new token is written at.  Returns logits f32 [batch][vocab]."""
+        c = self.c
+        hd, nh, nkv = c["head_dim"], c["n_heads"], c["n_kv_heads"]
+        groups = nh // nkv
+        B = len(tokens)
+        h = self.emb[np.asarray(tokens)].astype(np.float32)
+        for l in range(c["n_layers"]):
+            xn = self._rmsnorm(h, self.norms[(l, "attn")])
+            q = f16(xn @ self.w[(l, "q")].T).reshape(B, nh, hd)
+            k = f16(xn @ self.w[(l, "k")].T).reshape(B, nkv, hd)
+            v = f16(xn @ self.w[(l, "v")].T).reshape(B, nkv, hd)
+            ao = np.zeros((B, nh, hd), np.float32)
+            for b in range(B):
+                qr, kr = self._rope(q[b], pos), self._rope(k[b], pos)
+                self.kc[l][b] = np.concatenate([self.kc[l][b][:pos], kr[None]], 0)
+                self.vc[l][b] = np.concatenate([self.vc[l][b][:pos], v[b][None]], 0)
+                for qh in range(nh):
+                    kvh = qh // groups
+                    s = (self.kc[l][b][:, kvh, :] @ qr[qh]) * np.float32(1.0 / np.sqrt(hd))
+                    p = np.exp(s - s.max())
+                    p /= p.sum()
+                    ao[b, qh] = p @ self.vc[l][b][:, kvh, :]
+            ao = f16(ao.reshape(B, nh * hd))
+            h = h + ao @ self.w[(l, "o")].T
+            xn = self._rmsnorm(h, self.norms[(l, "ffn")])
+            gt = xn @ self.w[(l, "gate")].T
+            up = xn @ self.w[(l, "up")].T
+            act = f16(gt / (1.0 + np.exp(-gt)) * up)
+            h = h + act @ self.w[(l, "down")].T
+        xn = self._rmsnorm(h, self.norms[("final",)])
+        return (xn @ self.w[("lm_head",)].T).astype(np.float32)

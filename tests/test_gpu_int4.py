@@ -239,7 +239,7 @@ def test_invalid_arguments_are_rejected(K, torch_cuda):
     import yscv_amd
 
     with pytest.raises(yscv_amd.YscvHipError) as ei:
-        K.PackedInt4Weight(np.zeros(8, np.uint8), np.zeros(2, np.float32), 3, 2, 6 + 2)  # odd group size
+        K.PackedInt4Weight(np.zeros(9, np.uint8), np.zeros(6, np.float32), 3, 2, 9)  # odd group size
     assert ei.value.code == -1
     with pytest.raises(yscv_amd.YscvHipError):
         K.PackedInt4Weight(np.zeros(10, np.uint8), np.zeros(2, np.float32), 6, 2, 10)  # g does not divide k

@@ -14,6 +14,14 @@ _LIB_PATH = os.path.join(_HERE, "lib", "libyscv_hip.so")
 STATUS_NAMES = {0: "OK", -1: "INVALID_ARG", -2: "DEVICE", -3: "OOM", -4: "UNSUPPORTED", -5: "NO_DEVICE"}
 
 
+class DecoderConfig(C.Structure):
+    """yscv_hip_decoder_config."""
+
+    _fields_ = [(n, C.c_int32) for n in ("n_layers", "d_model", "n_heads", "n_kv_heads", "head_dim", "d_ff", "vocab",
+                                         "group_size", "max_batch", "max_ctx", "max_steps")] + \
+               [("rope_theta", C.c_float), ("rms_eps", C.c_float)]
+
+
 class YscvHipError(RuntimeError):
     def __init__(self, code: int, message: str):
         super().__init__(f"yscv_hip status {code} ({STATUS_NAMES.get(code, '?')}): {message}")
@@ -43,6 +51,8 @@ _SIGNATURES = {
     "yscv_hip_int4_matmul": [_vp, _vp, _i32, _vp, _i32, _sz, _vp],
     "yscv_hip_int4_gemv": [_vp, _vp, _i32, _vp, _i32, _sz, _vp],
     "yscv_hip_int4_gemm": [_vp, _vp, _i32, _vp, _i32, _sz, _vp],
+    "yscv_hip_int4_workspace_bytes": [_vp, _sz, _i32, C.POINTER(_sz)],
+    "yscv_hip_int4_matmul_ws": [_vp, _vp, _i32, _vp, _i32, _sz, _vp, _sz, _vp],
     "yscv_hip_packed_int4_gemv_dispatch": [_vp, _vp, _vp, _vp, _sz, _sz, _sz],
     "yscv_hip_packed_int4_gemm_dispatch": [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz],
     "yscv_hip_pack_int4_symmetric_per_group": [_vp, _sz, _sz, _sz, _vp, _vp],
@@ -62,6 +72,20 @@ _SIGNATURES = {
     "yscv_hip_requant_i8_per_channel_dispatch": [_vp, _sz, _vp, _vp, _f32, _vp, _sz],
     "yscv_hip_requant_i32_row_to_i8_dispatch": [_vp, _sz, _vp, _f32, _f32, _i32, _vp, _sz],
     "yscv_hip_dynamic_quantize_linear_host": [_vp, _sz, _vp, C.POINTER(_f32), C.POINTER(_f32)],
+    "yscv_hip_decoder_create": [_vp, C.POINTER(_vp)],
+    "yscv_hip_decoder_destroy": [_vp],
+    "yscv_hip_decoder_set_linear": [_vp, _i32, _i32, _vp, _vp, _sz, _sz],
+    "yscv_hip_decoder_set_norm": [_vp, _i32, _i32, _vp],
+    "yscv_hip_decoder_set_embedding": [_vp, _vp],
+    "yscv_hip_decoder_finalize": [_vp],
+    "yscv_hip_decoder_init_random": [_vp, C.c_uint64],
+    "yscv_hip_decoder_fill_kv_random": [_vp, C.c_uint64],
+    "yscv_hip_decoder_set_kv": [_vp, _i32, _vp, _vp, _i32, _i32],
+    "yscv_hip_decoder_reset": [_vp, _i32, _i32, _vp],
+    "yscv_hip_decoder_run": [_vp, _i32, _i32, _vp],
+    "yscv_hip_decoder_read_tokens": [_vp, _i32, _i32, _vp],
+    "yscv_hip_decoder_read_logits": [_vp, _vp],
+    "yscv_hip_decoder_weight_bytes": [_vp, C.POINTER(_sz)],
 }
 _SPECIAL = {
     "yscv_hip_abi_version": ([], C.c_uint32),
@@ -109,5 +133,9 @@ def lib() -> _Checked:
                 f"{_LIB_PATH} is missing: build it with `make -C yscv_amd/csrc -j8` "
                 "(or __graft_entry__.build()); there is no fallback path"
             )
+        # torch ships its own HIP runtime under the same soname as /opt/rocm's; a process can hold
+        # only one, and torch's must be the one that is loaded first or torch loses the GPU.
+        import torch  # noqa: F401
+
         _lib = _Checked(C.CDLL(_LIB_PATH))
     return _lib

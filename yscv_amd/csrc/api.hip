@@ -65,47 +65,99 @@ void drop_context() {
 static bool valid_act_dtype(int d) { return d == YSCV_HIP_F32 || d == YSCV_HIP_F16 || d == YSCV_HIP_BF16; }
 static size_t dtype_size(int d) { return d == YSCV_HIP_F32 ? 4 : 2; }
 
-// Runs the tiled int4 path: x_prep, then the skinny or the GEMM kernel.  All scratch comes
-// from the stream-ordered allocator, so concurrent callers on different streams never share it.
-static int32_t int4_run(const yscv_hip_int4_weight *w, const void *x, int x_dtype, void *y, int y_dtype,
-                        size_t m, int force /*0 auto, 1 skinny, 2 gemm*/, hipStream_t s) {
+// Scratch layout of one int4 call: [xh][xl][row_scale][partial], each part rounded to 256 B.
+// A fp16 activation whose row stride already equals the padded K needs no preparation at all.
+struct Int4Scratch {
+  bool direct;       // x is used in place as the fp16 `hi` operand
+  bool skinny;
+  int split;
+  size_t k_pad;
+  SkinnyPlan plan;
+  size_t xh_bytes, rs_bytes, part_bytes, total;
+};
+
+static Int4Scratch int4_scratch_layout(const yscv_hip_int4_weight *w, const void *x, int x_dtype, size_t m,
+                                       int force, int num_cus) {
+  Int4Scratch L{};
+  L.skinny = force == 1 || (force == 0 && m <= 16);
+  L.k_pad = w->kt * 128;
+  L.direct = x_dtype == YSCV_HIP_F16 && L.k_pad == w->k && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+  L.split = x_dtype == YSCV_HIP_F32 ? 2 : 1;
+  if (L.skinny) L.plan = plan_int4_skinny(w, m, L.split, num_cus);
+  L.xh_bytes = L.direct ? 0 : round_up(m * L.k_pad * sizeof(_Float16), 256);
+  L.rs_bytes = L.direct ? 0 : round_up(m * sizeof(float), 256);
+  L.part_bytes = L.skinny ? round_up(L.plan.partial_bytes, 256) : 0;
+  L.total = L.xh_bytes * L.split + L.rs_bytes + L.part_bytes;
+  return L;
+}
+
+int32_t int4_workspace_bytes(const yscv_hip_int4_weight *w, size_t m, int x_dtype, int force, size_t *bytes) {
+  const Context *ctx = nullptr;
+  YSCV_TRY(ensure_context(&ctx));
+  YSCV_REQUIRE(w != nullptr && bytes != nullptr, "null argument");
+  if (!w->tiled || m == 0) {
+    *bytes = 0;
+    return YSCV_HIP_OK;
+  }
+  // a 16-byte aligned pointer stands in for the activation: alignment is checked again at run time
+  Int4Scratch L = int4_scratch_layout(w, reinterpret_cast<const void *>(uintptr_t(256)), x_dtype, m, force, ctx->num_cus);
+  *bytes = L.total;
+  return YSCV_HIP_OK;
+}
+
+// Runs the int4 path: activation preparation if needed, then the skinny or the GEMM kernel.
+// `ws` may be null: scratch then comes from the stream-ordered allocator, so concurrent callers
+// on different streams never share it.
+int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, void *y, int y_dtype, size_t m,
+                    int force /*0 auto, 1 skinny, 2 gemm*/, int epi, void *ws, size_t ws_bytes, hipStream_t s) {
   const Context *ctx = nullptr;
   YSCV_TRY(ensure_context(&ctx));
   YSCV_REQUIRE(w != nullptr, "null int4 weight handle");
   YSCV_REQUIRE(x != nullptr && y != nullptr, "null activation / output pointer");
   YSCV_REQUIRE(valid_act_dtype(x_dtype) && valid_act_dtype(y_dtype), "unknown dtype code");
   if (m == 0) return YSCV_HIP_OK;
+  if (force == 1 && m > 16) return set_error(YSCV_HIP_ERR_INVALID_ARG, "gemv entry point handles m <= 16, got %zu", m);
   if (!w->tiled) {
-    if (force == 1 && m > 16) return set_error(YSCV_HIP_ERR_INVALID_ARG, "gemv entry point handles m <= 16, got %zu", m);
+    if (epi != EPI_STORE) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "fused epilogues need the tiled layout");
     return launch_int4_generic(w, x, x_dtype, y, y_dtype, m, s);
   }
-  const bool skinny = force == 1 || (force == 0 && m <= 16);
-  if (skinny && m > 16) return set_error(YSCV_HIP_ERR_INVALID_ARG, "gemv entry point handles m <= 16, got %zu", m);
-  const int split = x_dtype == YSCV_HIP_F32 ? 2 : 1;
-  const size_t k_pad = w->kt * 128;
-  SkinnyPlan plan{};
-  if (skinny) plan = plan_int4_skinny(w, m, split, ctx->num_cus);
-  const size_t xh_bytes = round_up(m * k_pad * sizeof(_Float16), 256);
-  const size_t rs_bytes = round_up(m * sizeof(float), 256);
-  const size_t part_bytes = skinny ? round_up(plan.partial_bytes, 256) : 0;
-  const size_t total = xh_bytes * split + rs_bytes + part_bytes;
-  char *scratch = nullptr;
-  YSCV_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&scratch), total, s));
-  _Float16 *xh = reinterpret_cast<_Float16 *>(scratch);
-  _Float16 *xl = split == 2 ? reinterpret_cast<_Float16 *>(scratch + xh_bytes) : nullptr;
-  float *row_scale = reinterpret_cast<float *>(scratch + xh_bytes * split);
-  float *partial = part_bytes ? reinterpret_cast<float *>(scratch + xh_bytes * split + rs_bytes) : nullptr;
-  int32_t st = launch_x_prep(x, x_dtype, m, w->k, k_pad, split, xh, xl, row_scale, s);
-  if (st == YSCV_HIP_OK) {
-    if (skinny)
-      st = launch_int4_skinny(w, plan, xh, xl, row_scale, k_pad, split, y, y_dtype, m, partial, s);
-    else
-      st = launch_int4_gemm(w, xh, xl, row_scale, k_pad, split, y, y_dtype, m, s);
+  Int4Scratch L = int4_scratch_layout(w, x, x_dtype, m, force, ctx->num_cus);
+  if (!L.skinny && epi != EPI_STORE) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "fused epilogues exist for m <= 16 only");
+  char *scratch = static_cast<char *>(ws);
+  bool own = false;
+  if (L.total > 0) {
+    if (scratch) {
+      YSCV_REQUIRE(ws_bytes >= L.total, "workspace too small: %zu < %zu bytes", ws_bytes, L.total);
+      YSCV_REQUIRE((reinterpret_cast<uintptr_t>(scratch) & 255) == 0, "workspace must be 256-byte aligned");
+    } else {
+      YSCV_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&scratch), L.total, s));
+      own = true;
+    }
   }
-  hipError_t fe = hipFreeAsync(scratch, s);
-  YSCV_TRY(st);
-  YSCV_HIP_TRY(fe);
-  return YSCV_HIP_OK;
+  const _Float16 *xh = L.direct ? static_cast<const _Float16 *>(x) : reinterpret_cast<_Float16 *>(scratch);
+  _Float16 *xl = (!L.direct && L.split == 2) ? reinterpret_cast<_Float16 *>(scratch + L.xh_bytes) : nullptr;
+  float *row_scale = L.direct ? nullptr : reinterpret_cast<float *>(scratch + L.xh_bytes * L.split);
+  float *partial = L.part_bytes ? reinterpret_cast<float *>(scratch + L.xh_bytes * L.split + L.rs_bytes) : nullptr;
+  int32_t st = YSCV_HIP_OK;
+  if (!L.direct)
+    st = launch_x_prep(x, x_dtype, m, w->k, L.k_pad, L.split, const_cast<_Float16 *>(xh), xl, row_scale, s);
+  if (st == YSCV_HIP_OK) {
+    if (L.skinny)
+      st = launch_int4_skinny(w, L.plan, xh, xl, row_scale, L.k_pad, L.split, y, y_dtype, m, partial, epi, s);
+    else
+      st = launch_int4_gemm(w, xh, xl, row_scale, L.k_pad, L.split, y, y_dtype, m, s);
+  }
+  if (own) {
+    hipError_t fe = hipFreeAsync(scratch, s);
+    YSCV_TRY(st);
+    YSCV_HIP_TRY(fe);
+  }
+  return st;
+}
+
+static int32_t int4_run(const yscv_hip_int4_weight *w, const void *x, int x_dtype, void *y, int y_dtype,
+                        size_t m, int force, hipStream_t s) {
+  return int4_run_ws(w, x, x_dtype, y, y_dtype, m, force, EPI_STORE, nullptr, 0, s);
 }
 
 static void free_int4(yscv_hip_int4_weight *w) {
@@ -321,6 +373,20 @@ int32_t yscv_hip_int4_gemv(const yscv_hip_int4_weight *w, const void *x_dev, int
 int32_t yscv_hip_int4_gemm(const yscv_hip_int4_weight *w, const void *x_dev, int32_t x_dtype, void *y_dev,
                            int32_t y_dtype, size_t m, void *stream) {
   return int4_run(w, x_dev, x_dtype, y_dev, y_dtype, m, 2, as_stream(stream));
+}
+
+int32_t yscv_hip_int4_workspace_bytes(const yscv_hip_int4_weight *w, size_t m, int32_t x_dtype, size_t *bytes) {
+  return int4_workspace_bytes(w, m, x_dtype, 0, bytes);
+}
+
+int32_t yscv_hip_int4_matmul_ws(const yscv_hip_int4_weight *w, const void *x_dev, int32_t x_dtype, void *y_dev,
+                                int32_t y_dtype, size_t m, void *workspace_dev, size_t workspace_bytes, void *stream) {
+  YSCV_REQUIRE(workspace_dev != nullptr || workspace_bytes == 0, "null workspace with non-zero size");
+  size_t need = 0;
+  YSCV_TRY(int4_workspace_bytes(w, m, x_dtype, 0, &need));
+  if (need > 0) YSCV_REQUIRE(workspace_dev != nullptr, "this call needs %zu bytes of workspace", need);
+  return int4_run_ws(w, x_dev, x_dtype, y_dev, y_dtype, m, 0, EPI_STORE, workspace_dev, workspace_bytes,
+                     as_stream(stream));
 }
 
 static int32_t int4_host_call(const uint8_t *weight_packed, const float *scales, const float *activation,

@@ -1,0 +1,556 @@
+// Llama-style decoder resident on the GPU: the decode loop of the llm-bench harness
+// (apps/llm-bench/src/main.rs:403-561: feed the last token plus the KV cache, take the greedy
+// pick, repeat) with every projection running through the skinny int4 kernel.
+// One decode step is a fixed sequence of kernel launches that reads the position from device
+// memory, so the step is captured once into a HIP graph and replayed for every token.
+#include <vector>
+
+#include "decoder.hpp"
+#include "int4_common.hpp"
+#include "kernels.hpp"
+
+namespace yscv {
+
+// ---- random-initialised tiled weights (benchmark setup) -------------------------------------------
+// Uniform nibbles and scales ~U(0.005, 0.02) written straight into the tiled layout: for random data
+// the tiling is just another arrangement of the same distribution, so no host round trip is needed.
+__global__ void random_tiles_kernel(uint32_t *__restrict__ words, size_t n_words, uint64_t seed) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n_words; i += (size_t)gridDim.x * blockDim.x) {
+    uint64_t z = (i + 1) * 0x9E3779B97F4A7C15ull + seed;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    words[i] = (uint32_t)(z ^ (z >> 31));
+  }
+}
+__global__ void random_scales_kernel(_Float16 *__restrict__ sc, size_t n, uint64_t seed, float lo, float hi) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    uint64_t z = (i + 1) * 0x9E3779B97F4A7C15ull + seed;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    const float u = (float)((z >> 40) & 0xFFFFFF) * (1.0f / 16777216.0f);
+    sc[i] = (_Float16)(lo + (hi - lo) * u);
+  }
+}
+__global__ void fill_f32_kernel(float *p, size_t n, float v) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+}
+__global__ void fill_i32_kernel(int32_t *p, size_t n, int32_t v) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
+static unsigned grid_for(size_t n) {
+  size_t b = ceil_div(n, (size_t)256);
+  return (unsigned)(b > 65535 ? 65535 : (b < 1 ? 1 : b));
+}
+
+static int32_t random_int4_weight(size_t n, size_t k, size_t g, uint64_t seed, yscv_hip_int4_weight **out) {
+  YSCV_REQUIRE(g == 32 || g == 64 || g % 128 == 0, "random weights need a tiled group size");
+  auto *w = new yscv_hip_int4_weight();
+  w->n = n;
+  w->k = k;
+  w->g = g;
+  w->scale_dtype = YSCV_HIP_F16;
+  w->has_zp = false;
+  w->tiled = true;
+  w->gm = g == 32 ? GM32 : (g == 64 ? GM64 : GM128);
+  w->nt = ceil_div(n, (size_t)16);
+  w->kt = ceil_div(k, (size_t)128);
+  w->chunks = w->gm == GM128 ? k / g : w->kt;
+  const size_t tile_bytes = w->nt * w->kt * (size_t)kTileBytes;
+  const size_t sc_elems = w->nt * w->chunks * 16 * (size_t)scales_per_chunk(w->gm);
+  hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->tiles), tile_bytes);
+  if (e == hipSuccess) e = hipMalloc(&w->tscales, sc_elems * 2);
+  if (e != hipSuccess) {
+    (void)hipFree(w->tiles);
+    delete w;
+    return set_error(e == hipErrorOutOfMemory ? YSCV_HIP_ERR_OOM : YSCV_HIP_ERR_DEVICE, "weight allocation failed: %s",
+                     hipGetErrorString(e));
+  }
+  hipLaunchKernelGGL(random_tiles_kernel, dim3(grid_for(tile_bytes / 4)), dim3(256), 0, nullptr,
+                     reinterpret_cast<uint32_t *>(w->tiles), tile_bytes / 4, seed);
+  hipLaunchKernelGGL(random_scales_kernel, dim3(grid_for(sc_elems)), dim3(256), 0, nullptr,
+                     static_cast<_Float16 *>(w->tscales), sc_elems, seed ^ 0x5ca1e5ull, 0.005f, 0.02f);
+  w->device_bytes = tile_bytes + sc_elems * 2;
+  *out = w;
+  return YSCV_HIP_OK;
+}
+
+static void destroy_int4(yscv_hip_int4_weight *w) {
+  if (!w) return;
+  (void)hipFree(w->tiles);
+  (void)hipFree(w->tscales);
+  (void)hipFree(w->tzps);
+  (void)hipFree(w->raw);
+  (void)hipFree(w->rscales);
+  (void)hipFree(w->rzps);
+  delete w;
+}
+
+}  // namespace yscv
+
+using namespace yscv;
+
+struct HostLinear {
+  std::vector<uint8_t> packed;
+  std::vector<uint16_t> scales;
+  size_t n = 0, k = 0;
+};
+
+struct yscv_hip_decoder {
+  yscv_hip_decoder_config cfg{};
+  struct Layer {
+    yscv_hip_int4_weight *wqkv = nullptr, *wo = nullptr, *wgu = nullptr, *wdown = nullptr;
+    float *attn_norm = nullptr, *ffn_norm = nullptr;
+    _Float16 *kc = nullptr, *vc = nullptr;
+    HostLinear stage[7];  // q k v o gate up down, kept until finalize
+  };
+  std::vector<Layer> layers;
+  yscv_hip_int4_weight *lm_head = nullptr;
+  float *final_norm = nullptr;
+  _Float16 *emb = nullptr;
+  // activations
+  float *h = nullptr, *logits = nullptr, *attn_part = nullptr;
+  _Float16 *xn = nullptr, *qkv = nullptr, *ao = nullptr, *act = nullptr;
+  void *ws = nullptr;
+  size_t ws_bytes = 0;
+  int32_t *tokens = nullptr, *history = nullptr, *pos = nullptr, *step = nullptr;
+  int batch = 0;
+  bool finalized = false;
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t graph_exec = nullptr;
+  int graph_batch = 0;
+  size_t weight_bytes = 0;
+};
+
+static void decoder_free(yscv_hip_decoder *d) {
+  if (!d) return;
+  if (d->graph_exec) (void)hipGraphExecDestroy(d->graph_exec);
+  if (d->graph) (void)hipGraphDestroy(d->graph);
+  for (auto &L : d->layers) {
+    destroy_int4(L.wqkv);
+    destroy_int4(L.wo);
+    destroy_int4(L.wgu);
+    destroy_int4(L.wdown);
+    (void)hipFree(L.attn_norm);
+    (void)hipFree(L.ffn_norm);
+    (void)hipFree(L.kc);
+    (void)hipFree(L.vc);
+  }
+  destroy_int4(d->lm_head);
+  (void)hipFree(d->final_norm);
+  (void)hipFree(d->emb);
+  (void)hipFree(d->h);
+  (void)hipFree(d->logits);
+  (void)hipFree(d->attn_part);
+  (void)hipFree(d->xn);
+  (void)hipFree(d->qkv);
+  (void)hipFree(d->ao);
+  (void)hipFree(d->act);
+  (void)hipFree(d->ws);
+  (void)hipFree(d->tokens);
+  (void)hipFree(d->history);
+  (void)hipFree(d->pos);
+  (void)hipFree(d->step);
+  delete d;
+}
+
+#define DEC_HIP(expr)                                                                                \
+  do {                                                                                               \
+    hipError_t _e = (expr);                                                                          \
+    if (_e != hipSuccess)                                                                            \
+      return set_error(_e == hipErrorOutOfMemory ? YSCV_HIP_ERR_OOM : YSCV_HIP_ERR_DEVICE, "%s failed: %s", #expr, \
+                       hipGetErrorString(_e));                                                       \
+  } while (0)
+
+static size_t kv_elems(const yscv_hip_decoder_config &c) {
+  return (size_t)c.max_batch * c.n_kv_heads * c.max_ctx * c.head_dim;
+}
+
+static int32_t make_fused(const HostLinear *parts, int count, bool interleave, size_t g, yscv_hip_int4_weight **out) {
+  const size_t k = parts[0].k;
+  size_t n_total = 0;
+  for (int i = 0; i < count; i++) {
+    YSCV_REQUIRE(parts[i].n > 0 && parts[i].k == k, "projection missing or with a different K");
+    n_total += parts[i].n;
+  }
+  const size_t row_b = k / 2, row_s = k / g;
+  std::vector<uint8_t> packed(n_total * row_b);
+  std::vector<uint16_t> scales(n_total * row_s);
+  if (interleave) {
+    YSCV_REQUIRE(count == 2 && parts[0].n == parts[1].n, "interleaving needs two equal projections");
+    for (size_t r = 0; r < parts[0].n; r++)
+      for (int p = 0; p < 2; p++) {
+        memcpy(&packed[(2 * r + p) * row_b], &parts[p].packed[r * row_b], row_b);
+        memcpy(&scales[(2 * r + p) * row_s], &parts[p].scales[r * row_s], row_s * 2);
+      }
+  } else {
+    size_t r0 = 0;
+    for (int i = 0; i < count; i++) {
+      memcpy(&packed[r0 * row_b], parts[i].packed.data(), parts[i].n * row_b);
+      memcpy(&scales[r0 * row_s], parts[i].scales.data(), parts[i].n * row_s * 2);
+      r0 += parts[i].n;
+    }
+  }
+  return yscv_hip_int4_weight_create(packed.data(), scales.data(), YSCV_HIP_F16, nullptr, YSCV_HIP_NIBBLE_UNSIGNED,
+                                     n_total, k, g, out);
+}
+
+static int32_t alloc_runtime(yscv_hip_decoder *d) {
+  const auto &c = d->cfg;
+  const size_t B = c.max_batch, D = c.d_model;
+  const size_t qkv_n = (size_t)(c.n_heads + 2 * c.n_kv_heads) * c.head_dim;
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->h), B * D * 4));
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->logits), B * c.vocab * 4));
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->xn), B * D * 2));
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->qkv), B * qkv_n * 2));
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->ao), B * (size_t)c.n_heads * c.head_dim * 2));
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->act), B * (size_t)c.d_ff * 2));
+  const size_t chunks = c.max_ctx / 128;
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->attn_part), B * c.n_heads * chunks * (c.head_dim + 2) * 4));
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->tokens), B * 4));
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->history), B * (size_t)c.max_steps * 4));
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->pos), 4));
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->step), 4));
+  DEC_HIP(hipMemset(d->tokens, 0, B * 4));
+  DEC_HIP(hipMemset(d->history, 0, B * (size_t)c.max_steps * 4));
+  DEC_HIP(hipMemset(d->pos, 0, 4));
+  DEC_HIP(hipMemset(d->step, 0, 4));
+  return YSCV_HIP_OK;
+}
+
+static int32_t finish_setup(yscv_hip_decoder *d) {
+  // workspace: the largest any projection needs at the maximum batch
+  size_t need = 0;
+  auto upd = [&](const yscv_hip_int4_weight *w) -> int32_t {
+    size_t b = 0;
+    YSCV_TRY(int4_workspace_bytes(w, d->cfg.max_batch, YSCV_HIP_F16, 1, &b));
+    if (b > need) need = b;
+    return YSCV_HIP_OK;
+  };
+  d->weight_bytes = 0;
+  for (auto &L : d->layers) {
+    for (auto *w : {L.wqkv, L.wo, L.wgu, L.wdown}) {
+      YSCV_REQUIRE(w != nullptr, "a projection was never set");
+      YSCV_TRY(upd(w));
+      d->weight_bytes += w->device_bytes;
+    }
+  }
+  YSCV_REQUIRE(d->lm_head != nullptr, "lm_head was never set");
+  YSCV_TRY(upd(d->lm_head));
+  d->weight_bytes += d->lm_head->device_bytes;
+  if (need > d->ws_bytes) {
+    (void)hipFree(d->ws);
+    d->ws = nullptr;
+    DEC_HIP(hipMalloc(&d->ws, need));
+    d->ws_bytes = need;
+  }
+  d->finalized = true;
+  return YSCV_HIP_OK;
+}
+
+// every launch of one decode step, in order, on stream s
+static int32_t enqueue_step(yscv_hip_decoder *d, int batch, hipStream_t s) {
+  const auto &c = d->cfg;
+  const int D = c.d_model;
+  YSCV_TRY(launch_embed(d->tokens, d->emb, batch, D, c.vocab, d->h, s));
+  for (auto &L : d->layers) {
+    YSCV_TRY(launch_rmsnorm(d->h, L.attn_norm, batch, D, c.rms_eps, d->xn, s));
+    YSCV_TRY(int4_run_ws(L.wqkv, d->xn, YSCV_HIP_F16, d->qkv, YSCV_HIP_F16, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s));
+    YSCV_TRY(launch_rope_append(d->qkv, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_theta, c.max_ctx,
+                                L.kc, L.vc, s));
+    YSCV_TRY(launch_attention(d->qkv, L.kc, L.vc, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim, c.max_ctx,
+                              d->attn_part, d->ao, s));
+    YSCV_TRY(int4_run_ws(L.wo, d->ao, YSCV_HIP_F16, d->h, YSCV_HIP_F32, batch, 1, EPI_ADD_F32, d->ws, d->ws_bytes, s));
+    YSCV_TRY(launch_rmsnorm(d->h, L.ffn_norm, batch, D, c.rms_eps, d->xn, s));
+    YSCV_TRY(int4_run_ws(L.wgu, d->xn, YSCV_HIP_F16, d->act, YSCV_HIP_F16, batch, 1, EPI_SWIGLU, d->ws, d->ws_bytes, s));
+    YSCV_TRY(int4_run_ws(L.wdown, d->act, YSCV_HIP_F16, d->h, YSCV_HIP_F32, batch, 1, EPI_ADD_F32, d->ws, d->ws_bytes, s));
+  }
+  YSCV_TRY(launch_rmsnorm(d->h, d->final_norm, batch, D, c.rms_eps, d->xn, s));
+  YSCV_TRY(int4_run_ws(d->lm_head, d->xn, YSCV_HIP_F16, d->logits, YSCV_HIP_F32, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s));
+  YSCV_TRY(launch_argmax(d->logits, batch, c.vocab, d->tokens, d->history, d->step, c.max_steps, s));
+  YSCV_TRY(launch_advance(d->pos, d->step, s));
+  return YSCV_HIP_OK;
+}
+
+extern "C" {
+
+int32_t yscv_hip_decoder_create(const yscv_hip_decoder_config *cfg, yscv_hip_decoder **out) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(cfg && out, "null argument");
+  *out = nullptr;
+  const auto &c = *cfg;
+  YSCV_REQUIRE(c.n_layers > 0 && c.d_model > 0 && c.n_heads > 0 && c.n_kv_heads > 0 && c.d_ff > 0 && c.vocab > 0,
+               "non-positive model dimension");
+  YSCV_REQUIRE(c.head_dim == 128, "head_dim must be 128 (got %d)", c.head_dim);
+  YSCV_REQUIRE(c.n_heads % c.n_kv_heads == 0 && c.n_heads / c.n_kv_heads <= 4, "1..4 query heads per kv head");
+  YSCV_REQUIRE(c.d_model % 128 == 0 && c.d_ff % 128 == 0 && (c.n_heads * c.head_dim) % 128 == 0,
+               "d_model, d_ff and n_heads*head_dim must be multiples of 128");
+  YSCV_REQUIRE(c.max_batch >= 1 && c.max_batch <= 16, "max_batch must be 1..16 (skinny kernel)");
+  YSCV_REQUIRE(c.max_ctx >= 128 && c.max_ctx % 128 == 0, "max_ctx must be a positive multiple of 128");
+  YSCV_REQUIRE(c.max_steps >= 1, "max_steps must be positive");
+  YSCV_REQUIRE(c.group_size == 32 || c.group_size == 64 || c.group_size % 128 == 0, "unsupported group size");
+  YSCV_REQUIRE(c.rms_eps > 0.0f, "rms_eps must be finite and > 0 (ops/norm.rs:1471)");
+  auto *d = new yscv_hip_decoder();
+  d->cfg = c;
+  d->layers.resize(c.n_layers);
+  int32_t st = alloc_runtime(d);
+  const size_t D = c.d_model;
+  for (auto &L : d->layers) {
+    if (st != YSCV_HIP_OK) break;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&L.attn_norm), D * 4);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&L.ffn_norm), D * 4);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&L.kc), kv_elems(c) * 2);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&L.vc), kv_elems(c) * 2);
+    if (e == hipSuccess) e = hipMemset(L.kc, 0, kv_elems(c) * 2);
+    if (e == hipSuccess) e = hipMemset(L.vc, 0, kv_elems(c) * 2);
+    if (e != hipSuccess)
+      st = set_error(e == hipErrorOutOfMemory ? YSCV_HIP_ERR_OOM : YSCV_HIP_ERR_DEVICE, "layer allocation failed: %s",
+                     hipGetErrorString(e));
+    else {
+      hipLaunchKernelGGL(fill_f32_kernel, dim3(grid_for(D)), dim3(256), 0, nullptr, L.attn_norm, D, 1.0f);
+      hipLaunchKernelGGL(fill_f32_kernel, dim3(grid_for(D)), dim3(256), 0, nullptr, L.ffn_norm, D, 1.0f);
+    }
+  }
+  if (st == YSCV_HIP_OK) {
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->final_norm), D * 4);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&d->emb), (size_t)c.vocab * D * 2);
+    if (e != hipSuccess)
+      st = set_error(e == hipErrorOutOfMemory ? YSCV_HIP_ERR_OOM : YSCV_HIP_ERR_DEVICE, "allocation failed: %s",
+                     hipGetErrorString(e));
+    else
+      hipLaunchKernelGGL(fill_f32_kernel, dim3(grid_for(D)), dim3(256), 0, nullptr, d->final_norm, D, 1.0f);
+  }
+  if (st == YSCV_HIP_OK) {
+    hipError_t e = hipDeviceSynchronize();
+    if (e != hipSuccess) st = set_error(YSCV_HIP_ERR_DEVICE, "setup failed: %s", hipGetErrorString(e));
+  }
+  if (st != YSCV_HIP_OK) {
+    decoder_free(d);
+    return st;
+  }
+  *out = d;
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_destroy(yscv_hip_decoder *d) {
+  decoder_free(d);
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_set_linear(yscv_hip_decoder *d, int32_t layer, int32_t kind, const uint8_t *packed,
+                                    const uint16_t *scales_f16, size_t n, size_t k) {
+  YSCV_REQUIRE(d && packed && scales_f16, "null argument");
+  YSCV_REQUIRE(kind >= 0 && kind <= YSCV_HIP_DEC_LM_HEAD, "unknown projection kind %d", kind);
+  const auto &c = d->cfg;
+  const size_t g = c.group_size;
+  YSCV_REQUIRE(k % g == 0, "group size does not divide k");
+  const size_t hq = (size_t)c.n_heads * c.head_dim, hkv = (size_t)c.n_kv_heads * c.head_dim;
+  const size_t exp_n[8] = {hq, hkv, hkv, (size_t)c.d_model, (size_t)c.d_ff, (size_t)c.d_ff, (size_t)c.d_model, (size_t)c.vocab};
+  const size_t exp_k[8] = {(size_t)c.d_model, (size_t)c.d_model, (size_t)c.d_model, hq, (size_t)c.d_model,
+                           (size_t)c.d_model, (size_t)c.d_ff, (size_t)c.d_model};
+  YSCV_REQUIRE(n == exp_n[kind] && k == exp_k[kind], "projection %d must be [%zu][%zu], got [%zu][%zu]", kind,
+               exp_n[kind], exp_k[kind], n, k);
+  d->finalized = false;
+  if (kind == YSCV_HIP_DEC_LM_HEAD) {
+    destroy_int4(d->lm_head);
+    d->lm_head = nullptr;
+    return yscv_hip_int4_weight_create(packed, scales_f16, YSCV_HIP_F16, nullptr, YSCV_HIP_NIBBLE_UNSIGNED, n, k, g,
+                                       &d->lm_head);
+  }
+  YSCV_REQUIRE(layer >= 0 && layer < c.n_layers, "layer %d out of range", layer);
+  HostLinear &hl = d->layers[layer].stage[kind];
+  hl.n = n;
+  hl.k = k;
+  hl.packed.assign(packed, packed + n * k / 2);
+  hl.scales.assign(scales_f16, scales_f16 + n * (k / g));
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_set_norm(yscv_hip_decoder *d, int32_t layer, int32_t kind, const float *gamma) {
+  YSCV_REQUIRE(d && gamma, "null argument");
+  float *dst = nullptr;
+  if (kind == YSCV_HIP_DEC_FINAL_NORM) {
+    dst = d->final_norm;
+  } else {
+    YSCV_REQUIRE(layer >= 0 && layer < d->cfg.n_layers, "layer %d out of range", layer);
+    YSCV_REQUIRE(kind == YSCV_HIP_DEC_ATTN_NORM || kind == YSCV_HIP_DEC_FFN_NORM, "unknown norm kind %d", kind);
+    dst = kind == YSCV_HIP_DEC_ATTN_NORM ? d->layers[layer].attn_norm : d->layers[layer].ffn_norm;
+  }
+  DEC_HIP(hipMemcpy(dst, gamma, (size_t)d->cfg.d_model * 4, hipMemcpyHostToDevice));
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_set_embedding(yscv_hip_decoder *d, const uint16_t *table_f16) {
+  YSCV_REQUIRE(d && table_f16, "null argument");
+  DEC_HIP(hipMemcpy(d->emb, table_f16, (size_t)d->cfg.vocab * d->cfg.d_model * 2, hipMemcpyHostToDevice));
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_finalize(yscv_hip_decoder *d) {
+  YSCV_REQUIRE(d != nullptr, "null decoder");
+  const size_t g = d->cfg.group_size;
+  for (auto &L : d->layers) {
+    if (L.stage[0].n) {  // q, k, v staged -> fused [q; k; v]
+      destroy_int4(L.wqkv);
+      L.wqkv = nullptr;
+      YSCV_TRY(make_fused(&L.stage[0], 3, false, g, &L.wqkv));
+      for (int i = 0; i < 3; i++) L.stage[i] = HostLinear();
+    }
+    if (L.stage[3].n) {
+      destroy_int4(L.wo);
+      L.wo = nullptr;
+      YSCV_TRY(make_fused(&L.stage[3], 1, false, g, &L.wo));
+      L.stage[3] = HostLinear();
+    }
+    if (L.stage[4].n) {  // gate, up staged -> rows interleaved gate_0, up_0, gate_1, ... for the SwiGLU epilogue
+      destroy_int4(L.wgu);
+      L.wgu = nullptr;
+      YSCV_TRY(make_fused(&L.stage[4], 2, true, g, &L.wgu));
+      L.stage[4] = HostLinear();
+      L.stage[5] = HostLinear();
+    }
+    if (L.stage[6].n) {
+      destroy_int4(L.wdown);
+      L.wdown = nullptr;
+      YSCV_TRY(make_fused(&L.stage[6], 1, false, g, &L.wdown));
+      L.stage[6] = HostLinear();
+    }
+  }
+  return finish_setup(d);
+}
+
+int32_t yscv_hip_decoder_init_random(yscv_hip_decoder *d, uint64_t seed) {
+  YSCV_REQUIRE(d != nullptr, "null decoder");
+  const auto &c = d->cfg;
+  const size_t g = c.group_size, D = c.d_model;
+  const size_t qkv_n = (size_t)(c.n_heads + 2 * c.n_kv_heads) * c.head_dim;
+  uint64_t sd = seed * 0x100000001B3ull + 1;
+  for (auto &L : d->layers) {
+    destroy_int4(L.wqkv);
+    destroy_int4(L.wo);
+    destroy_int4(L.wgu);
+    destroy_int4(L.wdown);
+    L.wqkv = L.wo = L.wgu = L.wdown = nullptr;
+    YSCV_TRY(random_int4_weight(qkv_n, D, g, sd++, &L.wqkv));
+    YSCV_TRY(random_int4_weight(D, (size_t)c.n_heads * c.head_dim, g, sd++, &L.wo));
+    YSCV_TRY(random_int4_weight(2 * (size_t)c.d_ff, D, g, sd++, &L.wgu));
+    YSCV_TRY(random_int4_weight(D, (size_t)c.d_ff, g, sd++, &L.wdown));
+  }
+  destroy_int4(d->lm_head);
+  d->lm_head = nullptr;
+  YSCV_TRY(random_int4_weight((size_t)c.vocab, D, g, sd++, &d->lm_head));
+  YSCV_TRY(launch_kv_random_fill(d->emb, (size_t)c.vocab * D, sd++, nullptr));
+  DEC_HIP(hipDeviceSynchronize());
+  return finish_setup(d);
+}
+
+int32_t yscv_hip_decoder_fill_kv_random(yscv_hip_decoder *d, uint64_t seed) {
+  YSCV_REQUIRE(d != nullptr, "null decoder");
+  uint64_t sd = seed * 0x9E3779B1ull + 7;
+  for (auto &L : d->layers) {
+    YSCV_TRY(launch_kv_random_fill(L.kc, kv_elems(d->cfg), sd++, nullptr));
+    YSCV_TRY(launch_kv_random_fill(L.vc, kv_elems(d->cfg), sd++, nullptr));
+  }
+  DEC_HIP(hipDeviceSynchronize());
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_set_kv(yscv_hip_decoder *d, int32_t layer, const uint16_t *k_f16, const uint16_t *v_f16,
+                                int32_t batch, int32_t n_positions) {
+  YSCV_REQUIRE(d && k_f16 && v_f16, "null argument");
+  const auto &c = d->cfg;
+  YSCV_REQUIRE(layer >= 0 && layer < c.n_layers, "layer %d out of range", layer);
+  YSCV_REQUIRE(batch >= 1 && batch <= c.max_batch && n_positions >= 0 && n_positions <= c.max_ctx, "bad batch / positions");
+  if (n_positions == 0) return YSCV_HIP_OK;
+  const size_t elems = (size_t)batch * n_positions * c.n_kv_heads * c.head_dim;
+  DevBuf dk, dv;
+  YSCV_TRY(dk.alloc(elems * 2));
+  YSCV_TRY(dv.alloc(elems * 2));
+  DEC_HIP(hipMemcpy(dk.p, k_f16, elems * 2, hipMemcpyHostToDevice));
+  DEC_HIP(hipMemcpy(dv.p, v_f16, elems * 2, hipMemcpyHostToDevice));
+  auto &L = d->layers[layer];
+  YSCV_TRY(launch_kv_relayout(dk.as<_Float16>(), dv.as<_Float16>(), batch, n_positions, c.n_kv_heads, c.head_dim,
+                              c.max_ctx, L.kc, L.vc, nullptr));
+  DEC_HIP(hipDeviceSynchronize());
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_reset(yscv_hip_decoder *d, int32_t batch, int32_t start_pos, const int32_t *tokens_host) {
+  YSCV_REQUIRE(d && tokens_host, "null argument");
+  const auto &c = d->cfg;
+  YSCV_REQUIRE(batch >= 1 && batch <= c.max_batch, "batch %d out of range 1..%d", batch, c.max_batch);
+  YSCV_REQUIRE(start_pos >= 0 && start_pos < c.max_ctx, "start position %d out of range", start_pos);
+  d->batch = batch;
+  DEC_HIP(hipMemcpy(d->tokens, tokens_host, (size_t)batch * 4, hipMemcpyHostToDevice));
+  DEC_HIP(hipMemcpy(d->pos, &start_pos, 4, hipMemcpyHostToDevice));
+  const int32_t zero = 0;
+  DEC_HIP(hipMemcpy(d->step, &zero, 4, hipMemcpyHostToDevice));
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_graph, void *stream) {
+  YSCV_REQUIRE(d != nullptr, "null decoder");
+  YSCV_REQUIRE(d->finalized, "decoder weights are not finalized");
+  YSCV_REQUIRE(d->batch >= 1, "call yscv_hip_decoder_reset first");
+  YSCV_REQUIRE(n_steps >= 0, "negative step count");
+  hipStream_t s = as_stream(stream);
+  // host-side bound check: the cache must hold every position this run appends
+  int32_t pos = 0, step = 0;
+  DEC_HIP(hipStreamSynchronize(s));
+  DEC_HIP(hipMemcpy(&pos, d->pos, 4, hipMemcpyDeviceToHost));
+  DEC_HIP(hipMemcpy(&step, d->step, 4, hipMemcpyDeviceToHost));
+  YSCV_REQUIRE(pos + n_steps <= d->cfg.max_ctx, "KV cache overflow: position %d + %d steps > max_ctx %d", pos, n_steps,
+               d->cfg.max_ctx);
+  YSCV_REQUIRE(step + n_steps <= d->cfg.max_steps, "token history overflow: %d + %d > max_steps %d", step, n_steps,
+               d->cfg.max_steps);
+  if (!use_graph) {
+    for (int i = 0; i < n_steps; i++) YSCV_TRY(enqueue_step(d, d->batch, s));
+    return YSCV_HIP_OK;
+  }
+  if (!d->graph_exec || d->graph_batch != d->batch) {
+    if (d->graph_exec) (void)hipGraphExecDestroy(d->graph_exec);
+    if (d->graph) (void)hipGraphDestroy(d->graph);
+    d->graph_exec = nullptr;
+    d->graph = nullptr;
+    hipStream_t cs = nullptr;
+    DEC_HIP(hipStreamCreateWithFlags(&cs, hipStreamNonBlocking));
+    hipError_t e = hipStreamBeginCapture(cs, hipStreamCaptureModeThreadLocal);
+    int32_t st = YSCV_HIP_OK;
+    if (e == hipSuccess) {
+      st = enqueue_step(d, d->batch, cs);
+      hipError_t e2 = hipStreamEndCapture(cs, &d->graph);
+      if (st == YSCV_HIP_OK && e2 != hipSuccess) e = e2;
+    }
+    if (st == YSCV_HIP_OK && e == hipSuccess) e = hipGraphInstantiate(&d->graph_exec, d->graph, nullptr, nullptr, 0);
+    (void)hipStreamDestroy(cs);
+    if (st != YSCV_HIP_OK) return st;
+    if (e != hipSuccess) return set_error(YSCV_HIP_ERR_DEVICE, "graph capture failed: %s", hipGetErrorString(e));
+    d->graph_batch = d->batch;
+  }
+  for (int i = 0; i < n_steps; i++) DEC_HIP(hipGraphLaunch(d->graph_exec, s));
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_read_tokens(yscv_hip_decoder *d, int32_t first_step, int32_t n_steps, int32_t *out_host) {
+  YSCV_REQUIRE(d && out_host, "null argument");
+  YSCV_REQUIRE(first_step >= 0 && n_steps >= 0 && first_step + n_steps <= d->cfg.max_steps, "step range out of bounds");
+  DEC_HIP(hipDeviceSynchronize());
+  DEC_HIP(hipMemcpy(out_host, d->history + (size_t)first_step * d->batch, (size_t)n_steps * d->batch * 4,
+                    hipMemcpyDeviceToHost));
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_read_logits(yscv_hip_decoder *d, float *out_host) {
+  YSCV_REQUIRE(d && out_host, "null argument");
+  DEC_HIP(hipDeviceSynchronize());
+  DEC_HIP(hipMemcpy(out_host, d->logits, (size_t)d->batch * d->cfg.vocab * 4, hipMemcpyDeviceToHost));
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_weight_bytes(const yscv_hip_decoder *d, size_t *bytes) {
+  YSCV_REQUIRE(d && bytes, "null argument");
+  *bytes = d->weight_bytes;
+  return YSCV_HIP_OK;
+}
+
+}  // extern "C"

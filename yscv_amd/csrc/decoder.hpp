@@ -1,0 +1,24 @@
+// Launchers of the decode-step glue kernels (decoder_kernels.hip), used by decoder.hip.
+#pragma once
+
+#include "common.hpp"
+
+namespace yscv {
+
+int32_t launch_embed(const int32_t *tokens, const _Float16 *table, int batch, int d, int vocab, float *h,
+                     hipStream_t s);
+int32_t launch_rmsnorm(const float *h, const float *gamma, int batch, int d, float eps, _Float16 *out,
+                       hipStream_t s);
+int32_t launch_rope_append(_Float16 *qkv, const int32_t *pos_ptr, int batch, int hq, int hkv, int hd, float theta,
+                           int max_ctx, _Float16 *kc, _Float16 *vc, hipStream_t s);
+int32_t launch_kv_relayout(const _Float16 *k_nat, const _Float16 *v_nat, int batch, int npos, int hkv, int hd,
+                           int max_ctx, _Float16 *kc, _Float16 *vc, hipStream_t s);
+int32_t launch_attention(const _Float16 *qkv, const _Float16 *kc, const _Float16 *vc, const int32_t *pos_ptr,
+                         int batch, int hq, int hkv, int hd, int max_ctx, float *part, _Float16 *out,
+                         hipStream_t s);
+int32_t launch_argmax(const float *logits, int batch, int vocab, int32_t *tokens, int32_t *history,
+                      int32_t *step_ptr, int max_steps, hipStream_t s);
+int32_t launch_advance(int32_t *pos_ptr, int32_t *step_ptr, hipStream_t s);
+int32_t launch_kv_random_fill(_Float16 *buf, size_t n, uint64_t seed, hipStream_t s);
+
+}  // namespace yscv

@@ -1,0 +1,421 @@
+// Glue kernels of the Llama-style decode step around the int4 projections: embedding lookup,
+// RMSNorm, rotary embedding + KV-cache append, single-token grouped-query attention over an fp16
+// KV cache, greedy pick.  Reference semantics (tolerance-checked, these use libm-class functions):
+//   RMSNorm  y = x * (1/sqrt(mean(x^2) + eps)) * gamma   crates/yscv-kernels/src/ops/norm.rs:1497-1518
+//   RoPE     rotate-half pairs (i, i + d/2), inv_freq[i] = 1/theta^(2i/d), angle = pos * inv_freq[i]
+//                                                        crates/yscv-kernels/src/ops/rope.rs:24-117
+//   GQA      kv_h = q_h / (Hq/Hkv), scores * 1/sqrt(d), max-subtracted softmax
+//                                                        crates/yscv-onnx/src/runner/linear.rs:552-646
+//   greedy   last index among equal maxima              apps/llm-bench/src/main.rs:538-543
+// The reference GQA op has no mask and no cache; attending to every cached position up to and
+// including the current token is the causal decode the llm-bench harness gets from its ONNX graph.
+//
+// KV cache layout (per layer, fp16), chosen so that both attention matmuls run on the matrix
+// cores with fully coalesced loads:
+//   K: [batch][kv_head][pos][head_dim]                      one 256 B row per position
+//   V: [batch][kv_head][pos / 8][head_dim][8]               8 positions interleaved per d
+// so a lane of v_mfma_f32_16x16x32_f16 reads 8 consecutive d of one position (K, B operand of
+// Q K^T) or 8 consecutive positions of one d (V, B operand of P V) as one 128-bit load.
+#include "decoder.hpp"
+#include "int4_common.hpp"
+
+namespace yscv {
+
+// ---- embedding: h[b][:] = table[token[b]][:] (fp16 -> f32 residual stream) ----------------------
+__global__ void embed_kernel(const int32_t *__restrict__ tokens, const _Float16 *__restrict__ table, int d,
+                             int vocab, float *__restrict__ h) {
+  const int b = blockIdx.x;
+  int tok = tokens[b];
+  tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+  for (int i = threadIdx.x; i < d; i += blockDim.x) h[(size_t)b * d + i] = (float)table[(size_t)tok * d + i];
+}
+
+// ---- RMSNorm: f32 residual -> fp16 normalised activations -----------------------------------------
+__global__ void __launch_bounds__(256) rmsnorm_kernel(const float *__restrict__ h, const float *__restrict__ gamma,
+                                                      int d, float eps, _Float16 *__restrict__ out) {
+  __shared__ float red[4];
+  const int b = blockIdx.x;
+  const float *row = h + (size_t)b * d;
+  float ss = 0.0f;
+  for (int i = threadIdx.x * 4; i < d; i += blockDim.x * 4) {
+    float4_t v = *reinterpret_cast<const float4_t *>(row + i);
+    ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+  }
+  for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  ss = red[0] + red[1] + red[2] + red[3];
+  const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+  for (int i = threadIdx.x * 4; i < d; i += blockDim.x * 4) {
+    float4_t v = *reinterpret_cast<const float4_t *>(row + i);
+    float4_t g = *reinterpret_cast<const float4_t *>(gamma + i);
+    half4_t o;
+#pragma unroll
+    for (int e = 0; e < 4; e++) o[e] = (_Float16)(v[e] * inv * g[e]);
+    *reinterpret_cast<half4_t *>(out + (size_t)b * d + i) = o;
+  }
+}
+
+// ---- RoPE on q (in place) and k, then append k / v to the cache -------------------------------------
+// qkv: [batch][(Hq + 2*Hkv) * D] fp16, q heads first, then k heads, then v heads.
+// one workgroup per (batch row, head slot); head slots: Hq q heads, Hkv k heads, Hkv v heads.
+__global__ void __launch_bounds__(64) rope_append_kernel(_Float16 *__restrict__ qkv, const int32_t *__restrict__ pos_ptr,
+                                                         int hq, int hkv, int hd, float theta, int max_ctx,
+                                                         _Float16 *__restrict__ kc, _Float16 *__restrict__ vc) {
+  const int b = blockIdx.y;
+  const int slot = blockIdx.x;
+  const int pos = *pos_ptr;
+  const int row_elems = (hq + 2 * hkv) * hd;
+  _Float16 *src = qkv + (size_t)b * row_elems + (size_t)slot * hd;
+  const int half_d = hd / 2;
+  if (slot < hq + hkv) {
+    // rotate-half: (x[i], x[i + d/2]) -> (x0 cos - x1 sin, x0 sin + x1 cos)
+    for (int i = threadIdx.x; i < half_d; i += blockDim.x) {
+      const float inv_freq = 1.0f / powf(theta, (float)(2 * i) / (float)hd);
+      const float ang = inv_freq * (float)pos;
+      float sn, cs;
+      sincosf(ang, &sn, &cs);
+      const float x0 = (float)src[i], x1 = (float)src[i + half_d];
+      const _Float16 y0 = (_Float16)(x0 * cs - x1 * sn), y1 = (_Float16)(x0 * sn + x1 * cs);
+      if (slot < hq) {
+        src[i] = y0;
+        src[i + half_d] = y1;
+      } else {
+        const int kvh = slot - hq;
+        _Float16 *dst = kc + (((size_t)b * hkv + kvh) * max_ctx + pos) * hd;
+        dst[i] = y0;
+        dst[i + half_d] = y1;
+      }
+    }
+  } else {
+    const int kvh = slot - hq - hkv;
+    _Float16 *dst = vc + ((((size_t)b * hkv + kvh) * (max_ctx / 8) + pos / 8) * hd) * 8 + (pos & 7);
+    for (int i = threadIdx.x; i < hd; i += blockDim.x) dst[(size_t)i * 8] = src[i];
+  }
+}
+
+// natural [batch][pos][kv_head][d] fp16 (host order) -> the two cache layouts, for positions [0, npos)
+__global__ void kv_relayout_kernel(const _Float16 *__restrict__ k_nat, const _Float16 *__restrict__ v_nat, int batch,
+                                   int npos, int hkv, int hd, int max_ctx, _Float16 *__restrict__ kc,
+                                   _Float16 *__restrict__ vc) {
+  const size_t total = (size_t)batch * npos * hkv * hd;
+  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * blockDim.x) {
+    const int i = idx % hd;
+    const int kvh = (idx / hd) % hkv;
+    const int pos = (idx / hd / hkv) % npos;
+    const int b = idx / hd / hkv / npos;
+    kc[(((size_t)b * hkv + kvh) * max_ctx + pos) * hd + i] = k_nat[idx];
+    vc[((((size_t)b * hkv + kvh) * (max_ctx / 8) + pos / 8) * hd + i) * 8 + (pos & 7)] = v_nat[idx];
+  }
+}
+
+// ---- single-token GQA attention, split over the context ----------------------------------------------
+// grid (chunks, Hkv, batch), 4 waves per workgroup, each wave owns 32 consecutive positions and the
+// GROUP = Hq/Hkv (<= 4) query heads that share this kv head.  Per wave:
+//   S = Q K^T   two 16-position blocks x 4 MFMAs (k = 128 d), Q rows sit at MFMA rows 4*h
+//   online-softmax statistics per head over its 32 positions
+//   O = P V     eight 16-wide d tiles x 1 MFMA (k = 32 positions), P as fp16 through LDS
+// then the 4 waves merge in LDS and write one (max, sum, o[128]) partial per (batch, head, chunk).
+constexpr int ATT_WAVES = 4;
+constexpr int ATT_POS_PER_WAVE = 32;
+constexpr int ATT_CHUNK = ATT_WAVES * ATT_POS_PER_WAVE;  // 128 positions per workgroup
+
+__global__ void __launch_bounds__(256) attn_partial_kernel(const _Float16 *__restrict__ qkv,
+                                                           const _Float16 *__restrict__ kc,
+                                                           const _Float16 *__restrict__ vc,
+                                                           const int32_t *__restrict__ pos_ptr, int hq, int hkv,
+                                                           int max_ctx, int max_chunks, float scale,
+                                                           float *__restrict__ part) {
+  constexpr int HD = 128;
+  __shared__ __attribute__((aligned(16))) _Float16 p_lds[ATT_WAVES][4][32];
+  __shared__ float w_m[ATT_WAVES][4], w_l[ATT_WAVES][4];
+  __shared__ float w_o[ATT_WAVES][4][HD];
+  const int chunk = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, c = lane >> 4;
+  const int group = hq / hkv;
+  const int n_ctx = *pos_ptr + 1;  // the current token was appended before this kernel
+  const int p0 = chunk * ATT_CHUNK + wave * ATT_POS_PER_WAVE;
+  const int row_elems = (hq + 2 * hkv) * HD;
+  const bool wave_live = p0 < n_ctx;
+
+  float m_h = -INFINITY, l_h = 0.0f;   // statistics of head c (lane group) -- valid for c < group
+  float o_acc[8];
+#pragma unroll
+  for (int t = 0; t < 8; t++) o_acc[t] = 0.0f;
+
+  if (wave_live) {
+    // Q operand: MFMA row 4*h carries head h of this group; lane (r, c) holds d = 32c + 8j + 0..7
+    half8_t qa[4];
+    {
+      const int h = r >> 2;
+      const bool valid = ((r & 3) == 0) && h < group;
+      const _Float16 *qsrc = qkv + (size_t)b * row_elems + (size_t)(kvh * group + h) * HD + 32 * c;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+        qa[j] = valid ? *reinterpret_cast<const half8_t *>(qsrc + 8 * j) : z;
+      }
+    }
+    const _Float16 *kbase = kc + (((size_t)b * hkv + kvh) * max_ctx + p0) * HD;
+    const _Float16 *vbase = vc + ((((size_t)b * hkv + kvh) * (max_ctx / 8) + p0 / 8) * HD) * 8;
+    // issue every load of this wave up front: 8 KiB of K, 8 KiB of V
+    half8_t kf[2][4], vf[8];
+#pragma unroll
+    for (int pb = 0; pb < 2; pb++)
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        kf[pb][j] = *reinterpret_cast<const half8_t *>(kbase + (size_t)(pb * 16 + r) * HD + 32 * c + 8 * j);
+#pragma unroll
+    for (int t = 0; t < 8; t++)
+      vf[t] = *reinterpret_cast<const half8_t *>(vbase + ((size_t)c * HD + t * 16 + r) * 8);
+
+    float s[2];
+#pragma unroll
+    for (int pb = 0; pb < 2; pb++) {
+      float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int j = 0; j < 4; j++) d = __builtin_amdgcn_mfma_f32_16x16x32_f16(qa[j], kf[pb][j], d, 0, 0, 0);
+      // lane (r, c): score of head c at position p0 + 16*pb + r
+      const int p = p0 + pb * 16 + r;
+      s[pb] = (p < n_ctx) ? d[0] * scale : -INFINITY;
+    }
+    float mx = fmaxf(s[0], s[1]);
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));  // within the 16 lanes of a group
+    const float e0 = (s[0] == -INFINITY) ? 0.0f : __expf(s[0] - mx);
+    const float e1 = (s[1] == -INFINITY) ? 0.0f : __expf(s[1] - mx);
+    float sum = e0 + e1;
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    m_h = mx;
+    l_h = sum;
+    if (c < 4) {
+      p_lds[wave][c][r] = (_Float16)e0;
+      p_lds[wave][c][16 + r] = (_Float16)e1;
+    }
+    __builtin_amdgcn_wave_barrier();  // LDS is in order per wave: the reads below see the writes above
+    // P operand: MFMA row 4*h = head h, lane (r, c) holds positions 8c .. 8c+7 of this wave's 32
+    half8_t pa = {0, 0, 0, 0, 0, 0, 0, 0};
+    if ((r & 3) == 0 && (r >> 2) < group) pa = *reinterpret_cast<const half8_t *>(&p_lds[wave][r >> 2][8 * c]);
+    // V rows past the context hold stale or unwritten bits; their weights are exactly 0, but 0 * NaN
+    // would poison the sum, so blank the operand where the whole 8-position slab is out of range.
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      half8_t vv = vf[t];
+      if (p0 + 8 * c >= n_ctx) vv = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      else if (p0 + 8 * c + 8 > n_ctx) {
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+          if (p0 + 8 * c + e >= n_ctx) vv[e] = (_Float16)0.0f;
+      }
+      float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
+      d = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vv, d, 0, 0, 0);
+      o_acc[t] = d[0];  // lane (r, c): o of head c at d = 16 t + r
+    }
+  }
+
+  // ---- merge the 4 waves ---------------------------------------------------------------------------
+  if (c < 4) {
+    if (r == 0) {
+      w_m[wave][c] = m_h;
+      w_l[wave][c] = l_h;
+    }
+#pragma unroll
+    for (int t = 0; t < 8; t++) w_o[wave][c][t * 16 + r] = o_acc[t];
+  }
+  __syncthreads();
+  // thread -> (head h = tid / 64 ... ) : 4 heads x 128 d = 512 values, 256 threads -> 2 each
+  for (int idx = threadIdx.x; idx < group * HD; idx += blockDim.x) {
+    const int h = idx / HD, dd = idx % HD;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < ATT_WAVES; w++) mx = fmaxf(mx, w_m[w][h]);
+    float l = 0.0f, o = 0.0f;
+#pragma unroll
+    for (int w = 0; w < ATT_WAVES; w++) {
+      const float f = (w_m[w][h] == -INFINITY) ? 0.0f : __expf(w_m[w][h] - mx);
+      l += w_l[w][h] * f;
+      o += w_o[w][h][dd] * f;
+    }
+    const int head = kvh * group + h;
+    float *dst = part + (((size_t)b * hq + head) * max_chunks + chunk) * (HD + 2);
+    dst[2 + dd] = o;
+    if (dd == 0) {
+      dst[0] = mx;
+      dst[1] = l;
+    }
+  }
+}
+
+// merge the per-chunk partials: one workgroup per (batch, head), 128 threads = one per d
+__global__ void __launch_bounds__(128) attn_combine_kernel(const float *__restrict__ part,
+                                                           const int32_t *__restrict__ pos_ptr, int hq,
+                                                           int max_chunks, _Float16 *__restrict__ out) {
+  constexpr int HD = 128;
+  const int head = blockIdx.x, b = blockIdx.y;
+  const int n_ctx = *pos_ptr + 1;
+  const int chunks = (n_ctx + ATT_CHUNK - 1) / ATT_CHUNK;
+  const float *src = part + (((size_t)b * hq + head) * max_chunks) * (HD + 2);
+  float mx = -INFINITY;
+  for (int ch = 0; ch < chunks; ch++) mx = fmaxf(mx, src[(size_t)ch * (HD + 2)]);
+  float l = 0.0f, o = 0.0f;
+  for (int ch = 0; ch < chunks; ch++) {
+    const float *p = src + (size_t)ch * (HD + 2);
+    const float f = (p[0] == -INFINITY) ? 0.0f : __expf(p[0] - mx);
+    l += p[1] * f;
+    o += p[2 + threadIdx.x] * f;
+  }
+  const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+  out[((size_t)b * hq + head) * HD + threadIdx.x] = (_Float16)(o * inv);
+}
+
+// ---- greedy pick: last index among equal maxima; also records the token and advances the position ------
+__global__ void __launch_bounds__(1024) argmax_kernel(const float *__restrict__ logits, int vocab,
+                                                      int32_t *__restrict__ tokens, int32_t *__restrict__ history,
+                                                      int32_t *__restrict__ step_ptr, int batch, int max_steps) {
+  __shared__ float sv[16];
+  __shared__ int si[16];
+  const int b = blockIdx.x;
+  const float *row = logits + (size_t)b * vocab;
+  float best = -INFINITY;
+  int bi = -1;
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+    const float v = row[i];
+    // max_by keeps the later element unless the earlier one compares Greater; NaN compares Equal
+    if (bi < 0 || !(best > v)) {
+      best = v;
+      bi = i;
+    }
+  }
+  // combine: higher value wins, equal values -> larger index; an unordered pair keeps the larger index too
+  auto better = [](float va, int ia, float vb, int ib) {
+    if (ia < 0) return false;
+    if (ib < 0) return true;
+    if (va > vb) return true;
+    if (vb > va) return false;
+    return ia > ib;
+  };
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(best, off, 64);
+    const int oi = __shfl_xor(bi, off, 64);
+    if (better(ov, oi, best, bi)) {
+      best = ov;
+      bi = oi;
+    }
+  }
+  if ((threadIdx.x & 63) == 0) {
+    sv[threadIdx.x >> 6] = best;
+    si[threadIdx.x >> 6] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (unsigned w = 1; w < (blockDim.x >> 6); w++)
+      if (better(sv[w], si[w], best, bi)) {
+        best = sv[w];
+        bi = si[w];
+      }
+    tokens[b] = bi;
+    const int step = *step_ptr;
+    if (history && step < max_steps) history[(size_t)step * batch + b] = bi;
+  }
+}
+
+// pos += 1, step += 1 (one thread) -- separate so every other kernel of the step sees one value
+__global__ void advance_kernel(int32_t *pos_ptr, int32_t *step_ptr) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    *pos_ptr += 1;
+    *step_ptr += 1;
+  }
+}
+
+// deterministic pseudo-random fill of a cache region with ~N(0,1) fp16 (sum of uniforms), for benchmarks
+__global__ void kv_random_fill_kernel(_Float16 *__restrict__ buf, size_t n, uint64_t seed) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    uint64_t z = (i + 1) * 0x9E3779B97F4A7C15ull + seed;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    // four 16-bit uniforms -> approximately normal with unit variance
+    float u = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 4; e++) u += (float)((z >> (16 * e)) & 0xFFFF) * (1.0f / 65536.0f);
+    buf[i] = (_Float16)((u - 2.0f) * 1.7320508f);
+  }
+}
+
+// ---- launchers -------------------------------------------------------------------------------------------
+int32_t launch_embed(const int32_t *tokens, const _Float16 *table, int batch, int d, int vocab, float *h,
+                     hipStream_t s) {
+  hipLaunchKernelGGL(embed_kernel, dim3(batch), dim3(256), 0, s, tokens, table, d, vocab, h);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_rmsnorm(const float *h, const float *gamma, int batch, int d, float eps, _Float16 *out,
+                       hipStream_t s) {
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3(batch), dim3(256), 0, s, h, gamma, d, eps, out);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_rope_append(_Float16 *qkv, const int32_t *pos_ptr, int batch, int hq, int hkv, int hd, float theta,
+                           int max_ctx, _Float16 *kc, _Float16 *vc, hipStream_t s) {
+  hipLaunchKernelGGL(rope_append_kernel, dim3(hq + 2 * hkv, batch), dim3(64), 0, s, qkv, pos_ptr, hq, hkv, hd,
+                     theta, max_ctx, kc, vc);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_kv_relayout(const _Float16 *k_nat, const _Float16 *v_nat, int batch, int npos, int hkv, int hd,
+                           int max_ctx, _Float16 *kc, _Float16 *vc, hipStream_t s) {
+  size_t total = (size_t)batch * npos * hkv * hd;
+  size_t blocks = ceil_div(total, (size_t)256);
+  if (blocks > 65535) blocks = 65535;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(kv_relayout_kernel, dim3((unsigned)blocks), dim3(256), 0, s, k_nat, v_nat, batch, npos, hkv,
+                     hd, max_ctx, kc, vc);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_attention(const _Float16 *qkv, const _Float16 *kc, const _Float16 *vc, const int32_t *pos_ptr,
+                         int batch, int hq, int hkv, int hd, int max_ctx, float *part, _Float16 *out,
+                         hipStream_t s) {
+  if (hd != 128) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "attention kernel is built for head_dim 128, got %d", hd);
+  if (hq % hkv != 0 || hq / hkv > 4)
+    return set_error(YSCV_HIP_ERR_UNSUPPORTED, "attention kernel handles 1..4 query heads per kv head");
+  const int max_chunks = max_ctx / ATT_CHUNK;
+  const float scale = 1.0f / sqrtf((float)hd);
+  hipLaunchKernelGGL(attn_partial_kernel, dim3(max_chunks, hkv, batch), dim3(256), 0, s, qkv, kc, vc, pos_ptr, hq,
+                     hkv, max_ctx, max_chunks, scale, part);
+  YSCV_HIP_TRY(hipGetLastError());
+  hipLaunchKernelGGL(attn_combine_kernel, dim3(hq, batch), dim3(128), 0, s, part, pos_ptr, hq, max_chunks, out);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_argmax(const float *logits, int batch, int vocab, int32_t *tokens, int32_t *history,
+                      int32_t *step_ptr, int max_steps, hipStream_t s) {
+  hipLaunchKernelGGL(argmax_kernel, dim3(batch), dim3(1024), 0, s, logits, vocab, tokens, history, step_ptr, batch,
+                     max_steps);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_advance(int32_t *pos_ptr, int32_t *step_ptr, hipStream_t s) {
+  hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, s, pos_ptr, step_ptr);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_kv_random_fill(_Float16 *buf, size_t n, uint64_t seed, hipStream_t s) {
+  size_t blocks = ceil_div(n, (size_t)256);
+  if (blocks > 65535) blocks = 65535;
+  hipLaunchKernelGGL(kv_random_fill_kernel, dim3((unsigned)blocks), dim3(256), 0, s, buf, n, seed);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+}  // namespace yscv

@@ -217,7 +217,7 @@ __global__ void __launch_bounds__(256) int4_gemm_kernel(GemmArgs a) {
     for (int i = 0; i < 4; i++) {
       const int row = m0 + mt * 16 + c * 4 + i;
       if (row >= a.m) continue;
-      const float rs = a.row_scale[row];
+      const float rs = a.row_scale ? a.row_scale[row] : 1.0f;
 #pragma unroll
       for (int t = 0; t < G_NTW; t++) {
         const int col = (nt0 + t) * 16 + r;

@@ -137,46 +137,99 @@ int32_t launch_xor88(uint8_t *buf, size_t bytes, hipStream_t s) {
 // fp16 `hi` and, for f32 input, a second fp16 `lo` = x' - hi.  hi + lo carries ~22
 // significant bits, f16/bf16 inputs are represented exactly by hi alone.  The power of
 // two is returned so the GEMV/GEMM epilogue can multiply it back (exactly).
-__global__ void __launch_bounds__(256) x_prep_kernel(const void *__restrict__ x, int x_dtype, size_t k,
-                                                     size_t k_pad, int split, _Float16 *__restrict__ xh,
-                                                     _Float16 *__restrict__ xl,
-                                                     float *__restrict__ row_scale) {
-  __shared__ float red[4];
-  size_t row = blockIdx.x;
-  size_t base = row * k;
+// load 8 consecutive activations starting at element `idx` (idx % 8 == 0 when VEC)
+template <bool VEC>
+__device__ __forceinline__ void load8(const void *x, size_t idx, int dtype, size_t limit, float v[8]) {
+  if constexpr (VEC) {
+    if (dtype == YSCV_HIP_F32) {
+      const float4_t *p = reinterpret_cast<const float4_t *>(reinterpret_cast<const float *>(x) + idx);
+      float4_t a = p[0], b = p[1];
+      v[0] = a[0]; v[1] = a[1]; v[2] = a[2]; v[3] = a[3];
+      v[4] = b[0]; v[5] = b[1]; v[6] = b[2]; v[7] = b[3];
+    } else if (dtype == YSCV_HIP_F16) {
+      half8_t h = *reinterpret_cast<const half8_t *>(reinterpret_cast<const _Float16 *>(x) + idx);
+#pragma unroll
+      for (int i = 0; i < 8; i++) v[i] = (float)h[i];
+    } else {
+      uint4_t u = *reinterpret_cast<const uint4_t *>(reinterpret_cast<const uint16_t *>(x) + idx);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        v[2 * i] = __uint_as_float(u[i] << 16);
+        v[2 * i + 1] = __uint_as_float(u[i] & 0xFFFF0000u);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = (idx + i < limit) ? load_in(x, idx + i, dtype) : 0.0f;
+  }
+}
+
+template <bool VEC>
+__global__ void __launch_bounds__(1024) x_prep_kernel(const void *__restrict__ x, int x_dtype, size_t k,
+                                                      size_t k_pad, int split, _Float16 *__restrict__ xh,
+                                                      _Float16 *__restrict__ xl,
+                                                      float *__restrict__ row_scale) {
+  __shared__ float red[16];
+  const size_t row = blockIdx.x;
+  const size_t base = row * k;
+  const size_t chunks = k_pad / 8;
+  // pass 1: abs-max of the row (values stay in registers when the row fits one sweep)
   float amax = 0.0f;
-  for (size_t i = threadIdx.x; i < k; i += blockDim.x) {
-    float v = fabsf(load_in(x, base + i, x_dtype));
-    amax = fmaxf(amax, v);  // NaN is ignored here; it still propagates through the values
+  for (size_t ch = threadIdx.x; ch < chunks; ch += blockDim.x) {
+    if (ch * 8 < k) {
+      float v[8];
+      load8<VEC>(x, base + ch * 8, x_dtype, base + k, v);
+#pragma unroll
+      for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(v[i]));  // NaN is ignored here, kept in the values
+    }
   }
   for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
   __syncthreads();
-  amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-  int e = 0;
+  amax = 0.0f;
+  for (unsigned w = 0; w < (blockDim.x >> 6); w++) amax = fmaxf(amax, red[w]);
+  int e = 14;
   if (amax > 0.0f && amax < 3.0e38f) {
     (void)frexpf(amax, &e);  // amax = f * 2^e, f in [0.5, 1)
     e -= 1;                  // amax in [2^e, 2^(e+1))
-  } else {
-    e = 14;  // all-zero or non-finite row: leave the values alone
-  }
+  }  // else: all-zero or non-finite row, leave the values alone
   int shift = 14 - e;
   shift = shift > 100 ? 100 : (shift < -100 ? -100 : shift);
-  float up = ldexpf(1.0f, shift);
+  const float up = ldexpf(1.0f, shift);
   if (threadIdx.x == 0) row_scale[row] = ldexpf(1.0f, -shift);
-  size_t obase = row * k_pad;
-  for (size_t i = threadIdx.x; i < k_pad; i += blockDim.x) {
-    float v = (i < k) ? load_in(x, base + i, x_dtype) * up : 0.0f;
-    _Float16 h = (_Float16)v;
-    xh[obase + i] = h;
-    if (split == 2) xl[obase + i] = (_Float16)(v - (float)h);
+  const size_t obase = row * k_pad;
+  for (size_t ch = threadIdx.x; ch < chunks; ch += blockDim.x) {
+    float v[8];
+    if (ch * 8 < k) {
+      load8<VEC>(x, base + ch * 8, x_dtype, base + k, v);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; i++) v[i] = 0.0f;
+    }
+    half8_t h, l;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const float s = v[i] * up;
+      h[i] = (_Float16)s;
+      l[i] = (_Float16)(s - (float)h[i]);
+    }
+    *reinterpret_cast<half8_t *>(xh + obase + ch * 8) = h;
+    if (split == 2) *reinterpret_cast<half8_t *>(xl + obase + ch * 8) = l;
   }
 }
 
 int32_t launch_x_prep(const void *x, int x_dtype, size_t m, size_t k, size_t k_pad, int split,
                       _Float16 *xh, _Float16 *xl, float *row_scale, hipStream_t s) {
-  hipLaunchKernelGGL(x_prep_kernel, dim3((unsigned)m), dim3(256), 0, s, x, x_dtype, k, k_pad, split,
-                     xh, xl, row_scale);
+  const size_t esz = x_dtype == YSCV_HIP_F32 ? 4 : 2;
+  const bool vec = (k % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) && ((k * esz) % 16 == 0);
+  size_t chunks = k_pad / 8;
+  unsigned threads = chunks >= 1024 ? 1024 : (unsigned)round_up(chunks < 64 ? 64 : chunks, 64);
+  if (vec)
+    hipLaunchKernelGGL(x_prep_kernel<true>, dim3((unsigned)m), dim3(threads), 0, s, x, x_dtype, k, k_pad, split,
+                       xh, xl, row_scale);
+  else
+    hipLaunchKernelGGL(x_prep_kernel<false>, dim3((unsigned)m), dim3(threads), 0, s, x, x_dtype, k, k_pad,
+                       split, xh, xl, row_scale);
   YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
 }

@@ -24,6 +24,8 @@
 
 namespace yscv {
 
+__device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
+
 struct SkinnyArgs {
   const uint8_t *tiles;
   const void *tscales;
@@ -40,6 +42,7 @@ struct SkinnyArgs {
   int k_pad;       // row stride of xh / xl
   int y_dtype;
   int ksg;
+  int epi;  // EPI_STORE / EPI_ADD_F32 / EPI_SWIGLU
 };
 
 // Scales of one (tile, row) kept in their storage type until used: 1, 2 or 4 values.
@@ -84,7 +87,7 @@ struct TileRegs {
   uint32_t z[TPW];
 };
 
-template <int TPW, int SPLIT, int NI, int GM, bool SF16>
+template <int TPW, int SPLIT, int NI, int GM, bool SF16, int P>
 __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
   extern __shared__ float red[];  // [2][waves][NI][64]
   const int lane = threadIdx.x & 63;
@@ -178,45 +181,87 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
         float v = 0.0f;
         for (int w = 0; w < waves; w++) v += buf[(w * NI + i) * 64 + lane];
         const int mrow = c * NI + i;
-        if (mrow < a.m && col < a.n) {
-          if (a.ksg > 1) {
-            a.partial[((size_t)blockIdx.y * a.m + mrow) * a.n + col] = v;
-          } else {
-            store_out(a.y, (size_t)mrow * a.n + col, v * a.row_scale[mrow], a.y_dtype);
+        const bool live = mrow < a.m && col < a.n;
+        if (a.ksg > 1) {
+          if (live) a.partial[((size_t)blockIdx.y * a.m + mrow) * a.n + col] = v;
+        } else {
+          if (a.row_scale && mrow < a.m) v *= a.row_scale[mrow];
+          if (a.epi == EPI_SWIGLU) {
+            // rows 2i / 2i+1 of the weight are gate_i / up_i: neighbours in the wave
+            const float up = __shfl_xor(v, 1, 64);
+            if (live && !(r & 1))
+              store_out(a.y, (size_t)mrow * (a.n >> 1) + (col >> 1), silu(v) * up, a.y_dtype);
+          } else if (a.epi == EPI_ADD_F32) {
+            if (live) {
+              float *dst = reinterpret_cast<float *>(a.y) + (size_t)mrow * a.n + col;
+              *dst = *dst + v;
+            }
+          } else if (live) {
+            store_out(a.y, (size_t)mrow * a.n + col, v, a.y_dtype);
           }
         }
       }
     }
   };
 
-  TileRegs<TPW, GM, SF16> ra, rb;
+  // Ring of P register slots: while one 16-row tile is being consumed, the loads of the next
+  // P-1 are in flight, so the memory pipeline never drains at the per-tile barrier.
+  TileRegs<TPW, GM, SF16> ring[P];
+  const int stride = gridDim.x;
   int nt = blockIdx.x;
+#pragma unroll
+  for (int sl = 0; sl < P; sl++) {
+    const int n = nt + sl * stride;
+    if (n < a.nt) issue(n, ring[sl]);
+  }
   int it = 0;
-  if (nt < a.nt) issue(nt, ra);
   while (nt < a.nt) {
-    int nx = nt + gridDim.x;
-    if (nx < a.nt) issue(nx, rb);
-    compute(nt, ra, it);
-    nt = nx;
-    it++;
-    if (nt >= a.nt) break;
-    nx = nt + gridDim.x;
-    if (nx < a.nt) issue(nx, ra);
-    compute(nt, rb, it);
-    nt = nx;
-    it++;
+#pragma unroll
+    for (int sl = 0; sl < P; sl++) {
+      if (nt < a.nt) {
+        compute(nt, ring[sl], it);
+        const int nn = nt + P * stride;
+        if (nn < a.nt) issue(nn, ring[sl]);
+        nt += stride;
+        it++;
+      }
+    }
   }
 }
 
-// partial [ksg][m][n] -> y[m][n], fixed summation order
+// partial [ksg][m][n] -> y, fixed summation order, same epilogues as the fused path
 __global__ void int4_skinny_finalize_kernel(const float *__restrict__ partial, int ksg, int m, int n,
-                                            const float *__restrict__ row_scale, void *y, int y_dtype) {
-  size_t total = (size_t)m * n;
+                                            const float *__restrict__ row_scale, void *y, int y_dtype, int epi) {
+  const size_t total = (size_t)m * n;
+  if (epi == EPI_SWIGLU) {
+    const size_t half_n = (size_t)(n >> 1);
+    for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < (size_t)m * half_n;
+         idx += (size_t)gridDim.x * blockDim.x) {
+      const size_t row = idx / half_n, j = idx % half_n;
+      float g = 0.0f, u = 0.0f;
+      for (int s = 0; s < ksg; s++) {
+        g += partial[(size_t)s * total + row * n + 2 * j];
+        u += partial[(size_t)s * total + row * n + 2 * j + 1];
+      }
+      if (row_scale) {
+        g *= row_scale[row];
+        u *= row_scale[row];
+      }
+      store_out(y, idx, silu(g) * u, y_dtype);
+    }
+    return;
+  }
   for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total;
        idx += (size_t)gridDim.x * blockDim.x) {
     float v = 0.0f;
     for (int s = 0; s < ksg; s++) v += partial[(size_t)s * total + idx];
-    store_out(y, idx, v * row_scale[idx / n], y_dtype);
+    if (row_scale) v *= row_scale[idx / n];
+    if (epi == EPI_ADD_F32) {
+      float *dst = reinterpret_cast<float *>(y) + idx;
+      *dst = *dst + v;
+    } else {
+      store_out(y, idx, v, y_dtype);
+    }
   }
 }
 
@@ -248,7 +293,7 @@ SkinnyPlan plan_int4_skinny(const yscv_hip_int4_weight *w, size_t m, int split, 
 template <int TPW, int SPLIT, int NI, int GM, bool SF16>
 static int32_t launch_one(const SkinnyArgs &a, const SkinnyPlan &plan, hipStream_t s) {
   size_t lds = (size_t)2 * plan.waves * NI * 64 * sizeof(float);
-  hipLaunchKernelGGL((int4_skinny_kernel<TPW, SPLIT, NI, GM, SF16>), dim3(plan.grid_x, plan.ksg),
+  hipLaunchKernelGGL((int4_skinny_kernel<TPW, SPLIT, NI, GM, SF16, (SPLIT == 2 ? 2 : 4)>), dim3(plan.grid_x, plan.ksg),
                      dim3(plan.waves * 64), lds, s, a);
   YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
@@ -263,7 +308,7 @@ static int32_t launch_gm(const SkinnyArgs &a, const SkinnyPlan &plan, int gm, bo
 
 int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan, const _Float16 *xh,
                            const _Float16 *xl, const float *row_scale, size_t k_pad, int split,
-                           void *y, int y_dtype, size_t m, float *partial, hipStream_t s) {
+                           void *y, int y_dtype, size_t m, float *partial, int epi, hipStream_t s) {
   if (!w->tiled) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "skinny int4 kernel needs the tiled layout");
   if (m == 0 || m > 16) return set_error(YSCV_HIP_ERR_INVALID_ARG, "skinny int4 kernel handles 1 <= m <= 16, got %zu", m);
   if (plan.ksg > 1 && !partial) return set_error(YSCV_HIP_ERR_INVALID_ARG, "k-split needs a partial buffer");
@@ -285,6 +330,9 @@ int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan
   a.k_pad = (int)k_pad;
   a.y_dtype = y_dtype;
   a.ksg = plan.ksg;
+  a.epi = epi;
+  if (epi == EPI_ADD_F32 && y_dtype != YSCV_HIP_F32) return set_error(YSCV_HIP_ERR_INVALID_ARG, "residual accumulation needs an f32 output");
+  if (epi == EPI_SWIGLU && (w->n & 1)) return set_error(YSCV_HIP_ERR_INVALID_ARG, "SwiGLU epilogue needs an even row count");
   const bool sf16 = w->scale_dtype == YSCV_HIP_F16;
   const bool small = m <= 4;
   int32_t st;
@@ -299,7 +347,7 @@ int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan
     int blocks = (int)ceil_div(total, (size_t)256);
     if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL(int4_skinny_finalize_kernel, dim3(blocks), dim3(256), 0, s, partial, plan.ksg,
-                       (int)m, (int)w->n, row_scale, y, y_dtype);
+                       (int)m, (int)w->n, row_scale, y, y_dtype, epi);
     YSCV_HIP_TRY(hipGetLastError());
   }
   return YSCV_HIP_OK;

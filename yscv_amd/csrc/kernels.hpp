@@ -53,6 +53,9 @@ int32_t launch_xor88(uint8_t *buf, size_t bytes, hipStream_t s);
 int32_t launch_x_prep(const void *x, int x_dtype, size_t m, size_t k, size_t k_pad, int split,
                       _Float16 *xh, _Float16 *xl, float *row_scale, hipStream_t s);
 
+// epilogues of the skinny kernel
+enum : int { EPI_STORE = 0, EPI_ADD_F32 = 1, EPI_SWIGLU = 2 };
+
 struct SkinnyPlan {
   int tpw;     // 128-k tiles per wave
   int waves;   // wavefronts per workgroup (= k-slices per workgroup)
@@ -63,12 +66,17 @@ struct SkinnyPlan {
 SkinnyPlan plan_int4_skinny(const yscv_hip_int4_weight *w, size_t m, int split, int num_cus);
 int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan, const _Float16 *xh,
                            const _Float16 *xl, const float *row_scale, size_t k_pad, int split,
-                           void *y, int y_dtype, size_t m, float *partial, hipStream_t s);
+                           void *y, int y_dtype, size_t m, float *partial, int epi, hipStream_t s);
 int32_t launch_int4_generic(const yscv_hip_int4_weight *w, const void *x, int x_dtype, void *y,
                             int y_dtype, size_t m, hipStream_t s);
 int32_t launch_int4_gemm(const yscv_hip_int4_weight *w, const _Float16 *xh, const _Float16 *xl,
                          const float *row_scale, size_t k_pad, int split, void *y, int y_dtype,
                          size_t m, hipStream_t s);
+
+// Whole int4 call (activation preparation + kernel) with caller-provided scratch; ws may be null.
+int32_t int4_workspace_bytes(const yscv_hip_int4_weight *w, size_t m, int x_dtype, int force, size_t *bytes);
+int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, void *y, int y_dtype, size_t m,
+                    int force, int epi, void *ws, size_t ws_bytes, hipStream_t s);
 
 int32_t launch_pack_int4_symmetric(const float *w, size_t m_w, size_t k, size_t g, uint8_t *packed,
                                    float *scales, hipStream_t s);

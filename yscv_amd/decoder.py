@@ -1,0 +1,89 @@
+"""Thin binding of the GPU-resident decoder (yscv_hip_decoder_* in include/yscv_hip.h)."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from .capi import DecoderConfig, lib
+
+KINDS = {"q": 0, "k": 1, "v": 2, "o": 3, "gate": 4, "up": 5, "down": 6, "lm_head": 7}
+NORMS = {"attn": 0, "ffn": 1, "final": 2}
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+class Decoder:
+    def __init__(self, **cfg):
+        self.cfg = dict(cfg)
+        c = DecoderConfig(**cfg)
+        h = C.c_void_p()
+        lib().decoder_create(C.byref(c), C.byref(h))
+        self._h = h
+        self.batch = 0
+
+    def set_linear(self, layer, kind, packed, scales16, n, k):
+        p = np.ascontiguousarray(packed, np.uint8)
+        s = np.ascontiguousarray(scales16)
+        assert s.dtype == np.float16
+        lib().decoder_set_linear(self._h, int(layer), KINDS[kind], _p(p), _p(s), C.c_size_t(n), C.c_size_t(k))
+
+    def set_norm(self, layer, kind, gamma):
+        g = np.ascontiguousarray(gamma, np.float32)
+        lib().decoder_set_norm(self._h, int(layer), NORMS[kind], _p(g))
+
+    def set_embedding(self, table16):
+        t = np.ascontiguousarray(table16)
+        assert t.dtype == np.float16
+        lib().decoder_set_embedding(self._h, _p(t))
+
+    def finalize(self):
+        lib().decoder_finalize(self._h)
+
+    def init_random(self, seed=0):
+        lib().decoder_init_random(self._h, C.c_uint64(seed))
+
+    def fill_kv_random(self, seed=0):
+        lib().decoder_fill_kv_random(self._h, C.c_uint64(seed))
+
+    def set_kv(self, layer, k16, v16):
+        k = np.ascontiguousarray(k16)
+        v = np.ascontiguousarray(v16)
+        assert k.dtype == np.float16 and v.dtype == np.float16 and k.shape == v.shape and k.ndim == 4
+        lib().decoder_set_kv(self._h, int(layer), _p(k), _p(v), int(k.shape[0]), int(k.shape[1]))
+
+    def reset(self, tokens, start_pos):
+        t = np.ascontiguousarray(tokens, np.int32)
+        self.batch = t.size
+        lib().decoder_reset(self._h, int(t.size), int(start_pos), _p(t))
+
+    def run(self, n_steps, use_graph=True, stream=None):
+        lib().decoder_run(self._h, int(n_steps), int(bool(use_graph)), C.c_void_p(stream) if stream else None)
+
+    def tokens(self, first_step, n_steps):
+        out = np.empty((n_steps, self.batch), np.int32)
+        lib().decoder_read_tokens(self._h, int(first_step), int(n_steps), _p(out))
+        return out
+
+    def logits(self):
+        out = np.empty((self.batch, self.cfg["vocab"]), np.float32)
+        lib().decoder_read_logits(self._h, _p(out))
+        return out
+
+    def weight_bytes(self) -> int:
+        b = C.c_size_t()
+        lib().decoder_weight_bytes(self._h, C.byref(b))
+        return b.value
+
+    def close(self):
+        if self._h:
+            lib().decoder_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
