@@ -1,0 +1,282 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-matmul hot path on one MI355X.
+
+Headline (BASELINE.json metric): int4 decode tokens/s on the 7B-shape Llama-style decoder
+(32 layers, d_model 4096, 32 q / 8 kv heads, head_dim 128, SwiGLU 14336, vocab 32000, every linear
+int4 with group size 32 and fp16 scales, fp16 KV cache pre-filled to context 2048), greedy, batch 1.
+One "step" = one decode step of the whole batch.  Weights are random-initialised on the device,
+inputs are synthetic, everything is resident in HBM before the timed region.
+
+The single JSON line also carries
+  roofline      -- the dominant kernel (the skinny int4 GEMV that runs every projection) against the
+                   8 TB/s HBM peak: algorithmic bytes per launch / its average launch duration, the
+                   latter measured here with HIP events around the projections of whole decode steps;
+  cpu_baseline  -- the restated reference CPU kernels timed on this host (bounded sample);
+  extra         -- batch-16 decode and the stand-alone kernels of the other BASELINE configs.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+MFMA_BF16_PEAK = 2500.0     # TFLOP/s dense (fp16 shares the rate)
+MFMA_I8_PEAK = 5000.0       # TOP/s dense
+
+CFG7B = dict(n_layers=32, d_model=4096, n_heads=32, n_kv_heads=8, head_dim=128, d_ff=14336, vocab=32000,
+             group_size=32, max_batch=16, max_ctx=2048 + 512, max_steps=1024, rope_theta=10000.0, rms_eps=1e-5)
+PREFILL = 2048
+
+
+def decode_bytes_per_step(cfg):
+    """Algorithmic bytes the projections of one decode step read: packed nibbles + fp16 scales."""
+    D, hd, g = cfg["d_model"], cfg["head_dim"], cfg["group_size"]
+    hq, hkv, ff = cfg["n_heads"] * hd, cfg["n_kv_heads"] * hd, cfg["d_ff"]
+    per_layer = (hq + 2 * hkv) * D + D * hq + 2 * ff * D + D * ff
+    params = cfg["n_layers"] * per_layer + cfg["vocab"] * D
+    return params // 2 + (params // g) * 2, params
+
+
+def event_time_ms(fn, torch):
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e)
+
+
+def bench_decode(dec, torch, batch, steps, warmup, stream_ptr):
+    import numpy as np
+
+    dec.reset(np.arange(1, batch + 1, dtype=np.int32), PREFILL)
+    dec.run(warmup, use_graph=True, stream=stream_ptr)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    dec.run(steps, use_graph=True, stream=stream_ptr)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    toks = dec.tokens(warmup, steps)
+    assert toks.shape == (steps, batch) and (toks >= 0).all() and (toks < dec.cfg["vocab"]).all()
+    return dt
+
+
+def bench_projections(dec, torch, batch, stream_ptr, reps=6):
+    """Average duration of one skinny-kernel launch over the projections of whole decode steps."""
+    import numpy as np
+
+    dec.reset(np.arange(1, batch + 1, dtype=np.int32), PREFILL)
+    dec.run_projections(2, stream=stream_ptr)
+    torch.cuda.synchronize()
+    ms = event_time_ms(lambda: dec.run_projections(reps, stream=stream_ptr), torch)
+    launches = reps * (4 * dec.cfg["n_layers"] + 1)
+    return ms * 1e-3 / launches, launches
+
+
+def cpu_baseline(cfg, seconds_budget=20.0):
+    """Restated reference CPU kernels (AVX-512 / AVX2 / scalar picked at run time, as the reference's
+    dispatchers do) on the projections of one decode step, batch 1, one thread -- what the reference
+    runs for MatMul-routed int4 weights.  Sample: one layer's seven projections + a 1/8 slice of lm_head."""
+    import numpy as np
+
+    from oracle import oracle as orc
+
+    orc.build()
+    D, hd, g = cfg["d_model"], cfg["head_dim"], cfg["group_size"]
+    hq, hkv, ff = cfg["n_heads"] * hd, cfg["n_kv_heads"] * hd, cfg["d_ff"]
+    shapes = [(hq, D), (hkv, D), (hkv, D), (D, hq), (ff, D), (ff, D), (D, ff)]
+    rng = np.random.default_rng(7)
+    ws = []
+    for (n, k) in shapes + [(cfg["vocab"] // 8, D)]:
+        ws.append((rng.integers(0, 256, n * k // 2, dtype=np.uint8), rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float32),
+                   rng.standard_normal(k).astype(np.float32), n, k))
+
+    def one_pass(threads):
+        t0 = time.perf_counter()
+        for (p, s, x, n, k) in ws[:-1]:
+            orc.simd_packed_int4_gemv_dispatch(p, s, x, n, k, g, threads=threads)
+        t_layer = time.perf_counter() - t0
+        p, s, x, n, k = ws[-1]
+        t0 = time.perf_counter()
+        orc.simd_packed_int4_gemv_dispatch(p, s, x, n, k, g, threads=threads)
+        t_head = (time.perf_counter() - t0) * 8
+        return t_layer * cfg["n_layers"] + t_head
+
+    one_pass(1)  # warm-up (page faults)
+    times, t_start = [], time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < seconds_budget / 2 and len(times) < 15):
+        times.append(one_pass(1))
+    t1 = sorted(times)[len(times) // 2]
+    cores = os.cpu_count() or 1
+    nthreads = min(cores, 64)
+    one_pass(nthreads)
+    tm = sorted(one_pass(nthreads) for _ in range(3))[1]
+    paths = orc.simd_paths(g)
+    return {
+        "value": round(1.0 / t1, 3), "unit": "tok/s", "cores": 1, "kind": "port",
+        "sample": "projections of 1 of 32 layers + 1/8 of lm_head at batch 1, median of %d, extrapolated to a "
+                  "full step; attention/norm glue not included (favours the CPU)" % len(times),
+        "kernel": "restated packed_int4_gemv_dispatch -> " + paths["int4_gemv"],
+        "all_cores": {"value": round(1.0 / tm, 3), "threads": nthreads,
+                      "note": "N-row partition; not present in the reference for MatMul"},
+    }
+
+
+def extra_kernels(torch, stream_ptr):
+    """Stand-alone kernels of BASELINE configs 1-3 (short runs; the parity tests cover correctness)."""
+    import numpy as np
+
+    from yscv_amd import kernels as K
+
+    out = {}
+    rng = np.random.default_rng(1)
+
+    def tavg(fn, iters, warm=3):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        return event_time_ms(lambda: [fn() for _ in range(iters)], torch) * 1e-3 / iters
+
+    # config 1: GEMV M1 K4096 N4096 g32, f32 scales, f32 activations; ring of weight copies > 256 MB
+    n = k = 4096
+    ring = []
+    for _ in range(32):
+        ring.append(K.PackedInt4Weight(rng.integers(0, 256, n * k // 2, dtype=np.uint8),
+                                       rng.uniform(0.005, 0.02, n * (k // 32)).astype(np.float32), 32, n, k,
+                                       nibble_format=K.NIBBLE_UNSIGNED))
+    x = torch.randn(1, k, device="cuda")
+    y = torch.empty(1, n, device="cuda")
+    i = [0]
+
+    def gemv():
+        ring[i[0] % len(ring)].matmul(x, out=y)
+        i[0] += 1
+
+    t = tavg(gemv, 128)
+    byt = n * k // 2 + n * (k // 32) * 4 + k * 4 + n * 4
+    out["config1_gemv_m1_k4096_n4096"] = {"us_per_call_whole_op": round(t * 1e6, 2), "GB/s_whole_op": round(byt / t / 1e9, 1),
+                                          "note": "x_prep + kernel, 32 rotating weight copies"}
+    del ring
+    # config 2: int8 M512 K4096 N4096
+    m, k, n = 512, 4096, 4096
+    pb = K.pack_i8_b_for_matmul(rng.integers(-127, 128, (k, n), dtype=np.int8), k, n)
+    a = torch.randint(0, 256, (m, k), device="cuda", dtype=torch.uint8)
+    o32 = torch.empty(m, n, device="cuda", dtype=torch.int32)
+    q8 = torch.empty(m, n, device="cuda", dtype=torch.uint8)
+    t = tavg(lambda: pb.matmul(a, a_zp=128, out=o32), 50)
+    t2 = tavg(lambda: pb.matmul_requant(a, 128, 1.0 / 4096, 128.0, K.ROUND_HALF_AWAY, 0, 255, out=q8), 50)
+    ops = 2.0 * m * k * n
+    out["config2_int8_m512_k4096_n4096"] = {"us_i32": round(t * 1e6, 2), "TOP/s_i32": round(ops / t / 1e12, 1),
+                                            "us_fused_requant": round(t2 * 1e6, 2), "TOP/s_fused_requant": round(ops / t2 / 1e12, 1),
+                                            "frac_of_i8_mfma_peak": round(ops / t2 / 1e12 / MFMA_I8_PEAK, 4)}
+    del pb
+    # config 3: int4 prefill M2048 K4096 N14336 g128, zero points 6..10, bf16
+    m, k, n, g = 2048, 4096, 14336, 128
+    zq = rng.integers(6, 11, (n, k // g))
+    zp = (zq[:, 0::2] | (zq[:, 1::2] << 4)).astype(np.uint8)
+    w = K.PackedInt4Weight(rng.integers(0, 256, n * k // 2, dtype=np.uint8), rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float16),
+                           g, n, k, zero_points=zp, nibble_format=K.NIBBLE_UNSIGNED)
+    xb = torch.randn(m, k, device="cuda").bfloat16()
+    yb = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
+    t = tavg(lambda: w.matmul(xb, out=yb), 10)
+    fl = 2.0 * m * k * n
+    out["config3_int4_prefill_m2048_k4096_n14336"] = {"us_whole_op": round(t * 1e6, 1), "TFLOP/s": round(fl / t / 1e12, 1),
+                                                      "frac_of_bf16_mfma_peak": round(fl / t / 1e12 / MFMA_BF16_PEAK, 4)}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--no-extra", action="store_true", help="skip the stand-alone kernels and the batch-16 run")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (every config of the metric fits one "
+              "MI355X); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import numpy as np  # noqa: F401
+    import torch
+
+    from yscv_amd.decoder import Decoder
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    assert 1 <= args.batch <= 16
+    cfg = dict(CFG7B)
+    need = PREFILL + args.steps + args.warmup
+    if need > cfg["max_ctx"]:
+        cfg["max_ctx"] = ((need + 127) // 128) * 128
+    cfg["max_steps"] = max(cfg["max_steps"], args.steps + args.warmup)
+    stream_ptr = torch.cuda.current_stream().cuda_stream
+
+    dec = Decoder(**cfg)
+    dec.init_random(seed=1)
+    dec.fill_kv_random(seed=2)
+    w_bytes, params = decode_bytes_per_step(cfg)
+    assert dec.weight_bytes() >= w_bytes
+
+    dt = bench_decode(dec, torch, args.batch, args.steps, args.warmup, stream_ptr)
+    tok_s = args.batch * args.steps / dt
+
+    avg_launch_s, launches = bench_projections(dec, torch, args.batch, stream_ptr)
+    n_proj = 4 * cfg["n_layers"] + 1
+    act_bytes = 0  # activations are < 0.1 % of the traffic and are left out of the algorithmic figure
+    bytes_per_launch = (w_bytes + act_bytes) / n_proj
+    achieved = bytes_per_launch / avg_launch_s / 1e9
+    kv_bytes_per_seq = 2 * cfg["n_layers"] * PREFILL * cfg["n_kv_heads"] * cfg["head_dim"] * 2
+    ideal_step_s = (w_bytes + args.batch * kv_bytes_per_seq) / (HBM_PEAK_GBS * 1e9)
+
+    result = {
+        "metric": "int4 decode tok/s (7B-shape) + matmul GB/s and % HBM/MFMA roofline, 1 GPU",
+        "value": round(tok_s, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(dt / args.steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int4 weights x fp16 activations, fp32 accumulate",
+        "data": "synthetic (random-init weights, random KV cache)",
+        "config": {"workload": "BASELINE configs[3]: Llama-style decoder 32L d4096 32q/8kv hd128 ffn14336 vocab32000, "
+                               "int4 g32 fp16 scales, fp16 KV ctx %d, greedy decode" % PREFILL,
+                   "batch": args.batch, "tokens_per_step": args.batch, "hip_graph": True},
+        "roofline": {
+            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "kernel": "int4_skinny_kernel (all %d projections of a decode step)" % n_proj,
+            "bytes_per_launch": int(bytes_per_launch), "avg_launch_us": round(avg_launch_s * 1e6, 3),
+            "launches_timed": launches,
+        },
+        "hbm_roofline_whole_step": {"ideal_ms": round(ideal_step_s * 1e3, 4), "frac": round(ideal_step_s / (dt / args.steps), 4),
+                                    "bytes_weights": w_bytes, "bytes_kv_per_seq": kv_bytes_per_seq},
+    }
+    extra = {}
+    if not args.no_extra:
+        if args.batch != 16:
+            dt16 = bench_decode(dec, torch, 16, min(args.steps, 64), 4, stream_ptr)
+            avg16, _ = bench_projections(dec, torch, 16, stream_ptr, reps=3)
+            extra["decode_batch16"] = {"tok/s": round(16 * min(args.steps, 64) / dt16, 1),
+                                       "ms_per_step": round(dt16 / min(args.steps, 64) * 1e3, 4),
+                                       "skinny_kernel_GB/s": round(bytes_per_launch / avg16 / 1e9, 1)}
+    del dec
+    torch.cuda.empty_cache()
+    if not args.no_extra:
+        extra.update(extra_kernels(torch, stream_ptr))
+        result["extra"] = extra
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(cfg)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -283,6 +283,10 @@ int32_t yscv_hip_decoder_reset(yscv_hip_decoder *d, int32_t batch, int32_t start
  * graph per step.  Fails if the KV cache or the token history would overflow (KvCache::append
  * returns an error in the same situation, kv_cache.rs:160-185). */
 int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_graph, void *stream);
+/* Measurement aid: enqueue only the int4 projections of n_steps decode steps (same weights, same
+ * order, same buffers as a real step, no attention / norm / sampling), so that the projections'
+ * share of a step can be timed on its own.  The activations it reads are whatever the buffers hold. */
+int32_t yscv_hip_decoder_run_projections(yscv_hip_decoder *d, int32_t n_steps, void *stream);
 /* Generated tokens of steps [first_step, first_step + n_steps), laid out [step][batch]. */
 int32_t yscv_hip_decoder_read_tokens(yscv_hip_decoder *d, int32_t first_step, int32_t n_steps,
                                      int32_t *out_host);

@@ -531,6 +531,24 @@ int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_g
   return YSCV_HIP_OK;
 }
 
+int32_t yscv_hip_decoder_run_projections(yscv_hip_decoder *d, int32_t n_steps, void *stream) {
+  YSCV_REQUIRE(d != nullptr, "null decoder");
+  YSCV_REQUIRE(d->finalized, "decoder weights are not finalized");
+  YSCV_REQUIRE(d->batch >= 1, "call yscv_hip_decoder_reset first");
+  hipStream_t s = as_stream(stream);
+  const int batch = d->batch;
+  for (int i = 0; i < n_steps; i++) {
+    for (auto &L : d->layers) {
+      YSCV_TRY(int4_run_ws(L.wqkv, d->xn, YSCV_HIP_F16, d->qkv, YSCV_HIP_F16, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s));
+      YSCV_TRY(int4_run_ws(L.wo, d->ao, YSCV_HIP_F16, d->h, YSCV_HIP_F32, batch, 1, EPI_ADD_F32, d->ws, d->ws_bytes, s));
+      YSCV_TRY(int4_run_ws(L.wgu, d->xn, YSCV_HIP_F16, d->act, YSCV_HIP_F16, batch, 1, EPI_SWIGLU, d->ws, d->ws_bytes, s));
+      YSCV_TRY(int4_run_ws(L.wdown, d->act, YSCV_HIP_F16, d->h, YSCV_HIP_F32, batch, 1, EPI_ADD_F32, d->ws, d->ws_bytes, s));
+    }
+    YSCV_TRY(int4_run_ws(d->lm_head, d->xn, YSCV_HIP_F16, d->logits, YSCV_HIP_F32, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s));
+  }
+  return YSCV_HIP_OK;
+}
+
 int32_t yscv_hip_decoder_read_tokens(yscv_hip_decoder *d, int32_t first_step, int32_t n_steps, int32_t *out_host) {
   YSCV_REQUIRE(d && out_host, "null argument");
   YSCV_REQUIRE(first_step >= 0 && n_steps >= 0 && first_step + n_steps <= d->cfg.max_steps, "step range out of bounds");

@@ -62,6 +62,9 @@ class Decoder:
     def run(self, n_steps, use_graph=True, stream=None):
         lib().decoder_run(self._h, int(n_steps), int(bool(use_graph)), C.c_void_p(stream) if stream else None)
 
+    def run_projections(self, n_steps, stream=None):
+        lib().decoder_run_projections(self._h, int(n_steps), C.c_void_p(stream) if stream else None)
+
     def tokens(self, first_step, n_steps):
         out = np.empty((n_steps, self.batch), np.int32)
         lib().decoder_read_tokens(self._h, int(first_step), int(n_steps), _p(out))
