@@ -80,7 +80,7 @@ static Int4Scratch int4_scratch_layout(const yscv_hip_int4_weight *w, const void
                                        int force, int num_cus) {
   Int4Scratch L{};
   L.skinny = force == 1 || (force == 0 && m <= 16);
-  L.k_pad = w->kt * 128;
+  L.k_pad = w->ktp * 128;
   L.direct = x_dtype == YSCV_HIP_F16 && L.k_pad == w->k && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
   L.split = x_dtype == YSCV_HIP_F32 ? 2 : 1;
   if (L.skinny) L.plan = plan_int4_skinny(w, m, L.split, num_cus);
@@ -246,14 +246,15 @@ static int32_t int4_create(const uint8_t *packed, const void *scales, int32_t sc
     w->gm = g == 32 ? GM32 : (g == 64 ? GM64 : GM128);
     w->nt = ceil_div(n, (size_t)16);
     w->kt = ceil_div(k, (size_t)128);
-    w->chunks = w->gm == GM128 ? groups : w->kt;
+    w->ktp = round_up(w->kt, (size_t)4);
+    w->chunks = w->gm == GM128 ? ceil_div(w->ktp, g / 128) : w->ktp;
     const int spt = scales_per_chunk(w->gm);
-    const size_t tile_bytes = w->nt * w->kt * (size_t)kTileBytes;
+    const size_t tile_bytes = w->nt * w->ktp * (size_t)kTileBytes;
     const size_t sc_elems = w->nt * w->chunks * 16 * (size_t)spt;
     CREATE_TRY(hipMalloc(reinterpret_cast<void **>(&w->tiles), tile_bytes));
     CREATE_TRY(hipMalloc(&w->tscales, sc_elems * ssz));
     if (has_zp) CREATE_TRY(hipMalloc(reinterpret_cast<void **>(&w->tzps), sc_elems));
-    CREATE_ST(launch_int4_retile(d_packed.as<uint8_t>(), nibble_format, n, k, w->nt, w->kt, w->tiles, s));
+    CREATE_ST(launch_int4_retile(d_packed.as<uint8_t>(), nibble_format, n, k, w->nt, w->ktp, w->tiles, s));
     CREATE_ST(launch_int4_retile_scales(d_scales.p, scale_dtype, has_zp ? d_zp.as<uint8_t>() : nullptr, n, k, g,
                                         w->gm, w->nt, w->chunks, w->tscales, w->tzps, s));
     w->device_bytes = tile_bytes + sc_elems * ssz + (has_zp ? sc_elems : 0);

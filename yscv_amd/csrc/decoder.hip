@@ -45,6 +45,7 @@ static unsigned grid_for(size_t n) {
 
 static int32_t random_int4_weight(size_t n, size_t k, size_t g, uint64_t seed, yscv_hip_int4_weight **out) {
   YSCV_REQUIRE(g == 32 || g == 64 || g % 128 == 0, "random weights need a tiled group size");
+  YSCV_REQUIRE(k % 512 == 0, "random weights need K to be a multiple of 512");
   auto *w = new yscv_hip_int4_weight();
   w->n = n;
   w->k = k;
@@ -55,8 +56,9 @@ static int32_t random_int4_weight(size_t n, size_t k, size_t g, uint64_t seed, y
   w->gm = g == 32 ? GM32 : (g == 64 ? GM64 : GM128);
   w->nt = ceil_div(n, (size_t)16);
   w->kt = ceil_div(k, (size_t)128);
-  w->chunks = w->gm == GM128 ? k / g : w->kt;
-  const size_t tile_bytes = w->nt * w->kt * (size_t)kTileBytes;
+  w->ktp = round_up(w->kt, (size_t)4);
+  w->chunks = w->gm == GM128 ? ceil_div(w->ktp, g / 128) : w->ktp;
+  const size_t tile_bytes = w->nt * w->ktp * (size_t)kTileBytes;
   const size_t sc_elems = w->nt * w->chunks * 16 * (size_t)scales_per_chunk(w->gm);
   hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->tiles), tile_bytes);
   if (e == hipSuccess) e = hipMalloc(&w->tscales, sc_elems * 2);

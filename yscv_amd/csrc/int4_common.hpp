@@ -45,6 +45,15 @@ enum : int { GM32 = 0, GM64 = 1, GM128 = 2 };
 
 __host__ __device__ inline int scales_per_chunk(int gm) { return gm == GM32 ? 4 : (gm == GM64 ? 2 : 1); }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
+// global load (s_waitcnt vmcnt(0)), which would drain the software-pipelined weight loads of the
+// streaming kernels at every tile; the kernels here exchange data through LDS alone.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 union U32H2 {
   uint32_t u;
   half2_t h;

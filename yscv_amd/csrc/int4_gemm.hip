@@ -29,7 +29,7 @@ struct GemmArgs {
   const float *row_scale;
   void *y;
   int m, n;
-  int nt, kt;
+  int nt, kt, ktp;
   int chunks, chunk_div;
   int k_pad;
   int y_dtype;
@@ -121,7 +121,7 @@ __global__ void __launch_bounds__(256) int4_gemm_kernel(GemmArgs a) {
     for (int t = 0; t < G_NTW; t++) {
       const int nt = nt0 + t;
       if (nt < a.nt) {
-        wraw[slot][t] = *(reinterpret_cast<const uint4_t *>(a.tiles + ((size_t)nt * a.kt + kt) * kTileBytes) + lane);
+        wraw[slot][t] = *(reinterpret_cast<const uint4_t *>(a.tiles + ((size_t)nt * a.ktp + kt) * kTileBytes) + lane);
         const size_t chunk = (size_t)nt * a.chunks + (GM == GM128 ? kt / a.chunk_div : kt);
         wsc[slot][t].load(a.tscales, chunk, r);
         if (has_zp) {
@@ -263,6 +263,7 @@ int32_t launch_int4_gemm(const yscv_hip_int4_weight *w, const _Float16 *xh, cons
   a.n = (int)w->n;
   a.nt = (int)w->nt;
   a.kt = (int)w->kt;
+  a.ktp = (int)w->ktp;
   a.chunks = (int)w->chunks;
   a.chunk_div = w->gm == GM128 ? (int)(w->g / 128) : 1;
   a.k_pad = (int)k_pad;

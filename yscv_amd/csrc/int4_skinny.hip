@@ -2,21 +2,28 @@
 // Replaces packed_int4_gemv_dispatch (crates/yscv-kernels/src/ops/int4_matmul.rs:310-377),
 // which the reference calls once per activation row (crates/yscv-onnx/src/runner/linear.rs:255-267).
 //
-// Bandwidth-bound design for gfx950:
-//   * weights stream from HBM exactly once, as 1 KiB coalesced tiles (one 128-bit load per
-//     lane, see int4_common.hpp), and are decoded to fp16 in registers;
-//   * the activation rows sit in registers for the whole kernel, pre-split into fp16
-//     hi (+ lo for f32 input) and already in MFMA A-operand order, so the inner loop touches
-//     neither LDS nor L2 for them;
-//   * v_mfma_f32_16x16x32_f16 does the dot products: A = activations (rows = up to 16
-//     batch rows, padded with zeros), B = decoded weights (16 output rows), one MFMA per
-//     32-k block, i.e. per quantisation group when group_size is 32;
-//   * group scales are applied in fp32 to the MFMA result (acc += scale * D), so the
-//     fp16 operands are exact integers and exact activation halves;
-//   * K is split across the wavefronts of a workgroup (each wave keeps its own K slice of
-//     the activations); the per-wave partial sums meet in LDS once per 16-row tile.
-//     When K is too long for one workgroup, a grid-level split writes fp32 partials that a
-//     second small kernel adds up in a fixed order (no atomics: results are deterministic).
+// Bandwidth-bound design for gfx950.  The kernel is limited by how many instructions a SIMD can
+// issue per byte streamed (about 80 VALU slots per KiB of weights at 8 TB/s), so everything in the
+// inner loop is there to keep that count low:
+//   * weights stream from HBM exactly once, as 1 KiB coalesced tiles (one 128-bit load per lane,
+//     layout in int4_common.hpp); a ring of P register slots keeps P-1 blocks in flight per wave;
+//     the steady-state loop has no conditional loads, so the compiler's s_waitcnt counts are exact;
+//   * the activation rows sit in registers for the whole kernel, as fp16 hi (+ lo for f32 input),
+//     already in MFMA A-operand order: the inner loop reads neither LDS nor L2 for them;
+//   * v_mfma_f32_16x16x32_f16 does the dot products (A = up to 16 activation rows, B = 16 weight
+//     rows), one MFMA per 32-k block = one quantisation group when group_size is 32;
+//   * nibbles become fp16 with one bit-field insert each: 0x6400 | q = 1024 + q and
+//     0x6400 | (q << 4) = 1024 + 16 q.  For symmetric weights (zero point 8), fp16/bf16
+//     activations and m <= 4 the offsets are not subtracted per weight: the activation slots that meet the
+//     16 q form are pre-divided by 16, and the offset term sum_k x_k * (1024 + 8 or 1024 + 128)
+//     -- which does not depend on the weight row -- is computed once per kernel by the same MFMA
+//     against a constant operand and removed from each group's result.  With explicit zero points,
+//     f32 activations or m > 4 the offsets are subtracted exactly in fp16 before the MFMA;
+//   * group scales are applied in fp32 to the MFMA result (acc += scale * D);
+//   * K is split across the wavefronts of a workgroup (each wave owns 512 k of the activations);
+//     the per-wave partial sums meet in LDS once per 16-row block behind an LDS-only barrier.
+//     When K is too long for one workgroup, a grid-level split writes fp32 partials that a second
+//     small kernel adds in a fixed order (no atomics on shared outputs: results are deterministic).
 #include <type_traits>
 
 #include "int4_common.hpp"
@@ -25,6 +32,8 @@
 namespace yscv {
 
 __device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
+
+constexpr int TPW = 4;  // 128-k tiles per wave: 512 k of activations live in 64 VGPRs (hi)
 
 struct SkinnyArgs {
   const uint8_t *tiles;
@@ -36,13 +45,14 @@ struct SkinnyArgs {
   void *y;
   float *partial;  // [ksg][m][n] when ksg > 1
   int m, n;
-  int nt, kt;      // tile counts
-  int chunks;      // scale chunks per n-tile
+  int nt, ktp;     // tile counts; ktp = 128-k tiles per 16-row block as stored (multiple of TPW)
+  int chunks;      // scale chunks per 16-row block
   int chunk_div;   // GM128: tiles per scale chunk (group_size / 128)
-  int k_pad;       // row stride of xh / xl
+  int k_pad;       // row stride of xh / xl, = ktp * 128
   int y_dtype;
   int ksg;
-  int epi;  // EPI_STORE / EPI_ADD_F32 / EPI_SWIGLU
+  int epi;         // EPI_STORE / EPI_ADD_F32 / EPI_SWIGLU
+  int slices;      // ktp / TPW: number of wave-sized k slices that exist
 };
 
 // Scales of one (tile, row) kept in their storage type until used: 1, 2 or 4 values.
@@ -52,128 +62,222 @@ struct ScaleRaw {
   typedef typename std::conditional<SF16, _Float16, float>::type elem_t;
   typedef elem_t vec_t __attribute__((ext_vector_type(SPT)));
   vec_t v;
-  __device__ __forceinline__ void load(const void *base, size_t chunk_idx, int r) {
-    const elem_t *p = reinterpret_cast<const elem_t *>(base) + (chunk_idx * 16 + r) * SPT;
-    v = *reinterpret_cast<const vec_t *>(p);
-  }
+  __device__ __forceinline__ void load(const char *p) { v = *reinterpret_cast<const vec_t *>(p); }
   __device__ __forceinline__ float get(int i) const { return (float)v[i]; }
 };
 
 template <int GM>
-__device__ __forceinline__ void load_zps(const uint8_t *base, size_t chunk_idx, int r, uint32_t &packed) {
+__device__ __forceinline__ uint32_t load_zp_raw(const uint8_t *p) {
   constexpr int SPT = GM == GM32 ? 4 : (GM == GM64 ? 2 : 1);
-  size_t off = (chunk_idx * 16 + r) * SPT;
-  if constexpr (SPT == 4)
-    packed = *reinterpret_cast<const uint32_t *>(base + off);
-  else if constexpr (SPT == 2)
-    packed = *reinterpret_cast<const uint16_t *>(base + off);
-  else
-    packed = base[off];
+  if constexpr (SPT == 4) return *reinterpret_cast<const uint32_t *>(p);
+  if constexpr (SPT == 2) return *reinterpret_cast<const uint16_t *>(p);
+  return *p;
+}
+
+// One wave's registers for one 16-row block: TPW weight tiles + their scales / zero points.
+template <int GM, bool SF16, bool HAS_ZP>
+struct TileRegs {
+  uint4_t w[TPW];
+  ScaleRaw<GM, SF16> s[TPW];
+  uint32_t z[HAS_ZP ? TPW : 1];
+};
+
+// (mask & s) | (~mask & magic): one v_bfi_b32
+__device__ __forceinline__ uint32_t bfi(uint32_t mask, uint32_t s, uint32_t magic) {
+  return (mask & s) | (~mask & magic);
+}
+
+// raw fp16 forms of the 8 weights of one word: {1024+q0, 1024+q1, 1024+16 q2, 1024+16 q3, ...}
+__device__ __forceinline__ half8_t extract8(uint32_t s, uint32_t magic) {
+  U32H2 r0, r1, r2, r3;
+  const uint32_t s2 = s >> 8;
+  r0.u = bfi(0x000F000Fu, s, magic);
+  r1.u = bfi(0x00F000F0u, s, magic);
+  r2.u = bfi(0x000F000Fu, s2, magic);
+  r3.u = bfi(0x00F000F0u, s2, magic);
+  half8_t out;
+  out[0] = r0.h[0];
+  out[1] = r0.h[1];
+  out[2] = r1.h[0];
+  out[3] = r1.h[1];
+  out[4] = r2.h[0];
+  out[5] = r2.h[1];
+  out[6] = r3.h[0];
+  out[7] = r3.h[1];
+  return out;
+}
+
+// exact (q - zp) in fp16: c1 = -(1024 + zp), c2 = -(64 + zp)
+__device__ __forceinline__ half8_t decode8_exact(uint32_t s, uint32_t magic, half2_t c1, half2_t c2) {
+  U32H2 r0, r1, r2, r3;
+  const uint32_t s2 = s >> 8;
+  r0.u = bfi(0x000F000Fu, s, magic);
+  r1.u = bfi(0x00F000F0u, s, magic);
+  r2.u = bfi(0x000F000Fu, s2, magic);
+  r3.u = bfi(0x00F000F0u, s2, magic);
+  const half2_t sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+  const half2_t h0 = r0.h + c1;
+  const half2_t h1 = r1.h * sixteenth + c2;
+  const half2_t h2 = r2.h + c1;
+  const half2_t h3 = r3.h * sixteenth + c2;
+  half8_t out;
+  out[0] = h0[0];
+  out[1] = h0[1];
+  out[2] = h1[0];
+  out[3] = h1[1];
+  out[4] = h2[0];
+  out[5] = h2[1];
+  out[6] = h3[0];
+  out[7] = h3[1];
+  return out;
 }
 
 __device__ __forceinline__ void zp_consts(uint32_t zp, half2_t &c1, half2_t &c2) {
-  _Float16 z = (_Float16)(float)zp;
-  _Float16 a = (_Float16)(-1024.0f) - z;
-  _Float16 b = (_Float16)(-64.0f) - z;
+  const _Float16 z = (_Float16)(float)zp;
+  const _Float16 a = (_Float16)(-1024.0f) - z;
+  const _Float16 b = (_Float16)(-64.0f) - z;
   c1 = half2_t{a, a};
   c2 = half2_t{b, b};
 }
 
-// One wave's registers for one 16-row tile: TPW weight tiles + their scales / zero points.
-template <int TPW, int GM, bool SF16>
-struct TileRegs {
-  uint4_t w[TPW];
-  ScaleRaw<GM, SF16> s[TPW];
-  uint32_t z[TPW];
-};
-
-template <int TPW, int SPLIT, int NI, int GM, bool SF16, int P>
+template <int SPLIT, int NI, int GM, bool SF16, bool HAS_ZP, int P>
 __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
+  // OFFSET mode: leave the 1024-offsets in the weights and cancel them per group (see file header)
+  constexpr bool OFFSET = (SPLIT == 1) && !HAS_ZP && (NI == 1);
+  constexpr int SPT = GM == GM32 ? 4 : (GM == GM64 ? 2 : 1);
+  constexpr int SC_BYTES = SPT * (SF16 ? 2 : 4);
   extern __shared__ float red[];  // [2][waves][NI][64]
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int waves = blockDim.x >> 6;
   const int r = lane & 15;
   const int c = lane >> 4;
-  const int t0 = (blockIdx.y * waves + wave) * TPW;  // first 128-k tile of this wave's K slice
+  const int slice = blockIdx.y * waves + wave;     // this wave's 512-k slice
+  const bool wave_active = slice < a.slices;       // trailing waves of the last k-split may be idle
+  const int t0 = (wave_active ? slice : 0) * TPW;  // first 128-k tile of the slice
+  const uint32_t magic = 0x64006400u;
 
-  // ---- activations -> registers, in A-operand order --------------------------------
-  // A row `r` of the MFMA carries batch row m when r == 4*(m / NI) + (m % NI): the
-  // useful results then sit in the first NI of the four accumulator registers.
+  // ---- activations -> registers, in A-operand order ------------------------------------------
+  // MFMA row `r` carries batch row m when r == 4*(m / NI) + (m % NI): the useful results then sit
+  // in the first NI of the four accumulator registers of each lane.
   half8_t xa[TPW][4][SPLIT];
   {
     const int i = r & 3;
     const int mrow = (r >> 2) * NI + i;
-    const bool valid = (i < NI) && (mrow < a.m);
+    const bool valid = wave_active && (i < NI) && (mrow < a.m);
+    const half8_t pre = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)0.0625f, (_Float16)0.0625f,
+                         (_Float16)1.0f, (_Float16)1.0f, (_Float16)0.0625f, (_Float16)0.0625f};
 #pragma unroll
     for (int t = 0; t < TPW; t++) {
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         half8_t h = {0, 0, 0, 0, 0, 0, 0, 0}, l = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (valid && (t0 + t) < a.kt) {
-          size_t off = (size_t)mrow * a.k_pad + (size_t)(t0 + t) * 128 + j * 32 + c * 8;
+        if (valid) {
+          const size_t off = (size_t)mrow * a.k_pad + (size_t)(t0 + t) * 128 + j * 32 + c * 8;
           h = *reinterpret_cast<const half8_t *>(a.xh + off);
           if constexpr (SPLIT == 2) l = *reinterpret_cast<const half8_t *>(a.xl + off);
         }
+        if constexpr (OFFSET) h = h * pre;  // slots that meet 1024 + 16 q carry x / 16 (a power of two)
         xa[t][j][0] = h;
         if constexpr (SPLIT == 2) xa[t][j][1] = l;
       }
     }
   }
-
-  const half2_t c1_default = {(_Float16)(-1032.0f), (_Float16)(-1032.0f)};
-  const half2_t c2_default = {(_Float16)(-72.0f), (_Float16)(-72.0f)};
-  const bool has_zp = a.tzps != nullptr;
-
-  auto issue = [&](int nt, TileRegs<TPW, GM, SF16> &tr) {
+  // offset term of every 32-k block: sum_k x'_k * (1024 + 8 | 1024 + 128), same register layout as D
+  float corr1[OFFSET ? TPW : 1][4];
+  if constexpr (OFFSET) {
+    const half8_t bc = {(_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f,
+                        (_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f};
 #pragma unroll
     for (int t = 0; t < TPW; t++) {
-      const int kt = t0 + t;
-      if (kt < a.kt) {
-        const uint4_t *src = reinterpret_cast<const uint4_t *>(a.tiles + ((size_t)nt * a.kt + kt) * kTileBytes) + lane;
-        tr.w[t] = __builtin_nontemporal_load(src);
-        size_t chunk = (size_t)nt * a.chunks + (GM == GM128 ? kt / a.chunk_div : kt);
-        tr.s[t].load(a.tscales, chunk, r);
-        if (has_zp) load_zps<GM>(a.tzps, chunk, r, tr.z[t]);
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        float4_t z = {0.0f, 0.0f, 0.0f, 0.0f};
+        z = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][j][0], bc, z, 0, 0, 0);
+        corr1[t][j] = z[0];
       }
+    }
+  }
+
+  // ---- per-wave stream pointers (advance by one grid stride of 16-row blocks per iteration) ----
+  const int stride = gridDim.x;
+  const size_t w_step = (size_t)stride * a.ktp * kTileBytes;
+  const size_t s_step = (size_t)stride * a.chunks * 16 * SC_BYTES;
+  const size_t z_step = (size_t)stride * a.chunks * 16 * SPT;
+  const char *wp = reinterpret_cast<const char *>(a.tiles) + ((size_t)blockIdx.x * a.ktp + t0) * kTileBytes + lane * 16;
+  const int chunk0 = GM == GM128 ? t0 / a.chunk_div : t0;
+  const char *sp = reinterpret_cast<const char *>(a.tscales) + (((size_t)blockIdx.x * a.chunks + chunk0) * 16 + r) * SC_BYTES;
+  const uint8_t *zp = HAS_ZP ? a.tzps + (((size_t)blockIdx.x * a.chunks + chunk0) * 16 + r) * SPT : nullptr;
+
+  using Regs = TileRegs<GM, SF16, HAS_ZP>;
+
+  // issue the loads of the block `ahead` grid strides after the current one
+  auto issue = [&](Regs &tr, int ahead) {
+    const char *wq = wp + (size_t)ahead * w_step;
+    const char *sq = sp + (size_t)ahead * s_step;
+#pragma unroll
+    for (int t = 0; t < TPW; t++) {
+      tr.w[t] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(wq + t * kTileBytes));
+      const int ch = GM == GM128 ? ((t0 + t) / a.chunk_div - chunk0) : t;
+      tr.s[t].load(sq + (size_t)ch * 16 * SC_BYTES);
+      if constexpr (HAS_ZP) tr.z[t] = load_zp_raw<GM>(zp + (size_t)ahead * z_step + (size_t)ch * 16 * SPT);
     }
   };
 
-  auto compute = [&](int nt, const TileRegs<TPW, GM, SF16> &tr, int it) {
-    float acc[NI];
+  auto advance = [&]() {
+    wp += w_step;
+    sp += s_step;
+    if constexpr (HAS_ZP) zp += z_step;
+  };
+
+  // dot products of one 16-row block against this wave's k slice
+  auto dots = [&](const Regs &tr, float acc[NI]) {
 #pragma unroll
     for (int i = 0; i < NI; i++) acc[i] = 0.0f;
 #pragma unroll
     for (int t = 0; t < TPW; t++) {
-      if ((t0 + t) < a.kt) {
-        const uint32_t wj[4] = {tr.w[t][0], tr.w[t][1], tr.w[t][2], tr.w[t][3]};
-        float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
+      float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
+      float csum = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-          half2_t c1 = c1_default, c2 = c2_default;
-          if (has_zp) {
-            uint32_t zp = GM == GM32 ? ((tr.z[t] >> (8 * j)) & 0xFF)
-                                     : (GM == GM64 ? ((tr.z[t] >> (8 * (j >> 1))) & 0xFF) : tr.z[t]);
-            zp_consts(zp, c1, c2);
+      for (int j = 0; j < 4; j++) {
+        const bool group_start = GM == GM32 || (GM == GM64 && !(j & 1)) || (GM == GM128 && j == 0);
+        const bool group_end = GM == GM32 || (GM == GM64 && (j & 1)) || (GM == GM128 && j == 3);
+        half8_t b;
+        if constexpr (OFFSET) {
+          b = extract8(tr.w[t][j], magic);
+          csum = group_start ? corr1[t][j] : csum + corr1[t][j];
+        } else {
+          half2_t c1 = {(_Float16)(-1032.0f), (_Float16)(-1032.0f)};
+          half2_t c2 = {(_Float16)(-72.0f), (_Float16)(-72.0f)};
+          if constexpr (HAS_ZP) {
+            const uint32_t z = GM == GM32 ? ((tr.z[t] >> (8 * j)) & 0xFF)
+                                          : (GM == GM64 ? ((tr.z[t] >> (8 * (j >> 1))) & 0xFF) : (tr.z[t] & 0xFF));
+            zp_consts(z, c1, c2);
           }
-          half8_t b = decode8(wj[j], c1, c2);
-          d = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][j][0], b, d, 0, 0, 0);
-          if constexpr (SPLIT == 2) d = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][j][1], b, d, 0, 0, 0);
-          const bool group_end = GM == GM32 || (GM == GM64 && (j & 1)) || (GM == GM128 && j == 3);
-          if (group_end) {
-            const float sc = tr.s[t].get(GM == GM32 ? j : (GM == GM64 ? (j >> 1) : 0));
+          b = decode8_exact(tr.w[t][j], magic, c1, c2);
+        }
+        d = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][j][0], b, d, 0, 0, 0);
+        if constexpr (SPLIT == 2) d = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][j][1], b, d, 0, 0, 0);
+        if (group_end) {
+          const float sc = tr.s[t].get(GM == GM32 ? j : (GM == GM64 ? (j >> 1) : 0));
+          if constexpr (OFFSET) {
+            acc[0] = fmaf(sc, d[0] - csum, acc[0]);
+          } else {
 #pragma unroll
             for (int i = 0; i < NI; i++) acc[i] = fmaf(sc, d[i], acc[i]);
-            d = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
           }
+          d = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
         }
       }
     }
-    // ---- meet the other K slices in LDS ---------------------------------------------
+  };
+
+  // meet the other k slices in LDS; one wave (rotating) sums them and writes the 16 x m results
+  auto reduce_store = [&](const float acc[NI], int nt, int it) {
     float *buf = red + (size_t)(it & 1) * waves * NI * 64;
 #pragma unroll
     for (int i = 0; i < NI; i++) buf[(wave * NI + i) * 64 + lane] = acc[i];
-    __syncthreads();
+    lds_barrier();
     if (wave == (it % waves)) {
       const int col = nt * 16 + r;
 #pragma unroll
@@ -192,10 +296,8 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
             if (live && !(r & 1))
               store_out(a.y, (size_t)mrow * (a.n >> 1) + (col >> 1), silu(v) * up, a.y_dtype);
           } else if (a.epi == EPI_ADD_F32) {
-            if (live) {
-              float *dst = reinterpret_cast<float *>(a.y) + (size_t)mrow * a.n + col;
-              *dst = *dst + v;
-            }
+            // single writer per element: a returnless add keeps the residual update off the load queue
+            if (live) unsafeAtomicAdd(reinterpret_cast<float *>(a.y) + (size_t)mrow * a.n + col, v);
           } else if (live) {
             store_out(a.y, (size_t)mrow * a.n + col, v, a.y_dtype);
           }
@@ -204,27 +306,59 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
     }
   };
 
-  // Ring of P register slots: while one 16-row tile is being consumed, the loads of the next
-  // P-1 are in flight, so the memory pipeline never drains at the per-tile barrier.
-  TileRegs<TPW, GM, SF16> ring[P];
-  const int stride = gridDim.x;
+  // ---- main loop over this workgroup's 16-row blocks: nt = blockIdx.x + i * stride ----------------
+  const int iters = (a.nt - (int)blockIdx.x + stride - 1) / stride;  // >= 1, uniform in the workgroup
   int nt = blockIdx.x;
-#pragma unroll
-  for (int sl = 0; sl < P; sl++) {
-    const int n = nt + sl * stride;
-    if (n < a.nt) issue(n, ring[sl]);
-  }
   int it = 0;
-  while (nt < a.nt) {
+  float acc[NI];
+
+  if (!wave_active) {
+    // an idle wave only takes part in the reductions
 #pragma unroll
-    for (int sl = 0; sl < P; sl++) {
-      if (nt < a.nt) {
-        compute(nt, ring[sl], it);
-        const int nn = nt + P * stride;
-        if (nn < a.nt) issue(nn, ring[sl]);
+    for (int i = 0; i < NI; i++) acc[i] = 0.0f;
+    for (; it < iters; it++, nt += stride) reduce_store(acc, nt, it);
+    return;
+  }
+
+  Regs ring[P];
+  // head: the iterations that do not fill whole groups of P are issued together, then consumed
+  const int head = iters < P ? iters : iters % P;
+  if (head > 0) {
+#pragma unroll
+    for (int sl = 0; sl < P - 1; sl++)
+      if (sl < head) issue(ring[sl], sl);
+#pragma unroll
+    for (int sl = 0; sl < P - 1; sl++) {
+      if (sl < head) {
+        dots(ring[sl], acc);
+        reduce_store(acc, nt, it);
+        advance();
         nt += stride;
         it++;
       }
+    }
+  }
+  const int groups = (iters - head) / P;  // whole groups of P iterations left
+  if (groups > 0) {
+#pragma unroll
+    for (int sl = 0; sl < P; sl++) issue(ring[sl], sl);
+    for (int g = 0; g + 1 < groups; g++) {
+#pragma unroll
+      for (int sl = 0; sl < P; sl++) {
+        dots(ring[sl], acc);
+        issue(ring[sl], P);  // refill the slot just consumed: stays P-1 blocks ahead
+        reduce_store(acc, nt, it);
+        advance();
+        nt += stride;
+        it++;
+      }
+    }
+#pragma unroll
+    for (int sl = 0; sl < P; sl++) {
+      dots(ring[sl], acc);
+      reduce_store(acc, nt, it);
+      nt += stride;
+      it++;
     }
   }
 }
@@ -253,8 +387,14 @@ __global__ void int4_skinny_finalize_kernel(const float *__restrict__ partial, i
   }
   for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total;
        idx += (size_t)gridDim.x * blockDim.x) {
+    // issue the loads of this element together (one memory round trip), then add in slice order
+    float p[8];
+#pragma unroll
+    for (int s = 0; s < 8; s++) p[s] = s < ksg ? partial[(size_t)s * total + idx] : 0.0f;
     float v = 0.0f;
-    for (int s = 0; s < ksg; s++) v += partial[(size_t)s * total + idx];
+#pragma unroll
+    for (int s = 0; s < 8; s++) v += p[s];
+    for (int s = 8; s < ksg; s++) v += partial[(size_t)s * total + idx];
     if (row_scale) v *= row_scale[idx / n];
     if (epi == EPI_ADD_F32) {
       float *dst = reinterpret_cast<float *>(y) + idx;
@@ -266,44 +406,50 @@ __global__ void int4_skinny_finalize_kernel(const float *__restrict__ partial, i
 }
 
 SkinnyPlan plan_int4_skinny(const yscv_hip_int4_weight *w, size_t m, int split, int num_cus) {
-  (void)m;
-  SkinnyPlan p;
-  // x registers per wave: 16 * tpw * split <= 128
   (void)split;
-  p.tpw = 4;
-  const int max_waves = 8;
-  int slices = (int)ceil_div(w->kt, (size_t)p.tpw);
+  SkinnyPlan p;
+  p.tpw = TPW;
+  const int max_waves = 8;  // 8 waves x <= 256 VGPRs: one workgroup per CU
+  const int slices = (int)(w->ktp / TPW);
   p.ksg = (int)ceil_div((size_t)slices, (size_t)max_waves);
   p.waves = (int)ceil_div((size_t)slices, (size_t)p.ksg);
   int gx = (int)w->nt;
-  int cap = num_cus > 0 ? num_cus : 256;
-  // one resident workgroup per CU and k-split slice; more tiles than that loop inside the kernel
+  const int cap = num_cus > 0 ? num_cus : 256;
+  // one resident workgroup per CU and k-split slice; more blocks than that loop inside the kernel
   int per = cap / p.ksg;
   if (per < 1) per = 1;
   if (gx > per) {
-    // spread the tiles evenly over the resident workgroups
-    int rounds = (int)ceil_div((size_t)gx, (size_t)per);
-    gx = (int)ceil_div((size_t)w->nt, (size_t)rounds);
+    const int rounds = (int)ceil_div((size_t)gx, (size_t)per);
+    gx = (int)ceil_div((size_t)w->nt, (size_t)rounds);  // spread the blocks evenly
   }
   p.grid_x = gx;
   p.partial_bytes = p.ksg > 1 ? (size_t)p.ksg * m * w->n * sizeof(float) : 0;
   return p;
 }
 
-template <int TPW, int SPLIT, int NI, int GM, bool SF16>
+template <int SPLIT, int NI, int GM, bool SF16, bool HAS_ZP>
 static int32_t launch_one(const SkinnyArgs &a, const SkinnyPlan &plan, hipStream_t s) {
-  size_t lds = (size_t)2 * plan.waves * NI * 64 * sizeof(float);
-  hipLaunchKernelGGL((int4_skinny_kernel<TPW, SPLIT, NI, GM, SF16, (SPLIT == 2 ? 2 : 4)>), dim3(plan.grid_x, plan.ksg),
+  // ring depth: bounded by the VGPR budget (activations: 64 per split, ring: ~26 per slot)
+  constexpr int P = SPLIT == 2 ? (NI == 1 ? 2 : 1) : (NI == 1 ? 4 : 3);
+  const size_t lds = (size_t)2 * plan.waves * NI * 64 * sizeof(float);
+  hipLaunchKernelGGL((int4_skinny_kernel<SPLIT, NI, GM, SF16, HAS_ZP, P>), dim3(plan.grid_x, plan.ksg),
                      dim3(plan.waves * 64), lds, s, a);
   YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
 }
 
-template <int TPW, int SPLIT, int NI>
-static int32_t launch_gm(const SkinnyArgs &a, const SkinnyPlan &plan, int gm, bool sf16, hipStream_t s) {
-  if (gm == GM32) return sf16 ? launch_one<TPW, SPLIT, NI, GM32, true>(a, plan, s) : launch_one<TPW, SPLIT, NI, GM32, false>(a, plan, s);
-  if (gm == GM64) return sf16 ? launch_one<TPW, SPLIT, NI, GM64, true>(a, plan, s) : launch_one<TPW, SPLIT, NI, GM64, false>(a, plan, s);
-  return sf16 ? launch_one<TPW, SPLIT, NI, GM128, true>(a, plan, s) : launch_one<TPW, SPLIT, NI, GM128, false>(a, plan, s);
+template <int SPLIT, int NI, int GM>
+static int32_t launch_sz(const SkinnyArgs &a, const SkinnyPlan &plan, bool sf16, bool has_zp, hipStream_t s) {
+  if (sf16)
+    return has_zp ? launch_one<SPLIT, NI, GM, true, true>(a, plan, s) : launch_one<SPLIT, NI, GM, true, false>(a, plan, s);
+  return has_zp ? launch_one<SPLIT, NI, GM, false, true>(a, plan, s) : launch_one<SPLIT, NI, GM, false, false>(a, plan, s);
+}
+
+template <int SPLIT, int NI>
+static int32_t launch_gm(const SkinnyArgs &a, const SkinnyPlan &plan, int gm, bool sf16, bool has_zp, hipStream_t s) {
+  if (gm == GM32) return launch_sz<SPLIT, NI, GM32>(a, plan, sf16, has_zp, s);
+  if (gm == GM64) return launch_sz<SPLIT, NI, GM64>(a, plan, sf16, has_zp, s);
+  return launch_sz<SPLIT, NI, GM128>(a, plan, sf16, has_zp, s);
 }
 
 int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan, const _Float16 *xh,
@@ -312,6 +458,8 @@ int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan
   if (!w->tiled) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "skinny int4 kernel needs the tiled layout");
   if (m == 0 || m > 16) return set_error(YSCV_HIP_ERR_INVALID_ARG, "skinny int4 kernel handles 1 <= m <= 16, got %zu", m);
   if (plan.ksg > 1 && !partial) return set_error(YSCV_HIP_ERR_INVALID_ARG, "k-split needs a partial buffer");
+  if (k_pad != w->ktp * 128)
+    return set_error(YSCV_HIP_ERR_INVALID_ARG, "activation row stride %zu != padded K %zu", k_pad, w->ktp * 128);
   SkinnyArgs a;
   a.tiles = w->tiles;
   a.tscales = w->tscales;
@@ -324,26 +472,27 @@ int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan
   a.m = (int)m;
   a.n = (int)w->n;
   a.nt = (int)w->nt;
-  a.kt = (int)w->kt;
+  a.ktp = (int)w->ktp;
   a.chunks = (int)w->chunks;
   a.chunk_div = w->gm == GM128 ? (int)(w->g / 128) : 1;
   a.k_pad = (int)k_pad;
   a.y_dtype = y_dtype;
   a.ksg = plan.ksg;
   a.epi = epi;
-  if (epi == EPI_ADD_F32 && y_dtype != YSCV_HIP_F32) return set_error(YSCV_HIP_ERR_INVALID_ARG, "residual accumulation needs an f32 output");
+  a.slices = (int)(w->ktp / TPW);
+  if (epi == EPI_ADD_F32 && y_dtype != YSCV_HIP_F32)
+    return set_error(YSCV_HIP_ERR_INVALID_ARG, "residual accumulation needs an f32 output");
   if (epi == EPI_SWIGLU && (w->n & 1)) return set_error(YSCV_HIP_ERR_INVALID_ARG, "SwiGLU epilogue needs an even row count");
   const bool sf16 = w->scale_dtype == YSCV_HIP_F16;
   const bool small = m <= 4;
   int32_t st;
-  if (split == 2) {
-    st = small ? launch_gm<4, 2, 1>(a, plan, w->gm, sf16, s) : launch_gm<4, 2, 4>(a, plan, w->gm, sf16, s);
-  } else {
-    st = small ? launch_gm<4, 1, 1>(a, plan, w->gm, sf16, s) : launch_gm<4, 1, 4>(a, plan, w->gm, sf16, s);
-  }
+  if (split == 2)
+    st = small ? launch_gm<2, 1>(a, plan, w->gm, sf16, w->has_zp, s) : launch_gm<2, 4>(a, plan, w->gm, sf16, w->has_zp, s);
+  else
+    st = small ? launch_gm<1, 1>(a, plan, w->gm, sf16, w->has_zp, s) : launch_gm<1, 4>(a, plan, w->gm, sf16, w->has_zp, s);
   YSCV_TRY(st);
   if (plan.ksg > 1) {
-    size_t total = m * w->n;
+    const size_t total = epi == EPI_SWIGLU ? m * (w->n / 2) : m * w->n;
     int blocks = (int)ceil_div(total, (size_t)256);
     if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL(int4_skinny_finalize_kernel, dim3(blocks), dim3(256), 0, s, partial, plan.ksg,

@@ -11,8 +11,9 @@ struct yscv_hip_int4_weight {
   bool tiled = false;              // fast layout built (g in {32,64} or g % 128 == 0)
   int gm = 0;                      // group mode of the tiled layout
   size_t nt = 0, kt = 0;           // tile counts: ceil(n/16), ceil(k/128)
+  size_t ktp = 0;                  // stored 128-k tiles per 16-row block: kt rounded up to 4 (zero tiles)
   size_t chunks = 0;               // scale chunks per n-tile
-  uint8_t *tiles = nullptr;        // [nt][kt][1 KiB]
+  uint8_t *tiles = nullptr;        // [nt][ktp][1 KiB]
   void *tscales = nullptr;         // [nt][chunks][16][spt]
   uint8_t *tzps = nullptr;         // same shape, one byte each; null when !has_zp
   // generic layout, kept only when the tiled one cannot be built
