@@ -27,6 +27,9 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_BF16_PEAK = 2500.0     # TFLOP/s dense (fp16 shares the rate)
 MFMA_I8_PEAK = 5000.0       # TOP/s dense
+# HBM bytes per skinny-kernel launch from rocprofv3 --pmc runs of this benchmark (fetch 15 306 KiB x 2.0, the factor a
+# plain 256 MiB copy gives for FETCH_SIZE on this GPU, + write 38 KiB x 1.0): profiles/int4_skinny_decode7b_graph_path.md
+SKINNY_TRAFFIC_BYTES = 31_385_000
 
 CFG7B = dict(n_layers=32, d_model=4096, n_heads=32, n_kv_heads=8, head_dim=128, d_ff=14336, vocab=32000,
              group_size=32, max_batch=16, max_ctx=2048 + 512, max_steps=1024, rope_theta=10000.0, rms_eps=1e-5)
@@ -198,6 +201,9 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-extra", action="store_true", help="skip the stand-alone kernels and the batch-16 run")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy (torch copy_ kernel, 3 launches): the known-size "
+                         "kernel that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (every config of the metric fits one "
@@ -216,6 +222,14 @@ def main():
         cfg["max_ctx"] = ((need + 127) // 128) * 128
     cfg["max_steps"] = max(cfg["max_steps"], args.steps + args.warmup)
     stream_ptr = torch.cuda.current_stream().cuda_stream
+
+    if args.calib_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     dec = Decoder(**cfg)
     dec.init_random(seed=1)
@@ -252,7 +266,7 @@ def main():
                    "batch": args.batch, "tokens_per_step": args.batch, "hip_graph": True},
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": SKINNY_TRAFFIC_BYTES,
             "kernel": "int4_skinny_kernel (all %d projections of a decode step)" % n_proj,
             "bytes_per_launch": int(bytes_per_launch), "avg_launch_us": round(avg_launch_s * 1e6, 3),
             "launches_timed": launches,
