@@ -105,3 +105,54 @@ def test_cache_overflow_is_an_error():
     dec.run(2)
     with pytest.raises(yscv_amd.YscvHipError):
         dec.run(1)
+
+
+# ---- single-launch (persistent) decode path ---------------------------------------------------------------
+# K = 2048 -> one 256-k tile per wave (single-tile records), K = 6144 -> three tiles (full + single record)
+PCFG = dict(n_layers=2, d_model=2048, n_heads=16, n_kv_heads=4, head_dim=128, d_ff=6144, vocab=1000, group_size=32,
+            max_batch=2, max_ctx=512, max_steps=32, rope_theta=10000.0, rms_eps=1e-5)
+
+
+def _prefill(rng, dec, ref, cfg, B, prefill):
+    for l in range(cfg["n_layers"]):
+        k = rng.standard_normal((B, prefill, cfg["n_kv_heads"], cfg["head_dim"])).astype(np.float16)
+        v = rng.standard_normal((B, prefill, cfg["n_kv_heads"], cfg["head_dim"])).astype(np.float16)
+        dec.set_kv(l, k, v)
+        if ref is not None:
+            ref.set_kv(l, k.astype(np.float32), v.astype(np.float32))
+
+
+@pytest.mark.parametrize("prefill", [0, 133, 300])
+def test_persistent_decode_matches_numpy_and_graph_path(prefill):
+    import torch
+
+    assert torch.cuda.is_available()
+    rng = np.random.default_rng(4100 + prefill)
+    cfg = dict(PCFG)
+    dec, ref = _build(rng, cfg)
+    _prefill(rng, dec, ref, cfg, 1, prefill)
+    tokens = np.array([7], np.int32)
+    dec.reset(tokens, prefill)
+    cur = tokens.copy()
+    for step in range(5):
+        dec.run(1, persistent=True)
+        got_logits = dec.logits()
+        got_tok = dec.tokens(step, 1)[0]
+        exp_logits = ref.step(cur, prefill + step)
+        err = np.abs(got_logits - exp_logits).max() / np.abs(exp_logits).max()
+        assert err < 2e-2, (step, err)
+        row = got_logits[0]
+        assert got_tok[0] == np.flatnonzero(row == row.max())[-1]
+        cur = got_tok.copy()
+    # several steps inside one launch reproduce the step-by-step token stream, and so does the graph path
+    first = dec.tokens(0, 5)[:, 0].copy()
+    logits5 = dec.logits().copy()
+    dec.reset(tokens, prefill)
+    dec.run(5, persistent=True)
+    assert np.array_equal(dec.tokens(0, 5)[:, 0], first)
+    assert np.abs(dec.logits() - logits5).max() <= 1e-5 * np.abs(logits5).max()
+    dec.reset(tokens, prefill)
+    dec.run(5, use_graph=True)
+    graph_logits = dec.logits()
+    assert np.array_equal(dec.tokens(0, 5)[:, 0], first)
+    assert np.abs(graph_logits - logits5).max() / np.abs(logits5).max() < 5e-3

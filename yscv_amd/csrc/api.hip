@@ -278,6 +278,49 @@ static int32_t int4_create(const uint8_t *packed, const void *scales, int32_t sc
   return YSCV_HIP_OK;
 }
 
+// Tiled weight from buffers that are already on the device (unsigned or signed nibbles in natural
+// [n][k/2] order, scales [n][k/g]); no zero points.  Used by the decoder's on-device random initialisation.
+int32_t int4_create_from_device(const uint8_t *d_packed, const void *d_scales, int scale_dtype, int nibble_format,
+                                size_t n, size_t k, size_t g, yscv_hip_int4_weight **out) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(out && d_packed && d_scales, "null argument");
+  *out = nullptr;
+  YSCV_REQUIRE(g == 32 || g == 64 || g % 128 == 0, "device-side creation needs a tiled group size");
+  YSCV_REQUIRE(k % g == 0 && n > 0 && k > 0, "bad shape n=%zu k=%zu group=%zu", n, k, g);
+  auto *w = new yscv_hip_int4_weight();
+  w->n = n;
+  w->k = k;
+  w->g = g;
+  w->scale_dtype = scale_dtype;
+  w->has_zp = false;
+  w->tiled = true;
+  w->gm = g == 32 ? GM32 : (g == 64 ? GM64 : GM128);
+  w->nt = ceil_div(n, (size_t)16);
+  w->kt = ceil_div(k, (size_t)128);
+  w->ktp = round_up(w->kt, (size_t)4);
+  w->chunks = w->gm == GM128 ? ceil_div(w->ktp, g / 128) : w->ktp;
+  const size_t ssz = dtype_size(scale_dtype);
+  const size_t tile_bytes = w->nt * w->ktp * (size_t)kTileBytes;
+  const size_t sc_elems = w->nt * w->chunks * 16 * (size_t)scales_per_chunk(w->gm);
+  hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->tiles), tile_bytes);
+  if (e == hipSuccess) e = hipMalloc(&w->tscales, sc_elems * ssz);
+  if (e != hipSuccess) {
+    free_int4(w);
+    return set_error(e == hipErrorOutOfMemory ? YSCV_HIP_ERR_OOM : YSCV_HIP_ERR_DEVICE, "weight allocation failed: %s",
+                     hipGetErrorString(e));
+  }
+  int32_t st = launch_int4_retile(d_packed, nibble_format, n, k, w->nt, w->ktp, w->tiles, nullptr);
+  if (st == YSCV_HIP_OK)
+    st = launch_int4_retile_scales(d_scales, scale_dtype, nullptr, n, k, g, w->gm, w->nt, w->chunks, w->tscales, nullptr, nullptr);
+  if (st != YSCV_HIP_OK) {
+    free_int4(w);
+    return st;
+  }
+  w->device_bytes = tile_bytes + sc_elems * ssz;
+  *out = w;
+  return YSCV_HIP_OK;
+}
+
 static void free_i8(yscv_hip_i8_weight *b) {
   if (!b) return;
   (void)hipFree(b->frag);

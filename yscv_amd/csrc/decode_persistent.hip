@@ -1,0 +1,930 @@
+// Persistent batch-1 decode: one cooperative launch runs whole decode steps of the Llama-style
+// decoder (the loop of apps/llm-bench/src/main.rs:525-548: feed the last token and the KV cache,
+// take the greedy pick, repeat) with the int4 weights streamed exactly once per step.
+//
+// Why one launch: at batch 1 a decode step is ~4.3 GB of HBM traffic cut into ~160 dependent
+// stages; as separate kernels every stage pays a launch and a cold start.  Here G workgroups (one per
+// CU, 8 waves each) stay resident and
+//   * every wave streams its own pre-ordered weight records (layout in persist.hpp) through a ring
+//     in LDS filled by direct global->LDS loads; the ring keeps running across stage boundaries, so
+//     the weights of the next stages are already in flight while a stage waits for its input;
+//   * stages exchange their small activation vectors through "tagged entries" in global memory:
+//     an 8-byte {payload, tag} word written with one agent-scope store and polled with coherent
+//     128-bit loads.  A consumer wave waits for exactly the entries it needs, so there is no grid
+//     barrier and no cache flush; the tag (step epoch, layer) makes stale data recognisable;
+//   * the residual stream lives in registers of the threads that own its rows.
+// Every wait is bounded: a wave that gives up sets abort_flag, every later wait returns at once and
+// the host reports the failure.
+//
+// Arithmetic per 32-k block: one v_mfma_f32_16x16x32_f16.  With a single activation row the 16 rows
+// of the A operand carry 16 different k-blocks of the activation (row i = k-block i of the wave's
+// 512-k fragment), and the 16 columns of B carry 8 weight rows x 2 k-blocks, so each MFMA produces
+// the dot products of 8 rows over two k-blocks in rows {j, j+4, ...} of D; the lanes that hold a
+// useful element apply the group scale in fp32.  Weights stay exact integers (0x6400 | q = 1024 + q);
+// the offset term sum_k x_k * (1024 + 8) is computed once per fragment by the same MFMA against a
+// constant operand and subtracted per group.
+//
+// Semantics of the glue (tolerance-checked against the numpy restatement, like the multi-kernel path):
+// RMSNorm crates/yscv-kernels/src/ops/norm.rs:1497-1518, RoPE ops/rope.rs:24-117, grouped-query
+// attention crates/yscv-onnx/src/runner/linear.rs:552-646 over the fp16 cache, greedy pick = last
+// maximal logit (apps/llm-bench/src/main.rs:538-543).
+#include <hip/hip_runtime.h>
+
+#include "int4_common.hpp"
+#include "persist.hpp"
+
+namespace yscv {
+
+typedef unsigned long long u64;
+
+constexpr int RING = 7;                        // records in flight per wave
+constexpr int SLOT = PS_REC_FULL;              // LDS bytes per ring slot
+constexpr int RING_BYTES = PS_WAVES * RING * SLOT;
+constexpr int PART_ROWS = 256;                 // rows a workgroup may own in one projection
+constexpr int PART_BYTES = 2 * PS_WAVES * PART_ROWS * 4;
+constexpr int ATT_BYTES = 10240;
+constexpr int PERSIST_LDS = RING_BYTES + PART_BYTES + ATT_BYTES;
+constexpr unsigned SPIN_LIMIT = 300000u;
+constexpr int ACHUNK = 128;                    // positions per attention work item (4 waves x 32)
+constexpr int PART_REC = 132;                  // entries per (head, chunk) partial: max, sum, o[128], pad
+
+#define AS1(p) ((const void __attribute__((address_space(1))) *)(p))
+#define AS3(p) ((void __attribute__((address_space(3))) *)(p))
+
+__device__ __forceinline__ void st_entry(u64 *p, uint32_t payload, uint32_t tag) {
+  __hip_atomic_store(p, ((u64)tag << 32) | payload, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// coherent 128-bit load (two entries); the result is valid only after wait_vm
+__device__ __forceinline__ uint4_t ld2(const void *p) {
+  uint4_t v;
+  asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+__device__ __forceinline__ void wait_vm(uint4_t &a) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(a)::"memory"); }
+__device__ __forceinline__ void wait_vm(uint4_t &a, uint4_t &b) {
+  asm volatile("s_waitcnt vmcnt(0)" : "+v"(a), "+v"(b)::"memory");
+}
+__device__ __forceinline__ void wait_vm(uint4_t &a, uint4_t &b, uint4_t &c, uint4_t &d) {
+  asm volatile("s_waitcnt vmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"memory");
+}
+__device__ __forceinline__ void wait_vm8(uint4_t *v) {
+  asm volatile("s_waitcnt vmcnt(0)"
+               : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7])::"memory");
+}
+// tags are compared on their low 24 bits; the top byte of the tag word may carry a block exponent
+__device__ __forceinline__ bool tag_ok(uint32_t word, uint32_t tag) { return ((word ^ tag) & 0xFFFFFFu) == 0; }
+__device__ __forceinline__ bool aborted(const PersistModel &m) {
+  return __hip_atomic_load(m.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+}
+__device__ __forceinline__ void set_abort(const PersistModel &m) {
+  __hip_atomic_store(m.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t pack_h2(float a, float b) {
+  a = fminf(fmaxf(a, -65504.0f), 65504.0f);
+  b = fminf(fmaxf(b, -65504.0f), 65504.0f);
+  U32H2 u;
+  u.h = half2_t{(_Float16)a, (_Float16)b};
+  return u.u;
+}
+__device__ __forceinline__ float h2_lo(uint32_t w) {
+  U32H2 u;
+  u.u = w;
+  return (float)u.h[0];
+}
+__device__ __forceinline__ float h2_hi(uint32_t w) {
+  U32H2 u;
+  u.u = w;
+  return (float)u.h[1];
+}
+__device__ __forceinline__ half8_t as_half8(uint4_t v) {
+  union {
+    uint4_t u;
+    half8_t h;
+  } x;
+  x.u = v;
+  return x.h;
+}
+// position of value i (even) of a k-vector inside its exchange buffer: fragment order of the consumer
+__device__ __forceinline__ int xidx(int i, int ks, int frags) {
+  const int v = i / ks;
+  const int kk = i - v * ks;
+  const int f = kk >> 9, k2 = kk & 511;
+  const int r = k2 >> 5, c = (k2 >> 3) & 3, q = (k2 & 7) >> 1;
+  return ((v * frags + f) << 8) + ((q >> 1) << 7) + 2 * (16 * c + r) + (q & 1);
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + __expf(-g)); }
+// order of the greedy pick: higher value wins, equal (or unordered) values -> larger index
+__device__ __forceinline__ bool better(float va, int ia, float vb, int ib) {
+  if (ia < 0) return false;
+  if (ib < 0) return true;
+  if (va > vb) return true;
+  if (vb > va) return false;
+  return ia > ib;
+}
+
+__global__ void __launch_bounds__(512, 1)
+decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int max_steps, uint32_t epoch0) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  float *part_lds = reinterpret_cast<float *>(lds + RING_BYTES);                 // [2][8][PART_ROWS]
+  unsigned char *att_lds = lds + RING_BYTES + PART_BYTES;
+  _Float16 *p_lds = reinterpret_cast<_Float16 *>(att_lds);                        // [4 waves][4 heads][32]
+  float *w_m = reinterpret_cast<float *>(att_lds + 1024);                         // [4][4]
+  float *w_l = reinterpret_cast<float *>(att_lds + 1024 + 64);                    // [4][4]
+  float *w_o = reinterpret_cast<float *>(att_lds + 1024 + 128);                   // [4][4][128]
+  int *tok_lds = reinterpret_cast<int *>(att_lds + 1024 + 128 + 8192);            // [1]
+  float *arg_v = reinterpret_cast<float *>(att_lds + 1024 + 128 + 8192 + 64);     // [8]
+  int *arg_i = reinterpret_cast<int *>(att_lds + 1024 + 128 + 8192 + 128);        // [8]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, c = lane >> 4;
+  const int wg = blockIdx.x;
+  const int G = m.G;
+  const int L = m.n_layers;
+  const int D = m.d_model;
+  const int HQ = m.n_heads, HKV = m.n_kv_heads, GROUP = HQ / HKV;
+  const int max_chunks = m.max_ctx / ACHUNK;
+  const uint32_t magic = 0x64006400u;
+
+  // ---- weight stream: prefetcher state (wave uniform) ------------------------------------------------
+  const unsigned char *const stream_base = m.stream + m.wg_off[wg] + (size_t)wave * m.wave_bytes[wg];
+  const unsigned char *pf_ptr = stream_base;
+  int pf_slot = 0, pf_kind = 0, pf_layer = 0, pf_blk = 0, pf_pair = 0;
+  auto nbw = [&](int kind) { return wg < m.ph[kind].nb ? (m.ph[kind].nb - wg + G - 1) / G : 0; };
+  const bool has_work = m.wave_bytes[wg] != 0;
+  unsigned char *const ring = lds + (size_t)wave * RING * SLOT;
+  const uint32_t ring_lds = (uint32_t)(size_t)ring;  // low 32 bits of an LDS pointer = LDS byte address
+
+  auto pf_next_kind = [&]() {
+    if (pf_kind == PK_DOWN) {
+      pf_layer++;
+      pf_kind = pf_layer == L ? PK_LM : PK_QKV;
+    } else if (pf_kind == PK_LM) {
+      pf_layer = 0;
+      pf_kind = PK_QKV;
+      pf_ptr = stream_base;
+    } else {
+      pf_kind++;
+    }
+  };
+  auto pf_issue = [&]() {
+    if (!has_work) return;
+    while (nbw(pf_kind) == 0) pf_next_kind();
+    const int pairs = m.ph[pf_kind].pairs;
+    const bool single = (pf_pair == pairs - 1) && (m.ph[pf_kind].tiles & 1);
+    unsigned char *dst = ring + pf_slot * SLOT;
+    __builtin_amdgcn_global_load_lds(AS1(pf_ptr + lane * 16), AS3(dst), 16, 0, 2);
+    __builtin_amdgcn_global_load_lds(AS1(pf_ptr + (single ? 0 : 1024) + lane * 16), AS3(dst + 1024), 16, 0, 2);
+    __builtin_amdgcn_global_load_lds(AS1(pf_ptr + (single ? 1024 : 2048) + lane * 4), AS3(dst + 2048), 4, 0, 2);
+    pf_ptr += single ? PS_REC_SINGLE : PS_REC_FULL;
+    pf_slot = pf_slot + 1 == RING ? 0 : pf_slot + 1;
+    if (++pf_pair == pairs) {
+      pf_pair = 0;
+      if (++pf_blk >= nbw(pf_kind)) {
+        pf_blk = 0;
+        pf_next_kind();
+      }
+    }
+  };
+#pragma unroll 1
+  for (int i = 0; i < RING - 1; i++) pf_issue();
+  int cslot = 0;  // ring slot of the next record to consume
+
+  // ---- one record: 8 rows x 512 k against the activation fragment xa ------------------------------
+  auto consume = [&](bool single, const half8_t &xa, const float4_t &z, float &acc) {
+    pf_issue();
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (RING - 1)) : "memory");
+    const uint32_t a_w = ring_lds + cslot * SLOT + lane * 16;
+    const uint32_t a_s = ring_lds + cslot * SLOT + (c >> 1) * 128 + r * 8;
+    uint4_t w0, w1;
+    typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+    uint2_t sc;
+    asm volatile(
+        "ds_read_b128 %0, %3\n\tds_read_b128 %1, %3 offset:1024\n\tds_read_b64 %2, %4 offset:2048\n\ts_waitcnt lgkmcnt(0)"
+        : "=&v"(w0), "=&v"(w1), "=&v"(sc)
+        : "v"(a_w), "v"(a_s)
+        : "memory");
+    cslot = cslot + 1 == RING ? 0 : cslot + 1;
+    const float4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    float d0[4], d1[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      U32H2 q0, q1, q2, q3;
+      const uint32_t s = w0[j], s2 = s >> 8;
+      q0.u = (s & 0x000F000Fu) | magic;
+      q1.u = (s & 0x00F000F0u) | magic;
+      q2.u = (s2 & 0x000F000Fu) | magic;
+      q3.u = (s2 & 0x00F000F0u) | magic;
+      const half8_t b = {q0.h[0], q0.h[1], q1.h[0], q1.h[1], q2.h[0], q2.h[1], q3.h[0], q3.h[1]};
+      const float4_t dd = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, b, zero, 0, 0, 0);
+      d0[j] = dd[j];
+    }
+    if (!single) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        U32H2 q0, q1, q2, q3;
+        const uint32_t s = w1[j], s2 = s >> 8;
+        q0.u = (s & 0x000F000Fu) | magic;
+        q1.u = (s & 0x00F000F0u) | magic;
+        q2.u = (s2 & 0x000F000Fu) | magic;
+        q3.u = (s2 & 0x00F000F0u) | magic;
+        const half8_t b = {q0.h[0], q0.h[1], q1.h[0], q1.h[1], q2.h[0], q2.h[1], q3.h[0], q3.h[1]};
+        const float4_t dd = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, b, zero, 0, 0, 0);
+        d1[j] = dd[j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; j++) d1[j] = 0.0f;
+    }
+    const bool second = (c >> 1) != 0;
+    const float s0 = h2_lo(sc[0]), s1 = h2_hi(sc[0]), s2 = h2_lo(sc[1]), s3 = h2_hi(sc[1]);
+    acc = fmaf(s0, (second ? d1[0] : d0[0]) - z[0], acc);
+    acc = fmaf(s1, (second ? d1[1] : d0[1]) - z[1], acc);
+    acc = fmaf(s2, (second ? d1[2] : d0[2]) - z[2], acc);
+    acc = fmaf(s3, (second ? d1[3] : d0[3]) - z[3], acc);
+  };
+
+  // ---- bounded waiting ------------------------------------------------------------------------------
+  unsigned spin_budget = SPIN_LIMIT;
+  auto poll_backoff = [&]() -> bool {  // false: give up (the budget ran out or another wave gave up)
+    __builtin_amdgcn_s_sleep(2);
+    if (spin_budget <= 1 || ((spin_budget & 63u) == 0 && aborted(m))) {
+      set_abort(m);
+      spin_budget = 1;
+      return false;
+    }
+    spin_budget--;
+    return true;
+  };
+  // Fragment f of this wave's slice of an exchange vector, as the A operand (row i = k-block i).
+  // With ss != null the per-workgroup sum-of-squares entries behind the vector are summed into 1/rms
+  // (returned through rstd).  A `normed` vector holds fp16(h * gamma * 2^-e) with the exponent e of each
+  // 8-row block in the top byte of its tag words; the operand is then fp16(h * gamma * rstd), the
+  // activation the multi-kernel path feeds (RMSNorm, crates/yscv-kernels/src/ops/norm.rs:1497-1518).
+  auto load_fragment = [&](const u64 *buf, int ks, int frags, int f, uint32_t tag, const u64 *ss, int ss_count,
+                           bool normed, float &rstd) -> half8_t {
+    const u64 *p = buf + (((size_t)wave * frags + f) << 8) + 2 * lane;
+    const bool valid = (512 * f + 32 * r) < ks;
+    const bool v0 = ss && 4 * lane < ss_count, v1 = ss && 4 * lane + 1 < ss_count, v2 = ss && 4 * lane + 2 < ss_count,
+               v3 = ss && 4 * lane + 3 < ss_count;
+    const u64 *sp = ss ? ss + 4 * lane : buf;
+    uint4_t a, b, sa, sb;
+    while (true) {
+      a = ld2(p);
+      b = ld2(p + 128);
+      sa = ld2(sp);
+      sb = ld2(sp + 2);
+      wait_vm(a, b, sa, sb);
+      bool ok = !valid || (tag_ok(a[1], tag) && tag_ok(a[3], tag) && tag_ok(b[1], tag) && tag_ok(b[3], tag));
+      ok = ok && (!v0 || tag_ok(sa[1], tag)) && (!v1 || tag_ok(sa[3], tag)) && (!v2 || tag_ok(sb[1], tag)) &&
+           (!v3 || tag_ok(sb[3], tag));
+      if (__all(ok)) break;
+      if (!poll_backoff()) break;
+    }
+    if (ss) {
+      const float sq = (v0 ? __uint_as_float(sa[0]) : 0.0f) + (v1 ? __uint_as_float(sa[2]) : 0.0f) +
+                       (v2 ? __uint_as_float(sb[0]) : 0.0f) + (v3 ? __uint_as_float(sb[2]) : 0.0f);
+      rstd = 1.0f / sqrtf(wave_sum(sq) / (float)D + m.eps);
+    }
+    U32H2 u0, u1, u2, u3;
+    u0.u = valid ? a[0] : 0u;
+    u1.u = valid ? a[2] : 0u;
+    u2.u = valid ? b[0] : 0u;
+    u3.u = valid ? b[2] : 0u;
+    if (normed) {
+      const float fac = valid ? ldexpf(rstd, (int)(a[1] >> 24) - 128) : 0.0f;
+      u0.h = half2_t{(_Float16)((float)u0.h[0] * fac), (_Float16)((float)u0.h[1] * fac)};
+      u1.h = half2_t{(_Float16)((float)u1.h[0] * fac), (_Float16)((float)u1.h[1] * fac)};
+      u2.h = half2_t{(_Float16)((float)u2.h[0] * fac), (_Float16)((float)u2.h[1] * fac)};
+      u3.h = half2_t{(_Float16)((float)u3.h[0] * fac), (_Float16)((float)u3.h[1] * fac)};
+    }
+    // the slots that meet 1024 + 16 q carry x / 16 (exact: a power of two)
+    const half2_t sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+    u1.h = u1.h * sixteenth;
+    u3.h = u3.h * sixteenth;
+    return half8_t{u0.h[0], u0.h[1], u1.h[0], u1.h[1], u2.h[0], u2.h[1], u3.h[0], u3.h[1]};
+  };
+
+  // ---- one projection: leaves the row sums of this workgroup in part_lds[pb]; returns 1/rms ------------
+  int pb = 0;
+  const half8_t bc = {(_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f,
+                      (_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f};
+  const int ss_count = m.ph[PK_O].nb < G ? m.ph[PK_O].nb : G;
+  auto gemv = [&](int kind, const u64 *in_buf, uint32_t tag, bool with_ss) {
+    const int ks = m.ph[kind].ks, frags = m.ph[kind].frags, pairs = m.ph[kind].pairs;
+    const bool odd = m.ph[kind].tiles & 1;
+    const int nb = nbw(kind);
+    half8_t xa[4];
+    float4_t z[4];
+    float rstd = 1.0f;
+    const u64 *ss = with_ss ? in_buf + persist_vec_entries(m.ph[kind].k) : nullptr;
+#pragma unroll
+    for (int f = 0; f < 4; f++) {
+      if (f < frags && nb > 0) {
+        xa[f] = load_fragment(in_buf, ks, frags, f, tag, f == 0 ? ss : nullptr, ss_count, with_ss, rstd);
+        const float4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+        z[f] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[f], bc, zero, 0, 0, 0);
+      } else {
+        xa[f] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        z[f] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+      }
+    }
+    float *dst = part_lds + ((size_t)pb * PS_WAVES + wave) * PART_ROWS;
+    const bool useful = (c & 1) == (r >> 3);
+#pragma unroll 1
+    for (int blk = 0; blk < nb; blk++) {
+      float acc = 0.0f;
+#pragma unroll
+      for (int p = 0; p < 4; p++)
+        if (p < pairs) consume(odd && p == pairs - 1, xa[p], z[p], acc);
+      acc = useful ? acc : 0.0f;
+      acc += __shfl_xor(acc, 8, 64);
+      acc += __shfl_xor(acc, 16, 64);
+      acc += __shfl_xor(acc, 32, 64);
+      if (lane < 8) dst[blk * 8 + lane] = acc;
+    }
+    lds_barrier();
+  };
+  auto row_sum = [&](int row_slot) -> float {
+    const float *src = part_lds + (size_t)pb * PS_WAVES * PART_ROWS + row_slot;
+    float v = 0.0f;
+#pragma unroll
+    for (int w = 0; w < PS_WAVES; w++) v += src[w * PART_ROWS];
+    return v;
+  };
+
+  // ---- residual stream: thread t < 8 * nbw(PK_O) owns row 8 * (wg + G * (t >> 3)) + (t & 7) ---------
+  const int nb_d = nbw(PK_O);
+  const bool own = tid < 8 * nb_d;  // 8 * nb_d <= 64: all owners sit in wave 0
+  const int own_row = 8 * (wg + G * (tid >> 3)) + (tid & 7);
+  float h = 0.0f;
+  // publish fp16(h * gamma * 2^-e) pairs (fragment order of a k = d_model consumer; e = exponent of the largest
+  // value of the 8-row block, carried in the top byte of the tag word) + this workgroup's sum of squares
+  auto publish_h = [&](u64 *buf, const float *gamma, uint32_t tag) {
+    if (tid < 64) {
+      const float xs = own ? h * gamma[own_row] : 0.0f;
+      float mx = fabsf(xs);
+      mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
+      int e = (mx > 0.0f && mx < INFINITY) ? ilogbf(mx) + 1 : 0;
+      e = e < -100 ? -100 : (e > 100 ? 100 : e);
+      const float sc = ldexpf(xs, -e);
+      const float nxt = __shfl_down(sc, 1, 64);
+      if (own && !(tid & 1))
+        st_entry(buf + xidx(own_row, m.ph[PK_QKV].ks, m.ph[PK_QKV].frags), pack_h2(sc, nxt), tag | ((uint32_t)(e + 128) << 24));
+      const float ss = wave_sum(own ? h * h : 0.0f);
+      if (tid == 0 && nb_d > 0) st_entry(buf + persist_vec_entries(D) + wg, __float_as_uint(ss), tag);
+    }
+  };
+
+  // ---- attention over the cached positions [0, pos): partials per (head, 128-position chunk) ---------
+  auto attention_items = [&](int layer, int pos, uint32_t tag) {
+    const int nchunks = (pos + ACHUNK - 1) / ACHUNK;
+    const int items = HKV * nchunks;
+    const _Float16 *kc = m.kc[layer];
+    const _Float16 *vc = m.vc[layer];
+    const float scale = 0.08838834764831845f;  // 1 / sqrt(128)
+#pragma unroll 1
+    for (int id = wg; id < items; id += G) {
+      const int chunk = id / HKV, kvh = id - chunk * HKV;
+      float m_h = -INFINITY, l_h = 0.0f;
+      float o_acc[8];
+#pragma unroll
+      for (int t = 0; t < 8; t++) o_acc[t] = 0.0f;
+      const int p0 = chunk * ACHUNK + wave * 32;
+      if (wave < 4 && p0 < pos) {
+        const _Float16 *kbase = kc + ((size_t)kvh * m.max_ctx + p0) * 128;
+        const _Float16 *vbase = vc + (((size_t)kvh * (m.max_ctx / 8) + p0 / 8) * 128) * 8;
+        half8_t kf[2][4], vf[8];
+        const half8_t hz = {0, 0, 0, 0, 0, 0, 0, 0};
+        // Blocks that were complete before this launch never change and are read with plain loads.
+        // Positions appended during this launch were written with agent-scope stores by another
+        // workgroup: their blocks are read with coherent loads, and only where already valid.
+        const bool recent = p0 + 32 > pos0;
+        if (!recent) {
+#pragma unroll
+          for (int pbk = 0; pbk < 2; pbk++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+              kf[pbk][j] = *reinterpret_cast<const half8_t *>(kbase + (size_t)(pbk * 16 + r) * 128 + 32 * c + 8 * j);
+#pragma unroll
+          for (int t = 0; t < 8; t++) vf[t] = *reinterpret_cast<const half8_t *>(vbase + ((size_t)c * 128 + t * 16 + r) * 8);
+        } else {
+          uint4_t tmp[8];
+#pragma unroll
+          for (int pbk = 0; pbk < 2; pbk++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) tmp[pbk * 4 + j] = ld2(kbase + (size_t)(pbk * 16 + r) * 128 + 32 * c + 8 * j);
+          wait_vm8(tmp);
+#pragma unroll
+          for (int pbk = 0; pbk < 2; pbk++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) kf[pbk][j] = (p0 + pbk * 16 + r) < pos ? as_half8(tmp[pbk * 4 + j]) : hz;
+#pragma unroll
+          for (int t = 0; t < 8; t++) tmp[t] = ld2(vbase + ((size_t)c * 128 + t * 16 + r) * 8);
+          wait_vm8(tmp);
+#pragma unroll
+          for (int t = 0; t < 8; t++) vf[t] = as_half8(tmp[t]);
+        }
+        // Q operand: MFMA row 4*hh carries head hh of this group; lane (r, c) holds d = 32c + 8j + 0..7.
+        // q arrives as fp16-pair entries in natural order: entry (head*128 + d) / 2.
+        half8_t qa[4];
+        {
+          const int hh = r >> 2;
+          const bool valid = ((r & 3) == 0) && hh < GROUP;
+          const u64 *qsrc = m.qkv + ((size_t)(kvh * GROUP + (valid ? hh : 0)) * 128 + 32 * c) / 2;
+          uint4_t qv[8];
+          while (true) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) qv[i] = ld2(qsrc + 2 * i);
+            wait_vm8(qv);
+            bool ok = true;
+#pragma unroll
+            for (int i = 0; i < 8; i++) ok = ok && tag_ok(qv[i][1], tag) && tag_ok(qv[i][3], tag);
+            if (__all(ok || !valid)) break;
+            if (!poll_backoff()) break;
+          }
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            U32H2 e0, e1, e2, e3;
+            e0.u = valid ? qv[2 * j][0] : 0u;
+            e1.u = valid ? qv[2 * j][2] : 0u;
+            e2.u = valid ? qv[2 * j + 1][0] : 0u;
+            e3.u = valid ? qv[2 * j + 1][2] : 0u;
+            qa[j] = half8_t{e0.h[0], e0.h[1], e1.h[0], e1.h[1], e2.h[0], e2.h[1], e3.h[0], e3.h[1]};
+          }
+        }
+        float sc2[2];
+#pragma unroll
+        for (int pbk = 0; pbk < 2; pbk++) {
+          float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+          for (int j = 0; j < 4; j++) d = __builtin_amdgcn_mfma_f32_16x16x32_f16(qa[j], kf[pbk][j], d, 0, 0, 0);
+          const int p = p0 + pbk * 16 + r;  // lane (r, c): score of head c at position p
+          sc2[pbk] = (p < pos) ? d[0] * scale : -INFINITY;
+        }
+        float mx = fmaxf(sc2[0], sc2[1]);
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+        const float e0 = (sc2[0] == -INFINITY) ? 0.0f : __expf(sc2[0] - mx);
+        const float e1 = (sc2[1] == -INFINITY) ? 0.0f : __expf(sc2[1] - mx);
+        float sum = e0 + e1;
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+        m_h = mx;
+        l_h = sum;
+        _Float16 *pw = p_lds + (size_t)wave * 4 * 32;
+        pw[c * 32 + r] = (_Float16)e0;
+        pw[c * 32 + 16 + r] = (_Float16)e1;
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+        half8_t pa = {0, 0, 0, 0, 0, 0, 0, 0};
+        if ((r & 3) == 0 && (r >> 2) < GROUP) pa = *reinterpret_cast<const half8_t *>(pw + (r >> 2) * 32 + 8 * c);
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+          half8_t vv = vf[t];
+          if (p0 + 8 * c >= pos) vv = hz;
+          else if (p0 + 8 * c + 8 > pos) {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+              if (p0 + 8 * c + e >= pos) vv[e] = (_Float16)0.0f;
+          }
+          float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
+          d = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vv, d, 0, 0, 0);
+          o_acc[t] = d[0];  // lane (r, c): o of head c at d = 16 t + r
+        }
+      }
+      if (wave < 4) {
+        if (r == 0) {
+          w_m[wave * 4 + c] = m_h;
+          w_l[wave * 4 + c] = l_h;
+        }
+#pragma unroll
+        for (int t = 0; t < 8; t++) w_o[((size_t)wave * 4 + c) * 128 + t * 16 + r] = o_acc[t];
+      }
+      lds_barrier();
+      if (wave < 4) {
+        for (int idx = tid; idx < GROUP * 128; idx += 256) {
+          const int hh = idx >> 7, dd = idx & 127;
+          float mx = -INFINITY;
+#pragma unroll
+          for (int w = 0; w < 4; w++) mx = fmaxf(mx, w_m[w * 4 + hh]);
+          float l = 0.0f, o = 0.0f;
+#pragma unroll
+          for (int w = 0; w < 4; w++) {
+            const float f = (w_m[w * 4 + hh] == -INFINITY) ? 0.0f : __expf(w_m[w * 4 + hh] - mx);
+            l += w_l[w * 4 + hh] * f;
+            o += w_o[((size_t)w * 4 + hh) * 128 + dd] * f;
+          }
+          u64 *dst = m.part + ((size_t)(kvh * GROUP + hh) * max_chunks + chunk) * PART_REC;
+          st_entry(dst + 2 + dd, __float_as_uint(o), tag);
+          if (dd == 0) {
+            st_entry(dst, __float_as_uint(mx), tag);
+            st_entry(dst + 1, __float_as_uint(l), tag);
+          }
+        }
+      }
+      lds_barrier();
+    }
+  };
+
+  // merge the chunk partials of one head with the new position; also appends k / v to the cache
+  auto attention_combine = [&](int layer, int head, int pos, uint32_t tag) {
+    const int nchunks = (pos + ACHUNK - 1) / ACHUNK;
+    const int kvh = head / GROUP;
+    float M = -INFINITY, Ls = 0.0f, O0 = 0.0f, O1 = 0.0f;
+    auto merge = [&](float mc, float lc, float o0, float o1) {
+      if (mc == -INFINITY) return;
+      const float Mn = fmaxf(M, mc);
+      const float a = (M == -INFINITY) ? 0.0f : __expf(M - Mn);
+      const float b = __expf(mc - Mn);
+      Ls = Ls * a + lc * b;
+      O0 = O0 * a + o0 * b;
+      O1 = O1 * a + o1 * b;
+      M = Mn;
+    };
+#pragma unroll 1
+    for (int ch = 0; ch < nchunks; ch++) {
+      const u64 *rec = m.part + ((size_t)head * max_chunks + ch) * PART_REC;
+      uint4_t a, b;
+      while (true) {
+        a = ld2(rec);
+        b = ld2(rec + 2 + 2 * lane);
+        wait_vm(a, b);
+        const bool ok = tag_ok(a[1], tag) && tag_ok(a[3], tag) && tag_ok(b[1], tag) && tag_ok(b[3], tag);
+        if (__all(ok)) break;
+        if (!poll_backoff()) break;
+      }
+      merge(__uint_as_float(a[0]), __uint_as_float(a[2]), __uint_as_float(b[0]), __uint_as_float(b[2]));
+    }
+    // the token of this step: q . k_new / sqrt(d) with k_new, v_new straight from the qkv exchange buffer
+    const u64 *qe = m.qkv + (size_t)head * 64 + lane;
+    const u64 *ke = m.qkv + (size_t)(HQ + kvh) * 64 + lane;
+    const u64 *ve = m.qkv + (size_t)(HQ + HKV + kvh) * 64 + lane;
+    u64 q, k, v;
+    while (true) {
+      q = __hip_atomic_load(qe, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      k = __hip_atomic_load(ke, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      v = __hip_atomic_load(ve, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool ok = tag_ok((uint32_t)(q >> 32), tag) && tag_ok((uint32_t)(k >> 32), tag) && tag_ok((uint32_t)(v >> 32), tag);
+      if (__all(ok)) break;
+      if (!poll_backoff()) break;
+    }
+    const uint32_t qw = (uint32_t)q, kw = (uint32_t)k, vw = (uint32_t)v;
+    const float s = wave_sum(h2_lo(qw) * h2_lo(kw) + h2_hi(qw) * h2_hi(kw)) * 0.08838834764831845f;
+    merge(s, 1.0f, h2_lo(vw), h2_hi(vw));
+    const float inv = Ls > 0.0f ? 1.0f / Ls : 0.0f;
+    st_entry(m.ao + xidx(head * 128 + 2 * lane, m.ph[PK_O].ks, m.ph[PK_O].frags), pack_h2(O0 * inv, O1 * inv), tag);
+    if (head == kvh * GROUP) {
+      // append: other workgroups read these lines in later steps of this launch -> agent-scope stores
+      _Float16 *kc = m.kc[layer];
+      _Float16 *vc = m.vc[layer];
+      uint32_t *krow = reinterpret_cast<uint32_t *>(kc + ((size_t)kvh * m.max_ctx + pos) * 128);
+      __hip_atomic_store(krow + lane, kw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      uint16_t *vslab = reinterpret_cast<uint16_t *>(vc + (((size_t)kvh * (m.max_ctx / 8) + pos / 8) * 128) * 8) + (pos & 7);
+      __hip_atomic_store(vslab + (size_t)(2 * lane) * 8, (uint16_t)(vw & 0xFFFFu), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(vslab + (size_t)(2 * lane + 1) * 8, (uint16_t)(vw >> 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  };
+
+  // ---- the decode loop ---------------------------------------------------------------------------------
+  if (tid == 0) tok_lds[0] = m.tokens[0];
+  lds_barrier();
+  int token = tok_lds[0];
+  const float *gam = m.gammas;
+
+#pragma unroll 1
+  for (int s = 0; s < n_steps; s++) {
+    const int pos = pos0 + s;
+    const uint32_t tag_base = (epoch0 + (uint32_t)s) * (uint32_t)(L + 2) + 1u;  // used modulo 2^24
+    spin_budget = spin_budget > 1 ? SPIN_LIMIT : 1;
+    token = token < 0 ? 0 : (token >= m.vocab ? m.vocab - 1 : token);
+    if (own) h = (float)m.emb[(size_t)token * D + own_row];
+    publish_h(m.xn, gam, tag_base & 0xFFFFFFu);
+
+#pragma unroll 1
+    for (int l = 0; l < L; l++) {
+      const uint32_t tag = (tag_base + (uint32_t)l) & 0xFFFFFFu;
+      // ---- q/k/v projection + rotary embedding ------------------------------------------------------------
+      {
+        const int nb = nbw(PK_QKV);
+        const bool act = tid < 8 * nb;
+        const int pr = 8 * (wg + G * (tid >> 3)) + (tid & 7);  // row in stream order
+        const bool rot = act && pr < (HQ + HKV) * 128;
+        float sn = 0.0f, cs = 1.0f;
+        if (rot) {
+          const int i = (pr & 127) >> 1;
+          const float inv_freq = 1.0f / powf(m.theta, (float)(2 * i) / 128.0f);
+          sincosf(inv_freq * (float)pos, &sn, &cs);
+        }
+        gemv(PK_QKV, m.xn, tag, true);
+        const float val = act ? row_sum(tid) : 0.0f;
+        const float partner = __shfl_xor(val, 1, 64);
+        const int which = pr & 1;
+        const float x0 = which ? partner : val, x1 = which ? val : partner;
+        const float rotated = which ? x0 * sn + x1 * cs : x0 * cs - x1 * sn;
+        const float out = rot ? rotated : val;
+        const float out2 = __shfl_down(out, 2, 64);  // same member of the next rotary pair
+        const float out1 = __shfl_down(out, 1, 64);  // next row (v rows are in natural order)
+        if (act) {
+          if (rot) {
+            if (!(tid & 2)) {
+              const int head = pr >> 7, i = (pr & 127) >> 1;
+              const int dim = i + 64 * which;
+              st_entry(m.qkv + (head * 128 + dim) / 2, pack_h2(out, out2), tag);
+            }
+          } else if (!(tid & 1)) {
+            st_entry(m.qkv + pr / 2, pack_h2(out, out1), tag);
+          }
+        }
+        pb ^= 1;
+      }
+      // ---- attention -------------------------------------------------------------------------------------
+      attention_items(l, pos, tag);
+      if (wave == 4)
+        for (int head = wg; head < HQ; head += G) attention_combine(l, head, pos, tag);
+      // ---- output projection + residual ------------------------------------------------------------------
+      {
+        gemv(PK_O, m.ao, tag, false);
+        if (own) h += row_sum(tid);
+        if (own && m.dbg_h) m.dbg_h[((size_t)l * 2) * D + own_row] = h;
+        publish_h(m.xn2, gam + (size_t)(2 * l + 1) * D, tag);
+        pb ^= 1;
+      }
+      // ---- gate / up projection + SwiGLU (rows interleaved: 2i = gate_i, 2i+1 = up_i) ---------------------
+      {
+        const int nb = nbw(PK_GU);
+        gemv(PK_GU, m.xn2, tag, true);
+        const bool act = tid < 8 * nb;
+        const int pr = 8 * (wg + G * (tid >> 3)) + (tid & 7);
+        const float val = act ? row_sum(tid) : 0.0f;
+        const float up = __shfl_down(val, 1, 64);
+        const float a = silu_f(val) * up;          // meaningful in even threads
+        const float a2 = __shfl_down(a, 2, 64);    // act value of the next pair of rows
+        if (act && !(tid & 3)) st_entry(m.act + xidx(pr / 2, m.ph[PK_DOWN].ks, m.ph[PK_DOWN].frags), pack_h2(a, a2), tag);
+        pb ^= 1;
+      }
+      // ---- down projection + residual; publishes the input of the next layer (or of lm_head) ---------------
+      {
+        gemv(PK_DOWN, m.act, tag, false);
+        if (own) h += row_sum(tid);
+        if (own && m.dbg_h) m.dbg_h[((size_t)l * 2 + 1) * D + own_row] = h;
+        publish_h(m.xn, gam + (size_t)(l + 1 < L ? 2 * (l + 1) : 2 * L) * D, (tag + 1) & 0xFFFFFFu);
+        pb ^= 1;
+      }
+    }
+    // ---- lm_head + greedy pick -----------------------------------------------------------------------------
+    {
+      const uint32_t tag = (tag_base + (uint32_t)L) & 0xFFFFFFu;
+      const int nb = nbw(PK_LM);
+      gemv(PK_LM, m.xn, tag, true);
+      const bool act = tid < 8 * nb;
+      const int row = 8 * (wg + G * (tid >> 3)) + (tid & 7);
+      float best = 0.0f;
+      int bi = -1;
+      if (act) {
+        best = row_sum(tid);
+        bi = row;
+        m.logits[row] = best;
+      }
+      pb ^= 1;
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(best, off, 64);
+        const int oi = __shfl_xor(bi, off, 64);
+        if (better(ov, oi, best, bi)) {
+          best = ov;
+          bi = oi;
+        }
+      }
+      if (lane == 0) {
+        arg_v[wave] = best;
+        arg_i[wave] = bi;
+      }
+      lds_barrier();
+      if (wave == 0) {
+        if (lane == 0 && nb > 0) {
+          for (int w = 1; w < PS_WAVES; w++)
+            if (better(arg_v[w], arg_i[w], best, bi)) {
+              best = arg_v[w];
+              bi = arg_i[w];
+            }
+          st_entry(m.arg + 2 * wg, __float_as_uint(best), tag);
+          st_entry(m.arg + 2 * wg + 1, (uint32_t)bi, tag);
+        }
+        // every workgroup merges the per-workgroup picks itself: no second exchange for the token
+        const int cnt = m.ph[PK_LM].nb < G ? m.ph[PK_LM].nb : G;
+        float gv = 0.0f;
+        int gi = -1;
+        for (int w0 = 0; w0 < cnt; w0 += 64) {
+          const int w = w0 + lane;
+          uint4_t e;
+          while (true) {
+            e = ld2(m.arg + 2 * (w < cnt ? w : 0));
+            wait_vm(e);
+            const bool ok = w >= cnt || (tag_ok(e[1], tag) && tag_ok(e[3], tag));
+            if (__all(ok)) break;
+            if (!poll_backoff()) break;
+          }
+          if (w < cnt && better(__uint_as_float(e[0]), (int)e[2], gv, gi)) {
+            gv = __uint_as_float(e[0]);
+            gi = (int)e[2];
+          }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+          const float ov = __shfl_xor(gv, off, 64);
+          const int oi = __shfl_xor(gi, off, 64);
+          if (better(ov, oi, gv, gi)) {
+            gv = ov;
+            gi = oi;
+          }
+        }
+        if (lane == 0) {
+          tok_lds[0] = gi;
+          if (wg == 0) {
+            m.tokens[0] = gi;
+            if (step0 + s < max_steps) m.history[step0 + s] = gi;
+          }
+        }
+      }
+      lds_barrier();
+      token = tok_lds[0];
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+// ---- stream packing --------------------------------------------------------------------------------------
+__device__ __forceinline__ int pk_nbw(const PersistModel &m, int kind, int w) {
+  return w < m.ph[kind].nb ? (m.ph[kind].nb - w + m.G - 1) / m.G : 0;
+}
+__device__ __host__ inline size_t pk_seq_offset(const PersistModel &m, int w, int layer, int kind) {
+  size_t per_layer = 0, before = 0;
+  for (int k = 0; k < 4; k++) {
+    const int nb = w < m.ph[k].nb ? (m.ph[k].nb - w + m.G - 1) / m.G : 0;
+    const size_t b = (size_t)nb * m.ph[k].blk_bytes;
+    per_layer += b;
+    if (k < kind) before += b;
+  }
+  if (kind == PK_LM) return (size_t)m.n_layers * per_layer;
+  return (size_t)layer * per_layer + before;
+}
+
+__global__ void __launch_bounds__(256) persist_pack_kernel(PersistModel m, int layer, int kind,
+                                                           const uint8_t *__restrict__ packed,
+                                                           const _Float16 *__restrict__ scales, uint8_t *stream) {
+  const int gb = blockIdx.x;   // global 8-row block
+  const int v = blockIdx.y;    // wave (k slice)
+  const PersistPhase ph = m.ph[kind];
+  const int w = gb % m.G, bi = gb / m.G;
+  uint8_t *dest = stream + m.wg_off[w] + (size_t)v * m.wave_bytes[w] + pk_seq_offset(m, w, layer, kind) +
+                  (size_t)bi * ph.blk_bytes;
+  const int tid = threadIdx.x;
+  const size_t row_bytes = (size_t)ph.k / 2, row_groups = (size_t)ph.k / 32;
+  const int rot_rows = kind == PK_QKV ? (m.n_heads + m.n_kv_heads) * 128 : 0;
+  auto logical_row = [&](int pr) {
+    if (pr < rot_rows) {
+      const int head = pr >> 7, p2 = pr & 127;
+      return head * 128 + (p2 >> 1) + 64 * (p2 & 1);
+    }
+    return pr;
+  };
+  for (int p = 0; p < ph.pairs; p++) {
+    const bool single = (ph.tiles & 1) && p == ph.pairs - 1;
+    uint8_t *rec = dest + (size_t)p * PS_REC_FULL;
+    if (tid < 128) {
+      const int t = tid >> 6, ln = tid & 63;
+      if (!(t == 1 && single)) {
+        const int r = ln & 15, c = ln >> 4;
+        const int row = logical_row(8 * gb + (r & 7));
+        const int kbase = v * ph.ks + 256 * (2 * p + t);
+        uint4_t out;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const int kb = (r < 8) ? j : 4 + j;
+          const int k = kbase + 32 * kb + 8 * c;
+          const uint32_t raw = *reinterpret_cast<const uint32_t *>(packed + (size_t)row * row_bytes + k / 2);
+          // raw: element i in bits [4i, 4i+4)  ->  e0 e2 e4 e6 | e1 e3 e5 e7 (int4_common.hpp)
+          uint32_t wv = 0;
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            const uint32_t q = (raw >> (4 * e)) & 0xFu;
+            const int slot = (e & 1) ? 4 + (e >> 1) : (e >> 1);
+            wv |= q << (4 * slot);
+          }
+          out[j] = wv;
+        }
+        *reinterpret_cast<uint4_t *>(rec + t * 1024 + ln * 16) = out;
+      }
+    } else if (tid < 192) {
+      const int sl = tid - 128;  // two fp16 scales at byte sl * 4 of the 256-byte scale block
+      const int t = sl >> 5, r = (sl & 31) >> 1, j0 = (sl & 1) * 2;
+      uint32_t word = 0;
+      if (!(t == 1 && single)) {
+        const int row = logical_row(8 * gb + (r & 7));
+        const int kbase = v * ph.ks + 256 * (2 * p + t);
+        U32H2 u;
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++) {
+          const int kb = (r < 8) ? (j0 + jj) : 4 + j0 + jj;
+          u.h[jj] = scales[(size_t)row * row_groups + (kbase + 32 * kb) / 32];
+        }
+        word = u.u;
+      }
+      *reinterpret_cast<uint32_t *>(rec + (single ? 1024 : 2048) + sl * 4) = word;
+    }
+  }
+}
+
+// ---- host side ---------------------------------------------------------------------------------------------
+bool persist_supported(const yscv_hip_decoder_config &c, int num_cus, const char **why) {
+  const char *dummy;
+  if (!why) why = &dummy;
+  const int G = num_cus;
+  const int hq = c.n_heads * c.head_dim;
+  auto bad_k = [](int k) { return k % 2048 != 0 || k > 16384 || k <= 0; };
+  if (c.head_dim != 128) { *why = "head_dim must be 128"; return false; }
+  if (c.group_size != 32) { *why = "group size must be 32"; return false; }
+  if (bad_k(c.d_model) || bad_k(hq) || bad_k(c.d_ff)) { *why = "d_model, n_heads*128 and d_ff must be multiples of 2048, at most 16384"; return false; }
+  if (c.vocab % 8 != 0) { *why = "vocab must be a multiple of 8"; return false; }
+  if (c.n_heads % c.n_kv_heads != 0 || c.n_heads / c.n_kv_heads > 4) { *why = "1..4 query heads per kv head"; return false; }
+  if (G < 16 || G > 1024) { *why = "unsupported CU count"; return false; }
+  auto rows_per_wg = [&](int n) { return ((n / 8 + G - 1) / G) * 8; };
+  if (rows_per_wg(c.d_model) > 64) { *why = "d_model too large for the CU count"; return false; }
+  const int qkv_n = (c.n_heads + 2 * c.n_kv_heads) * 128;
+  if (rows_per_wg(qkv_n) > PART_ROWS || rows_per_wg(2 * c.d_ff) > PART_ROWS || rows_per_wg(c.vocab) > PART_ROWS) {
+    *why = "a projection has more rows per workgroup than the reduction buffer holds";
+    return false;
+  }
+  if (c.max_ctx % 128 != 0) { *why = "max_ctx must be a multiple of 128"; return false; }
+  return true;
+}
+
+void persist_fill_phases(const yscv_hip_decoder_config &c, int G, PersistModel *m) {
+  m->n_layers = c.n_layers;
+  m->d_model = c.d_model;
+  m->n_heads = c.n_heads;
+  m->n_kv_heads = c.n_kv_heads;
+  m->d_ff = c.d_ff;
+  m->vocab = c.vocab;
+  m->max_ctx = c.max_ctx;
+  m->theta = c.rope_theta;
+  m->eps = c.rms_eps;
+  m->G = G;
+  const int hq = c.n_heads * 128;
+  const int n[PK_COUNT] = {(c.n_heads + 2 * c.n_kv_heads) * 128, c.d_model, 2 * c.d_ff, c.d_model, c.vocab};
+  const int k[PK_COUNT] = {c.d_model, hq, c.d_model, c.d_ff, c.d_model};
+  for (int i = 0; i < PK_COUNT; i++) {
+    PersistPhase &p = m->ph[i];
+    p.n = n[i];
+    p.k = k[i];
+    p.ks = k[i] / 8;
+    p.tiles = p.ks / 256;
+    p.pairs = (p.tiles + 1) / 2;
+    p.frags = p.pairs;
+    p.nb = n[i] / 8;
+    p.blk_bytes = (p.tiles / 2) * PS_REC_FULL + (p.tiles & 1) * PS_REC_SINGLE;
+  }
+}
+
+size_t persist_wave_bytes(const PersistModel &m, int w) { return pk_seq_offset(m, w, 0, PK_LM) + (size_t)(w < m.ph[PK_LM].nb ? (m.ph[PK_LM].nb - w + m.G - 1) / m.G : 0) * m.ph[PK_LM].blk_bytes; }
+size_t persist_seq_offset(const PersistModel &m, int w, int layer, int kind) { return pk_seq_offset(m, w, layer, kind); }
+
+int32_t launch_persist_pack(const PersistModel &m, int layer, int kind, const uint8_t *packed_dev,
+                            const _Float16 *scales_dev, uint8_t *stream, hipStream_t s) {
+  if (kind < 0 || kind >= PK_COUNT) return set_error(YSCV_HIP_ERR_INVALID_ARG, "bad projection kind %d", kind);
+  hipLaunchKernelGGL(persist_pack_kernel, dim3(m.ph[kind].nb, PS_WAVES), dim3(256), 0, s, m, layer, kind, packed_dev,
+                     scales_dev, stream);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_persist_decode(const PersistModel &m, int n_steps, int pos0, int step0, int max_steps,
+                              uint32_t epoch0, hipStream_t s) {
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(once, [] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(decode_persistent_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, PERSIST_LDS);
+  });
+  if (attr_err != hipSuccess)
+    return set_error(YSCV_HIP_ERR_DEVICE, "cannot reserve %d bytes of LDS: %s", PERSIST_LDS, hipGetErrorString(attr_err));
+  int max_blocks = 0;
+  YSCV_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&max_blocks, decode_persistent_kernel, 512, PERSIST_LDS));
+  if (max_blocks < 1) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the persistent decode kernel does not fit a CU");
+  PersistModel mm = m;
+  void *args[] = {&mm, &n_steps, &pos0, &step0, &max_steps, &epoch0};
+  YSCV_HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<const void *>(decode_persistent_kernel), dim3(m.G), dim3(512),
+                                          args, PERSIST_LDS, s));
+  return YSCV_HIP_OK;
+}
+
+}  // namespace yscv

@@ -3,11 +3,13 @@
 // pick, repeat) with every projection running through the skinny int4 kernel.
 // One decode step is a fixed sequence of kernel launches that reads the position from device
 // memory, so the step is captured once into a HIP graph and replayed for every token.
+#include <algorithm>
 #include <vector>
 
 #include "decoder.hpp"
 #include "int4_common.hpp"
 #include "kernels.hpp"
+#include "persist.hpp"
 
 namespace yscv {
 
@@ -34,6 +36,12 @@ __global__ void random_scales_kernel(_Float16 *__restrict__ sc, size_t n, uint64
 __global__ void fill_f32_kernel(float *p, size_t n, float v) {
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
 }
+__global__ void set_counters_kernel(int32_t *pos, int32_t *step, int32_t p, int32_t s) {
+  if (threadIdx.x == 0) {
+    *pos = p;
+    *step = s;
+  }
+}
 __global__ void fill_i32_kernel(int32_t *p, size_t n, int32_t v) {
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
 }
@@ -43,37 +51,15 @@ static unsigned grid_for(size_t n) {
   return (unsigned)(b > 65535 ? 65535 : (b < 1 ? 1 : b));
 }
 
-static int32_t random_int4_weight(size_t n, size_t k, size_t g, uint64_t seed, yscv_hip_int4_weight **out) {
-  YSCV_REQUIRE(g == 32 || g == 64 || g % 128 == 0, "random weights need a tiled group size");
-  YSCV_REQUIRE(k % 512 == 0, "random weights need K to be a multiple of 512");
-  auto *w = new yscv_hip_int4_weight();
-  w->n = n;
-  w->k = k;
-  w->g = g;
-  w->scale_dtype = YSCV_HIP_F16;
-  w->has_zp = false;
-  w->tiled = true;
-  w->gm = g == 32 ? GM32 : (g == 64 ? GM64 : GM128);
-  w->nt = ceil_div(n, (size_t)16);
-  w->kt = ceil_div(k, (size_t)128);
-  w->ktp = round_up(w->kt, (size_t)4);
-  w->chunks = w->gm == GM128 ? ceil_div(w->ktp, g / 128) : w->ktp;
-  const size_t tile_bytes = w->nt * w->ktp * (size_t)kTileBytes;
-  const size_t sc_elems = w->nt * w->chunks * 16 * (size_t)scales_per_chunk(w->gm);
-  hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->tiles), tile_bytes);
-  if (e == hipSuccess) e = hipMalloc(&w->tscales, sc_elems * 2);
-  if (e != hipSuccess) {
-    (void)hipFree(w->tiles);
-    delete w;
-    return set_error(e == hipErrorOutOfMemory ? YSCV_HIP_ERR_OOM : YSCV_HIP_ERR_DEVICE, "weight allocation failed: %s",
-                     hipGetErrorString(e));
-  }
-  hipLaunchKernelGGL(random_tiles_kernel, dim3(grid_for(tile_bytes / 4)), dim3(256), 0, nullptr,
-                     reinterpret_cast<uint32_t *>(w->tiles), tile_bytes / 4, seed);
-  hipLaunchKernelGGL(random_scales_kernel, dim3(grid_for(sc_elems)), dim3(256), 0, nullptr,
-                     static_cast<_Float16 *>(w->tscales), sc_elems, seed ^ 0x5ca1e5ull, 0.005f, 0.02f);
-  w->device_bytes = tile_bytes + sc_elems * 2;
-  *out = w;
+// Random raw weight on the device: [n][k/2] uniform nibble bytes and fp16 scales ~U(0.005, 0.02) in natural
+// order, so that every layout built from it (tiled, persistent stream) holds the same logical matrix.
+static int32_t random_raw_weight(size_t n, size_t k, size_t g, uint64_t seed, uint8_t *raw, _Float16 *scales) {
+  const size_t words = n * k / 8, sc = n * (k / g);
+  hipLaunchKernelGGL(random_tiles_kernel, dim3(grid_for(words)), dim3(256), 0, nullptr, reinterpret_cast<uint32_t *>(raw),
+                     words, seed);
+  hipLaunchKernelGGL(random_scales_kernel, dim3(grid_for(sc)), dim3(256), 0, nullptr, scales, sc, seed ^ 0x5ca1e5ull, 0.005f,
+                     0.02f);
+  YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
 }
 
@@ -122,6 +108,18 @@ struct yscv_hip_decoder {
   hipGraphExec_t graph_exec = nullptr;
   int graph_batch = 0;
   size_t weight_bytes = 0;
+  // persistent single-launch path (batch 1)
+  bool persist_ok = false;     // the shape is supported and the buffers exist
+  PersistModel pm{};
+  uint8_t *p_stream = nullptr;
+  uint64_t *p_wg_off = nullptr;
+  uint32_t *p_wave_bytes = nullptr;
+  float *p_gammas = nullptr;
+  _Float16 **p_kc = nullptr, **p_vc = nullptr;
+  unsigned long long *p_exch = nullptr;
+  uint32_t *p_abort = nullptr;
+  size_t p_stream_bytes = 0;
+  uint32_t epoch = 1;          // tag epoch of the next persistent step; never reused
 };
 
 static void decoder_free(yscv_hip_decoder *d) {
@@ -153,6 +151,14 @@ static void decoder_free(yscv_hip_decoder *d) {
   (void)hipFree(d->history);
   (void)hipFree(d->pos);
   (void)hipFree(d->step);
+  (void)hipFree(d->p_stream);
+  (void)hipFree(d->p_wg_off);
+  (void)hipFree(d->p_wave_bytes);
+  (void)hipFree(d->p_gammas);
+  (void)hipFree(d->p_kc);
+  (void)hipFree(d->p_vc);
+  (void)hipFree(d->p_exch);
+  (void)hipFree(d->p_abort);
   delete d;
 }
 
@@ -168,7 +174,98 @@ static size_t kv_elems(const yscv_hip_decoder_config &c) {
   return (size_t)c.max_batch * c.n_kv_heads * c.max_ctx * c.head_dim;
 }
 
-static int32_t make_fused(const HostLinear *parts, int count, bool interleave, size_t g, yscv_hip_int4_weight **out) {
+// Allocate the persistent path's stream and exchange buffers when the shape allows it.
+static int32_t persist_setup(yscv_hip_decoder *d) {
+  const Context *ctx = nullptr;
+  YSCV_TRY(ensure_context(&ctx));
+  const auto &c = d->cfg;
+  const char *why = "";
+  if (!persist_supported(c, ctx->num_cus, &why)) return YSCV_HIP_OK;  // the multi-kernel path remains
+  PersistModel &m = d->pm;
+  persist_fill_phases(c, ctx->num_cus, &m);
+  const int G = m.G;
+  std::vector<uint64_t> off(G);
+  std::vector<uint32_t> wb(G);
+  size_t total = 0;
+  for (int w = 0; w < G; w++) {
+    const size_t b = persist_wave_bytes(m, w);
+    YSCV_REQUIRE(b < (1ull << 32), "weight stream of one wave exceeds 4 GiB");
+    off[w] = total;
+    wb[w] = (uint32_t)b;
+    total += b * PS_WAVES;
+  }
+  d->p_stream_bytes = total;
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->p_stream), total + 4096));  // slack: the prefetcher reads a dword lane pattern
+  DEC_HIP(hipMemset(d->p_stream, 0, total + 4096));
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->p_wg_off), G * 8));
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->p_wave_bytes), G * 4));
+  DEC_HIP(hipMemcpy(d->p_wg_off, off.data(), G * 8, hipMemcpyHostToDevice));
+  DEC_HIP(hipMemcpy(d->p_wave_bytes, wb.data(), G * 4, hipMemcpyHostToDevice));
+  const size_t D = c.d_model;
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->p_gammas), (2 * (size_t)c.n_layers + 1) * D * 4));
+  std::vector<_Float16 *> kc(c.n_layers), vc(c.n_layers);
+  for (int l = 0; l < c.n_layers; l++) {
+    kc[l] = d->layers[l].kc;
+    vc[l] = d->layers[l].vc;
+  }
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->p_kc), c.n_layers * sizeof(void *)));
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->p_vc), c.n_layers * sizeof(void *)));
+  DEC_HIP(hipMemcpy(d->p_kc, kc.data(), c.n_layers * sizeof(void *), hipMemcpyHostToDevice));
+  DEC_HIP(hipMemcpy(d->p_vc, vc.data(), c.n_layers * sizeof(void *), hipMemcpyHostToDevice));
+  // exchange buffers, one allocation: xn | xn2 | qkv | ao | act | part | arg
+  const size_t e_xn = persist_vec_entries(c.d_model) + G;
+  const size_t e_qkv = (size_t)(c.n_heads + 2 * c.n_kv_heads) * 64;
+  const size_t e_ao = persist_vec_entries(c.n_heads * 128);
+  const size_t e_act = persist_vec_entries(c.d_ff);
+  const size_t e_part = (size_t)c.n_heads * (c.max_ctx / 128) * 132;
+  const size_t e_arg = 2 * (size_t)G;
+  auto up = [](size_t e) { return (e + 31) & ~(size_t)31; };  // keep every buffer 256-byte aligned
+  const size_t total_e = 2 * up(e_xn) + up(e_qkv) + up(e_ao) + up(e_act) + up(e_part) + up(e_arg);
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->p_exch), total_e * 8));
+  DEC_HIP(hipMemset(d->p_exch, 0, total_e * 8));
+  unsigned long long *p = d->p_exch;
+  m.xn = p;   p += up(e_xn);
+  m.xn2 = p;  p += up(e_xn);
+  m.qkv = p;  p += up(e_qkv);
+  m.ao = p;   p += up(e_ao);
+  m.act = p;  p += up(e_act);
+  m.part = p; p += up(e_part);
+  m.arg = p;
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->p_abort), 4));
+  DEC_HIP(hipMemset(d->p_abort, 0, 4));
+  m.stream = d->p_stream;
+  m.wg_off = d->p_wg_off;
+  m.wave_bytes = d->p_wave_bytes;
+  m.gammas = d->p_gammas;
+  m.emb = d->emb;
+  m.kc = d->p_kc;
+  m.vc = d->p_vc;
+  m.logits = d->logits;
+  m.tokens = d->tokens;
+  m.history = d->history;
+  m.abort_flag = d->p_abort;
+  m.dbg_h = nullptr;
+  if (getenv("YSCV_DBG_H")) { (void)hipMalloc(reinterpret_cast<void **>(&m.dbg_h), (size_t)c.n_layers * 2 * D * 4); }
+  d->persist_ok = true;
+  return YSCV_HIP_OK;
+}
+
+// pack one projection given on the host (fused, natural row order) into the persistent streams
+static int32_t persist_pack_host(yscv_hip_decoder *d, int layer, int kind, const uint8_t *packed, const uint16_t *scales,
+                                 size_t n, size_t k) {
+  if (!d->persist_ok) return YSCV_HIP_OK;
+  DevBuf dp, ds;
+  YSCV_TRY(dp.alloc(n * k / 2));
+  YSCV_TRY(ds.alloc(n * (k / 32) * 2));
+  DEC_HIP(hipMemcpy(dp.p, packed, n * k / 2, hipMemcpyHostToDevice));
+  DEC_HIP(hipMemcpy(ds.p, scales, n * (k / 32) * 2, hipMemcpyHostToDevice));
+  YSCV_TRY(launch_persist_pack(d->pm, layer, kind, dp.as<uint8_t>(), ds.as<_Float16>(), d->p_stream, nullptr));
+  DEC_HIP(hipDeviceSynchronize());
+  return YSCV_HIP_OK;
+}
+
+static int32_t make_fused(yscv_hip_decoder *d, int layer, int pkind, const HostLinear *parts, int count, bool interleave,
+                          size_t g, yscv_hip_int4_weight **out) {
   const size_t k = parts[0].k;
   size_t n_total = 0;
   for (int i = 0; i < count; i++) {
@@ -193,6 +290,7 @@ static int32_t make_fused(const HostLinear *parts, int count, bool interleave, s
       r0 += parts[i].n;
     }
   }
+  YSCV_TRY(persist_pack_host(d, layer, pkind, packed.data(), scales.data(), n_total, k));
   return yscv_hip_int4_weight_create(packed.data(), scales.data(), YSCV_HIP_F16, nullptr, YSCV_HIP_NIBBLE_UNSIGNED,
                                      n_total, k, g, out);
 }
@@ -246,6 +344,14 @@ static int32_t finish_setup(yscv_hip_decoder *d) {
     DEC_HIP(hipMalloc(&d->ws, need));
     d->ws_bytes = need;
   }
+  if (d->persist_ok) {
+    const size_t D = d->cfg.d_model;
+    for (size_t l = 0; l < d->layers.size(); l++) {
+      DEC_HIP(hipMemcpy(d->p_gammas + (2 * l) * D, d->layers[l].attn_norm, D * 4, hipMemcpyDeviceToDevice));
+      DEC_HIP(hipMemcpy(d->p_gammas + (2 * l + 1) * D, d->layers[l].ffn_norm, D * 4, hipMemcpyDeviceToDevice));
+    }
+    DEC_HIP(hipMemcpy(d->p_gammas + 2 * d->layers.size() * D, d->final_norm, D * 4, hipMemcpyDeviceToDevice));
+  }
   d->finalized = true;
   return YSCV_HIP_OK;
 }
@@ -271,6 +377,17 @@ static int32_t enqueue_step(yscv_hip_decoder *d, int batch, hipStream_t s) {
   YSCV_TRY(int4_run_ws(d->lm_head, d->xn, YSCV_HIP_F16, d->logits, YSCV_HIP_F32, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s));
   YSCV_TRY(launch_argmax(d->logits, batch, c.vocab, d->tokens, d->history, d->step, c.max_steps, s));
   YSCV_TRY(launch_advance(d->pos, d->step, s));
+  return YSCV_HIP_OK;
+}
+
+static int32_t check_persist_abort(yscv_hip_decoder *d) {
+  if (!d->persist_ok) return YSCV_HIP_OK;
+  uint32_t flag = 0;
+  DEC_HIP(hipMemcpy(&flag, d->p_abort, 4, hipMemcpyDeviceToHost));
+  if (flag) {
+    DEC_HIP(hipMemset(d->p_abort, 0, 4));
+    return set_error(YSCV_HIP_ERR_DEVICE, "the single-launch decode kernel gave up waiting for a stage (bounded wait expired)");
+  }
   return YSCV_HIP_OK;
 }
 
@@ -326,6 +443,7 @@ int32_t yscv_hip_decoder_create(const yscv_hip_decoder_config *cfg, yscv_hip_dec
     hipError_t e = hipDeviceSynchronize();
     if (e != hipSuccess) st = set_error(YSCV_HIP_ERR_DEVICE, "setup failed: %s", hipGetErrorString(e));
   }
+  if (st == YSCV_HIP_OK && c.max_batch >= 1) st = persist_setup(d);
   if (st != YSCV_HIP_OK) {
     decoder_free(d);
     return st;
@@ -356,6 +474,7 @@ int32_t yscv_hip_decoder_set_linear(yscv_hip_decoder *d, int32_t layer, int32_t 
   if (kind == YSCV_HIP_DEC_LM_HEAD) {
     destroy_int4(d->lm_head);
     d->lm_head = nullptr;
+    YSCV_TRY(persist_pack_host(d, 0, PK_LM, packed, scales_f16, n, k));
     return yscv_hip_int4_weight_create(packed, scales_f16, YSCV_HIP_F16, nullptr, YSCV_HIP_NIBBLE_UNSIGNED, n, k, g,
                                        &d->lm_head);
   }
@@ -379,6 +498,7 @@ int32_t yscv_hip_decoder_set_norm(yscv_hip_decoder *d, int32_t layer, int32_t ki
     dst = kind == YSCV_HIP_DEC_ATTN_NORM ? d->layers[layer].attn_norm : d->layers[layer].ffn_norm;
   }
   DEC_HIP(hipMemcpy(dst, gamma, (size_t)d->cfg.d_model * 4, hipMemcpyHostToDevice));
+  d->finalized = false;  // the persistent path keeps its own contiguous copy, refreshed by finalize
   return YSCV_HIP_OK;
 }
 
@@ -391,30 +511,31 @@ int32_t yscv_hip_decoder_set_embedding(yscv_hip_decoder *d, const uint16_t *tabl
 int32_t yscv_hip_decoder_finalize(yscv_hip_decoder *d) {
   YSCV_REQUIRE(d != nullptr, "null decoder");
   const size_t g = d->cfg.group_size;
-  for (auto &L : d->layers) {
+  for (int li = 0; li < (int)d->layers.size(); li++) {
+    auto &L = d->layers[li];
     if (L.stage[0].n) {  // q, k, v staged -> fused [q; k; v]
       destroy_int4(L.wqkv);
       L.wqkv = nullptr;
-      YSCV_TRY(make_fused(&L.stage[0], 3, false, g, &L.wqkv));
+      YSCV_TRY(make_fused(d, li, PK_QKV, &L.stage[0], 3, false, g, &L.wqkv));
       for (int i = 0; i < 3; i++) L.stage[i] = HostLinear();
     }
     if (L.stage[3].n) {
       destroy_int4(L.wo);
       L.wo = nullptr;
-      YSCV_TRY(make_fused(&L.stage[3], 1, false, g, &L.wo));
+      YSCV_TRY(make_fused(d, li, PK_O, &L.stage[3], 1, false, g, &L.wo));
       L.stage[3] = HostLinear();
     }
     if (L.stage[4].n) {  // gate, up staged -> rows interleaved gate_0, up_0, gate_1, ... for the SwiGLU epilogue
       destroy_int4(L.wgu);
       L.wgu = nullptr;
-      YSCV_TRY(make_fused(&L.stage[4], 2, true, g, &L.wgu));
+      YSCV_TRY(make_fused(d, li, PK_GU, &L.stage[4], 2, true, g, &L.wgu));
       L.stage[4] = HostLinear();
       L.stage[5] = HostLinear();
     }
     if (L.stage[6].n) {
       destroy_int4(L.wdown);
       L.wdown = nullptr;
-      YSCV_TRY(make_fused(&L.stage[6], 1, false, g, &L.wdown));
+      YSCV_TRY(make_fused(d, li, PK_DOWN, &L.stage[6], 1, false, g, &L.wdown));
       L.stage[6] = HostLinear();
     }
   }
@@ -427,20 +548,34 @@ int32_t yscv_hip_decoder_init_random(yscv_hip_decoder *d, uint64_t seed) {
   const size_t g = c.group_size, D = c.d_model;
   const size_t qkv_n = (size_t)(c.n_heads + 2 * c.n_kv_heads) * c.head_dim;
   uint64_t sd = seed * 0x100000001B3ull + 1;
-  for (auto &L : d->layers) {
+  // one raw buffer, sized for the largest projection, reused for every weight
+  const size_t max_elems = std::max(std::max(qkv_n, 2 * (size_t)c.d_ff) * D, std::max((size_t)c.vocab * D, D * (size_t)c.d_ff));
+  DevBuf raw, rsc;
+  YSCV_TRY(raw.alloc(max_elems / 2));
+  YSCV_TRY(rsc.alloc(max_elems / g * 2));
+  auto make = [&](int layer, int pkind, size_t n, size_t k, yscv_hip_int4_weight **out) -> int32_t {
+    YSCV_REQUIRE(g == 32 || g == 64 || g % 128 == 0, "random weights need a tiled group size");
+    YSCV_TRY(random_raw_weight(n, k, g, sd++, raw.as<uint8_t>(), rsc.as<_Float16>()));
+    YSCV_TRY(int4_create_from_device(raw.as<uint8_t>(), rsc.p, YSCV_HIP_F16, YSCV_HIP_NIBBLE_UNSIGNED, n, k, g, out));
+    if (d->persist_ok) YSCV_TRY(launch_persist_pack(d->pm, layer, pkind, raw.as<uint8_t>(), rsc.as<_Float16>(), d->p_stream, nullptr));
+    DEC_HIP(hipDeviceSynchronize());  // the raw buffer is reused by the next weight
+    return YSCV_HIP_OK;
+  };
+  for (int li = 0; li < (int)d->layers.size(); li++) {
+    auto &L = d->layers[li];
     destroy_int4(L.wqkv);
     destroy_int4(L.wo);
     destroy_int4(L.wgu);
     destroy_int4(L.wdown);
     L.wqkv = L.wo = L.wgu = L.wdown = nullptr;
-    YSCV_TRY(random_int4_weight(qkv_n, D, g, sd++, &L.wqkv));
-    YSCV_TRY(random_int4_weight(D, (size_t)c.n_heads * c.head_dim, g, sd++, &L.wo));
-    YSCV_TRY(random_int4_weight(2 * (size_t)c.d_ff, D, g, sd++, &L.wgu));
-    YSCV_TRY(random_int4_weight(D, (size_t)c.d_ff, g, sd++, &L.wdown));
+    YSCV_TRY(make(li, PK_QKV, qkv_n, D, &L.wqkv));
+    YSCV_TRY(make(li, PK_O, D, (size_t)c.n_heads * c.head_dim, &L.wo));
+    YSCV_TRY(make(li, PK_GU, 2 * (size_t)c.d_ff, D, &L.wgu));
+    YSCV_TRY(make(li, PK_DOWN, D, (size_t)c.d_ff, &L.wdown));
   }
   destroy_int4(d->lm_head);
   d->lm_head = nullptr;
-  YSCV_TRY(random_int4_weight((size_t)c.vocab, D, g, sd++, &d->lm_head));
+  YSCV_TRY(make(0, PK_LM, (size_t)c.vocab, D, &d->lm_head));
   YSCV_TRY(launch_kv_random_fill(d->emb, (size_t)c.vocab * D, sd++, nullptr));
   DEC_HIP(hipDeviceSynchronize());
   return finish_setup(d);
@@ -505,6 +640,18 @@ int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_g
                d->cfg.max_ctx);
   YSCV_REQUIRE(step + n_steps <= d->cfg.max_steps, "token history overflow: %d + %d > max_steps %d", step, n_steps,
                d->cfg.max_steps);
+  if (use_graph == 2) {
+    if (!d->persist_ok)
+      return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the single-launch decode path does not support this model shape");
+    if (d->batch != 1) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the single-launch decode path runs batch 1 only");
+    if (n_steps == 0) return YSCV_HIP_OK;
+    YSCV_TRY(launch_persist_decode(d->pm, n_steps, pos, step, d->cfg.max_steps, d->epoch, s));
+    d->epoch += (uint32_t)n_steps;
+    // position and step counters live on the device for the multi-kernel path: keep them in step
+    hipLaunchKernelGGL(set_counters_kernel, dim3(1), dim3(64), 0, s, d->pos, d->step, pos + n_steps, step + n_steps);
+    DEC_HIP(hipGetLastError());
+    return YSCV_HIP_OK;
+  }
   if (!use_graph) {
     for (int i = 0; i < n_steps; i++) YSCV_TRY(enqueue_step(d, d->batch, s));
     return YSCV_HIP_OK;
@@ -555,6 +702,7 @@ int32_t yscv_hip_decoder_read_tokens(yscv_hip_decoder *d, int32_t first_step, in
   YSCV_REQUIRE(d && out_host, "null argument");
   YSCV_REQUIRE(first_step >= 0 && n_steps >= 0 && first_step + n_steps <= d->cfg.max_steps, "step range out of bounds");
   DEC_HIP(hipDeviceSynchronize());
+  YSCV_TRY(check_persist_abort(d));
   DEC_HIP(hipMemcpy(out_host, d->history + (size_t)first_step * d->batch, (size_t)n_steps * d->batch * 4,
                     hipMemcpyDeviceToHost));
   return YSCV_HIP_OK;
@@ -563,8 +711,16 @@ int32_t yscv_hip_decoder_read_tokens(yscv_hip_decoder *d, int32_t first_step, in
 int32_t yscv_hip_decoder_read_logits(yscv_hip_decoder *d, float *out_host) {
   YSCV_REQUIRE(d && out_host, "null argument");
   DEC_HIP(hipDeviceSynchronize());
+  YSCV_TRY(check_persist_abort(d));
   DEC_HIP(hipMemcpy(out_host, d->logits, (size_t)d->batch * d->cfg.vocab * 4, hipMemcpyDeviceToHost));
   return YSCV_HIP_OK;
+}
+
+__attribute__((visibility("default"))) int32_t yscv_hip_decoder_dbg_h(yscv_hip_decoder *d, float *out) {
+  if (!d->pm.dbg_h) return -1;
+  (void)hipDeviceSynchronize();
+  (void)hipMemcpy(out, d->pm.dbg_h, (size_t)d->cfg.n_layers * 2 * d->cfg.d_model * 4, hipMemcpyDeviceToHost);
+  return 0;
 }
 
 int32_t yscv_hip_decoder_weight_bytes(const yscv_hip_decoder *d, size_t *bytes) {

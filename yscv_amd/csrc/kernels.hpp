@@ -79,6 +79,9 @@ int32_t int4_workspace_bytes(const yscv_hip_int4_weight *w, size_t m, int x_dtyp
 int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, void *y, int y_dtype, size_t m,
                     int force, int epi, void *ws, size_t ws_bytes, hipStream_t s);
 
+int32_t int4_create_from_device(const uint8_t *d_packed, const void *d_scales, int scale_dtype, int nibble_format,
+                                size_t n, size_t k, size_t g, yscv_hip_int4_weight **out);
+
 int32_t launch_pack_int4_symmetric(const float *w, size_t m_w, size_t k, size_t g, uint8_t *packed,
                                    float *scales, hipStream_t s);
 int32_t launch_dequantize_int4(const uint8_t *packed, size_t n_bytes, float scale, int zp,

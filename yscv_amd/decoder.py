@@ -59,8 +59,11 @@ class Decoder:
         self.batch = t.size
         lib().decoder_reset(self._h, int(t.size), int(start_pos), _p(t))
 
-    def run(self, n_steps, use_graph=True, stream=None):
-        lib().decoder_run(self._h, int(n_steps), int(bool(use_graph)), C.c_void_p(stream) if stream else None)
+    def run(self, n_steps, use_graph=True, stream=None, persistent=False):
+        """use_graph: replay one captured HIP graph per step; persistent: run all steps inside one
+        cooperative launch (batch 1, shapes the single-launch kernel supports)."""
+        mode = 2 if persistent else int(bool(use_graph))
+        lib().decoder_run(self._h, int(n_steps), mode, C.c_void_p(stream) if stream else None)
 
     def run_projections(self, n_steps, stream=None):
         lib().decoder_run_projections(self._h, int(n_steps), C.c_void_p(stream) if stream else None)
