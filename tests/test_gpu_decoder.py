@@ -108,8 +108,8 @@ def test_cache_overflow_is_an_error():
 
 
 # ---- single-launch (persistent) decode path ---------------------------------------------------------------
-# K = 2048 -> one 256-k tile per wave (single-tile records), K = 6144 -> three tiles (full + single record)
-PCFG = dict(n_layers=2, d_model=2048, n_heads=16, n_kv_heads=4, head_dim=128, d_ff=6144, vocab=1000, group_size=32,
+# per-wave k slice = K / 4: K = 2048 -> two 256-k tiles (one full record), K = 3072 -> three tiles (full + single record)
+PCFG = dict(n_layers=2, d_model=2048, n_heads=16, n_kv_heads=4, head_dim=128, d_ff=3072, vocab=1000, group_size=32,
             max_batch=2, max_ctx=512, max_steps=32, rope_theta=10000.0, rms_eps=1e-5)
 
 

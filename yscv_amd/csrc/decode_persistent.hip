@@ -36,14 +36,28 @@
 namespace yscv {
 
 typedef unsigned long long u64;
+#ifndef DBG_WAIT_ALL
+#define DBG_WAIT_ALL 0
+#endif
+#ifndef GEMV_INL
+#define GEMV_INL __noinline__
+#endif
+#ifndef ATTN_INL
+#define ATTN_INL __noinline__
+#endif
 
-constexpr int RING = 7;                        // records in flight per wave
+constexpr int CW = PS_WAVES;                   // compute waves per workgroup (waves 0 .. CW-1)
+constexpr int PW = 2;                          // producer waves (waves CW .. CW+PW-1), each feeds CW/PW compute waves
+constexpr int THREADS = 64 * (CW + PW);
+constexpr int RING = 14;                       // ring slots (records) per compute wave
 constexpr int SLOT = PS_REC_FULL;              // LDS bytes per ring slot
-constexpr int RING_BYTES = PS_WAVES * RING * SLOT;
+constexpr int RING_BYTES = CW * RING * SLOT;
 constexpr int PART_ROWS = 256;                 // rows a workgroup may own in one projection
-constexpr int PART_BYTES = 2 * PS_WAVES * PART_ROWS * 4;
+constexpr int PART_BYTES = 2 * CW * PART_ROWS * 4;
 constexpr int ATT_BYTES = 10240;
-constexpr int PERSIST_LDS = RING_BYTES + PART_BYTES + ATT_BYTES;
+constexpr int SYNC_BYTES = 256;                // landed[CW], consumed[CW], barrier counter
+constexpr int PERSIST_LDS = RING_BYTES + PART_BYTES + ATT_BYTES + SYNC_BYTES;
+constexpr int MAXF = 8;                        // 512-k fragments per compute wave: k <= 4 * 8 * 512
 constexpr unsigned SPIN_LIMIT = 300000u;
 constexpr int ACHUNK = 128;                    // positions per attention work item (4 waves x 32)
 constexpr int PART_REC = 132;                  // entries per (head, chunk) partial: max, sum, o[128], pad
@@ -70,6 +84,15 @@ __device__ __forceinline__ void wait_vm(uint4_t &a, uint4_t &b, uint4_t &c, uint
 __device__ __forceinline__ void wait_vm8(uint4_t *v) {
   asm volatile("s_waitcnt vmcnt(0)"
                : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7])::"memory");
+}
+// LDS word access that the compiler does not order against outstanding global->LDS loads
+__device__ __forceinline__ uint32_t lds_peek(uint32_t addr) {
+  uint32_t v;
+  asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
+  return v;
+}
+__device__ __forceinline__ void lds_poke(uint32_t addr, uint32_t v) {
+  asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(addr), "v"(v) : "memory");
 }
 // tags are compared on their low 24 bits; the top byte of the tag word may carry a block exponent
 __device__ __forceinline__ bool tag_ok(uint32_t word, uint32_t tag) { return ((word ^ tag) & 0xFFFFFFu) == 0; }
@@ -127,7 +150,476 @@ __device__ __forceinline__ bool better(float va, int ia, float vb, int ib) {
   return ia > ib;
 }
 
-__global__ void __launch_bounds__(512, 1)
+typedef __attribute__((address_space(3))) uint32_t lds_u32;
+typedef __attribute__((address_space(3))) float lds_f32;
+typedef __attribute__((address_space(3))) _Float16 lds_f16;
+
+// state of the bounded waits and of the compute-wave barrier, carried by value through the noinline stages
+struct WaitState {
+  unsigned spin_budget;
+  unsigned bar_gen;
+};
+__device__ __forceinline__ bool poll_backoff_ws(WaitState &ws, uint32_t *abort_flag) {
+  __builtin_amdgcn_s_sleep(2);
+  if (ws.spin_budget <= 1 ||
+      ((ws.spin_budget & 63u) == 0 && __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
+    __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    ws.spin_budget = 1;
+    return false;
+  }
+  ws.spin_budget--;
+  return true;
+}
+// barrier of the compute waves (the producer waves never join, so s_barrier cannot be used)
+__device__ __forceinline__ void compute_barrier(WaitState &ws, lds_u32 *ctr, int n_waves) {
+  ws.bar_gen += n_waves;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  if ((threadIdx.x & 63) == 0) {
+    __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    while ((int)(__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) - ws.bar_gen) < 0)
+      __builtin_amdgcn_s_sleep(0);
+  }
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+__device__ __forceinline__ half8_t gload_h8(const _Float16 *p) {
+  return *reinterpret_cast<const half8_t __attribute__((address_space(1))) *>(reinterpret_cast<uintptr_t>(p));
+}
+
+struct AttnArgs {
+  u64 *qkv, *part, *ao;
+  _Float16 *kc, *vc;       // caches of this layer, batch row 0
+  uint32_t *abort_flag;
+  int HQ, HKV, GROUP, max_ctx, G, pos, pos0, wg;
+  int ks_o, frags_o;       // k slice / fragments of the output projection (layout of `ao`)
+  uint32_t tag;
+  uint32_t att_off, bar_off;  // LDS byte offsets: attention scratch, barrier counter
+};
+
+// Attention of the new token over the cached positions [0, pos): one work item = (kv head, 128 positions),
+// four waves x 32 positions; writes one (max, sum, o[128]) partial per query head of the group.
+__device__ ATTN_INL WaitState attn_items(AttnArgs a, WaitState ws) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, c = lane >> 4;
+  lds_f16 *p_lds = (lds_f16 *)(uintptr_t)a.att_off;                 // [4 waves][4 heads][32]
+  lds_f32 *w_m = (lds_f32 *)(uintptr_t)(a.att_off + 1024);          // [4][4]
+  lds_f32 *w_l = (lds_f32 *)(uintptr_t)(a.att_off + 1024 + 64);     // [4][4]
+  lds_f32 *w_o = (lds_f32 *)(uintptr_t)(a.att_off + 1024 + 128);    // [4][4][128]
+  lds_u32 *bar = (lds_u32 *)(uintptr_t)a.bar_off;
+  const int pos = a.pos, GROUP = a.GROUP, HKV = a.HKV;
+  const int nchunks = (pos + ACHUNK - 1) / ACHUNK;
+  const int items = HKV * nchunks;
+  const int max_chunks = a.max_ctx / ACHUNK;
+  const uint32_t tag = a.tag;
+  const float scale = 0.08838834764831845f;  // 1 / sqrt(128)
+#pragma unroll 1
+  for (int id = a.wg; id < items; id += a.G) {
+    const int chunk = id / HKV, kvh = id - chunk * HKV;
+    float m_h = -INFINITY, l_h = 0.0f;
+    float o_acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) o_acc[t] = 0.0f;
+    const int p0 = chunk * ACHUNK + wave * 32;
+    if (p0 < pos) {
+      const _Float16 *kbase = a.kc + ((size_t)kvh * a.max_ctx + p0) * 128;
+      const _Float16 *vbase = a.vc + (((size_t)kvh * (a.max_ctx / 8) + p0 / 8) * 128) * 8;
+      half8_t kf[2][4], vf[8];
+      const half8_t hz = {0, 0, 0, 0, 0, 0, 0, 0};
+      // Blocks that were complete before this launch never change and are read with plain loads (issued
+      // before the wait for q).  Positions appended during this launch were written with agent-scope
+      // stores by another workgroup: their blocks are read with coherent loads, and only where valid.
+      const bool recent = p0 + 32 > a.pos0;
+      if (!recent) {
+#pragma unroll
+        for (int pbk = 0; pbk < 2; pbk++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) kf[pbk][j] = gload_h8(kbase + (size_t)(pbk * 16 + r) * 128 + 32 * c + 8 * j);
+#pragma unroll
+        for (int t = 0; t < 8; t++) vf[t] = gload_h8(vbase + ((size_t)c * 128 + t * 16 + r) * 8);
+      } else {
+        uint4_t tmp[8];
+#pragma unroll
+        for (int pbk = 0; pbk < 2; pbk++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) tmp[pbk * 4 + j] = ld2(kbase + (size_t)(pbk * 16 + r) * 128 + 32 * c + 8 * j);
+        wait_vm8(tmp);
+#pragma unroll
+        for (int pbk = 0; pbk < 2; pbk++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) kf[pbk][j] = (p0 + pbk * 16 + r) < pos ? as_half8(tmp[pbk * 4 + j]) : hz;
+#pragma unroll
+        for (int t = 0; t < 8; t++) tmp[t] = ld2(vbase + ((size_t)c * 128 + t * 16 + r) * 8);
+        wait_vm8(tmp);
+#pragma unroll
+        for (int t = 0; t < 8; t++) vf[t] = as_half8(tmp[t]);
+      }
+      // Q operand: MFMA row 4*hh carries head hh of this group; lane (r, c) holds d = 32c + 8j + 0..7.
+      // q arrives as fp16-pair entries in natural order: entry (head*128 + d) / 2.
+      half8_t qa[4];
+      {
+        const int hh = r >> 2;
+        const bool valid = ((r & 3) == 0) && hh < GROUP;
+        const u64 *qsrc = a.qkv + ((size_t)(kvh * GROUP + (valid ? hh : 0)) * 128 + 32 * c) / 2;
+        uint4_t qv[8];
+        while (true) {
+#pragma unroll
+          for (int i = 0; i < 8; i++) qv[i] = ld2(qsrc + 2 * i);
+          wait_vm8(qv);
+          bool ok = true;
+#pragma unroll
+          for (int i = 0; i < 8; i++) ok = ok && tag_ok(qv[i][1], tag) && tag_ok(qv[i][3], tag);
+          if (__all(ok || !valid)) break;
+          if (!poll_backoff_ws(ws, a.abort_flag)) break;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          U32H2 e0, e1, e2, e3;
+          e0.u = valid ? qv[2 * j][0] : 0u;
+          e1.u = valid ? qv[2 * j][2] : 0u;
+          e2.u = valid ? qv[2 * j + 1][0] : 0u;
+          e3.u = valid ? qv[2 * j + 1][2] : 0u;
+          qa[j] = half8_t{e0.h[0], e0.h[1], e1.h[0], e1.h[1], e2.h[0], e2.h[1], e3.h[0], e3.h[1]};
+        }
+      }
+      float sc2[2];
+#pragma unroll
+      for (int pbk = 0; pbk < 2; pbk++) {
+        float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < 4; j++) d = __builtin_amdgcn_mfma_f32_16x16x32_f16(qa[j], kf[pbk][j], d, 0, 0, 0);
+        const int p = p0 + pbk * 16 + r;  // lane (r, c): score of head c at position p
+        sc2[pbk] = (p < pos) ? d[0] * scale : -INFINITY;
+      }
+      float mx = fmaxf(sc2[0], sc2[1]);
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+      const float e0 = (sc2[0] == -INFINITY) ? 0.0f : __expf(sc2[0] - mx);
+      const float e1 = (sc2[1] == -INFINITY) ? 0.0f : __expf(sc2[1] - mx);
+      float sum = e0 + e1;
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+      m_h = mx;
+      l_h = sum;
+      lds_f16 *pw = p_lds + (size_t)wave * 4 * 32;
+      pw[c * 32 + r] = (_Float16)e0;
+      pw[c * 32 + 16 + r] = (_Float16)e1;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+      half8_t pa = {0, 0, 0, 0, 0, 0, 0, 0};
+      if ((r & 3) == 0 && (r >> 2) < GROUP) {
+        typedef __attribute__((address_space(3))) half8_t lds_h8;
+        pa = *(const lds_h8 *)(pw + (r >> 2) * 32 + 8 * c);
+      }
+#pragma unroll
+      for (int t = 0; t < 8; t++) {
+        half8_t vv = vf[t];
+        if (p0 + 8 * c >= pos) vv = hz;
+        else if (p0 + 8 * c + 8 > pos) {
+#pragma unroll
+          for (int e = 0; e < 8; e++)
+            if (p0 + 8 * c + e >= pos) vv[e] = (_Float16)0.0f;
+        }
+        float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
+        d = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vv, d, 0, 0, 0);
+        o_acc[t] = d[0];  // lane (r, c): o of head c at d = 16 t + r
+      }
+    }
+    if (r == 0) {
+      w_m[wave * 4 + c] = m_h;
+      w_l[wave * 4 + c] = l_h;
+    }
+#pragma unroll
+    for (int t = 0; t < 8; t++) w_o[((size_t)wave * 4 + c) * 128 + t * 16 + r] = o_acc[t];
+    compute_barrier(ws, bar, CW);
+    for (int idx = tid; idx < GROUP * 128; idx += 64 * CW) {
+      const int hh = idx >> 7, dd = idx & 127;
+      float mx = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < 4; w++) mx = fmaxf(mx, w_m[w * 4 + hh]);
+      float l = 0.0f, o = 0.0f;
+#pragma unroll
+      for (int w = 0; w < 4; w++) {
+        const float wm = w_m[w * 4 + hh];
+        const float f = (wm == -INFINITY) ? 0.0f : __expf(wm - mx);
+        l += w_l[w * 4 + hh] * f;
+        o += w_o[((size_t)w * 4 + hh) * 128 + dd] * f;
+      }
+      u64 *dst = a.part + ((size_t)(kvh * GROUP + hh) * max_chunks + chunk) * PART_REC;
+      st_entry(dst + 2 + dd, __float_as_uint(o), tag);
+      if (dd == 0) {
+        st_entry(dst, __float_as_uint(mx), tag);
+        st_entry(dst + 1, __float_as_uint(l), tag);
+      }
+    }
+    compute_barrier(ws, bar, CW);
+  }
+  return ws;
+}
+
+// Merge the chunk partials of one head with the token of this step (its k / v come straight from the qkv
+// exchange buffer), publish the head's output, and append k / v to the cache (first head of each group).
+__device__ ATTN_INL WaitState attn_combine(AttnArgs a, WaitState ws, int head) {
+  const int lane = threadIdx.x & 63;
+  const int pos = a.pos;
+  const uint32_t tag = a.tag;
+  const int nchunks = (pos + ACHUNK - 1) / ACHUNK;
+  const int max_chunks = a.max_ctx / ACHUNK;
+  const int kvh = head / a.GROUP;
+  float M = -INFINITY, Ls = 0.0f, O0 = 0.0f, O1 = 0.0f;
+  auto merge = [&](float mc, float lc, float o0, float o1) {
+    if (mc == -INFINITY) return;
+    const float Mn = fmaxf(M, mc);
+    const float fa = (M == -INFINITY) ? 0.0f : __expf(M - Mn);
+    const float fb = __expf(mc - Mn);
+    Ls = Ls * fa + lc * fb;
+    O0 = O0 * fa + o0 * fb;
+    O1 = O1 * fa + o1 * fb;
+    M = Mn;
+  };
+#pragma unroll 1
+  for (int ch0 = 0; ch0 < nchunks; ch0 += 4) {  // four chunks per round trip
+    uint4_t v[8];
+    while (true) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int ch = ch0 + i < nchunks ? ch0 + i : nchunks - 1;
+        const u64 *rec = a.part + ((size_t)head * max_chunks + ch) * PART_REC;
+        v[2 * i] = ld2(rec);
+        v[2 * i + 1] = ld2(rec + 2 + 2 * lane);
+      }
+      wait_vm8(v);
+      bool ok = true;
+#pragma unroll
+      for (int i = 0; i < 8; i++) ok = ok && tag_ok(v[i][1], tag) && tag_ok(v[i][3], tag);
+      if (__all(ok)) break;
+      if (!poll_backoff_ws(ws, a.abort_flag)) break;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      if (ch0 + i < nchunks)
+        merge(__uint_as_float(v[2 * i][0]), __uint_as_float(v[2 * i][2]), __uint_as_float(v[2 * i + 1][0]),
+              __uint_as_float(v[2 * i + 1][2]));
+  }
+  const u64 *qe = a.qkv + (size_t)head * 64 + lane;
+  const u64 *ke = a.qkv + (size_t)(a.HQ + kvh) * 64 + lane;
+  const u64 *ve = a.qkv + (size_t)(a.HQ + a.HKV + kvh) * 64 + lane;
+  u64 q, k, v;
+  while (true) {
+    q = __hip_atomic_load(qe, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    k = __hip_atomic_load(ke, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    v = __hip_atomic_load(ve, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool ok = tag_ok((uint32_t)(q >> 32), tag) && tag_ok((uint32_t)(k >> 32), tag) && tag_ok((uint32_t)(v >> 32), tag);
+    if (__all(ok)) break;
+    if (!poll_backoff_ws(ws, a.abort_flag)) break;
+  }
+  const uint32_t qw = (uint32_t)q, kw = (uint32_t)k, vw = (uint32_t)v;
+  const float s = wave_sum(h2_lo(qw) * h2_lo(kw) + h2_hi(qw) * h2_hi(kw)) * 0.08838834764831845f;
+  merge(s, 1.0f, h2_lo(vw), h2_hi(vw));
+  const float inv = Ls > 0.0f ? 1.0f / Ls : 0.0f;
+  st_entry(a.ao + xidx(head * 128 + 2 * lane, a.ks_o, a.frags_o), pack_h2(O0 * inv, O1 * inv), tag);
+  if (head == kvh * a.GROUP) {
+    // append: other workgroups read these lines in later steps of this launch -> agent-scope stores
+    uint32_t *krow = reinterpret_cast<uint32_t *>(a.kc + ((size_t)kvh * a.max_ctx + pos) * 128);
+    __hip_atomic_store(krow + lane, kw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint16_t *vslab = reinterpret_cast<uint16_t *>(a.vc + (((size_t)kvh * (a.max_ctx / 8) + pos / 8) * 128) * 8) + (pos & 7);
+    __hip_atomic_store(vslab + (size_t)(2 * lane) * 8, (uint16_t)(vw & 0xFFFFu), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(vslab + (size_t)(2 * lane + 1) * 8, (uint16_t)(vw >> 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  return ws;
+}
+
+struct GemvArgs {
+  const u64 *in_buf, *ss;        // exchange vector of the activation; sum-of-squares entries behind it or null
+  uint32_t *abort_flag;
+  unsigned long long *dbg_t;     // null or two timestamp slots (input arrived, blocks done)
+  uint32_t tag;
+  int ks, frags, pairs, odd, nb, ss_count, d_model;
+  float eps;
+  uint32_t ring_off, part_off, sync_off;  // LDS byte addresses: this wave's ring, its row-sum slots, sync words
+};
+struct GemvState {
+  unsigned crec;   // weight records this wave has consumed in this launch
+  WaitState ws;
+};
+
+// One projection for one compute wave: waits for its slice of the activation, then consumes the records
+// of every 8-row block this workgroup owns and leaves one partial row sum per row in LDS (the caller adds
+// the CW slices).  Ends with the barrier of the compute waves.
+__device__ GEMV_INL GemvState gemv_stage(GemvArgs a, GemvState st) {
+  // arguments of a non-kernel function arrive in vector registers: tell the compiler which are wave-uniform
+  a.tag = __builtin_amdgcn_readfirstlane(a.tag);
+  a.ks = __builtin_amdgcn_readfirstlane(a.ks);
+  a.frags = __builtin_amdgcn_readfirstlane(a.frags);
+  a.pairs = __builtin_amdgcn_readfirstlane(a.pairs);
+  a.odd = __builtin_amdgcn_readfirstlane(a.odd);
+  a.nb = __builtin_amdgcn_readfirstlane(a.nb);
+  a.ss_count = __builtin_amdgcn_readfirstlane(a.ss_count);
+  a.ring_off = __builtin_amdgcn_readfirstlane(a.ring_off);
+  a.part_off = __builtin_amdgcn_readfirstlane(a.part_off);
+  a.sync_off = __builtin_amdgcn_readfirstlane(a.sync_off);
+  st.crec = __builtin_amdgcn_readfirstlane(st.crec);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int r = lane & 15, c = lane >> 4;
+  lds_u32 *sync = (lds_u32 *)(uintptr_t)a.sync_off;
+  lds_f32 *dst = (lds_f32 *)(uintptr_t)a.part_off;
+  // The decode constants are kept in registers the compiler cannot see through, so that (s & mask) | magic
+  // becomes one three-register v_and_or_b32 instead of two literal-operand instructions.  (An inline-asm
+  // v_and_or_b32 is not an option: the hazard recognizer does not see it overwrite a register that a
+  // matrix instruction is still writing.)
+  uint32_t magic = 0x64006400u, mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u;
+  asm volatile("" : "+v"(magic), "+v"(mask_lo), "+v"(mask_hi));
+  const uint32_t tag = a.tag;
+  half8_t xa[MAXF];
+  float4_t z[MAXF];
+  float rstd = 1.0f;
+  const half8_t bc = {(_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f,
+                      (_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f};
+  const bool normed = a.ss != nullptr;
+  // ---- activation fragments (A operand: row i = k-block i of the fragment) ------------------------------
+  // A `normed` vector holds fp16(h * gamma * 2^-e) with the exponent e of each 8-row block in the top byte
+  // of its tag words; the operand is then fp16(h * gamma / rms), the activation RMSNorm feeds
+  // (crates/yscv-kernels/src/ops/norm.rs:1497-1518); 1/rms comes from the sum-of-squares entries.
+#pragma unroll
+  for (int f = 0; f < MAXF; f++) {
+    if (f < a.frags && a.nb > 0) {
+      const u64 *p = a.in_buf + (((size_t)wave * a.frags + f) << 8) + 2 * lane;
+      const bool valid = (512 * f + 32 * r) < a.ks;
+      const bool with_ss = normed && f == 0;
+      const bool v0 = with_ss && 4 * lane < a.ss_count, v1 = with_ss && 4 * lane + 1 < a.ss_count,
+                 v2 = with_ss && 4 * lane + 2 < a.ss_count, v3 = with_ss && 4 * lane + 3 < a.ss_count;
+      const u64 *sp = with_ss ? a.ss + 4 * lane : a.in_buf;
+      uint4_t qa, qb, sa, sb;
+      while (true) {
+        qa = ld2(p);
+        qb = ld2(p + 128);
+        sa = ld2(sp);
+        sb = ld2(sp + 2);
+        wait_vm(qa, qb, sa, sb);
+        bool ok = !valid || (tag_ok(qa[1], tag) && tag_ok(qa[3], tag) && tag_ok(qb[1], tag) && tag_ok(qb[3], tag));
+        ok = ok && (!v0 || tag_ok(sa[1], tag)) && (!v1 || tag_ok(sa[3], tag)) && (!v2 || tag_ok(sb[1], tag)) &&
+             (!v3 || tag_ok(sb[3], tag));
+        if (__all(ok)) break;
+        if (!poll_backoff_ws(st.ws, a.abort_flag)) break;
+      }
+      if (with_ss) {
+        const float sq = (v0 ? __uint_as_float(sa[0]) : 0.0f) + (v1 ? __uint_as_float(sa[2]) : 0.0f) +
+                         (v2 ? __uint_as_float(sb[0]) : 0.0f) + (v3 ? __uint_as_float(sb[2]) : 0.0f);
+        rstd = 1.0f / sqrtf(wave_sum(sq) / (float)a.d_model + a.eps);
+      }
+      U32H2 u0, u1, u2, u3;
+      u0.u = valid ? qa[0] : 0u;
+      u1.u = valid ? qa[2] : 0u;
+      u2.u = valid ? qb[0] : 0u;
+      u3.u = valid ? qb[2] : 0u;
+      if (normed) {
+        const float fac = valid ? ldexpf(rstd, (int)(qa[1] >> 24) - 128) : 0.0f;
+        u0.h = half2_t{(_Float16)((float)u0.h[0] * fac), (_Float16)((float)u0.h[1] * fac)};
+        u1.h = half2_t{(_Float16)((float)u1.h[0] * fac), (_Float16)((float)u1.h[1] * fac)};
+        u2.h = half2_t{(_Float16)((float)u2.h[0] * fac), (_Float16)((float)u2.h[1] * fac)};
+        u3.h = half2_t{(_Float16)((float)u3.h[0] * fac), (_Float16)((float)u3.h[1] * fac)};
+      }
+      // the slots that meet 1024 + 16 q carry x / 16 (exact: a power of two)
+      const half2_t sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+      u1.h = u1.h * sixteenth;
+      u3.h = u3.h * sixteenth;
+      xa[f] = half8_t{u0.h[0], u0.h[1], u1.h[0], u1.h[1], u2.h[0], u2.h[1], u3.h[0], u3.h[1]};
+      const float4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+      z[f] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[f], bc, zero, 0, 0, 0);  // offset term of every k-block
+    } else {
+      xa[f] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      z[f] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+  }
+  if (a.dbg_t && threadIdx.x == 0) a.dbg_t[0] = wall_clock64();
+
+  // ---- one record: 8 rows x 512 k against fragment xa ------------------------------------------------------
+  unsigned crec = st.crec;
+  auto consume = [&](bool single, const half8_t &xf, const float4_t &zf, float &acc) {
+    {
+      unsigned spins = 0;
+      while ((int)(__hip_atomic_load(sync + wave, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) - (crec + 1)) < 0) {
+        __builtin_amdgcn_s_sleep(0);
+        if (++spins > 40000000u) {  // the stream stalled: never expected, but no wait here is unbounded
+          __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+      }
+    }
+    const uint32_t slot = crec % RING;
+    const uint32_t a_w = a.ring_off + slot * SLOT + lane * 16;
+    const uint32_t a_s = a.ring_off + slot * SLOT + (c >> 1) * 128 + r * 8;
+    uint4_t w0, w1;
+    typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+    uint2_t sc;
+    asm volatile(
+        "ds_read_b128 %0, %3\n\tds_read_b128 %1, %3 offset:1024\n\tds_read_b64 %2, %4 offset:2048\n\ts_waitcnt lgkmcnt(0)"
+        : "=&v"(w0), "=&v"(w1), "=&v"(sc)
+        : "v"(a_w), "v"(a_s)
+        : "memory");
+    crec++;
+    if (lane == 0) __hip_atomic_store(sync + 8 + wave, crec, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    const float4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    float d0[4], d1[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      U32H2 q0, q1, q2, q3;
+      const uint32_t s = w0[j], s2 = s >> 8;
+      q0.u = (s & mask_lo) | magic;
+      q1.u = (s & mask_hi) | magic;
+      q2.u = (s2 & mask_lo) | magic;
+      q3.u = (s2 & mask_hi) | magic;
+      const half8_t b = {q0.h[0], q0.h[1], q1.h[0], q1.h[1], q2.h[0], q2.h[1], q3.h[0], q3.h[1]};
+      const float4_t dd = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf, b, zero, 0, 0, 0);
+      d0[j] = dd[j];
+    }
+    if (!single) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        U32H2 q0, q1, q2, q3;
+        const uint32_t s = w1[j], s2 = s >> 8;
+        q0.u = (s & mask_lo) | magic;
+        q1.u = (s & mask_hi) | magic;
+        q2.u = (s2 & mask_lo) | magic;
+        q3.u = (s2 & mask_hi) | magic;
+        const half8_t b = {q0.h[0], q0.h[1], q1.h[0], q1.h[1], q2.h[0], q2.h[1], q3.h[0], q3.h[1]};
+        const float4_t dd = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf, b, zero, 0, 0, 0);
+        d1[j] = dd[j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; j++) d1[j] = 0.0f;
+    }
+    const bool second = (c >> 1) != 0;
+    const float s0 = h2_lo(sc[0]), s1 = h2_hi(sc[0]), s2 = h2_lo(sc[1]), s3 = h2_hi(sc[1]);
+    acc = fmaf(s0, (second ? d1[0] : d0[0]) - zf[0], acc);
+    acc = fmaf(s1, (second ? d1[1] : d0[1]) - zf[1], acc);
+    acc = fmaf(s2, (second ? d1[2] : d0[2]) - zf[2], acc);
+    acc = fmaf(s3, (second ? d1[3] : d0[3]) - zf[3], acc);
+  };
+
+  const bool useful = (c & 1) == (r >> 3);
+#pragma unroll 1
+  for (int blk = 0; blk < a.nb; blk++) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int p = 0; p < MAXF; p++)
+      if (p < a.pairs) consume(a.odd && p == a.pairs - 1, xa[p], z[p], acc);
+    acc = useful ? acc : 0.0f;
+    acc += __shfl_xor(acc, 8, 64);
+    acc += __shfl_xor(acc, 16, 64);
+    acc += __shfl_xor(acc, 32, 64);
+    if (lane < 8) dst[blk * 8 + lane] = acc;
+  }
+  if (a.dbg_t && threadIdx.x == 0) a.dbg_t[1] = wall_clock64();
+  st.crec = crec;
+  compute_barrier(st.ws, sync + 16, CW);
+  return st;
+}
+
+__global__ void __launch_bounds__(THREADS, 1)
 decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int max_steps, uint32_t epoch0) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   float *part_lds = reinterpret_cast<float *>(lds + RING_BYTES);                 // [2][8][PART_ROWS]
@@ -139,6 +631,7 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
   int *tok_lds = reinterpret_cast<int *>(att_lds + 1024 + 128 + 8192);            // [1]
   float *arg_v = reinterpret_cast<float *>(att_lds + 1024 + 128 + 8192 + 64);     // [8]
   int *arg_i = reinterpret_cast<int *>(att_lds + 1024 + 128 + 8192 + 128);        // [8]
+  lds_u32 *sync = (lds_u32 *)(lds + RING_BYTES + PART_BYTES + ATT_BYTES);  // [0..CW) landed, [8..8+CW) consumed, [16] barrier
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -152,210 +645,153 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
   const int max_chunks = m.max_ctx / ACHUNK;
   const uint32_t magic = 0x64006400u;
 
-  // ---- weight stream: prefetcher state (wave uniform) ------------------------------------------------
-  const unsigned char *const stream_base = m.stream + m.wg_off[wg] + (size_t)wave * m.wave_bytes[wg];
-  const unsigned char *pf_ptr = stream_base;
-  int pf_slot = 0, pf_kind = 0, pf_layer = 0, pf_blk = 0, pf_pair = 0;
   auto nbw = [&](int kind) { return wg < m.ph[kind].nb ? (m.ph[kind].nb - wg + G - 1) / G : 0; };
-  const bool has_work = m.wave_bytes[wg] != 0;
-  unsigned char *const ring = lds + (size_t)wave * RING * SLOT;
-  const uint32_t ring_lds = (uint32_t)(size_t)ring;  // low 32 bits of an LDS pointer = LDS byte address
-
-  auto pf_next_kind = [&]() {
-    if (pf_kind == PK_DOWN) {
-      pf_layer++;
-      pf_kind = pf_layer == L ? PK_LM : PK_QKV;
-    } else if (pf_kind == PK_LM) {
-      pf_layer = 0;
-      pf_kind = PK_QKV;
-      pf_ptr = stream_base;
-    } else {
-      pf_kind++;
-    }
+  int dbg_layer = 0;
+  auto mark = [&](int idx) {
+    if (m.dbg_t && tid == 0) m.dbg_t[((size_t)wg * L + dbg_layer) * 16 + idx] = wall_clock64();
   };
-  auto pf_issue = [&]() {
-    if (!has_work) return;
-    while (nbw(pf_kind) == 0) pf_next_kind();
-    const int pairs = m.ph[pf_kind].pairs;
-    const bool single = (pf_pair == pairs - 1) && (m.ph[pf_kind].tiles & 1);
-    unsigned char *dst = ring + pf_slot * SLOT;
-    __builtin_amdgcn_global_load_lds(AS1(pf_ptr + lane * 16), AS3(dst), 16, 0, 2);
-    __builtin_amdgcn_global_load_lds(AS1(pf_ptr + (single ? 0 : 1024) + lane * 16), AS3(dst + 1024), 16, 0, 2);
-    __builtin_amdgcn_global_load_lds(AS1(pf_ptr + (single ? 1024 : 2048) + lane * 4), AS3(dst + 2048), 4, 0, 2);
-    pf_ptr += single ? PS_REC_SINGLE : PS_REC_FULL;
-    pf_slot = pf_slot + 1 == RING ? 0 : pf_slot + 1;
-    if (++pf_pair == pairs) {
-      pf_pair = 0;
-      if (++pf_blk >= nbw(pf_kind)) {
-        pf_blk = 0;
-        pf_next_kind();
+  if (tid < 32) sync[tid] = 0;
+  __syncthreads();
+
+  // ---- producer waves: stream the weight records of their compute waves into the LDS rings -------------
+  // A producer issues a record (3 direct global->LDS loads) whenever a ring of one of its waves has a free
+  // slot, and publishes how many records have landed from its own outstanding-load counter (loads return in
+  // order).  Compute waves never have a weight load of their own in flight, so their polls are not queued
+  // behind the stream.
+  // ---- producer waves: stream the weight records of their compute waves into the LDS rings -------------
+  // A producer issues a record (3 direct global->LDS loads) whenever a ring of one of its waves has a free
+  // slot, and publishes how many records have landed, which it reads from its own outstanding-load counter
+  // (loads return in order).  Compute waves never have a weight load of their own in flight, so their polls
+  // are not queued behind the stream.  The LDS words shared with the compute waves are accessed with explicit
+  // ds instructions: a compiler-visible LDS read would be ordered behind every outstanding LDS-bound load.
+  if (wave >= CW) {
+    const uint32_t sync_lds = (uint32_t)(size_t)(lds + RING_BYTES + PART_BYTES + ATT_BYTES);
+  {
+    constexpr int SERVED = CW / PW;
+    const int p = wave - CW;
+    const uint32_t lds_base = (uint32_t)(size_t)lds;
+    int nb_k[PK_COUNT], pairs_k[PK_COUNT], odd_k[PK_COUNT];
+    unsigned per_step = 0;
+#pragma unroll
+    for (int k = 0; k < PK_COUNT; k++) {
+      nb_k[k] = nbw(k);
+      pairs_k[k] = m.ph[k].pairs;
+      odd_k[k] = m.ph[k].tiles & 1;
+      per_step += (unsigned)nb_k[k] * pairs_k[k] * (k == PK_LM ? 1 : L);
+    }
+    const unsigned total = per_step * (unsigned)n_steps;  // records per compute wave in this launch
+    const unsigned char *base[SERVED], *ptr[SERVED];
+    int kind[SERVED], layer[SERVED], blk[SERVED], pair[SERVED];
+    unsigned issued[SERVED], landed_cnt[SERVED];
+#pragma unroll
+    for (int j = 0; j < SERVED; j++) {
+      const int w = p * SERVED + j;
+      base[j] = ptr[j] = m.stream + m.wg_off[wg] + (size_t)w * m.wave_bytes[wg];
+      kind[j] = layer[j] = blk[j] = pair[j] = 0;
+      issued[j] = landed_cnt[j] = 0;
+    }
+    unsigned long long fifo = 0;  // bit (i & 63): which served wave the i-th issued record belongs to
+    unsigned n_issued = 0, n_retired = 0;
+    auto kv = [&](const int *arr, int k) {  // 5-entry table lookup without dynamic register indexing
+      return k == 0 ? arr[0] : (k == 1 ? arr[1] : (k == 2 ? arr[2] : (k == 3 ? arr[3] : arr[4])));
+    };
+    if (total > 0) {
+      while (n_retired < total * SERVED) {
+        bool did = false;
+#pragma unroll
+        for (int j = 0; j < SERVED; j++) {
+          const int w = p * SERVED + j;
+          if (issued[j] < total && n_issued - n_retired < 20 &&
+              issued[j] - lds_peek(sync_lds + 4 * (8 + w)) < RING) {
+            while (kv(nb_k, kind[j]) == 0) {  // kinds this workgroup has no rows of
+              if (kind[j] == PK_DOWN) { layer[j]++; kind[j] = layer[j] == L ? PK_LM : PK_QKV; }
+              else if (kind[j] == PK_LM) { layer[j] = 0; kind[j] = PK_QKV; ptr[j] = base[j]; }
+              else kind[j]++;
+            }
+            const int pairs = kv(pairs_k, kind[j]);
+            const bool single = (pair[j] == pairs - 1) && kv(odd_k, kind[j]);
+            const uint32_t dst = lds_base + (uint32_t)((w * RING + issued[j] % RING) * SLOT);
+            const unsigned char *src = ptr[j];
+            __builtin_amdgcn_global_load_lds(AS1(src + lane * 16), (void __attribute__((address_space(3))) *)(uintptr_t)(dst), 16, 0, 2);
+            __builtin_amdgcn_global_load_lds(AS1(src + (single ? 0 : 1024) + lane * 16), (void __attribute__((address_space(3))) *)(uintptr_t)(dst + 1024), 16, 0, 2);
+            __builtin_amdgcn_global_load_lds(AS1(src + (single ? 1024 : 2048) + lane * 4), (void __attribute__((address_space(3))) *)(uintptr_t)(dst + 2048), 4, 0, 2);
+            ptr[j] += single ? PS_REC_SINGLE : PS_REC_FULL;
+            issued[j]++;
+            fifo = (fifo & ~(1ull << (n_issued & 63))) | ((unsigned long long)j << (n_issued & 63));
+            n_issued++;
+            did = true;
+            if (++pair[j] == pairs) {
+              pair[j] = 0;
+              if (++blk[j] >= kv(nb_k, kind[j])) {
+                blk[j] = 0;
+                if (kind[j] == PK_DOWN) { layer[j]++; kind[j] = layer[j] == L ? PK_LM : PK_QKV; }
+                else if (kind[j] == PK_LM) { layer[j] = 0; kind[j] = PK_QKV; ptr[j] = base[j]; }
+                else kind[j]++;
+              }
+            }
+          }
+        }
+        // outstanding vector-memory operations of this wave: IB_STS.vm_cnt (bits 3:0 and 23:22)
+        // (read after the issues above: the clobber keeps the compiler from moving it across them)
+        unsigned ib_sts;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_IB_STS)" : "=s"(ib_sts)::"memory");
+        const unsigned vm = (ib_sts & 15u) | (((ib_sts >> 22) & 3u) << 4);
+        const unsigned done = n_issued - (vm + 2) / 3;
+        bool dirty = false;
+        while ((int)(done - n_retired) > 0) {
+          const int j = (int)((fifo >> (n_retired & 63)) & 1ull);
+          if (j == 0) landed_cnt[0]++; else landed_cnt[SERVED - 1]++;
+          n_retired++;
+          dirty = true;
+        }
+        if (dirty) {
+          if (DBG_WAIT_ALL) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+          for (int j = 0; j < SERVED; j++)
+            lds_poke(sync_lds + 4 * (p * SERVED + j), landed_cnt[j]);
+        }
+        if (!did && !dirty) __builtin_amdgcn_s_sleep(1);
       }
     }
-  };
-#pragma unroll 1
-  for (int i = 0; i < RING - 1; i++) pf_issue();
-  int cslot = 0;  // ring slot of the next record to consume
+  }
+    return;
+  }
 
-  // ---- one record: 8 rows x 512 k against the activation fragment xa ------------------------------
-  auto consume = [&](bool single, const half8_t &xa, const float4_t &z, float &acc) {
-    pf_issue();
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (RING - 1)) : "memory");
-    const uint32_t a_w = ring_lds + cslot * SLOT + lane * 16;
-    const uint32_t a_s = ring_lds + cslot * SLOT + (c >> 1) * 128 + r * 8;
-    uint4_t w0, w1;
-    typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
-    uint2_t sc;
-    asm volatile(
-        "ds_read_b128 %0, %3\n\tds_read_b128 %1, %3 offset:1024\n\tds_read_b64 %2, %4 offset:2048\n\ts_waitcnt lgkmcnt(0)"
-        : "=&v"(w0), "=&v"(w1), "=&v"(sc)
-        : "v"(a_w), "v"(a_s)
-        : "memory");
-    cslot = cslot + 1 == RING ? 0 : cslot + 1;
-    const float4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
-    float d0[4], d1[4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      U32H2 q0, q1, q2, q3;
-      const uint32_t s = w0[j], s2 = s >> 8;
-      q0.u = (s & 0x000F000Fu) | magic;
-      q1.u = (s & 0x00F000F0u) | magic;
-      q2.u = (s2 & 0x000F000Fu) | magic;
-      q3.u = (s2 & 0x00F000F0u) | magic;
-      const half8_t b = {q0.h[0], q0.h[1], q1.h[0], q1.h[1], q2.h[0], q2.h[1], q3.h[0], q3.h[1]};
-      const float4_t dd = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, b, zero, 0, 0, 0);
-      d0[j] = dd[j];
-    }
-    if (!single) {
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        U32H2 q0, q1, q2, q3;
-        const uint32_t s = w1[j], s2 = s >> 8;
-        q0.u = (s & 0x000F000Fu) | magic;
-        q1.u = (s & 0x00F000F0u) | magic;
-        q2.u = (s2 & 0x000F000Fu) | magic;
-        q3.u = (s2 & 0x00F000F0u) | magic;
-        const half8_t b = {q0.h[0], q0.h[1], q1.h[0], q1.h[1], q2.h[0], q2.h[1], q3.h[0], q3.h[1]};
-        const float4_t dd = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, b, zero, 0, 0, 0);
-        d1[j] = dd[j];
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; j++) d1[j] = 0.0f;
-    }
-    const bool second = (c >> 1) != 0;
-    const float s0 = h2_lo(sc[0]), s1 = h2_hi(sc[0]), s2 = h2_lo(sc[1]), s3 = h2_hi(sc[1]);
-    acc = fmaf(s0, (second ? d1[0] : d0[0]) - z[0], acc);
-    acc = fmaf(s1, (second ? d1[1] : d0[1]) - z[1], acc);
-    acc = fmaf(s2, (second ? d1[2] : d0[2]) - z[2], acc);
-    acc = fmaf(s3, (second ? d1[3] : d0[3]) - z[3], acc);
-  };
+  // ---- compute waves ---------------------------------------------------------------------------------
+  const uint32_t ring_lds = (uint32_t)(size_t)(lds + (size_t)wave * RING * SLOT);  // LDS byte address of this wave's ring
+  WaitState ws{SPIN_LIMIT, 0};
+  auto cbar = [&]() { compute_barrier(ws, sync + 16, CW); };
 
-  // ---- bounded waiting ------------------------------------------------------------------------------
-  unsigned spin_budget = SPIN_LIMIT;
-  auto poll_backoff = [&]() -> bool {  // false: give up (the budget ran out or another wave gave up)
-    __builtin_amdgcn_s_sleep(2);
-    if (spin_budget <= 1 || ((spin_budget & 63u) == 0 && aborted(m))) {
-      set_abort(m);
-      spin_budget = 1;
-      return false;
-    }
-    spin_budget--;
-    return true;
-  };
-  // Fragment f of this wave's slice of an exchange vector, as the A operand (row i = k-block i).
-  // With ss != null the per-workgroup sum-of-squares entries behind the vector are summed into 1/rms
-  // (returned through rstd).  A `normed` vector holds fp16(h * gamma * 2^-e) with the exponent e of each
-  // 8-row block in the top byte of its tag words; the operand is then fp16(h * gamma * rstd), the
-  // activation the multi-kernel path feeds (RMSNorm, crates/yscv-kernels/src/ops/norm.rs:1497-1518).
-  auto load_fragment = [&](const u64 *buf, int ks, int frags, int f, uint32_t tag, const u64 *ss, int ss_count,
-                           bool normed, float &rstd) -> half8_t {
-    const u64 *p = buf + (((size_t)wave * frags + f) << 8) + 2 * lane;
-    const bool valid = (512 * f + 32 * r) < ks;
-    const bool v0 = ss && 4 * lane < ss_count, v1 = ss && 4 * lane + 1 < ss_count, v2 = ss && 4 * lane + 2 < ss_count,
-               v3 = ss && 4 * lane + 3 < ss_count;
-    const u64 *sp = ss ? ss + 4 * lane : buf;
-    uint4_t a, b, sa, sb;
-    while (true) {
-      a = ld2(p);
-      b = ld2(p + 128);
-      sa = ld2(sp);
-      sb = ld2(sp + 2);
-      wait_vm(a, b, sa, sb);
-      bool ok = !valid || (tag_ok(a[1], tag) && tag_ok(a[3], tag) && tag_ok(b[1], tag) && tag_ok(b[3], tag));
-      ok = ok && (!v0 || tag_ok(sa[1], tag)) && (!v1 || tag_ok(sa[3], tag)) && (!v2 || tag_ok(sb[1], tag)) &&
-           (!v3 || tag_ok(sb[3], tag));
-      if (__all(ok)) break;
-      if (!poll_backoff()) break;
-    }
-    if (ss) {
-      const float sq = (v0 ? __uint_as_float(sa[0]) : 0.0f) + (v1 ? __uint_as_float(sa[2]) : 0.0f) +
-                       (v2 ? __uint_as_float(sb[0]) : 0.0f) + (v3 ? __uint_as_float(sb[2]) : 0.0f);
-      rstd = 1.0f / sqrtf(wave_sum(sq) / (float)D + m.eps);
-    }
-    U32H2 u0, u1, u2, u3;
-    u0.u = valid ? a[0] : 0u;
-    u1.u = valid ? a[2] : 0u;
-    u2.u = valid ? b[0] : 0u;
-    u3.u = valid ? b[2] : 0u;
-    if (normed) {
-      const float fac = valid ? ldexpf(rstd, (int)(a[1] >> 24) - 128) : 0.0f;
-      u0.h = half2_t{(_Float16)((float)u0.h[0] * fac), (_Float16)((float)u0.h[1] * fac)};
-      u1.h = half2_t{(_Float16)((float)u1.h[0] * fac), (_Float16)((float)u1.h[1] * fac)};
-      u2.h = half2_t{(_Float16)((float)u2.h[0] * fac), (_Float16)((float)u2.h[1] * fac)};
-      u3.h = half2_t{(_Float16)((float)u3.h[0] * fac), (_Float16)((float)u3.h[1] * fac)};
-    }
-    // the slots that meet 1024 + 16 q carry x / 16 (exact: a power of two)
-    const half2_t sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
-    u1.h = u1.h * sixteenth;
-    u3.h = u3.h * sixteenth;
-    return half8_t{u0.h[0], u0.h[1], u1.h[0], u1.h[1], u2.h[0], u2.h[1], u3.h[0], u3.h[1]};
-  };
-
-  // ---- one projection: leaves the row sums of this workgroup in part_lds[pb]; returns 1/rms ------------
   int pb = 0;
-  const half8_t bc = {(_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f,
-                      (_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f};
   const int ss_count = m.ph[PK_O].nb < G ? m.ph[PK_O].nb : G;
-  auto gemv = [&](int kind, const u64 *in_buf, uint32_t tag, bool with_ss) {
-    const int ks = m.ph[kind].ks, frags = m.ph[kind].frags, pairs = m.ph[kind].pairs;
-    const bool odd = m.ph[kind].tiles & 1;
-    const int nb = nbw(kind);
-    half8_t xa[4];
-    float4_t z[4];
-    float rstd = 1.0f;
-    const u64 *ss = with_ss ? in_buf + persist_vec_entries(m.ph[kind].k) : nullptr;
-#pragma unroll
-    for (int f = 0; f < 4; f++) {
-      if (f < frags && nb > 0) {
-        xa[f] = load_fragment(in_buf, ks, frags, f, tag, f == 0 ? ss : nullptr, ss_count, with_ss, rstd);
-        const float4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
-        z[f] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[f], bc, zero, 0, 0, 0);
-      } else {
-        xa[f] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-        z[f] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-      }
-    }
-    float *dst = part_lds + ((size_t)pb * PS_WAVES + wave) * PART_ROWS;
-    const bool useful = (c & 1) == (r >> 3);
-#pragma unroll 1
-    for (int blk = 0; blk < nb; blk++) {
-      float acc = 0.0f;
-#pragma unroll
-      for (int p = 0; p < 4; p++)
-        if (p < pairs) consume(odd && p == pairs - 1, xa[p], z[p], acc);
-      acc = useful ? acc : 0.0f;
-      acc += __shfl_xor(acc, 8, 64);
-      acc += __shfl_xor(acc, 16, 64);
-      acc += __shfl_xor(acc, 32, 64);
-      if (lane < 8) dst[blk * 8 + lane] = acc;
-    }
-    lds_barrier();
+  unsigned crec = 0;  // weight records this wave has consumed in this launch
+  auto gemv = [&](int kind, const u64 *in_buf, uint32_t tag, bool with_ss, int mk) {
+    GemvArgs ga;
+    ga.in_buf = in_buf;
+    ga.ss = with_ss ? in_buf + persist_vec_entries(m.ph[kind].k) : nullptr;
+    ga.abort_flag = m.abort_flag;
+    ga.dbg_t = m.dbg_t ? m.dbg_t + ((size_t)wg * L + dbg_layer) * 16 + mk : nullptr;
+    ga.tag = tag;
+    ga.ks = m.ph[kind].ks;
+    ga.frags = m.ph[kind].frags;
+    ga.pairs = m.ph[kind].pairs;
+    ga.odd = m.ph[kind].tiles & 1;
+    ga.nb = nbw(kind);
+    ga.ss_count = ss_count;
+    ga.d_model = D;
+    ga.eps = m.eps;
+    ga.ring_off = ring_lds;
+    ga.part_off = (uint32_t)(size_t)(part_lds + ((size_t)pb * CW + wave) * PART_ROWS);
+    ga.sync_off = (uint32_t)(size_t)(lds + RING_BYTES + PART_BYTES + ATT_BYTES);
+    const GemvState gs = gemv_stage(ga, GemvState{crec, ws});
+    crec = gs.crec;
+    ws = gs.ws;
   };
   auto row_sum = [&](int row_slot) -> float {
-    const float *src = part_lds + (size_t)pb * PS_WAVES * PART_ROWS + row_slot;
+    const float *src = part_lds + (size_t)pb * CW * PART_ROWS + row_slot;
     float v = 0.0f;
 #pragma unroll
-    for (int w = 0; w < PS_WAVES; w++) v += src[w * PART_ROWS];
+    for (int w = 0; w < CW; w++) v += src[w * PART_ROWS];
     return v;
   };
 
@@ -384,219 +820,9 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
     }
   };
 
-  // ---- attention over the cached positions [0, pos): partials per (head, 128-position chunk) ---------
-  auto attention_items = [&](int layer, int pos, uint32_t tag) {
-    const int nchunks = (pos + ACHUNK - 1) / ACHUNK;
-    const int items = HKV * nchunks;
-    const _Float16 *kc = m.kc[layer];
-    const _Float16 *vc = m.vc[layer];
-    const float scale = 0.08838834764831845f;  // 1 / sqrt(128)
-#pragma unroll 1
-    for (int id = wg; id < items; id += G) {
-      const int chunk = id / HKV, kvh = id - chunk * HKV;
-      float m_h = -INFINITY, l_h = 0.0f;
-      float o_acc[8];
-#pragma unroll
-      for (int t = 0; t < 8; t++) o_acc[t] = 0.0f;
-      const int p0 = chunk * ACHUNK + wave * 32;
-      if (wave < 4 && p0 < pos) {
-        const _Float16 *kbase = kc + ((size_t)kvh * m.max_ctx + p0) * 128;
-        const _Float16 *vbase = vc + (((size_t)kvh * (m.max_ctx / 8) + p0 / 8) * 128) * 8;
-        half8_t kf[2][4], vf[8];
-        const half8_t hz = {0, 0, 0, 0, 0, 0, 0, 0};
-        // Blocks that were complete before this launch never change and are read with plain loads.
-        // Positions appended during this launch were written with agent-scope stores by another
-        // workgroup: their blocks are read with coherent loads, and only where already valid.
-        const bool recent = p0 + 32 > pos0;
-        if (!recent) {
-#pragma unroll
-          for (int pbk = 0; pbk < 2; pbk++)
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-              kf[pbk][j] = *reinterpret_cast<const half8_t *>(kbase + (size_t)(pbk * 16 + r) * 128 + 32 * c + 8 * j);
-#pragma unroll
-          for (int t = 0; t < 8; t++) vf[t] = *reinterpret_cast<const half8_t *>(vbase + ((size_t)c * 128 + t * 16 + r) * 8);
-        } else {
-          uint4_t tmp[8];
-#pragma unroll
-          for (int pbk = 0; pbk < 2; pbk++)
-#pragma unroll
-            for (int j = 0; j < 4; j++) tmp[pbk * 4 + j] = ld2(kbase + (size_t)(pbk * 16 + r) * 128 + 32 * c + 8 * j);
-          wait_vm8(tmp);
-#pragma unroll
-          for (int pbk = 0; pbk < 2; pbk++)
-#pragma unroll
-            for (int j = 0; j < 4; j++) kf[pbk][j] = (p0 + pbk * 16 + r) < pos ? as_half8(tmp[pbk * 4 + j]) : hz;
-#pragma unroll
-          for (int t = 0; t < 8; t++) tmp[t] = ld2(vbase + ((size_t)c * 128 + t * 16 + r) * 8);
-          wait_vm8(tmp);
-#pragma unroll
-          for (int t = 0; t < 8; t++) vf[t] = as_half8(tmp[t]);
-        }
-        // Q operand: MFMA row 4*hh carries head hh of this group; lane (r, c) holds d = 32c + 8j + 0..7.
-        // q arrives as fp16-pair entries in natural order: entry (head*128 + d) / 2.
-        half8_t qa[4];
-        {
-          const int hh = r >> 2;
-          const bool valid = ((r & 3) == 0) && hh < GROUP;
-          const u64 *qsrc = m.qkv + ((size_t)(kvh * GROUP + (valid ? hh : 0)) * 128 + 32 * c) / 2;
-          uint4_t qv[8];
-          while (true) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) qv[i] = ld2(qsrc + 2 * i);
-            wait_vm8(qv);
-            bool ok = true;
-#pragma unroll
-            for (int i = 0; i < 8; i++) ok = ok && tag_ok(qv[i][1], tag) && tag_ok(qv[i][3], tag);
-            if (__all(ok || !valid)) break;
-            if (!poll_backoff()) break;
-          }
-#pragma unroll
-          for (int j = 0; j < 4; j++) {
-            U32H2 e0, e1, e2, e3;
-            e0.u = valid ? qv[2 * j][0] : 0u;
-            e1.u = valid ? qv[2 * j][2] : 0u;
-            e2.u = valid ? qv[2 * j + 1][0] : 0u;
-            e3.u = valid ? qv[2 * j + 1][2] : 0u;
-            qa[j] = half8_t{e0.h[0], e0.h[1], e1.h[0], e1.h[1], e2.h[0], e2.h[1], e3.h[0], e3.h[1]};
-          }
-        }
-        float sc2[2];
-#pragma unroll
-        for (int pbk = 0; pbk < 2; pbk++) {
-          float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-          for (int j = 0; j < 4; j++) d = __builtin_amdgcn_mfma_f32_16x16x32_f16(qa[j], kf[pbk][j], d, 0, 0, 0);
-          const int p = p0 + pbk * 16 + r;  // lane (r, c): score of head c at position p
-          sc2[pbk] = (p < pos) ? d[0] * scale : -INFINITY;
-        }
-        float mx = fmaxf(sc2[0], sc2[1]);
-#pragma unroll
-        for (int off = 8; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
-        const float e0 = (sc2[0] == -INFINITY) ? 0.0f : __expf(sc2[0] - mx);
-        const float e1 = (sc2[1] == -INFINITY) ? 0.0f : __expf(sc2[1] - mx);
-        float sum = e0 + e1;
-#pragma unroll
-        for (int off = 8; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
-        m_h = mx;
-        l_h = sum;
-        _Float16 *pw = p_lds + (size_t)wave * 4 * 32;
-        pw[c * 32 + r] = (_Float16)e0;
-        pw[c * 32 + 16 + r] = (_Float16)e1;
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
-        half8_t pa = {0, 0, 0, 0, 0, 0, 0, 0};
-        if ((r & 3) == 0 && (r >> 2) < GROUP) pa = *reinterpret_cast<const half8_t *>(pw + (r >> 2) * 32 + 8 * c);
-#pragma unroll
-        for (int t = 0; t < 8; t++) {
-          half8_t vv = vf[t];
-          if (p0 + 8 * c >= pos) vv = hz;
-          else if (p0 + 8 * c + 8 > pos) {
-#pragma unroll
-            for (int e = 0; e < 8; e++)
-              if (p0 + 8 * c + e >= pos) vv[e] = (_Float16)0.0f;
-          }
-          float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
-          d = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vv, d, 0, 0, 0);
-          o_acc[t] = d[0];  // lane (r, c): o of head c at d = 16 t + r
-        }
-      }
-      if (wave < 4) {
-        if (r == 0) {
-          w_m[wave * 4 + c] = m_h;
-          w_l[wave * 4 + c] = l_h;
-        }
-#pragma unroll
-        for (int t = 0; t < 8; t++) w_o[((size_t)wave * 4 + c) * 128 + t * 16 + r] = o_acc[t];
-      }
-      lds_barrier();
-      if (wave < 4) {
-        for (int idx = tid; idx < GROUP * 128; idx += 256) {
-          const int hh = idx >> 7, dd = idx & 127;
-          float mx = -INFINITY;
-#pragma unroll
-          for (int w = 0; w < 4; w++) mx = fmaxf(mx, w_m[w * 4 + hh]);
-          float l = 0.0f, o = 0.0f;
-#pragma unroll
-          for (int w = 0; w < 4; w++) {
-            const float f = (w_m[w * 4 + hh] == -INFINITY) ? 0.0f : __expf(w_m[w * 4 + hh] - mx);
-            l += w_l[w * 4 + hh] * f;
-            o += w_o[((size_t)w * 4 + hh) * 128 + dd] * f;
-          }
-          u64 *dst = m.part + ((size_t)(kvh * GROUP + hh) * max_chunks + chunk) * PART_REC;
-          st_entry(dst + 2 + dd, __float_as_uint(o), tag);
-          if (dd == 0) {
-            st_entry(dst, __float_as_uint(mx), tag);
-            st_entry(dst + 1, __float_as_uint(l), tag);
-          }
-        }
-      }
-      lds_barrier();
-    }
-  };
-
-  // merge the chunk partials of one head with the new position; also appends k / v to the cache
-  auto attention_combine = [&](int layer, int head, int pos, uint32_t tag) {
-    const int nchunks = (pos + ACHUNK - 1) / ACHUNK;
-    const int kvh = head / GROUP;
-    float M = -INFINITY, Ls = 0.0f, O0 = 0.0f, O1 = 0.0f;
-    auto merge = [&](float mc, float lc, float o0, float o1) {
-      if (mc == -INFINITY) return;
-      const float Mn = fmaxf(M, mc);
-      const float a = (M == -INFINITY) ? 0.0f : __expf(M - Mn);
-      const float b = __expf(mc - Mn);
-      Ls = Ls * a + lc * b;
-      O0 = O0 * a + o0 * b;
-      O1 = O1 * a + o1 * b;
-      M = Mn;
-    };
-#pragma unroll 1
-    for (int ch = 0; ch < nchunks; ch++) {
-      const u64 *rec = m.part + ((size_t)head * max_chunks + ch) * PART_REC;
-      uint4_t a, b;
-      while (true) {
-        a = ld2(rec);
-        b = ld2(rec + 2 + 2 * lane);
-        wait_vm(a, b);
-        const bool ok = tag_ok(a[1], tag) && tag_ok(a[3], tag) && tag_ok(b[1], tag) && tag_ok(b[3], tag);
-        if (__all(ok)) break;
-        if (!poll_backoff()) break;
-      }
-      merge(__uint_as_float(a[0]), __uint_as_float(a[2]), __uint_as_float(b[0]), __uint_as_float(b[2]));
-    }
-    // the token of this step: q . k_new / sqrt(d) with k_new, v_new straight from the qkv exchange buffer
-    const u64 *qe = m.qkv + (size_t)head * 64 + lane;
-    const u64 *ke = m.qkv + (size_t)(HQ + kvh) * 64 + lane;
-    const u64 *ve = m.qkv + (size_t)(HQ + HKV + kvh) * 64 + lane;
-    u64 q, k, v;
-    while (true) {
-      q = __hip_atomic_load(qe, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      k = __hip_atomic_load(ke, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      v = __hip_atomic_load(ve, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const bool ok = tag_ok((uint32_t)(q >> 32), tag) && tag_ok((uint32_t)(k >> 32), tag) && tag_ok((uint32_t)(v >> 32), tag);
-      if (__all(ok)) break;
-      if (!poll_backoff()) break;
-    }
-    const uint32_t qw = (uint32_t)q, kw = (uint32_t)k, vw = (uint32_t)v;
-    const float s = wave_sum(h2_lo(qw) * h2_lo(kw) + h2_hi(qw) * h2_hi(kw)) * 0.08838834764831845f;
-    merge(s, 1.0f, h2_lo(vw), h2_hi(vw));
-    const float inv = Ls > 0.0f ? 1.0f / Ls : 0.0f;
-    st_entry(m.ao + xidx(head * 128 + 2 * lane, m.ph[PK_O].ks, m.ph[PK_O].frags), pack_h2(O0 * inv, O1 * inv), tag);
-    if (head == kvh * GROUP) {
-      // append: other workgroups read these lines in later steps of this launch -> agent-scope stores
-      _Float16 *kc = m.kc[layer];
-      _Float16 *vc = m.vc[layer];
-      uint32_t *krow = reinterpret_cast<uint32_t *>(kc + ((size_t)kvh * m.max_ctx + pos) * 128);
-      __hip_atomic_store(krow + lane, kw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      uint16_t *vslab = reinterpret_cast<uint16_t *>(vc + (((size_t)kvh * (m.max_ctx / 8) + pos / 8) * 128) * 8) + (pos & 7);
-      __hip_atomic_store(vslab + (size_t)(2 * lane) * 8, (uint16_t)(vw & 0xFFFFu), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(vslab + (size_t)(2 * lane + 1) * 8, (uint16_t)(vw >> 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  };
-
   // ---- the decode loop ---------------------------------------------------------------------------------
   if (tid == 0) tok_lds[0] = m.tokens[0];
-  lds_barrier();
+  cbar();
   int token = tok_lds[0];
   const float *gam = m.gammas;
 
@@ -604,7 +830,7 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
   for (int s = 0; s < n_steps; s++) {
     const int pos = pos0 + s;
     const uint32_t tag_base = (epoch0 + (uint32_t)s) * (uint32_t)(L + 2) + 1u;  // used modulo 2^24
-    spin_budget = spin_budget > 1 ? SPIN_LIMIT : 1;
+    ws.spin_budget = ws.spin_budget > 1 ? SPIN_LIMIT : 1;
     token = token < 0 ? 0 : (token >= m.vocab ? m.vocab - 1 : token);
     if (own) h = (float)m.emb[(size_t)token * D + own_row];
     publish_h(m.xn, gam, tag_base & 0xFFFFFFu);
@@ -612,6 +838,8 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
 #pragma unroll 1
     for (int l = 0; l < L; l++) {
       const uint32_t tag = (tag_base + (uint32_t)l) & 0xFFFFFFu;
+      dbg_layer = l;
+      mark(0);
       // ---- q/k/v projection + rotary embedding ------------------------------------------------------------
       {
         const int nb = nbw(PK_QKV);
@@ -624,7 +852,7 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
           const float inv_freq = 1.0f / powf(m.theta, (float)(2 * i) / 128.0f);
           sincosf(inv_freq * (float)pos, &sn, &cs);
         }
-        gemv(PK_QKV, m.xn, tag, true);
+        gemv(PK_QKV, m.xn, tag, true, 1);
         const float val = act ? row_sum(tid) : 0.0f;
         const float partner = __shfl_xor(val, 1, 64);
         const int which = pr & 1;
@@ -645,23 +873,37 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
           }
         }
         pb ^= 1;
+        mark(3);
       }
       // ---- attention -------------------------------------------------------------------------------------
-      attention_items(l, pos, tag);
-      if (wave == 4)
-        for (int head = wg; head < HQ; head += G) attention_combine(l, head, pos, tag);
+      {
+        AttnArgs aa;
+        aa.qkv = m.qkv; aa.part = m.part; aa.ao = m.ao;
+        aa.kc = m.kc[l]; aa.vc = m.vc[l];
+        aa.abort_flag = m.abort_flag;
+        aa.HQ = HQ; aa.HKV = HKV; aa.GROUP = GROUP; aa.max_ctx = m.max_ctx; aa.G = G; aa.pos = pos; aa.pos0 = pos0; aa.wg = wg;
+        aa.ks_o = m.ph[PK_O].ks; aa.frags_o = m.ph[PK_O].frags;
+        aa.tag = tag;
+        aa.att_off = (uint32_t)(size_t)att_lds;
+        aa.bar_off = (uint32_t)(size_t)(lds + RING_BYTES + PART_BYTES + ATT_BYTES) + 64;
+        ws = attn_items(aa, ws);
+        mark(4);
+        if (wave == 0)
+          for (int head = G - 1 - wg; head < HQ; head += G) ws = attn_combine(aa, ws, head);
+      }
       // ---- output projection + residual ------------------------------------------------------------------
       {
-        gemv(PK_O, m.ao, tag, false);
+        gemv(PK_O, m.ao, tag, false, 5);
         if (own) h += row_sum(tid);
         if (own && m.dbg_h) m.dbg_h[((size_t)l * 2) * D + own_row] = h;
         publish_h(m.xn2, gam + (size_t)(2 * l + 1) * D, tag);
         pb ^= 1;
+        mark(7);
       }
       // ---- gate / up projection + SwiGLU (rows interleaved: 2i = gate_i, 2i+1 = up_i) ---------------------
       {
         const int nb = nbw(PK_GU);
-        gemv(PK_GU, m.xn2, tag, true);
+        gemv(PK_GU, m.xn2, tag, true, 8);
         const bool act = tid < 8 * nb;
         const int pr = 8 * (wg + G * (tid >> 3)) + (tid & 7);
         const float val = act ? row_sum(tid) : 0.0f;
@@ -670,21 +912,23 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
         const float a2 = __shfl_down(a, 2, 64);    // act value of the next pair of rows
         if (act && !(tid & 3)) st_entry(m.act + xidx(pr / 2, m.ph[PK_DOWN].ks, m.ph[PK_DOWN].frags), pack_h2(a, a2), tag);
         pb ^= 1;
+        mark(10);
       }
       // ---- down projection + residual; publishes the input of the next layer (or of lm_head) ---------------
       {
-        gemv(PK_DOWN, m.act, tag, false);
+        gemv(PK_DOWN, m.act, tag, false, 11);
         if (own) h += row_sum(tid);
         if (own && m.dbg_h) m.dbg_h[((size_t)l * 2 + 1) * D + own_row] = h;
         publish_h(m.xn, gam + (size_t)(l + 1 < L ? 2 * (l + 1) : 2 * L) * D, (tag + 1) & 0xFFFFFFu);
         pb ^= 1;
+        mark(13);
       }
     }
     // ---- lm_head + greedy pick -----------------------------------------------------------------------------
     {
       const uint32_t tag = (tag_base + (uint32_t)L) & 0xFFFFFFu;
       const int nb = nbw(PK_LM);
-      gemv(PK_LM, m.xn, tag, true);
+      gemv(PK_LM, m.xn, tag, true, 14);
       const bool act = tid < 8 * nb;
       const int row = 8 * (wg + G * (tid >> 3)) + (tid & 7);
       float best = 0.0f;
@@ -708,10 +952,10 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
         arg_v[wave] = best;
         arg_i[wave] = bi;
       }
-      lds_barrier();
+      cbar();
       if (wave == 0) {
         if (lane == 0 && nb > 0) {
-          for (int w = 1; w < PS_WAVES; w++)
+          for (int w = 1; w < CW; w++)
             if (better(arg_v[w], arg_i[w], best, bi)) {
               best = arg_v[w];
               bi = arg_i[w];
@@ -731,7 +975,7 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
             wait_vm(e);
             const bool ok = w >= cnt || (tag_ok(e[1], tag) && tag_ok(e[3], tag));
             if (__all(ok)) break;
-            if (!poll_backoff()) break;
+            if (!poll_backoff_ws(ws, m.abort_flag)) break;
           }
           if (w < cnt && better(__uint_as_float(e[0]), (int)e[2], gv, gi)) {
             gv = __uint_as_float(e[0]);
@@ -755,7 +999,7 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
           }
         }
       }
-      lds_barrier();
+      cbar();
       token = tok_lds[0];
     }
   }
@@ -850,10 +1094,10 @@ bool persist_supported(const yscv_hip_decoder_config &c, int num_cus, const char
   if (!why) why = &dummy;
   const int G = num_cus;
   const int hq = c.n_heads * c.head_dim;
-  auto bad_k = [](int k) { return k % 2048 != 0 || k > 16384 || k <= 0; };
+  auto bad_k = [](int k) { return k % (256 * PS_WAVES) != 0 || k > PS_WAVES * 512 * MAXF || k <= 0; };
   if (c.head_dim != 128) { *why = "head_dim must be 128"; return false; }
   if (c.group_size != 32) { *why = "group size must be 32"; return false; }
-  if (bad_k(c.d_model) || bad_k(hq) || bad_k(c.d_ff)) { *why = "d_model, n_heads*128 and d_ff must be multiples of 2048, at most 16384"; return false; }
+  if (bad_k(c.d_model) || bad_k(hq) || bad_k(c.d_ff)) { *why = "d_model, n_heads*128 and d_ff must be multiples of 1024, at most 16384"; return false; }
   if (c.vocab % 8 != 0) { *why = "vocab must be a multiple of 8"; return false; }
   if (c.n_heads % c.n_kv_heads != 0 || c.n_heads / c.n_kv_heads > 4) { *why = "1..4 query heads per kv head"; return false; }
   if (G < 16 || G > 1024) { *why = "unsupported CU count"; return false; }
@@ -886,7 +1130,7 @@ void persist_fill_phases(const yscv_hip_decoder_config &c, int G, PersistModel *
     PersistPhase &p = m->ph[i];
     p.n = n[i];
     p.k = k[i];
-    p.ks = k[i] / 8;
+    p.ks = k[i] / PS_WAVES;
     p.tiles = p.ks / 256;
     p.pairs = (p.tiles + 1) / 2;
     p.frags = p.pairs;
@@ -901,7 +1145,7 @@ size_t persist_seq_offset(const PersistModel &m, int w, int layer, int kind) { r
 int32_t launch_persist_pack(const PersistModel &m, int layer, int kind, const uint8_t *packed_dev,
                             const _Float16 *scales_dev, uint8_t *stream, hipStream_t s) {
   if (kind < 0 || kind >= PK_COUNT) return set_error(YSCV_HIP_ERR_INVALID_ARG, "bad projection kind %d", kind);
-  hipLaunchKernelGGL(persist_pack_kernel, dim3(m.ph[kind].nb, PS_WAVES), dim3(256), 0, s, m, layer, kind, packed_dev,
+  hipLaunchKernelGGL(persist_pack_kernel, dim3(m.ph[kind].nb, CW), dim3(256), 0, s, m, layer, kind, packed_dev,
                      scales_dev, stream);
   YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
@@ -918,11 +1162,11 @@ int32_t launch_persist_decode(const PersistModel &m, int n_steps, int pos0, int 
   if (attr_err != hipSuccess)
     return set_error(YSCV_HIP_ERR_DEVICE, "cannot reserve %d bytes of LDS: %s", PERSIST_LDS, hipGetErrorString(attr_err));
   int max_blocks = 0;
-  YSCV_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&max_blocks, decode_persistent_kernel, 512, PERSIST_LDS));
+  YSCV_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&max_blocks, decode_persistent_kernel, THREADS, PERSIST_LDS));
   if (max_blocks < 1) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the persistent decode kernel does not fit a CU");
   PersistModel mm = m;
   void *args[] = {&mm, &n_steps, &pos0, &step0, &max_steps, &epoch0};
-  YSCV_HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<const void *>(decode_persistent_kernel), dim3(m.G), dim3(512),
+  YSCV_HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<const void *>(decode_persistent_kernel), dim3(m.G), dim3(THREADS),
                                           args, PERSIST_LDS, s));
   return YSCV_HIP_OK;
 }

@@ -245,6 +245,8 @@ static int32_t persist_setup(yscv_hip_decoder *d) {
   m.history = d->history;
   m.abort_flag = d->p_abort;
   m.dbg_h = nullptr;
+  m.dbg_t = nullptr;
+  if (getenv("YSCV_DBG_T")) { (void)hipMalloc(reinterpret_cast<void **>(&m.dbg_t), (size_t)G * c.n_layers * 16 * 8); (void)hipMemset(m.dbg_t, 0, (size_t)G * c.n_layers * 16 * 8); }
   if (getenv("YSCV_DBG_H")) { (void)hipMalloc(reinterpret_cast<void **>(&m.dbg_h), (size_t)c.n_layers * 2 * D * 4); }
   d->persist_ok = true;
   return YSCV_HIP_OK;
@@ -716,6 +718,12 @@ int32_t yscv_hip_decoder_read_logits(yscv_hip_decoder *d, float *out_host) {
   return YSCV_HIP_OK;
 }
 
+__attribute__((visibility("default"))) int32_t yscv_hip_decoder_dbg_t(yscv_hip_decoder *d, unsigned long long *out) {
+  if (!d->pm.dbg_t) return -1;
+  (void)hipDeviceSynchronize();
+  (void)hipMemcpy(out, d->pm.dbg_t, (size_t)d->pm.G * d->cfg.n_layers * 16 * 8, hipMemcpyDeviceToHost);
+  return 0;
+}
 __attribute__((visibility("default"))) int32_t yscv_hip_decoder_dbg_h(yscv_hip_decoder *d, float *out) {
   if (!d->pm.dbg_h) return -1;
   (void)hipDeviceSynchronize();

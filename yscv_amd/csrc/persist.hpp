@@ -3,8 +3,8 @@
 //
 // Weight stream
 // -------------
-// The persistent kernel runs G workgroups of 8 wavefronts, one workgroup per CU.  For a projection
-// W[n][k] (k a multiple of 2048) wave v of every workgroup owns the k range [v*k/8, (v+1)*k/8), and
+// The persistent kernel runs G workgroups, one per CU, each with PS_WAVES compute wavefronts.  For a projection
+// W[n][k] (k a multiple of 1024) compute wave v of every workgroup owns the k range [v*k/4, (v+1)*k/4), and
 // workgroup w owns the 8-row blocks w, w+G, w+2G, ...  A tile is 8 rows x 256 k = 1 KiB: lane
 // L = 16*c + r of a wavefront holds four 32-bit words, word j = the eight weights
 //     W[8*blk + (r & 7)][k0 + 32*(j + 4*(r >> 3)) + 8*c + 0..7]
@@ -14,7 +14,7 @@
 // tile t and lane-row r, four fp16 values at byte t*128 + r*8: the scales of row (r & 7), groups
 // (k0 + 256*t)/32 + j + 4*(r >> 3), j = 0..3.
 // Every wave has one contiguous stream holding its records in the order the kernel consumes them:
-// layer 0 {qkv, o, gate/up, down}, layer 1 ..., lm_head; the streams of the 8 waves of workgroup w
+// layer 0 {qkv, o, gate/up, down}, layer 1 ..., lm_head; the streams of the compute waves of workgroup w
 // sit back to back at wg_off[w].
 #pragma once
 
@@ -24,7 +24,7 @@
 
 namespace yscv {
 
-constexpr int PS_WAVES = 8;
+constexpr int PS_WAVES = 4;   // compute waves per workgroup = k slices of every projection
 constexpr int PS_REC_FULL = 2304;
 constexpr int PS_REC_SINGLE = 1280;
 enum : int { PK_QKV = 0, PK_O = 1, PK_GU = 2, PK_DOWN = 3, PK_LM = 4, PK_COUNT = 5 };
@@ -32,7 +32,7 @@ enum : int { PK_QKV = 0, PK_O = 1, PK_GU = 2, PK_DOWN = 3, PK_LM = 4, PK_COUNT =
 struct PersistPhase {
   int n;       // output rows
   int k;       // input channels
-  int ks;      // k per wave = k / 8
+  int ks;      // k per wave = k / PS_WAVES
   int tiles;   // 256-k tiles per wave and block = ks / 256
   int pairs;   // records per wave and block = ceil(tiles / 2)
   int frags;   // 512-k A fragments per wave = pairs
@@ -66,14 +66,15 @@ struct PersistModel {
   int32_t *tokens;              // [1] current token (in: first token; out: last pick)
   int32_t *history;             // [max_steps]
   uint32_t *abort_flag;         // set when a bounded wait gave up
+  unsigned long long *dbg_t;    // debug: [G][n_layers][16] timestamps of wave 0
   float *dbg_h;                 // debug: [n_layers][2][d_model] residual after o-proj / down
 };
 
 // entries an exchange vector of k values occupies (padded to whole 512-k fragments per wave)
 __host__ __device__ inline size_t persist_vec_entries(int k) {
-  const int ks = k / 8;
+  const int ks = k / PS_WAVES;
   const int frags = (ks + 511) / 512;
-  return (size_t)8 * frags * 256;
+  return (size_t)PS_WAVES * frags * 256;
 }
 
 // true when the shape can run on the persistent path
