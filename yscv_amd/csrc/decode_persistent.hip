@@ -39,6 +39,9 @@ typedef unsigned long long u64;
 #ifndef DBG_WAIT_ALL
 #define DBG_WAIT_ALL 0
 #endif
+#ifndef INFLIGHT_CAP
+#define INFLIGHT_CAP 20
+#endif
 #ifndef GEMV_INL
 #define GEMV_INL __noinline__
 #endif
@@ -47,7 +50,7 @@ typedef unsigned long long u64;
 #endif
 
 constexpr int CW = PS_WAVES;                   // compute waves per workgroup (waves 0 .. CW-1)
-constexpr int PW = 2;                          // producer waves (waves CW .. CW+PW-1), each feeds CW/PW compute waves
+constexpr int PW = 4;                          // producer waves (waves CW .. CW+PW-1), each feeds CW/PW compute waves
 constexpr int THREADS = 64 * (CW + PW);
 constexpr int RING = 14;                       // ring slots (records) per compute wave
 constexpr int SLOT = PS_REC_FULL;              // LDS bytes per ring slot
@@ -71,7 +74,7 @@ __device__ __forceinline__ void st_entry(u64 *p, uint32_t payload, uint32_t tag)
 // coherent 128-bit load (two entries); the result is valid only after wait_vm
 __device__ __forceinline__ uint4_t ld2(const void *p) {
   uint4_t v;
-  asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
+  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
   return v;
 }
 __device__ __forceinline__ void wait_vm(uint4_t &a) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(a)::"memory"); }
@@ -194,6 +197,7 @@ struct AttnArgs {
   int ks_o, frags_o;       // k slice / fragments of the output projection (layout of `ao`)
   uint32_t tag;
   uint32_t att_off, bar_off;  // LDS byte offsets: attention scratch, barrier counter
+  unsigned long long *dbg_t;  // null or timestamp slots
 };
 
 // Attention of the new token over the cached positions [0, pos): one work item = (kv head, 128 positions),
@@ -213,6 +217,7 @@ __device__ ATTN_INL WaitState attn_items(AttnArgs a, WaitState ws) {
   const int max_chunks = a.max_ctx / ACHUNK;
   const uint32_t tag = a.tag;
   const float scale = 0.08838834764831845f;  // 1 / sqrt(128)
+  if (a.dbg_t && tid == 0) a.dbg_t[14] = wall_clock64();
 #pragma unroll 1
   for (int id = a.wg; id < items; id += a.G) {
     const int chunk = id / HKV, kvh = id - chunk * HKV;
@@ -272,6 +277,7 @@ __device__ ATTN_INL WaitState attn_items(AttnArgs a, WaitState ws) {
           if (__all(ok || !valid)) break;
           if (!poll_backoff_ws(ws, a.abort_flag)) break;
         }
+        if (a.dbg_t && tid == 0) a.dbg_t[15] = wall_clock64();
 #pragma unroll
         for (int j = 0; j < 4; j++) {
           U32H2 e0, e1, e2, e3;
@@ -360,13 +366,18 @@ __device__ ATTN_INL WaitState attn_items(AttnArgs a, WaitState ws) {
 
 // Merge the chunk partials of one head with the token of this step (its k / v come straight from the qkv
 // exchange buffer), publish the head's output, and append k / v to the cache (first head of each group).
+// All compute waves of the workgroup take part: wave w merges chunks w, w + CW, ... (one round trip for up
+// to five of them), the last wave also takes the token of this step, and wave 0 merges the CW states.
 __device__ ATTN_INL WaitState attn_combine(AttnArgs a, WaitState ws, int head) {
   const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int pos = a.pos;
   const uint32_t tag = a.tag;
   const int nchunks = (pos + ACHUNK - 1) / ACHUNK;
   const int max_chunks = a.max_ctx / ACHUNK;
   const int kvh = head / a.GROUP;
+  lds_f32 *cst = (lds_f32 *)(uintptr_t)(a.att_off + 1024 + 128);  // [CW][4][64] merge states (the w_o area)
+  lds_u32 *bar = (lds_u32 *)(uintptr_t)a.bar_off;
   float M = -INFINITY, Ls = 0.0f, O0 = 0.0f, O1 = 0.0f;
   auto merge = [&](float mc, float lc, float o0, float o1) {
     if (mc == -INFINITY) return;
@@ -379,54 +390,75 @@ __device__ ATTN_INL WaitState attn_combine(AttnArgs a, WaitState ws, int head) {
     M = Mn;
   };
 #pragma unroll 1
-  for (int ch0 = 0; ch0 < nchunks; ch0 += 4) {  // four chunks per round trip
-    uint4_t v[8];
+  for (int c0 = wave; c0 < nchunks; c0 += 5 * CW) {
+    uint4_t v[10];
     while (true) {
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const int ch = ch0 + i < nchunks ? ch0 + i : nchunks - 1;
+      for (int i = 0; i < 5; i++) {
+        const int ch = c0 + i * CW < nchunks ? c0 + i * CW : c0;
         const u64 *rec = a.part + ((size_t)head * max_chunks + ch) * PART_REC;
         v[2 * i] = ld2(rec);
         v[2 * i + 1] = ld2(rec + 2 + 2 * lane);
       }
-      wait_vm8(v);
+      asm volatile("s_waitcnt vmcnt(0)"
+                   : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]), "+v"(v[8]),
+                     "+v"(v[9])::"memory");
       bool ok = true;
 #pragma unroll
-      for (int i = 0; i < 8; i++) ok = ok && tag_ok(v[i][1], tag) && tag_ok(v[i][3], tag);
+      for (int i = 0; i < 10; i++) ok = ok && tag_ok(v[i][1], tag) && tag_ok(v[i][3], tag);
       if (__all(ok)) break;
       if (!poll_backoff_ws(ws, a.abort_flag)) break;
     }
 #pragma unroll
-    for (int i = 0; i < 4; i++)
-      if (ch0 + i < nchunks)
+    for (int i = 0; i < 5; i++)
+      if (c0 + i * CW < nchunks)
         merge(__uint_as_float(v[2 * i][0]), __uint_as_float(v[2 * i][2]), __uint_as_float(v[2 * i + 1][0]),
               __uint_as_float(v[2 * i + 1][2]));
   }
-  const u64 *qe = a.qkv + (size_t)head * 64 + lane;
-  const u64 *ke = a.qkv + (size_t)(a.HQ + kvh) * 64 + lane;
-  const u64 *ve = a.qkv + (size_t)(a.HQ + a.HKV + kvh) * 64 + lane;
-  u64 q, k, v;
-  while (true) {
-    q = __hip_atomic_load(qe, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    k = __hip_atomic_load(ke, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    v = __hip_atomic_load(ve, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const bool ok = tag_ok((uint32_t)(q >> 32), tag) && tag_ok((uint32_t)(k >> 32), tag) && tag_ok((uint32_t)(v >> 32), tag);
-    if (__all(ok)) break;
-    if (!poll_backoff_ws(ws, a.abort_flag)) break;
+  uint32_t kw = 0, vw = 0;
+  if (wave == CW - 1) {
+    const u64 *qe = a.qkv + (size_t)head * 64 + lane;
+    const u64 *ke = a.qkv + (size_t)(a.HQ + kvh) * 64 + lane;
+    const u64 *ve = a.qkv + (size_t)(a.HQ + a.HKV + kvh) * 64 + lane;
+    u64 q, k, v;
+    while (true) {
+      q = __hip_atomic_load(qe, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      k = __hip_atomic_load(ke, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      v = __hip_atomic_load(ve, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool ok = tag_ok((uint32_t)(q >> 32), tag) && tag_ok((uint32_t)(k >> 32), tag) && tag_ok((uint32_t)(v >> 32), tag);
+      if (__all(ok)) break;
+      if (!poll_backoff_ws(ws, a.abort_flag)) break;
+    }
+    const uint32_t qw = (uint32_t)q;
+    kw = (uint32_t)k;
+    vw = (uint32_t)v;
+    const float s = wave_sum(h2_lo(qw) * h2_lo(kw) + h2_hi(qw) * h2_hi(kw)) * 0.08838834764831845f;
+    merge(s, 1.0f, h2_lo(vw), h2_hi(vw));
+    if (head == kvh * a.GROUP) {
+      // append: other workgroups read these lines in later steps of this launch -> agent-scope stores
+      uint32_t *krow = reinterpret_cast<uint32_t *>(a.kc + ((size_t)kvh * a.max_ctx + pos) * 128);
+      __hip_atomic_store(krow + lane, kw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      uint16_t *vslab = reinterpret_cast<uint16_t *>(a.vc + (((size_t)kvh * (a.max_ctx / 8) + pos / 8) * 128) * 8) + (pos & 7);
+      __hip_atomic_store(vslab + (size_t)(2 * lane) * 8, (uint16_t)(vw & 0xFFFFu), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(vslab + (size_t)(2 * lane + 1) * 8, (uint16_t)(vw >> 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
   }
-  const uint32_t qw = (uint32_t)q, kw = (uint32_t)k, vw = (uint32_t)v;
-  const float s = wave_sum(h2_lo(qw) * h2_lo(kw) + h2_hi(qw) * h2_hi(kw)) * 0.08838834764831845f;
-  merge(s, 1.0f, h2_lo(vw), h2_hi(vw));
-  const float inv = Ls > 0.0f ? 1.0f / Ls : 0.0f;
-  st_entry(a.ao + xidx(head * 128 + 2 * lane, a.ks_o, a.frags_o), pack_h2(O0 * inv, O1 * inv), tag);
-  if (head == kvh * a.GROUP) {
-    // append: other workgroups read these lines in later steps of this launch -> agent-scope stores
-    uint32_t *krow = reinterpret_cast<uint32_t *>(a.kc + ((size_t)kvh * a.max_ctx + pos) * 128);
-    __hip_atomic_store(krow + lane, kw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    uint16_t *vslab = reinterpret_cast<uint16_t *>(a.vc + (((size_t)kvh * (a.max_ctx / 8) + pos / 8) * 128) * 8) + (pos & 7);
-    __hip_atomic_store(vslab + (size_t)(2 * lane) * 8, (uint16_t)(vw & 0xFFFFu), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(vslab + (size_t)(2 * lane + 1) * 8, (uint16_t)(vw >> 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  lds_f32 *mine = cst + (size_t)wave * 256;
+  mine[lane] = M;
+  mine[64 + lane] = Ls;
+  mine[128 + lane] = O0;
+  mine[192 + lane] = O1;
+  compute_barrier(ws, bar, CW);
+  if (wave == 0) {
+#pragma unroll
+    for (int w = 1; w < CW; w++) {
+      const lds_f32 *o = cst + (size_t)w * 256;
+      merge(o[lane], o[64 + lane], o[128 + lane], o[192 + lane]);
+    }
+    const float inv = Ls > 0.0f ? 1.0f / Ls : 0.0f;
+    st_entry(a.ao + xidx(head * 128 + 2 * lane, a.ks_o, a.frags_o), pack_h2(O0 * inv, O1 * inv), tag);
   }
+  compute_barrier(ws, bar, CW);  // the merge states are reused by the next head / the next attention item
   return ws;
 }
 
@@ -478,62 +510,81 @@ __device__ GEMV_INL GemvState gemv_stage(GemvArgs a, GemvState st) {
   const half8_t bc = {(_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f,
                       (_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f};
   const bool normed = a.ss != nullptr;
+  unsigned dbg_polls = 0;
   // ---- activation fragments (A operand: row i = k-block i of the fragment) ------------------------------
   // A `normed` vector holds fp16(h * gamma * 2^-e) with the exponent e of each 8-row block in the top byte
   // of its tag words; the operand is then fp16(h * gamma / rms), the activation RMSNorm feeds
   // (crates/yscv-kernels/src/ops/norm.rs:1497-1518); 1/rms comes from the sum-of-squares entries.
+  {
+    uint4_t qa[MAXF], qb[MAXF], sa, sb;
+    const bool v0 = normed && 4 * lane < a.ss_count, v1 = normed && 4 * lane + 1 < a.ss_count,
+               v2 = normed && 4 * lane + 2 < a.ss_count, v3 = normed && 4 * lane + 3 < a.ss_count;
+    const u64 *sp = normed ? a.ss + 4 * lane : a.in_buf;
+    const u64 *p0 = a.in_buf + (((size_t)wave * a.frags) << 8) + 2 * lane;
+    if (a.nb > 0) {
+      while (true) {  // one round trip for all fragments and the sum-of-squares entries
 #pragma unroll
-  for (int f = 0; f < MAXF; f++) {
-    if (f < a.frags && a.nb > 0) {
-      const u64 *p = a.in_buf + (((size_t)wave * a.frags + f) << 8) + 2 * lane;
-      const bool valid = (512 * f + 32 * r) < a.ks;
-      const bool with_ss = normed && f == 0;
-      const bool v0 = with_ss && 4 * lane < a.ss_count, v1 = with_ss && 4 * lane + 1 < a.ss_count,
-                 v2 = with_ss && 4 * lane + 2 < a.ss_count, v3 = with_ss && 4 * lane + 3 < a.ss_count;
-      const u64 *sp = with_ss ? a.ss + 4 * lane : a.in_buf;
-      uint4_t qa, qb, sa, sb;
-      while (true) {
-        qa = ld2(p);
-        qb = ld2(p + 128);
+        for (int f = 0; f < MAXF; f++) {
+          if (f < a.frags) {  // wave-uniform
+            qa[f] = ld2(p0 + ((size_t)f << 8));
+            qb[f] = ld2(p0 + ((size_t)f << 8) + 128);
+          }
+        }
         sa = ld2(sp);
         sb = ld2(sp + 2);
-        wait_vm(qa, qb, sa, sb);
-        bool ok = !valid || (tag_ok(qa[1], tag) && tag_ok(qa[3], tag) && tag_ok(qb[1], tag) && tag_ok(qb[3], tag));
-        ok = ok && (!v0 || tag_ok(sa[1], tag)) && (!v1 || tag_ok(sa[3], tag)) && (!v2 || tag_ok(sb[1], tag)) &&
-             (!v3 || tag_ok(sb[3], tag));
+        asm volatile("s_waitcnt vmcnt(0)"
+                     : "+v"(qa[0]), "+v"(qa[1]), "+v"(qa[2]), "+v"(qa[3]), "+v"(qa[4]), "+v"(qa[5]), "+v"(qa[6]), "+v"(qa[7]),
+                       "+v"(qb[0]), "+v"(qb[1]), "+v"(qb[2]), "+v"(qb[3]), "+v"(qb[4]), "+v"(qb[5]), "+v"(qb[6]), "+v"(qb[7]),
+                       "+v"(sa), "+v"(sb)::"memory");
+        dbg_polls++;
+        bool ok = (!v0 || tag_ok(sa[1], tag)) && (!v1 || tag_ok(sa[3], tag)) && (!v2 || tag_ok(sb[1], tag)) &&
+                  (!v3 || tag_ok(sb[3], tag));
+#pragma unroll
+        for (int f = 0; f < MAXF; f++) {
+          const bool valid = f < a.frags && (512 * f + 32 * r) < a.ks;
+          ok = ok && (!valid || (tag_ok(qa[f][1], tag) && tag_ok(qa[f][3], tag) && tag_ok(qb[f][1], tag) && tag_ok(qb[f][3], tag)));
+        }
         if (__all(ok)) break;
         if (!poll_backoff_ws(st.ws, a.abort_flag)) break;
       }
-      if (with_ss) {
-        const float sq = (v0 ? __uint_as_float(sa[0]) : 0.0f) + (v1 ? __uint_as_float(sa[2]) : 0.0f) +
-                         (v2 ? __uint_as_float(sb[0]) : 0.0f) + (v3 ? __uint_as_float(sb[2]) : 0.0f);
-        rstd = 1.0f / sqrtf(wave_sum(sq) / (float)a.d_model + a.eps);
+    }
+    if (normed) {
+      const float sq = (v0 ? __uint_as_float(sa[0]) : 0.0f) + (v1 ? __uint_as_float(sa[2]) : 0.0f) +
+                       (v2 ? __uint_as_float(sb[0]) : 0.0f) + (v3 ? __uint_as_float(sb[2]) : 0.0f);
+      rstd = 1.0f / sqrtf(wave_sum(sq) / (float)a.d_model + a.eps);
+    }
+#pragma unroll
+    for (int f = 0; f < MAXF; f++) {
+      if (f < a.frags && a.nb > 0) {
+        const bool valid = (512 * f + 32 * r) < a.ks;
+        U32H2 u0, u1, u2, u3;
+        u0.u = valid ? qa[f][0] : 0u;
+        u1.u = valid ? qa[f][2] : 0u;
+        u2.u = valid ? qb[f][0] : 0u;
+        u3.u = valid ? qb[f][2] : 0u;
+        if (normed) {
+          const float fac = valid ? ldexpf(rstd, (int)(qa[f][1] >> 24) - 128) : 0.0f;
+          u0.h = half2_t{(_Float16)((float)u0.h[0] * fac), (_Float16)((float)u0.h[1] * fac)};
+          u1.h = half2_t{(_Float16)((float)u1.h[0] * fac), (_Float16)((float)u1.h[1] * fac)};
+          u2.h = half2_t{(_Float16)((float)u2.h[0] * fac), (_Float16)((float)u2.h[1] * fac)};
+          u3.h = half2_t{(_Float16)((float)u3.h[0] * fac), (_Float16)((float)u3.h[1] * fac)};
+        }
+        // the slots that meet 1024 + 16 q carry x / 16 (exact: a power of two)
+        const half2_t sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+        u1.h = u1.h * sixteenth;
+        u3.h = u3.h * sixteenth;
+        xa[f] = half8_t{u0.h[0], u0.h[1], u1.h[0], u1.h[1], u2.h[0], u2.h[1], u3.h[0], u3.h[1]};
+        const float4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+        z[f] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[f], bc, zero, 0, 0, 0);  // offset term of every k-block
+      } else {
+        xa[f] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        z[f] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
       }
-      U32H2 u0, u1, u2, u3;
-      u0.u = valid ? qa[0] : 0u;
-      u1.u = valid ? qa[2] : 0u;
-      u2.u = valid ? qb[0] : 0u;
-      u3.u = valid ? qb[2] : 0u;
-      if (normed) {
-        const float fac = valid ? ldexpf(rstd, (int)(qa[1] >> 24) - 128) : 0.0f;
-        u0.h = half2_t{(_Float16)((float)u0.h[0] * fac), (_Float16)((float)u0.h[1] * fac)};
-        u1.h = half2_t{(_Float16)((float)u1.h[0] * fac), (_Float16)((float)u1.h[1] * fac)};
-        u2.h = half2_t{(_Float16)((float)u2.h[0] * fac), (_Float16)((float)u2.h[1] * fac)};
-        u3.h = half2_t{(_Float16)((float)u3.h[0] * fac), (_Float16)((float)u3.h[1] * fac)};
-      }
-      // the slots that meet 1024 + 16 q carry x / 16 (exact: a power of two)
-      const half2_t sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
-      u1.h = u1.h * sixteenth;
-      u3.h = u3.h * sixteenth;
-      xa[f] = half8_t{u0.h[0], u0.h[1], u1.h[0], u1.h[1], u2.h[0], u2.h[1], u3.h[0], u3.h[1]};
-      const float4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
-      z[f] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[f], bc, zero, 0, 0, 0);  // offset term of every k-block
-    } else {
-      xa[f] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      z[f] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
     }
   }
-  if (a.dbg_t && threadIdx.x == 0) a.dbg_t[0] = wall_clock64();
+  if (a.dbg_t && threadIdx.x == 0) {
+    a.dbg_t[0] = wall_clock64();
+  }
 
   // ---- one record: 8 rows x 512 k against fragment xa ------------------------------------------------------
   unsigned crec = st.crec;
@@ -701,7 +752,7 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
 #pragma unroll
         for (int j = 0; j < SERVED; j++) {
           const int w = p * SERVED + j;
-          if (issued[j] < total && n_issued - n_retired < 20 &&
+          if (issued[j] < total && n_issued - n_retired < INFLIGHT_CAP &&
               issued[j] - lds_peek(sync_lds + 4 * (8 + w)) < RING) {
             while (kv(nb_k, kind[j]) == 0) {  // kinds this workgroup has no rows of
               if (kind[j] == PK_DOWN) { layer[j]++; kind[j] = layer[j] == L ? PK_LM : PK_QKV; }
@@ -802,9 +853,9 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
   float h = 0.0f;
   // publish fp16(h * gamma * 2^-e) pairs (fragment order of a k = d_model consumer; e = exponent of the largest
   // value of the 8-row block, carried in the top byte of the tag word) + this workgroup's sum of squares
-  auto publish_h = [&](u64 *buf, const float *gamma, uint32_t tag) {
+  auto publish_h = [&](u64 *buf, float gamma, uint32_t tag) {
     if (tid < 64) {
-      const float xs = own ? h * gamma[own_row] : 0.0f;
+      const float xs = own ? h * gamma : 0.0f;
       float mx = fabsf(xs);
       mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
@@ -833,7 +884,7 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
     ws.spin_budget = ws.spin_budget > 1 ? SPIN_LIMIT : 1;
     token = token < 0 ? 0 : (token >= m.vocab ? m.vocab - 1 : token);
     if (own) h = (float)m.emb[(size_t)token * D + own_row];
-    publish_h(m.xn, gam, tag_base & 0xFFFFFFu);
+    publish_h(m.xn, own ? gam[own_row] : 0.0f, tag_base & 0xFFFFFFu);
 
 #pragma unroll 1
     for (int l = 0; l < L; l++) {
@@ -886,17 +937,18 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
         aa.tag = tag;
         aa.att_off = (uint32_t)(size_t)att_lds;
         aa.bar_off = (uint32_t)(size_t)(lds + RING_BYTES + PART_BYTES + ATT_BYTES) + 64;
+        aa.dbg_t = m.dbg_t ? m.dbg_t + ((size_t)wg * L + l) * 16 : nullptr;
         ws = attn_items(aa, ws);
         mark(4);
-        if (wave == 0)
-          for (int head = G - 1 - wg; head < HQ; head += G) ws = attn_combine(aa, ws, head);
+        for (int head = G - 1 - wg; head < HQ; head += G) ws = attn_combine(aa, ws, head);
       }
       // ---- output projection + residual ------------------------------------------------------------------
       {
+        const float g_next = own ? gam[(size_t)(2 * l + 1) * D + own_row] : 0.0f;  // in flight during the stage
         gemv(PK_O, m.ao, tag, false, 5);
         if (own) h += row_sum(tid);
         if (own && m.dbg_h) m.dbg_h[((size_t)l * 2) * D + own_row] = h;
-        publish_h(m.xn2, gam + (size_t)(2 * l + 1) * D, tag);
+        publish_h(m.xn2, g_next, tag);
         pb ^= 1;
         mark(7);
       }
@@ -916,10 +968,11 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
       }
       // ---- down projection + residual; publishes the input of the next layer (or of lm_head) ---------------
       {
+        const float g_next = own ? gam[(size_t)(l + 1 < L ? 2 * (l + 1) : 2 * L) * D + own_row] : 0.0f;
         gemv(PK_DOWN, m.act, tag, false, 11);
         if (own) h += row_sum(tid);
         if (own && m.dbg_h) m.dbg_h[((size_t)l * 2 + 1) * D + own_row] = h;
-        publish_h(m.xn, gam + (size_t)(l + 1 < L ? 2 * (l + 1) : 2 * L) * D, (tag + 1) & 0xFFFFFFu);
+        publish_h(m.xn, g_next, (tag + 1) & 0xFFFFFFu);
         pb ^= 1;
         mark(13);
       }
