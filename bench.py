@@ -8,9 +8,11 @@ One "step" = one decode step of the whole batch.  Weights are random-initialised
 inputs are synthetic, everything is resident in HBM before the timed region.
 
 The single JSON line also carries
-  roofline      -- the dominant kernel (the skinny int4 GEMV that runs every projection) against the
-                   8 TB/s HBM peak: algorithmic bytes per launch / its average launch duration, the
-                   latter measured here with HIP events around the projections of whole decode steps;
+  roofline      -- the dominant kernel against the 8 TB/s HBM peak.  At batch 1 that is the single-launch
+                   decode kernel (one cooperative launch runs all timed steps): algorithmic bytes per launch
+                   (per step: packed weights + scales once, plus the KV cache rows read) / the launch duration
+                   measured with HIP events on the launch stream.  With --graph-path or batch > 1 it is the
+                   skinny int4 GEMV of the multi-kernel path, timed around the projections of whole steps;
   cpu_baseline  -- the restated reference CPU kernels timed on this host (bounded sample);
   extra         -- batch-16 decode and the stand-alone kernels of the other BASELINE configs.
 """
@@ -30,6 +32,8 @@ MFMA_I8_PEAK = 5000.0       # TOP/s dense
 # HBM bytes per skinny-kernel launch from rocprofv3 --pmc runs of this benchmark (fetch 15 306 KiB x 2.0, the factor a
 # plain 256 MiB copy gives for FETCH_SIZE on this GPU, + write 38 KiB x 1.0): profiles/int4_skinny_decode7b_graph_path.md
 SKINNY_TRAFFIC_BYTES = 31_385_000
+# HBM bytes per decode step of the single-launch kernel from the same kind of counter runs (None until measured)
+PERSIST_TRAFFIC_BYTES_PER_STEP = 4_787_000_000  # fetch 4.35 GB (x2.0 scale) + write 0.44 GB: profiles/decode_persistent_7b.md
 
 CFG7B = dict(n_layers=32, d_model=4096, n_heads=32, n_kv_heads=8, head_dim=128, d_ff=14336, vocab=32000,
              group_size=32, max_batch=16, max_ctx=2048 + 512, max_steps=1024, rope_theta=10000.0, rms_eps=1e-5)
@@ -54,19 +58,24 @@ def event_time_ms(fn, torch):
     return s.elapsed_time(e)
 
 
-def bench_decode(dec, torch, batch, steps, warmup, stream_ptr):
+def bench_decode(dec, torch, batch, steps, warmup, stream_ptr, persistent=False):
+    """Wall time of `steps` decode steps after `warmup` untimed ones.  persistent: every run() call is ONE
+    cooperative launch that executes all its steps on the device; otherwise one HIP-graph replay per step."""
     import numpy as np
 
     dec.reset(np.arange(1, batch + 1, dtype=np.int32), PREFILL)
-    dec.run(warmup, use_graph=True, stream=stream_ptr)
+    dec.run(warmup, use_graph=True, stream=stream_ptr, persistent=persistent)
     torch.cuda.synchronize()
+    s_ev, e_ev = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
-    dec.run(steps, use_graph=True, stream=stream_ptr)
+    s_ev.record()
+    dec.run(steps, use_graph=True, stream=stream_ptr, persistent=persistent)
+    e_ev.record()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     toks = dec.tokens(warmup, steps)
     assert toks.shape == (steps, batch) and (toks >= 0).all() and (toks < dec.cfg["vocab"]).all()
-    return dt
+    return dt, s_ev.elapsed_time(e_ev) * 1e-3
 
 
 def bench_projections(dec, torch, batch, stream_ptr, reps=6):
@@ -201,6 +210,8 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-extra", action="store_true", help="skip the stand-alone kernels and the batch-16 run")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--graph-path", action="store_true",
+                    help="time the multi-kernel path (one HIP-graph replay per step) instead of the single-launch kernel")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (torch copy_ kernel, 3 launches): the known-size "
                          "kernel that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
@@ -237,16 +248,28 @@ def main():
     w_bytes, params = decode_bytes_per_step(cfg)
     assert dec.weight_bytes() >= w_bytes
 
-    dt = bench_decode(dec, torch, args.batch, args.steps, args.warmup, stream_ptr)
+    persistent = args.batch == 1 and not args.graph_path
+    dt, dt_events = bench_decode(dec, torch, args.batch, args.steps, args.warmup, stream_ptr, persistent=persistent)
     tok_s = args.batch * args.steps / dt
-
-    avg_launch_s, launches = bench_projections(dec, torch, args.batch, stream_ptr)
-    n_proj = 4 * cfg["n_layers"] + 1
-    act_bytes = 0  # activations are < 0.1 % of the traffic and are left out of the algorithmic figure
-    bytes_per_launch = (w_bytes + act_bytes) / n_proj
-    achieved = bytes_per_launch / avg_launch_s / 1e9
-    kv_bytes_per_seq = 2 * cfg["n_layers"] * PREFILL * cfg["n_kv_heads"] * cfg["head_dim"] * 2
+    kv_row_bytes = 2 * cfg["n_layers"] * cfg["n_kv_heads"] * cfg["head_dim"] * 2  # K + V bytes one cached position adds
+    kv_bytes_per_seq = kv_row_bytes * PREFILL
     ideal_step_s = (w_bytes + args.batch * kv_bytes_per_seq) / (HBM_PEAK_GBS * 1e9)
+    if persistent:
+        # dominant kernel = the single-launch decode kernel: one launch runs all timed steps.  Algorithmic bytes
+        # per launch = per step, the packed weights + scales (read once) + the KV cache rows attended to.
+        first = PREFILL + args.warmup
+        kv_bytes = sum(kv_row_bytes * (first + i) for i in range(args.steps))
+        bytes_per_launch = w_bytes * args.steps + kv_bytes
+        launch_s, launches = dt_events, 1
+        kernel = "decode_persistent_kernel (one launch = %d decode steps)" % args.steps
+        traffic = PERSIST_TRAFFIC_BYTES_PER_STEP * args.steps if PERSIST_TRAFFIC_BYTES_PER_STEP else None
+    else:
+        launch_s, launches = bench_projections(dec, torch, args.batch, stream_ptr)
+        n_proj = 4 * cfg["n_layers"] + 1
+        bytes_per_launch = w_bytes / n_proj  # activations are < 0.1 % of the traffic and are left out
+        kernel = "int4_skinny_kernel (all %d projections of a decode step)" % n_proj
+        traffic = SKINNY_TRAFFIC_BYTES
+    achieved = bytes_per_launch / launch_s / 1e9
 
     result = {
         "metric": "int4 decode tok/s (7B-shape) + matmul GB/s and % HBM/MFMA roofline, 1 GPU",
@@ -259,16 +282,17 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int4 weights x fp16 activations, fp32 accumulate",
-        "data": "synthetic (random-init weights, random KV cache)",
+        "dtype": "f16",
+        "data": "synthetic (random-init int4 weights, random fp16 KV cache)",
         "config": {"workload": "BASELINE configs[3]: Llama-style decoder 32L d4096 32q/8kv hd128 ffn14336 vocab32000, "
                                "int4 g32 fp16 scales, fp16 KV ctx %d, greedy decode" % PREFILL,
-                   "batch": args.batch, "tokens_per_step": args.batch, "hip_graph": True},
+                   "batch": args.batch, "tokens_per_step": args.batch,
+                   "path": "single cooperative launch for all steps" if persistent else "one HIP-graph replay per step",
+                   "arithmetic": "int4 weights (exact in fp16) x fp16 activations on v_mfma_f32_16x16x32_f16, fp32 accumulate"},
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": SKINNY_TRAFFIC_BYTES,
-            "kernel": "int4_skinny_kernel (all %d projections of a decode step)" % n_proj,
-            "bytes_per_launch": int(bytes_per_launch), "avg_launch_us": round(avg_launch_s * 1e6, 3),
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+            "kernel": kernel, "bytes_per_launch": int(bytes_per_launch), "avg_launch_us": round(launch_s * 1e6, 3),
             "launches_timed": launches,
         },
         "hbm_roofline_whole_step": {"ideal_ms": round(ideal_step_s * 1e3, 4), "frac": round(ideal_step_s / (dt / args.steps), 4),
@@ -276,12 +300,20 @@ def main():
     }
     extra = {}
     if not args.no_extra:
+        n_proj = 4 * cfg["n_layers"] + 1
+        if persistent:
+            dtg, _ = bench_decode(dec, torch, 1, min(args.steps, 64), 4, stream_ptr)
+            avg1, _ = bench_projections(dec, torch, 1, stream_ptr)
+            extra["decode_batch1_graph_path"] = {"tok/s": round(min(args.steps, 64) / dtg, 1),
+                                                 "ms_per_step": round(dtg / min(args.steps, 64) * 1e3, 4),
+                                                 "skinny_kernel_GB/s": round(w_bytes / n_proj / avg1 / 1e9, 1)}
         if args.batch != 16:
-            dt16 = bench_decode(dec, torch, 16, min(args.steps, 64), 4, stream_ptr)
+            dt16, _ = bench_decode(dec, torch, 16, min(args.steps, 64), 4, stream_ptr)
             avg16, _ = bench_projections(dec, torch, 16, stream_ptr, reps=3)
             extra["decode_batch16"] = {"tok/s": round(16 * min(args.steps, 64) / dt16, 1),
                                        "ms_per_step": round(dt16 / min(args.steps, 64) * 1e3, 4),
-                                       "skinny_kernel_GB/s": round(bytes_per_launch / avg16 / 1e9, 1)}
+                                       "path": "one HIP-graph replay per step",
+                                       "skinny_kernel_GB/s": round(w_bytes / n_proj / avg16 / 1e9, 1)}
     del dec
     torch.cuda.empty_cache()
     if not args.no_extra:

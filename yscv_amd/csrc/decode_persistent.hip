@@ -36,8 +36,10 @@
 namespace yscv {
 
 typedef unsigned long long u64;
-#ifndef DBG_WAIT_ALL
-#define DBG_WAIT_ALL 0
+// Stage timestamps (wall clock, per workgroup and layer) for performance work: build with
+// -DYSCV_PERSIST_TRACE=1 and point PersistModel::dbg_t at a [G][n_layers][16] buffer.
+#ifndef YSCV_PERSIST_TRACE
+#define YSCV_PERSIST_TRACE 0
 #endif
 #ifndef INFLIGHT_CAP
 #define INFLIGHT_CAP 20
@@ -217,7 +219,7 @@ __device__ ATTN_INL WaitState attn_items(AttnArgs a, WaitState ws) {
   const int max_chunks = a.max_ctx / ACHUNK;
   const uint32_t tag = a.tag;
   const float scale = 0.08838834764831845f;  // 1 / sqrt(128)
-  if (a.dbg_t && tid == 0) a.dbg_t[14] = wall_clock64();
+  if (YSCV_PERSIST_TRACE && a.dbg_t && tid == 0) a.dbg_t[14] = wall_clock64();
 #pragma unroll 1
   for (int id = a.wg; id < items; id += a.G) {
     const int chunk = id / HKV, kvh = id - chunk * HKV;
@@ -277,7 +279,7 @@ __device__ ATTN_INL WaitState attn_items(AttnArgs a, WaitState ws) {
           if (__all(ok || !valid)) break;
           if (!poll_backoff_ws(ws, a.abort_flag)) break;
         }
-        if (a.dbg_t && tid == 0) a.dbg_t[15] = wall_clock64();
+        if (YSCV_PERSIST_TRACE && a.dbg_t && tid == 0) a.dbg_t[15] = wall_clock64();
 #pragma unroll
         for (int j = 0; j < 4; j++) {
           U32H2 e0, e1, e2, e3;
@@ -510,7 +512,6 @@ __device__ GEMV_INL GemvState gemv_stage(GemvArgs a, GemvState st) {
   const half8_t bc = {(_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f,
                       (_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f};
   const bool normed = a.ss != nullptr;
-  unsigned dbg_polls = 0;
   // ---- activation fragments (A operand: row i = k-block i of the fragment) ------------------------------
   // A `normed` vector holds fp16(h * gamma * 2^-e) with the exponent e of each 8-row block in the top byte
   // of its tag words; the operand is then fp16(h * gamma / rms), the activation RMSNorm feeds
@@ -536,7 +537,6 @@ __device__ GEMV_INL GemvState gemv_stage(GemvArgs a, GemvState st) {
                      : "+v"(qa[0]), "+v"(qa[1]), "+v"(qa[2]), "+v"(qa[3]), "+v"(qa[4]), "+v"(qa[5]), "+v"(qa[6]), "+v"(qa[7]),
                        "+v"(qb[0]), "+v"(qb[1]), "+v"(qb[2]), "+v"(qb[3]), "+v"(qb[4]), "+v"(qb[5]), "+v"(qb[6]), "+v"(qb[7]),
                        "+v"(sa), "+v"(sb)::"memory");
-        dbg_polls++;
         bool ok = (!v0 || tag_ok(sa[1], tag)) && (!v1 || tag_ok(sa[3], tag)) && (!v2 || tag_ok(sb[1], tag)) &&
                   (!v3 || tag_ok(sb[3], tag));
 #pragma unroll
@@ -582,9 +582,7 @@ __device__ GEMV_INL GemvState gemv_stage(GemvArgs a, GemvState st) {
       }
     }
   }
-  if (a.dbg_t && threadIdx.x == 0) {
-    a.dbg_t[0] = wall_clock64();
-  }
+  if (YSCV_PERSIST_TRACE && a.dbg_t && threadIdx.x == 0) a.dbg_t[0] = wall_clock64();
 
   // ---- one record: 8 rows x 512 k against fragment xa ------------------------------------------------------
   unsigned crec = st.crec;
@@ -664,7 +662,7 @@ __device__ GEMV_INL GemvState gemv_stage(GemvArgs a, GemvState st) {
     acc += __shfl_xor(acc, 32, 64);
     if (lane < 8) dst[blk * 8 + lane] = acc;
   }
-  if (a.dbg_t && threadIdx.x == 0) a.dbg_t[1] = wall_clock64();
+  if (YSCV_PERSIST_TRACE && a.dbg_t && threadIdx.x == 0) a.dbg_t[1] = wall_clock64();
   st.crec = crec;
   compute_barrier(st.ws, sync + 16, CW);
   return st;
@@ -675,10 +673,6 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   float *part_lds = reinterpret_cast<float *>(lds + RING_BYTES);                 // [2][8][PART_ROWS]
   unsigned char *att_lds = lds + RING_BYTES + PART_BYTES;
-  _Float16 *p_lds = reinterpret_cast<_Float16 *>(att_lds);                        // [4 waves][4 heads][32]
-  float *w_m = reinterpret_cast<float *>(att_lds + 1024);                         // [4][4]
-  float *w_l = reinterpret_cast<float *>(att_lds + 1024 + 64);                    // [4][4]
-  float *w_o = reinterpret_cast<float *>(att_lds + 1024 + 128);                   // [4][4][128]
   int *tok_lds = reinterpret_cast<int *>(att_lds + 1024 + 128 + 8192);            // [1]
   float *arg_v = reinterpret_cast<float *>(att_lds + 1024 + 128 + 8192 + 64);     // [8]
   int *arg_i = reinterpret_cast<int *>(att_lds + 1024 + 128 + 8192 + 128);        // [8]
@@ -687,19 +681,16 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r = lane & 15, c = lane >> 4;
   const int wg = blockIdx.x;
   const int G = m.G;
   const int L = m.n_layers;
   const int D = m.d_model;
   const int HQ = m.n_heads, HKV = m.n_kv_heads, GROUP = HQ / HKV;
-  const int max_chunks = m.max_ctx / ACHUNK;
-  const uint32_t magic = 0x64006400u;
 
   auto nbw = [&](int kind) { return wg < m.ph[kind].nb ? (m.ph[kind].nb - wg + G - 1) / G : 0; };
   int dbg_layer = 0;
   auto mark = [&](int idx) {
-    if (m.dbg_t && tid == 0) m.dbg_t[((size_t)wg * L + dbg_layer) * 16 + idx] = wall_clock64();
+    if (YSCV_PERSIST_TRACE && m.dbg_t && tid == 0) m.dbg_t[((size_t)wg * L + dbg_layer) * 16 + idx] = wall_clock64();
   };
   if (tid < 32) sync[tid] = 0;
   __syncthreads();
@@ -796,7 +787,6 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
           dirty = true;
         }
         if (dirty) {
-          if (DBG_WAIT_ALL) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
           for (int j = 0; j < SERVED; j++)
             lds_poke(sync_lds + 4 * (p * SERVED + j), landed_cnt[j]);
@@ -821,7 +811,7 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
     ga.in_buf = in_buf;
     ga.ss = with_ss ? in_buf + persist_vec_entries(m.ph[kind].k) : nullptr;
     ga.abort_flag = m.abort_flag;
-    ga.dbg_t = m.dbg_t ? m.dbg_t + ((size_t)wg * L + dbg_layer) * 16 + mk : nullptr;
+    ga.dbg_t = (YSCV_PERSIST_TRACE && m.dbg_t) ? m.dbg_t + ((size_t)wg * L + dbg_layer) * 16 + mk : nullptr;
     ga.tag = tag;
     ga.ks = m.ph[kind].ks;
     ga.frags = m.ph[kind].frags;
@@ -937,7 +927,7 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
         aa.tag = tag;
         aa.att_off = (uint32_t)(size_t)att_lds;
         aa.bar_off = (uint32_t)(size_t)(lds + RING_BYTES + PART_BYTES + ATT_BYTES) + 64;
-        aa.dbg_t = m.dbg_t ? m.dbg_t + ((size_t)wg * L + l) * 16 : nullptr;
+        aa.dbg_t = (YSCV_PERSIST_TRACE && m.dbg_t) ? m.dbg_t + ((size_t)wg * L + l) * 16 : nullptr;
         ws = attn_items(aa, ws);
         mark(4);
         for (int head = G - 1 - wg; head < HQ; head += G) ws = attn_combine(aa, ws, head);
@@ -947,7 +937,6 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
         const float g_next = own ? gam[(size_t)(2 * l + 1) * D + own_row] : 0.0f;  // in flight during the stage
         gemv(PK_O, m.ao, tag, false, 5);
         if (own) h += row_sum(tid);
-        if (own && m.dbg_h) m.dbg_h[((size_t)l * 2) * D + own_row] = h;
         publish_h(m.xn2, g_next, tag);
         pb ^= 1;
         mark(7);
@@ -971,7 +960,6 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
         const float g_next = own ? gam[(size_t)(l + 1 < L ? 2 * (l + 1) : 2 * L) * D + own_row] : 0.0f;
         gemv(PK_DOWN, m.act, tag, false, 11);
         if (own) h += row_sum(tid);
-        if (own && m.dbg_h) m.dbg_h[((size_t)l * 2 + 1) * D + own_row] = h;
         publish_h(m.xn, g_next, (tag + 1) & 0xFFFFFFu);
         pb ^= 1;
         mark(13);

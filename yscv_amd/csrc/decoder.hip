@@ -244,10 +244,7 @@ static int32_t persist_setup(yscv_hip_decoder *d) {
   m.tokens = d->tokens;
   m.history = d->history;
   m.abort_flag = d->p_abort;
-  m.dbg_h = nullptr;
   m.dbg_t = nullptr;
-  if (getenv("YSCV_DBG_T")) { (void)hipMalloc(reinterpret_cast<void **>(&m.dbg_t), (size_t)G * c.n_layers * 16 * 8); (void)hipMemset(m.dbg_t, 0, (size_t)G * c.n_layers * 16 * 8); }
-  if (getenv("YSCV_DBG_H")) { (void)hipMalloc(reinterpret_cast<void **>(&m.dbg_h), (size_t)c.n_layers * 2 * D * 4); }
   d->persist_ok = true;
   return YSCV_HIP_OK;
 }
@@ -716,19 +713,6 @@ int32_t yscv_hip_decoder_read_logits(yscv_hip_decoder *d, float *out_host) {
   YSCV_TRY(check_persist_abort(d));
   DEC_HIP(hipMemcpy(out_host, d->logits, (size_t)d->batch * d->cfg.vocab * 4, hipMemcpyDeviceToHost));
   return YSCV_HIP_OK;
-}
-
-__attribute__((visibility("default"))) int32_t yscv_hip_decoder_dbg_t(yscv_hip_decoder *d, unsigned long long *out) {
-  if (!d->pm.dbg_t) return -1;
-  (void)hipDeviceSynchronize();
-  (void)hipMemcpy(out, d->pm.dbg_t, (size_t)d->pm.G * d->cfg.n_layers * 16 * 8, hipMemcpyDeviceToHost);
-  return 0;
-}
-__attribute__((visibility("default"))) int32_t yscv_hip_decoder_dbg_h(yscv_hip_decoder *d, float *out) {
-  if (!d->pm.dbg_h) return -1;
-  (void)hipDeviceSynchronize();
-  (void)hipMemcpy(out, d->pm.dbg_h, (size_t)d->cfg.n_layers * 2 * d->cfg.d_model * 4, hipMemcpyDeviceToHost);
-  return 0;
 }
 
 int32_t yscv_hip_decoder_weight_bytes(const yscv_hip_decoder *d, size_t *bytes) {

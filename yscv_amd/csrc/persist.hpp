@@ -66,8 +66,7 @@ struct PersistModel {
   int32_t *tokens;              // [1] current token (in: first token; out: last pick)
   int32_t *history;             // [max_steps]
   uint32_t *abort_flag;         // set when a bounded wait gave up
-  unsigned long long *dbg_t;    // debug: [G][n_layers][16] timestamps of wave 0
-  float *dbg_h;                 // debug: [n_layers][2][d_model] residual after o-proj / down
+  unsigned long long *dbg_t;    // null, or [G][n_layers][16] stage timestamps (builds with YSCV_PERSIST_TRACE)
 };
 
 // entries an exchange vector of k values occupies (padded to whole 512-k fragments per wave)
