@@ -216,6 +216,72 @@ int32_t yscv_hip_requant_i32_row_to_i8_dispatch(const int32_t *acc, size_t len,
 int32_t yscv_hip_dynamic_quantize_linear_host(const float *x, size_t len, uint8_t *y,
                                               float *scale, float *zero_point);
 
+/* ---- ONNX operators on f32 carriers (device pointers) ------------------------------------- */
+
+/* The reference runner keeps every quantised tensor as f32 values holding integers; these entry points
+ * take and return such tensors in device memory, so a graph executor calls them where the reference
+ * calls the function cited.  Operands are rank 2 (callers flatten leading dimensions of A into m). */
+
+/* Which route a call took (written to *path_out when it is not null). */
+#define YSCV_HIP_PATH_FAST 0            /* both zero points 0: integer kernel, as the reference's fast path */
+#define YSCV_HIP_PATH_FALLBACK_EXACT 1  /* non-zero zero point, 8-bit integer operands: exact integer route */
+#define YSCV_HIP_PATH_FALLBACK_F32 2    /* non-zero zero point, other operands: f32 products added in k order */
+
+/* QuantRuntimeStats (crates/yscv-onnx/src/runner/quant_stats.rs:6-22) restricted to this path, plus the
+ * int4_fast / int4_fallback split docs/int4-quant-pipeline-plan.md:25-34 asks a runtime to report and the
+ * same split for MatMulInteger.  "fallback" counts every call the reference would send to its f32 matmul
+ * (linear.rs:494), whichever device route served it here.  int4_fast counts calls served by the tiled MFMA
+ * kernels, int4_fallback calls served by the generic per-group kernel. */
+typedef struct yscv_hip_quant_stats {
+  uint64_t qlinear_matmul_fast;
+  uint64_t qlinear_matmul_fallback;
+  uint64_t matmul_integer_fast;
+  uint64_t matmul_integer_fallback;
+  uint64_t int4_fast;
+  uint64_t int4_fallback;
+} yscv_hip_quant_stats;
+/* quant_runtime_stats / reset_quant_runtime_stats (quant_stats.rs:24-62): process-wide, relaxed atomics. */
+int32_t yscv_hip_quant_runtime_stats(yscv_hip_quant_stats *out);
+int32_t yscv_hip_reset_quant_runtime_stats(void);
+/* quant_int8_fast_enabled (quant_stats.rs:64-69): 0 only when YSCV_QUANT_INT8_FAST is exactly "0". */
+int32_t yscv_hip_quant_int8_fast_enabled(void);
+/* should_use_prepacked_i8_b (crates/yscv-onnx/src/runner/layout.rs:6-11) and the load-time gate
+ * should_prepack_i8_b (crates/yscv-onnx/src/plan/build.rs:1371-1377); 1 = yes. */
+int32_t yscv_hip_should_use_prepacked_i8_b(size_t m, size_t k, size_t n);
+int32_t yscv_hip_should_prepack_i8_b(size_t k, size_t n);
+/* Load-time prepack of a weight initialiser held as an f32 carrier [k][n] on the device: `v.round() as i8`
+ * per element (tensor_data_as_i8, plan/build.rs:1367-1369), then the layout of
+ * yscv_hip_pack_i8_b_for_matmul (plan/build.rs:1416-1454). */
+int32_t yscv_hip_i8_weight_from_f32(const float *b_dev, size_t k, size_t n, void *stream,
+                                    yscv_hip_i8_weight **out);
+/* exec_matmul_integer (crates/yscv-onnx/src/runner/linear.rs:648-737).  out_dev[m][n] f32.  Pass the
+ * unpacked B (b_dev, [k][n]), a prepacked one, or both; absent ONNX zero points are 0.  A prepacked B
+ * alone serves b_zp == 0 only. */
+int32_t yscv_hip_exec_matmul_integer(const float *a_dev, const float *b_dev,
+                                     const yscv_hip_i8_weight *b_packed, float a_zp, float b_zp, size_t m,
+                                     size_t k, size_t n, float *out_dev, int32_t *path_out, void *stream);
+/* exec_qlinear_matmul (crates/yscv-onnx/src/runner/linear.rs:438-538): scalar scales and zero points,
+ * output clamp(round_half_away(.), -128, 127) as f32.  A prepacked B whose shape differs from (k, n) is
+ * an error, as in the reference (linear.rs:468-475). */
+int32_t yscv_hip_exec_qlinear_matmul(const float *a_dev, float a_scale, float a_zp, const float *b_dev,
+                                     const yscv_hip_i8_weight *b_packed, float b_scale, float b_zp,
+                                     float y_scale, float y_zp, size_t m, size_t k, size_t n,
+                                     float *out_dev, int32_t *path_out, void *stream);
+/* exec_quantize_linear, f32-carrier arm (crates/yscv-onnx/src/runner/misc.rs:42-80) =
+ * quantize_linear_f32_to_f32_i8_scalar (crates/yscv-kernels/src/ops/quantize.rs:226-238). */
+int32_t yscv_hip_exec_quantize_linear(const float *x_dev, size_t len, float scale, float zero_point,
+                                      float *out_dev, void *stream);
+/* exec_dequantize_linear (crates/yscv-onnx/src/runner/misc.rs:110-239) on a tensor viewed as
+ * [outer][chan][inner] around the quantisation axis.  n_scales = 1: per tensor; n_scales = chan: per
+ * channel; anything else is the reference's "scale len" error.  zps_dev may be null (all zero). */
+int32_t yscv_hip_exec_dequantize_linear(const float *q_dev, size_t outer, size_t chan, size_t inner,
+                                        const float *scales_dev, const float *zps_dev, size_t n_scales,
+                                        float *out_dev, void *stream);
+/* exec_dynamic_quantize_linear (crates/yscv-onnx/src/runner/misc.rs:241-289) with its three f32 outputs:
+ * y_dev[len], *y_scale_dev, *y_zp_dev. */
+int32_t yscv_hip_exec_dynamic_quantize_linear(const float *x_dev, size_t len, float *y_dev,
+                                              float *y_scale_dev, float *y_zp_dev, void *stream);
+
 /* ---- decode loop (Llama-style decoder, int4 projections, fp16 KV cache) ----------------- */
 
 /* GPU-resident counterpart of the llm-bench decode loop (apps/llm-bench/src/main.rs:403-561:
@@ -279,9 +345,12 @@ int32_t yscv_hip_decoder_set_kv(yscv_hip_decoder *d, int32_t layer, const uint16
 /* Start a generation: batch rows, the position the next token is written at, one input token per row. */
 int32_t yscv_hip_decoder_reset(yscv_hip_decoder *d, int32_t batch, int32_t start_pos,
                                const int32_t *tokens_host);
-/* Run n_steps decode steps (asynchronously on `stream`).  use_graph != 0 replays one captured HIP
- * graph per step.  Fails if the KV cache or the token history would overflow (KvCache::append
- * returns an error in the same situation, kv_cache.rs:160-185). */
+/* Run n_steps decode steps (asynchronously on `stream`).  use_graph = 0 launches the kernels of a step one
+ * by one, 1 replays one captured HIP graph per step, 2 runs all n_steps in ONE cooperative launch of the
+ * persistent decode kernel (batch 1 only; YSCV_HIP_ERR_UNSUPPORTED with the reason in the error text when
+ * the model shape or the device cannot run it).  All three produce the same tokens.  Fails if the KV cache
+ * or the token history would overflow (KvCache::append returns an error in the same situation,
+ * kv_cache.rs:160-185). */
 int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_graph, void *stream);
 /* Measurement aid: enqueue only the int4 projections of n_steps decode steps (same weights, same
  * order, same buffers as a real step, no attention / norm / sampling), so that the projections'

@@ -1,0 +1,255 @@
+"""GPU parity of the operator layer (MatMulInteger, QLinearMatMul, QuantizeLinear, DequantizeLinear,
+DynamicQuantizeLinear on f32 carriers) against the CPU restatement of the reference runner, through the C ABI."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+KATS = json.load(open(os.path.join(HERE, "golden", "reference_kats.json")))
+
+SHAPES = [(1, 1, 1), (2, 3, 4), (5, 17, 6), (4, 64, 16), (8, 127, 33), (33, 200, 70), (64, 512, 128)]
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+
+    assert torch.cuda.is_available()
+    return torch
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from yscv_amd import onnx_ops
+
+    return onnx_ops
+
+
+def _dev(torch, a, shape=None):
+    t = torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+    return t.reshape(shape) if shape is not None else t
+
+
+def test_reference_known_answers(torch_cuda, ops):
+    torch = torch_cuda
+    for c in KATS["matmul_integer"]["cases"]:  # coverage.rs:359-390, gemm_matmul.rs:73-87
+        out, path = ops.exec_matmul_integer(_dev(torch, c["a"], (c["m"], c["k"])), _dev(torch, c["b"], (c["k"], c["n"])),
+                                            a_zp=float(c["a_zp"]))
+        assert out.cpu().numpy().ravel().tolist() == [float(v) for v in c["expected"]]
+        assert path == (ops.PATH_FAST if c["a_zp"] == 0 else ops.PATH_FALLBACK_EXACT)
+    q = KATS["qlinear_matmul"]  # qlinear.rs:150-194
+    m, k, n = q["m"], q["k"], q["n"]
+    a = np.array([v - 16 for v in range(m * k)], np.float32)
+    b = np.array([(7 * v) % 31 - 15 for v in range(k * n)], np.float32)
+    comp = np.float32(np.float32(q["a_scale"]) * np.float32(q["b_scale"])) / np.float32(q["y_scale"])
+    acc = a.reshape(m, k).astype(np.int64) @ b.reshape(k, n).astype(np.int64)
+    v = acc.astype(np.float32) * comp
+    exp = np.clip(np.where(v >= 0, np.floor(v + np.float32(0.5)), -np.floor(-v + np.float32(0.5))), -128, 127)
+    out, path = ops.exec_qlinear_matmul(_dev(torch, a, (m, k)), q["a_scale"], 0.0, _dev(torch, b, (k, n)), q["b_scale"], 0.0,
+                                        q["y_scale"], 0.0)
+    assert path == ops.PATH_FAST and np.array_equal(out.cpu().numpy(), exp.astype(np.float32))
+    for c in KATS["dynamic_quantize_linear"]["cases"]:  # coverage.rs:210-249
+        y, s, z = ops.exec_dynamic_quantize_linear(_dev(torch, c["x"]))
+        assert abs(float(s) - c["scale"]) < 1e-6 and float(z) == c["zero_point"] and y.cpu().numpy().tolist() == c["y"]
+    for c in KATS["quantize_linear"]["cases"]:
+        out = ops.exec_quantize_linear(_dev(torch, c["data"]), c["scale"], c["zero_point"])
+        assert out.cpu().numpy().tolist() == [float(v) for v in c["expected"]]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_matmul_integer_fast_path_bit_exact(oracle, torch_cuda, ops, shape):
+    torch = torch_cuda
+    m, k, n = shape
+    rng = np.random.default_rng(m * 1000 + k * 10 + n)
+    a = rng.integers(-128, 128, m * k).astype(np.float32)
+    b = rng.integers(-128, 128, k * n).astype(np.float32)
+    # carriers outside the i8 range and non-integers exercise the saturating, truncating `as i8` cast
+    a[:: 7] = a[:: 7] * 3.5 + 0.75
+    b[:: 5] = b[:: 5] * 2.25 - 0.5
+    if a.size > 3:
+        a[3] = np.nan
+    exp, fast = oracle.exec_matmul_integer(a, b, 0.0, 0.0, m, k, n)
+    assert fast
+    out, path = ops.exec_matmul_integer(_dev(torch, a, (m, k)), _dev(torch, b, (k, n)))
+    assert path == ops.PATH_FAST and np.array_equal(out.cpu().numpy(), exp)
+    # the load-time prepack rounds before the cast (plan/build.rs:1367-1369): same result on integer weights
+    bi = np.trunc(np.clip(b, -128, 127))
+    pre = ops.PrepackedI8B(_dev(torch, bi, (k, n)))
+    exp2, _ = oracle.exec_matmul_integer(a, bi, 0.0, 0.0, m, k, n)
+    out2, _ = ops.exec_matmul_integer(_dev(torch, a, (m, k)), None, prepacked=pre)
+    assert np.array_equal(out2.cpu().numpy(), exp2)
+    pre.close()
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("domain", ["u8_i8", "i8_u8", "u8_u8"])
+def test_matmul_integer_asymmetric_is_integer_exact(oracle, torch_cuda, ops, shape, domain):
+    torch = torch_cuda
+    m, k, n = shape
+    rng = np.random.default_rng(m * 77 + k * 3 + n + len(domain))
+    alo, ahi = (0, 256) if domain.startswith("u8") else (-128, 128)
+    blo, bhi = (0, 256) if domain.endswith("u8") else (-128, 128)
+    a = rng.integers(alo, ahi, (m, k))
+    b = rng.integers(blo, bhi, (k, n))
+    a_zp = int(rng.integers(alo, ahi))
+    b_zp = int(rng.integers(blo, bhi)) if domain != "u8_i8" else 0
+    if a_zp == 0 and b_zp == 0:
+        a_zp = 1 if alo == 0 else -1
+    exact = (a.astype(np.int64) - a_zp) @ (b.astype(np.int64) - b_zp)
+    out, path = ops.exec_matmul_integer(_dev(torch, a), _dev(torch, b), a_zp=float(a_zp), b_zp=float(b_zp))
+    assert path == ops.PATH_FALLBACK_EXACT
+    assert np.array_equal(out.cpu().numpy(), exact.astype(np.float32))
+    if np.abs(a - a_zp).max() * np.abs(b - b_zp).max() * k < 2 ** 24:
+        # every partial sum is exact in f32, so the reference's float fallback gives the same numbers
+        exp, fast = oracle.exec_matmul_integer(a.ravel(), b.ravel(), float(a_zp), float(b_zp), m, k, n)
+        assert not fast and np.array_equal(out.cpu().numpy(), exp)
+
+
+def test_matmul_integer_f32_route_follows_the_float_fallback(oracle, torch_cuda, ops):
+    torch = torch_cuda
+    m, k, n = 7, 45, 19
+    rng = np.random.default_rng(5)
+    a = (rng.integers(0, 256, m * k) + rng.choice([0.0, 0.25, 0.5], m * k)).astype(np.float32)
+    b = rng.integers(-128, 128, k * n).astype(np.float32)
+    exp, fast = oracle.exec_matmul_integer(a, b, 3.0, 1.0, m, k, n)
+    out, path = ops.exec_matmul_integer(_dev(torch, a, (m, k)), _dev(torch, b, (k, n)), a_zp=3.0, b_zp=1.0)
+    assert not fast and path == ops.PATH_FALLBACK_F32
+    assert np.array_equal(out.cpu().numpy(), exp)
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_qlinear_matmul_fast_path_bit_exact(oracle, torch_cuda, ops, shape):
+    torch = torch_cuda
+    m, k, n = shape
+    rng = np.random.default_rng(m + 31 * k + 977 * n)
+    a = rng.integers(-128, 128, m * k).astype(np.float32)
+    b = rng.integers(-128, 128, k * n).astype(np.float32)
+    for a_s, b_s, y_s, y_zp in ((0.05, 0.1, 0.25, 0.0), (0.02, 0.004, 0.5, -7.0), (1.0, 0.5, 64.0, 3.0)):
+        exp, fast = oracle.exec_qlinear_matmul(a, a_s, 0.0, b, b_s, 0.0, y_s, y_zp, m, k, n)
+        out, path = ops.exec_qlinear_matmul(_dev(torch, a, (m, k)), a_s, 0.0, _dev(torch, b, (k, n)), b_s, 0.0, y_s, y_zp)
+        assert fast and path == ops.PATH_FAST
+        assert np.array_equal(out.cpu().numpy(), exp)
+        if ops.should_use_prepacked_i8_b(m, k, n):
+            pre = ops.PrepackedI8B(_dev(torch, b, (k, n)))
+            out2, _ = ops.exec_qlinear_matmul(_dev(torch, a, (m, k)), a_s, 0.0, None, b_s, 0.0, y_s, y_zp, prepacked=pre)
+            assert np.array_equal(out2.cpu().numpy(), exp)
+            pre.close()
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_qlinear_matmul_asymmetric(oracle, torch_cuda, ops, shape):
+    """Asymmetric zero points: the exact sum, scaled once, against (a) the same expression in float64 and (b) the
+    reference's float fallback, whose per-product rounding can move a value sitting on a rounding boundary by one."""
+    torch = torch_cuda
+    m, k, n = shape
+    rng = np.random.default_rng(k * 13 + n)
+    a = rng.integers(0, 256, (m, k))
+    b = rng.integers(-128, 128, (k, n))
+    a_zp, b_zp, a_s, b_s, y_s, y_zp = 128.0, 0.0, 0.02, 0.01, 0.8, 5.0
+    out, path = ops.exec_qlinear_matmul(_dev(torch, a), a_s, a_zp, _dev(torch, b), b_s, b_zp, y_s, y_zp)
+    assert path == ops.PATH_FALLBACK_EXACT
+    got = out.cpu().numpy()
+    acc = (a.astype(np.int64) - 128) @ b.astype(np.int64)
+    v = (acc.astype(np.float64) * (float(np.float32(a_s)) * float(np.float32(b_s)))).astype(np.float32)
+    t = v / np.float32(y_s) + np.float32(y_zp)
+    want = np.clip(np.where(t >= 0, np.floor(t + np.float32(0.5)), -np.floor(-t + np.float32(0.5))), -128, 127)
+    assert np.array_equal(got, want.astype(np.float32))
+    exp, fast = oracle.exec_qlinear_matmul(a.ravel(), a_s, a_zp, b.ravel(), b_s, b_zp, y_s, y_zp, m, k, n)
+    assert not fast
+    assert np.abs(got - exp).max() <= 1.0
+    assert (got != exp).mean() <= 0.02
+
+
+def test_qlinear_prepacked_shape_mismatch_is_an_error(torch_cuda, ops):
+    import yscv_amd
+
+    torch = torch_cuda
+    pre = ops.PrepackedI8B(torch.zeros(8, 32, device="cuda"))
+    with pytest.raises(yscv_amd.YscvHipError) as ei:  # linear.rs:468-475
+        yscv_amd.lib().exec_qlinear_matmul(torch.zeros(4, 16, device="cuda").data_ptr(), 1.0, 0.0, None, pre.handle, 1.0, 0.0,
+                                           1.0, 0.0, 4, 16, 32, torch.zeros(4, 32, device="cuda").data_ptr(), None, None)
+    assert ei.value.code == -1 and "shape mismatch" in ei.value.message
+    pre.close()
+
+
+def test_counters_follow_the_reference_gates(torch_cuda, ops):
+    torch = torch_cuda
+    a = torch.ones(4, 8, device="cuda")
+    b = torch.ones(8, 16, device="cuda")
+    ops.reset_quant_runtime_stats()
+    ops.exec_qlinear_matmul(a, 1.0, 0.0, b, 1.0, 0.0, 1.0, 0.0)
+    ops.exec_qlinear_matmul(a, 1.0, 0.0, b, 1.0, 0.0, 1.0, 0.0)
+    ops.exec_qlinear_matmul(a, 1.0, 1.0, b, 1.0, 0.0, 1.0, 0.0)
+    ops.exec_matmul_integer(a, b)
+    ops.exec_matmul_integer(a, b, a_zp=2.0)
+    ops.exec_matmul_integer(a, b, b_zp=2.0)
+    s = ops.quant_runtime_stats()
+    assert (s.qlinear_matmul_fast, s.qlinear_matmul_fallback, s.matmul_integer_fast, s.matmul_integer_fallback) == (2, 1, 1, 2)
+    # int4: tiled layouts count as fast, the generic per-group kernel as fallback
+    from yscv_amd import kernels as K
+
+    rng = np.random.default_rng(0)
+    for g, want in ((32, "int4_fast"), (16, "int4_fallback")):
+        n, k = 16, 128
+        w = K.PackedInt4Weight(rng.integers(0, 256, n * k // 2, dtype=np.uint8), np.ones(n * k // g, np.float32), g, n, k)
+        before = ops.quant_runtime_stats()
+        w.matmul(torch.ones(1, k, device="cuda"))
+        after = ops.quant_runtime_stats()
+        assert getattr(after, want) == getattr(before, want) + 1
+        w.close()
+    ops.reset_quant_runtime_stats()
+    assert ops.quant_runtime_stats() == ops.QuantRuntimeStats()
+
+
+def test_quantize_dequantize_linear(oracle, torch_cuda, ops):
+    torch = torch_cuda
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal(10_007) * 40).astype(np.float32)
+    x[:8] = [0.5, 1.5, 2.5, -0.5, -1.5, np.nan, 1e9, -1e9]
+    for scale, zp in ((1.0, 0.0), (0.37, 3.0), (0.011, -100.0)):
+        exp = oracle.quantize_linear_f32_to_f32_i8(x, scale, zp)
+        got = ops.exec_quantize_linear(_dev(torch, x), scale, zp).cpu().numpy()
+        assert np.array_equal(got, exp, equal_nan=True)
+        back = ops.exec_dequantize_linear(_dev(torch, np.nan_to_num(exp)), torch.tensor([scale], device="cuda"),
+                                          torch.tensor([zp], device="cuda")).cpu().numpy()
+        assert np.array_equal(back, oracle.dequantize_linear(np.nan_to_num(exp), scale, zp))
+    # per-channel along axis 1 and along the last axis (misc.rs:136-170), written out with numpy broadcasting
+    q = rng.integers(-128, 128, (3, 5, 4, 2)).astype(np.float32)
+    for axis in (1, -1, 0):
+        chan = q.shape[axis]
+        s = (rng.random(chan) + 0.1).astype(np.float32)
+        z = rng.integers(-5, 5, chan).astype(np.float32)
+        shp = [1] * q.ndim
+        shp[axis] = chan
+        want = (q - z.reshape(shp)) * s.reshape(shp)
+        got = ops.exec_dequantize_linear(_dev(torch, q), _dev(torch, s), _dev(torch, z), axis=axis).cpu().numpy()
+        assert np.array_equal(got, want)
+        got = ops.exec_dequantize_linear(_dev(torch, q), _dev(torch, s), None, axis=axis).cpu().numpy()
+        assert np.array_equal(got, q * s.reshape(shp))
+    import yscv_amd
+
+    with pytest.raises(yscv_amd.YscvHipError):  # misc.rs:146-153: scale length must equal the axis extent
+        ops.exec_dequantize_linear(_dev(torch, q), _dev(torch, np.ones(3, np.float32)), None, axis=1)
+
+
+def test_dynamic_quantize_linear_matches_checker(oracle, torch_cuda, ops):
+    torch = torch_cuda
+    rng = np.random.default_rng(3)
+    for x in (rng.standard_normal(4099).astype(np.float32) * 3, np.abs(rng.standard_normal(300)).astype(np.float32),
+              np.zeros(17, np.float32), -np.abs(rng.standard_normal(64)).astype(np.float32)):
+        ey, es, ez = oracle.dynamic_quantize_linear(x)
+        y, s, z = ops.exec_dynamic_quantize_linear(_dev(torch, x))
+        assert float(s) == float(es) and float(z) == float(ez)
+        assert np.array_equal(y.cpu().numpy(), np.asarray(ey, np.float32))
+    # DynamicQuantizeLinear -> MatMulInteger, the dynamic-quantisation pattern: integer-exact downstream
+    x = (rng.standard_normal((6, 96)) * 2).astype(np.float32)
+    w = rng.integers(-128, 128, (96, 48))
+    y, s, z = ops.exec_dynamic_quantize_linear(_dev(torch, x))
+    out, path = ops.exec_matmul_integer(y, _dev(torch, w), a_zp=float(z))
+    assert path == ops.PATH_FALLBACK_EXACT
+    exact = (y.cpu().numpy().astype(np.int64) - int(float(z))) @ w.astype(np.int64)
+    assert np.array_equal(out.cpu().numpy(), exact.astype(np.float32))

@@ -22,6 +22,16 @@ class DecoderConfig(C.Structure):
                [("rope_theta", C.c_float), ("rms_eps", C.c_float)]
 
 
+class QuantStats(C.Structure):
+    """yscv_hip_quant_stats."""
+
+    _fields_ = [(n, C.c_uint64) for n in ("qlinear_matmul_fast", "qlinear_matmul_fallback", "matmul_integer_fast",
+                                          "matmul_integer_fallback", "int4_fast", "int4_fallback")]
+
+
+PATH_FAST, PATH_FALLBACK_EXACT, PATH_FALLBACK_F32 = 0, 1, 2
+
+
 class YscvHipError(RuntimeError):
     def __init__(self, code: int, message: str):
         super().__init__(f"yscv_hip status {code} ({STATUS_NAMES.get(code, '?')}): {message}")
@@ -72,6 +82,15 @@ _SIGNATURES = {
     "yscv_hip_requant_i8_per_channel_dispatch": [_vp, _sz, _vp, _vp, _f32, _vp, _sz],
     "yscv_hip_requant_i32_row_to_i8_dispatch": [_vp, _sz, _vp, _f32, _f32, _i32, _vp, _sz],
     "yscv_hip_dynamic_quantize_linear_host": [_vp, _sz, _vp, C.POINTER(_f32), C.POINTER(_f32)],
+    "yscv_hip_quant_runtime_stats": [_vp],
+    "yscv_hip_reset_quant_runtime_stats": [],
+    "yscv_hip_i8_weight_from_f32": [_vp, _sz, _sz, _vp, C.POINTER(_vp)],
+    "yscv_hip_exec_matmul_integer": [_vp, _vp, _vp, _f32, _f32, _sz, _sz, _sz, _vp, C.POINTER(_i32), _vp],
+    "yscv_hip_exec_qlinear_matmul": [_vp, _f32, _f32, _vp, _vp, _f32, _f32, _f32, _f32, _sz, _sz, _sz, _vp,
+                                     C.POINTER(_i32), _vp],
+    "yscv_hip_exec_quantize_linear": [_vp, _sz, _f32, _f32, _vp, _vp],
+    "yscv_hip_exec_dequantize_linear": [_vp, _sz, _sz, _sz, _vp, _vp, _sz, _vp, _vp],
+    "yscv_hip_exec_dynamic_quantize_linear": [_vp, _sz, _vp, _vp, _vp, _vp],
     "yscv_hip_decoder_create": [_vp, C.POINTER(_vp)],
     "yscv_hip_decoder_destroy": [_vp],
     "yscv_hip_decoder_set_linear": [_vp, _i32, _i32, _vp, _vp, _sz, _sz],
@@ -91,6 +110,10 @@ _SIGNATURES = {
 _SPECIAL = {
     "yscv_hip_abi_version": ([], C.c_uint32),
     "yscv_hip_last_error": ([], C.c_char_p),
+    # predicates: the return value is the answer, not a status
+    "yscv_hip_quant_int8_fast_enabled": ([], _i32),
+    "yscv_hip_should_use_prepacked_i8_b": ([_sz, _sz, _sz], _i32),
+    "yscv_hip_should_prepack_i8_b": ([_sz, _sz], _i32),
 }
 
 EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + list(_SPECIAL))

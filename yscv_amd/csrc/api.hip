@@ -119,8 +119,10 @@ int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, v
   if (force == 1 && m > 16) return set_error(YSCV_HIP_ERR_INVALID_ARG, "gemv entry point handles m <= 16, got %zu", m);
   if (!w->tiled) {
     if (epi != EPI_STORE) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "fused epilogues need the tiled layout");
+    note_int4_fallback();
     return launch_int4_generic(w, x, x_dtype, y, y_dtype, m, s);
   }
+  note_int4_fast();
   Int4Scratch L = int4_scratch_layout(w, x, x_dtype, m, force, ctx->num_cus);
   if (!L.skinny && epi != EPI_STORE) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "fused epilogues exist for m <= 16 only");
   char *scratch = static_cast<char *>(ws);

@@ -87,6 +87,10 @@ int32_t launch_pack_int4_symmetric(const float *w, size_t m_w, size_t k, size_t 
 int32_t launch_dequantize_int4(const uint8_t *packed, size_t n_bytes, float scale, int zp,
                                float *out, hipStream_t s);
 
+// runtime counters: a call served by the tiled MFMA kernels / by the generic per-group kernel
+void note_int4_fast();
+void note_int4_fallback();
+
 // ---- int8 --------------------------------------------------------------------------
 int32_t launch_i8_pack_b(const int8_t *b_kn, size_t k, size_t n, size_t kp, size_t np,
                          int8_t *frag, int32_t *col_sum, hipStream_t s);

@@ -1,0 +1,491 @@
+// ONNX operator entry points of the quantised matmul path.  Tensors are device-resident f32
+// "carriers" exactly as the reference runner keeps them (every quantised value is an f32 holding an
+// integer), so a graph executor can call these where the reference calls
+//   exec_matmul_integer          crates/yscv-onnx/src/runner/linear.rs:648-737
+//   exec_qlinear_matmul          crates/yscv-onnx/src/runner/linear.rs:438-538
+//   exec_quantize_linear         crates/yscv-onnx/src/runner/misc.rs:42-108 (f32-carrier arm)
+//   exec_dequantize_linear       crates/yscv-onnx/src/runner/misc.rs:110-239
+//   exec_dynamic_quantize_linear crates/yscv-onnx/src/runner/misc.rs:241-289
+// and read the same fast/fallback counters (crates/yscv-onnx/src/runner/quant_stats.rs:6-92).
+//
+// Fast path (both zero points 0): operands are cast with Rust's saturating `as i8`, the product runs on the
+// int8 MFMA kernel, the epilogue follows the reference expression by expression.
+//
+// Fallback (a zero point is non-zero): the reference dequantises to f32 and calls its float matmul.  When
+// every operand value is an integer that fits 8 bits the same quantity is computed exactly here,
+//   sum_k (a - a_zp)(b - b_zp) = sum_k A'B' - a_zp' colsum(B')[j] - b_zp' (rowsum(A')[i] - K a_zp'),
+// with A' the operand shifted into u8, B' shifted into i8 and the zero points shifted alike, on the
+// same MFMA kernel.  That equals the reference's f32 result whenever the latter is exact (all partial
+// sums below 2^24) and is the correctly rounded value otherwise.  Operands that are not 8-bit integers
+// take a plain f32 kernel that adds the products in k order with separately rounded multiply and add.
+#include <atomic>
+#include <cstdlib>
+
+#include "int4_common.hpp"
+#include "kernels.hpp"
+
+namespace yscv {
+namespace {
+
+std::atomic<uint64_t> g_qlinear_fast{0}, g_qlinear_fallback{0}, g_mmi_fast{0}, g_mmi_fallback{0},
+    g_int4_fast{0}, g_int4_fallback{0};
+
+__device__ __forceinline__ float round_half_away(float v) {
+  float t = truncf(v);
+  float d = fabsf(__fsub_rn(v, t));
+  return (d >= 0.5f) ? __fadd_rn(t, copysignf(1.0f, v)) : t;
+}
+// f32::clamp: NaN stays NaN
+__device__ __forceinline__ float clamp_keep_nan(float r, float lo, float hi) {
+  return (r != r) ? r : fminf(fmaxf(r, lo), hi);
+}
+// Rust `v as i8`: NaN -> 0, saturating, truncation toward zero
+__device__ __forceinline__ int8_t f32_as_i8(float v) {
+  if (v != v) return 0;
+  if (v <= -128.0f) return -128;
+  if (v >= 127.0f) return 127;
+  return (int8_t)(int)v;
+}
+
+inline unsigned grid_for(size_t len, unsigned per_block = 256) {
+  size_t blocks = ceil_div(len, (size_t)per_block);
+  if (blocks > 16384) blocks = 16384;
+  if (blocks < 1) blocks = 1;
+  return (unsigned)blocks;
+}
+
+#define GRID_STRIDE(i, len) \
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < (len); i += (size_t)gridDim.x * blockDim.x)
+
+// round_first: `v.round() as i8` (load-time prepack), else `v as i8` (per-call cast)
+__global__ void cast_as_i8_kernel(const float *__restrict__ x, size_t len, int round_first, int8_t *__restrict__ out) {
+  GRID_STRIDE(i, len) out[i] = f32_as_i8(round_first ? round_half_away(x[i]) : x[i]);
+}
+
+// info[0] = min, info[1] = max (as integers), info[2] != 0 when a value is not an integer in [-1024, 1024]
+__global__ void scan_int_range_kernel(const float *__restrict__ x, size_t len, int *__restrict__ info) {
+  int lo = 1 << 20, hi = -(1 << 20), bad = 0;
+  GRID_STRIDE(i, len) {
+    float v = x[i];
+    if (!(fabsf(v) <= 1024.0f) || truncf(v) != v) {
+      bad = 1;
+    } else {
+      int q = (int)v;
+      lo = min(lo, q);
+      hi = max(hi, q);
+    }
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    lo = min(lo, __shfl_xor(lo, o));
+    hi = max(hi, __shfl_xor(hi, o));
+    bad |= __shfl_xor(bad, o);
+  }
+  if ((threadIdx.x & 63) == 0) {
+    atomicMin(&info[0], lo);
+    atomicMax(&info[1], hi);
+    if (bad) atomicOr(&info[2], 1);
+  }
+}
+__global__ void init_range_kernel(int *info) {
+  if (threadIdx.x < 2) {
+    info[threadIdx.x * 4 + 0] = 1 << 20;
+    info[threadIdx.x * 4 + 1] = -(1 << 20);
+    info[threadIdx.x * 4 + 2] = 0;
+    info[threadIdx.x * 4 + 3] = 0;
+  }
+}
+
+__global__ void cast_shift_kernel(const float *__restrict__ x, size_t len, int shift, uint8_t *__restrict__ out) {
+  GRID_STRIDE(i, len) out[i] = (uint8_t)((int)x[i] + shift);
+}
+
+// one wavefront per row of the u8 matrix
+__global__ void row_sum_u8_kernel(const uint8_t *__restrict__ a, size_t m, size_t k, int32_t *__restrict__ rs) {
+  const size_t row = blockIdx.x * (size_t)(blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= m) return;
+  const int lane = threadIdx.x & 63;
+  int s = 0;
+  for (size_t c = lane; c < k; c += 64) s += a[row * k + c];
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+  if (lane == 0) rs[row] = s;
+}
+
+// mode 0: out = f32(acc')                 (MatMulInteger)
+// mode 1: out = clamp(round(f32(acc') * composite + y_zp))       (QLinearMatMul fast path)
+// mode 2: out = clamp(round(f32(acc' * ab_scale) / y_scale + y_zp))  (QLinearMatMul, asymmetric)
+// acc' = acc - b_zp * (rs[i] - k_azp) when rs != null
+__global__ void mm_post_kernel(const int32_t *__restrict__ acc, const int32_t *__restrict__ rs, int b_zp, int k_azp,
+                               size_t m, size_t n, int mode, float composite, double ab_scale, float y_scale,
+                               float y_zp, float *__restrict__ out) {
+  GRID_STRIDE(i, m * n) {
+    int32_t a = acc[i];
+    if (rs) a = (int32_t)((uint32_t)a - (uint32_t)b_zp * ((uint32_t)rs[i / n] - (uint32_t)k_azp));  // wraps like the sum itself
+    float r;
+    if (mode == 0) {
+      r = (float)a;
+    } else if (mode == 1) {
+      r = clamp_keep_nan(round_half_away(__fadd_rn(__fmul_rn((float)a, composite), y_zp)), -128.0f, 127.0f);
+    } else {
+      float v = (float)((double)a * ab_scale);
+      r = clamp_keep_nan(round_half_away(__fadd_rn(__fdiv_rn(v, y_scale), y_zp)), -128.0f, 127.0f);
+    }
+    out[i] = r;
+  }
+}
+
+// Plain f32 product of the dequantised operands in k order; mode as in mm_post_kernel (0 rounds the sum,
+// 2 requantises it).  One output element per lane, B read coalesced along n.
+__global__ void f32_fallback_kernel(const float *__restrict__ a, const float *__restrict__ b, size_t m, size_t k,
+                                    size_t n, float a_zp, float a_scale, float b_zp, float b_scale, int mode,
+                                    float y_scale, float y_zp, float *__restrict__ out) {
+  const size_t j = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  const size_t i = blockIdx.y;
+  if (j >= n || i >= m) return;
+  float s = 0.0f;
+  for (size_t kk = 0; kk < k; kk++) {
+    float av = __fsub_rn(a[i * k + kk], a_zp);
+    float bv = __fsub_rn(b[kk * n + j], b_zp);
+    if (mode == 2) {
+      av = __fmul_rn(av, a_scale);
+      bv = __fmul_rn(bv, b_scale);
+    }
+    s = __fadd_rn(s, __fmul_rn(av, bv));
+  }
+  out[i * n + j] = (mode == 0)
+                       ? round_half_away(s)
+                       : clamp_keep_nan(round_half_away(__fadd_rn(__fdiv_rn(s, y_scale), y_zp)), -128.0f, 127.0f);
+}
+
+__global__ void quantize_linear_f32_kernel(const float *__restrict__ x, size_t len, float scale, float zp,
+                                           float *__restrict__ out) {
+  GRID_STRIDE(i, len) out[i] = clamp_keep_nan(rintf(__fadd_rn(__fdiv_rn(x[i], scale), zp)), -128.0f, 127.0f);
+}
+
+// scales / zps: one entry (chan == 1) or one per index of the quantisation axis
+__global__ void dequantize_linear_f32_kernel(const float *__restrict__ q, size_t len, size_t chan, size_t inner,
+                                             const float *__restrict__ scales, const float *__restrict__ zps,
+                                             float *__restrict__ out) {
+  GRID_STRIDE(i, len) {
+    const size_t c = chan == 1 ? 0 : (i / inner) % chan;
+    const float zp = zps ? zps[c] : 0.0f;
+    out[i] = __fmul_rn(__fsub_rn(q[i], zp), scales[c]);
+  }
+}
+
+__global__ void u8_to_f32_kernel(const uint8_t *__restrict__ q, size_t len, const float *__restrict__ scale_zp,
+                                 float *__restrict__ y, float *__restrict__ scale_out, float *__restrict__ zp_out) {
+  GRID_STRIDE(i, len) y[i] = (float)q[i];
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *scale_out = scale_zp[0];
+    *zp_out = scale_zp[1];
+  }
+}
+
+struct Operand8 {
+  DevBuf buf;
+  int shift = 0;    // added to every value
+  bool ok = false;  // values are integers that fit the 8-bit target after the shift
+};
+
+bool is_int_in(float v, int lo, int hi) { return v == (float)(int)v && (int)v >= lo && (int)v <= hi; }
+
+int32_t free_weight(yscv_hip_i8_weight *w) {
+  if (!w) return YSCV_HIP_OK;
+  if (w->frag) (void)hipFree(w->frag);
+  if (w->col_sum) (void)hipFree(w->col_sum);
+  delete w;
+  return YSCV_HIP_OK;
+}
+
+// device i8 [k][n] -> fragment layout + column sums
+int32_t pack_device_i8(const int8_t *b_kn, size_t k, size_t n, hipStream_t s, yscv_hip_i8_weight **out) {
+  auto *b = new yscv_hip_i8_weight();
+  b->k = k;
+  b->n = n;
+  b->kp = round_up(k, 64);
+  b->np = round_up(n, 16);
+  hipError_t e = hipMalloc(reinterpret_cast<void **>(&b->frag), b->kp * b->np);
+  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&b->col_sum), b->np * sizeof(int32_t));
+  int32_t st = YSCV_HIP_OK;
+  if (e == hipSuccess) st = launch_i8_pack_b(b_kn, k, n, b->kp, b->np, b->frag, b->col_sum, s);
+  if (e != hipSuccess || st != YSCV_HIP_OK) {
+    free_weight(b);
+    if (st != YSCV_HIP_OK) return st;
+    return set_error(e == hipErrorOutOfMemory ? YSCV_HIP_ERR_OOM : YSCV_HIP_ERR_DEVICE, "packing B failed: %s",
+                     hipGetErrorString(e));
+  }
+  b->device_bytes = b->kp * b->np + b->np * sizeof(int32_t);
+  *out = b;
+  return YSCV_HIP_OK;
+}
+
+struct TempWeight {
+  yscv_hip_i8_weight *w = nullptr;
+  ~TempWeight() { free_weight(w); }
+};
+
+enum : int { OP_MATMUL_INTEGER = 0, OP_QLINEAR = 1 };
+
+struct MatmulArgs {
+  int op;
+  const float *a;
+  const float *b;                     // [k][n] carrier or null
+  const yscv_hip_i8_weight *b_packed;  // or null
+  size_t m, k, n;
+  float a_scale, a_zp, b_scale, b_zp, y_scale, y_zp;
+  float *out;
+  hipStream_t s;
+};
+
+int32_t run_fast(const MatmulArgs &g) {
+  DevBuf a8, b8, acc;
+  YSCV_TRY(a8.alloc(g.m * g.k));
+  YSCV_TRY(acc.alloc(g.m * g.n * sizeof(int32_t)));
+  hipLaunchKernelGGL(cast_as_i8_kernel, dim3(grid_for(g.m * g.k)), dim3(256), 0, g.s, g.a, g.m * g.k, 0, a8.as<int8_t>());
+  TempWeight tmp;
+  const yscv_hip_i8_weight *w = g.b_packed;
+  if (!w) {
+    YSCV_TRY(b8.alloc(g.k * g.n));
+    hipLaunchKernelGGL(cast_as_i8_kernel, dim3(grid_for(g.k * g.n)), dim3(256), 0, g.s, g.b, g.k * g.n, 0,
+                       b8.as<int8_t>());
+    YSCV_TRY(pack_device_i8(b8.as<int8_t>(), g.k, g.n, g.s, &tmp.w));
+    w = tmp.w;
+  }
+  I8Epilogue ep{};
+  ep.mode = 0;
+  YSCV_TRY(launch_i8_gemm(a8.p, 0, 0, w, g.m, acc.p, ep, g.s));
+  const float composite = g.op == OP_QLINEAR ? (g.a_scale * g.b_scale) / g.y_scale : 0.0f;
+  hipLaunchKernelGGL(mm_post_kernel, dim3(grid_for(g.m * g.n)), dim3(256), 0, g.s, acc.as<int32_t>(),
+                     (const int32_t *)nullptr, 0, 0, g.m, g.n, g.op == OP_QLINEAR ? 1 : 0, composite, 0.0, g.y_scale,
+                     g.y_zp, g.out);
+  YSCV_HIP_TRY(hipGetLastError());
+  YSCV_HIP_TRY(hipStreamSynchronize(g.s));  // the scratch buffers are released on return
+  return YSCV_HIP_OK;
+}
+
+int32_t run_fallback(const MatmulArgs &g, int *took_integer_route) {
+  *took_integer_route = 0;
+  // operand ranges decide whether the exact integer route applies
+  DevBuf info;
+  YSCV_TRY(info.alloc(8 * sizeof(int)));
+  int h[8] = {0};
+  bool integer_route = g.k * (size_t)65025 < ((size_t)1 << 31) && is_int_in(g.a_zp, -128, 255) &&
+                       is_int_in(g.b_zp, -128, 255);
+  if (integer_route && !g.b) integer_route = g.b_zp == 0.0f;  // a packed B was cast without a shift
+  if (integer_route) {
+    hipLaunchKernelGGL(init_range_kernel, dim3(1), dim3(64), 0, g.s, info.as<int>());
+    hipLaunchKernelGGL(scan_int_range_kernel, dim3(grid_for(g.m * g.k)), dim3(256), 0, g.s, g.a, g.m * g.k,
+                       info.as<int>());
+    if (g.b)
+      hipLaunchKernelGGL(scan_int_range_kernel, dim3(grid_for(g.k * g.n)), dim3(256), 0, g.s, g.b, g.k * g.n,
+                         info.as<int>() + 4);
+    YSCV_HIP_TRY(hipMemcpyAsync(h, info.p, sizeof(h), hipMemcpyDeviceToHost, g.s));
+    YSCV_HIP_TRY(hipStreamSynchronize(g.s));
+  }
+  // shift A into u8 (by 0 or 128) so that its zero point fits as well; shift B into i8 (by 0 or -128)
+  int sa = 0, sb = 0;
+  if (integer_route) {
+    const int zp = (int)g.a_zp;
+    auto fits = [&](int sh) { return h[0] + sh >= 0 && h[1] + sh <= 255 && zp + sh >= 0 && zp + sh <= 255; };
+    if (h[2] || (g.m * g.k > 0 && !fits(0) && !fits(128))) integer_route = false;
+    else sa = fits(0) ? 0 : 128;
+  }
+  if (integer_route && g.b) {
+    if (h[6]) integer_route = false;
+    else if (h[4] >= -128 && h[5] <= 127) sb = 0;
+    else if (h[4] >= 0 && h[5] <= 255) sb = -128;
+    else integer_route = false;
+  }
+  const int azp = (int)g.a_zp + sa, bzp = (int)g.b_zp + sb;
+
+  if (!integer_route) {
+    YSCV_REQUIRE(g.b != nullptr,
+                 "operands are not 8-bit integers (or the zero points do not fit); the f32 route needs the unpacked B");
+    dim3 grid((unsigned)ceil_div(g.n, (size_t)256), (unsigned)g.m);
+    YSCV_REQUIRE(g.m <= 65535, "f32 route: m=%zu exceeds 65535 rows", g.m);
+    hipLaunchKernelGGL(f32_fallback_kernel, grid, dim3(256), 0, g.s, g.a, g.b, g.m, g.k, g.n, g.a_zp, g.a_scale,
+                       g.b_zp, g.b_scale, g.op == OP_QLINEAR ? 2 : 0, g.y_scale, g.y_zp, g.out);
+    YSCV_HIP_TRY(hipGetLastError());
+    return YSCV_HIP_OK;
+  }
+
+  *took_integer_route = 1;
+  DevBuf a8, b8, acc, rs;
+  YSCV_TRY(a8.alloc(g.m * g.k));
+  YSCV_TRY(acc.alloc(g.m * g.n * sizeof(int32_t)));
+  YSCV_TRY(rs.alloc(g.m * sizeof(int32_t)));
+  hipLaunchKernelGGL(cast_shift_kernel, dim3(grid_for(g.m * g.k)), dim3(256), 0, g.s, g.a, g.m * g.k, sa,
+                     a8.as<uint8_t>());
+  TempWeight tmp;
+  const yscv_hip_i8_weight *w = g.b_packed;
+  if (g.b) {
+    YSCV_TRY(b8.alloc(g.k * g.n));
+    hipLaunchKernelGGL(cast_shift_kernel, dim3(grid_for(g.k * g.n)), dim3(256), 0, g.s, g.b, g.k * g.n, sb,
+                       b8.as<uint8_t>());
+    YSCV_TRY(pack_device_i8(b8.as<int8_t>(), g.k, g.n, g.s, &tmp.w));
+    w = tmp.w;
+  }
+  const bool need_rs = bzp != 0;
+  if (need_rs)
+    hipLaunchKernelGGL(row_sum_u8_kernel, dim3((unsigned)ceil_div(g.m, (size_t)4)), dim3(256), 0, g.s,
+                       a8.as<uint8_t>(), g.m, g.k, rs.as<int32_t>());
+  I8Epilogue ep{};
+  ep.mode = 0;
+  YSCV_TRY(launch_i8_gemm(a8.p, 1, azp, w, g.m, acc.p, ep, g.s));
+  hipLaunchKernelGGL(mm_post_kernel, dim3(grid_for(g.m * g.n)), dim3(256), 0, g.s, acc.as<int32_t>(),
+                     need_rs ? rs.as<int32_t>() : (const int32_t *)nullptr, bzp, (int)g.k * azp, g.m, g.n,
+                     g.op == OP_QLINEAR ? 2 : 0, 0.0f, (double)g.a_scale * (double)g.b_scale, g.y_scale, g.y_zp,
+                     g.out);
+  YSCV_HIP_TRY(hipGetLastError());
+  YSCV_HIP_TRY(hipStreamSynchronize(g.s));
+  return YSCV_HIP_OK;
+}
+
+int32_t run_matmul(const MatmulArgs &g, int32_t *path_out) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(g.b || g.b_packed, "neither an unpacked nor a packed B given");
+  YSCV_REQUIRE(g.k > 0 && g.n > 0, "bad shape k=%zu n=%zu", g.k, g.n);
+  if (g.b_packed)
+    YSCV_REQUIRE(g.b_packed->k == g.k && g.b_packed->n == g.n, "prepacked weight shape mismatch: packed %zux%zu, op %zux%zu",
+                 g.b_packed->k, g.b_packed->n, g.k, g.n);
+  const bool fast = g.a_zp == 0.0f && g.b_zp == 0.0f;
+  auto &fast_ctr = g.op == OP_QLINEAR ? g_qlinear_fast : g_mmi_fast;
+  auto &fb_ctr = g.op == OP_QLINEAR ? g_qlinear_fallback : g_mmi_fallback;
+  int32_t path = fast ? YSCV_HIP_PATH_FAST : YSCV_HIP_PATH_FALLBACK_F32;
+  if (g.m > 0) {
+    YSCV_REQUIRE(g.a && g.out, "null a / out pointer");
+    if (fast) {
+      YSCV_TRY(run_fast(g));
+    } else {
+      int integer_route = 0;
+      YSCV_TRY(run_fallback(g, &integer_route));
+      if (integer_route) path = YSCV_HIP_PATH_FALLBACK_EXACT;
+    }
+  }
+  (fast ? fast_ctr : fb_ctr).fetch_add(1, std::memory_order_relaxed);
+  if (path_out) *path_out = path;
+  return YSCV_HIP_OK;
+}
+
+}  // namespace
+
+void note_int4_fast() { g_int4_fast.fetch_add(1, std::memory_order_relaxed); }
+void note_int4_fallback() { g_int4_fallback.fetch_add(1, std::memory_order_relaxed); }
+
+}  // namespace yscv
+
+using namespace yscv;
+
+extern "C" {
+
+int32_t yscv_hip_quant_runtime_stats(yscv_hip_quant_stats *out) {
+  YSCV_REQUIRE(out != nullptr, "null stats pointer");
+  out->qlinear_matmul_fast = g_qlinear_fast.load(std::memory_order_relaxed);
+  out->qlinear_matmul_fallback = g_qlinear_fallback.load(std::memory_order_relaxed);
+  out->matmul_integer_fast = g_mmi_fast.load(std::memory_order_relaxed);
+  out->matmul_integer_fallback = g_mmi_fallback.load(std::memory_order_relaxed);
+  out->int4_fast = g_int4_fast.load(std::memory_order_relaxed);
+  out->int4_fallback = g_int4_fallback.load(std::memory_order_relaxed);
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_reset_quant_runtime_stats(void) {
+  for (auto *c : {&g_qlinear_fast, &g_qlinear_fallback, &g_mmi_fast, &g_mmi_fallback, &g_int4_fast, &g_int4_fallback})
+    c->store(0, std::memory_order_relaxed);
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_quant_int8_fast_enabled(void) {
+  const char *v = std::getenv("YSCV_QUANT_INT8_FAST");
+  return (v != nullptr && v[0] == '0' && v[1] == '\0') ? 0 : 1;
+}
+
+int32_t yscv_hip_should_use_prepacked_i8_b(size_t m, size_t k, size_t n) {
+  return ((m >= 4 && k >= 4 && n >= 32 && n % 16 == 0) || (m <= 64 && k >= 512 && n >= 1024)) ? 1 : 0;
+}
+
+int32_t yscv_hip_should_prepack_i8_b(size_t k, size_t n) {
+  return ((k >= 4 && n % 16 == 0) || (k >= 512 && n >= 1024)) ? 1 : 0;
+}
+
+int32_t yscv_hip_i8_weight_from_f32(const float *b_dev, size_t k, size_t n, void *stream, yscv_hip_i8_weight **out) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(out != nullptr, "null output handle pointer");
+  *out = nullptr;
+  YSCV_REQUIRE(b_dev != nullptr, "null b");
+  YSCV_REQUIRE(k > 0 && n > 0 && k < (1u << 30) && n < (1u << 30), "bad shape k=%zu n=%zu", k, n);
+  hipStream_t s = as_stream(stream);
+  DevBuf b8;
+  YSCV_TRY(b8.alloc(k * n));
+  hipLaunchKernelGGL(cast_as_i8_kernel, dim3(grid_for(k * n)), dim3(256), 0, s, b_dev, k * n, 1, b8.as<int8_t>());
+  YSCV_TRY(pack_device_i8(b8.as<int8_t>(), k, n, s, out));
+  hipError_t e = hipStreamSynchronize(s);
+  if (e != hipSuccess) {
+    free_weight(*out);
+    *out = nullptr;
+    return set_error(YSCV_HIP_ERR_DEVICE, "packing B failed: %s", hipGetErrorString(e));
+  }
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_exec_matmul_integer(const float *a_dev, const float *b_dev, const yscv_hip_i8_weight *b_packed,
+                                     float a_zp, float b_zp, size_t m, size_t k, size_t n, float *out_dev,
+                                     int32_t *path_out, void *stream) {
+  MatmulArgs g{OP_MATMUL_INTEGER, a_dev, b_dev, b_packed, m, k, n, 1.0f, a_zp, 1.0f, b_zp, 1.0f, 0.0f, out_dev,
+               as_stream(stream)};
+  return run_matmul(g, path_out);
+}
+
+int32_t yscv_hip_exec_qlinear_matmul(const float *a_dev, float a_scale, float a_zp, const float *b_dev,
+                                     const yscv_hip_i8_weight *b_packed, float b_scale, float b_zp, float y_scale,
+                                     float y_zp, size_t m, size_t k, size_t n, float *out_dev, int32_t *path_out,
+                                     void *stream) {
+  MatmulArgs g{OP_QLINEAR, a_dev, b_dev, b_packed, m, k, n, a_scale, a_zp, b_scale, b_zp, y_scale, y_zp, out_dev,
+               as_stream(stream)};
+  return run_matmul(g, path_out);
+}
+
+int32_t yscv_hip_exec_quantize_linear(const float *x_dev, size_t len, float scale, float zero_point, float *out_dev,
+                                      void *stream) {
+  YSCV_TRY(ensure_context(nullptr));
+  if (len == 0) return YSCV_HIP_OK;
+  YSCV_REQUIRE(x_dev && out_dev, "null pointer");
+  hipLaunchKernelGGL(quantize_linear_f32_kernel, dim3(grid_for(len)), dim3(256), 0, as_stream(stream), x_dev, len,
+                     scale, zero_point, out_dev);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_exec_dequantize_linear(const float *q_dev, size_t outer, size_t chan, size_t inner,
+                                        const float *scales_dev, const float *zps_dev, size_t n_scales,
+                                        float *out_dev, void *stream) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(scales_dev != nullptr, "null scale pointer");
+  YSCV_REQUIRE(n_scales == 1 || n_scales == chan, "DequantizeLinear: scale len=%zu but axis dim=%zu", n_scales, chan);
+  const size_t len = outer * chan * inner;
+  if (len == 0) return YSCV_HIP_OK;
+  YSCV_REQUIRE(q_dev && out_dev, "null pointer");
+  hipLaunchKernelGGL(dequantize_linear_f32_kernel, dim3(grid_for(len)), dim3(256), 0, as_stream(stream), q_dev, len,
+                     n_scales == 1 ? (size_t)1 : chan, inner, scales_dev, zps_dev, out_dev);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_exec_dynamic_quantize_linear(const float *x_dev, size_t len, float *y_dev, float *y_scale_dev,
+                                              float *y_zp_dev, void *stream) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(y_scale_dev && y_zp_dev, "null scale / zero-point pointer");
+  YSCV_REQUIRE(len == 0 || (x_dev && y_dev), "null pointer");
+  hipStream_t s = as_stream(stream);
+  DevBuf q, sz;
+  YSCV_TRY(q.alloc(len));
+  YSCV_TRY(sz.alloc(2 * sizeof(float)));
+  YSCV_TRY(launch_dynamic_quantize_linear(x_dev, len, q.as<uint8_t>(), sz.as<float>(), s));
+  hipLaunchKernelGGL(u8_to_f32_kernel, dim3(grid_for(len)), dim3(256), 0, s, q.as<uint8_t>(), len, sz.as<float>(),
+                     y_dev, y_scale_dev, y_zp_dev);
+  YSCV_HIP_TRY(hipGetLastError());
+  YSCV_HIP_TRY(hipStreamSynchronize(s));
+  return YSCV_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,184 @@
+"""Host-side mirror of the reference runner's quantised operators over the C ABI.
+
+Function names and argument meaning follow crates/yscv-onnx/src/runner/linear.rs (exec_matmul_integer :648,
+exec_qlinear_matmul :438), crates/yscv-onnx/src/runner/misc.rs (exec_quantize_linear :42, exec_dequantize_linear
+:110, exec_dynamic_quantize_linear :241) and crates/yscv-onnx/src/runner/quant_stats.rs.  Tensors are torch CUDA
+f32 tensors used as device buffers (the reference keeps every quantised value in an f32 tensor as well); all
+arithmetic happens inside libyscv_hip.so.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+from .capi import PATH_FALLBACK_EXACT, PATH_FALLBACK_F32, PATH_FAST, QuantStats, lib  # noqa: F401
+
+_sz = C.c_size_t
+
+
+def _stream_ptr():
+    import torch
+
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev_f32(t, name):
+    import torch
+
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float32):
+        raise TypeError(f"{name}: expected a CUDA float32 tensor")
+    return t.contiguous()
+
+
+def _p(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+@dataclass(frozen=True)
+class QuantRuntimeStats:
+    """quant_stats.rs:6-22, restricted to the matmul path, plus the int4 and MatMulInteger splits."""
+
+    qlinear_matmul_fast: int = 0
+    qlinear_matmul_fallback: int = 0
+    matmul_integer_fast: int = 0
+    matmul_integer_fallback: int = 0
+    int4_fast: int = 0
+    int4_fallback: int = 0
+
+
+def quant_runtime_stats() -> QuantRuntimeStats:
+    s = QuantStats()
+    lib().quant_runtime_stats(C.byref(s))
+    return QuantRuntimeStats(**{n: int(getattr(s, n)) for n, _ in QuantStats._fields_})
+
+
+def reset_quant_runtime_stats() -> None:
+    lib().reset_quant_runtime_stats()
+
+
+def quant_int8_fast_enabled() -> bool:
+    return bool(lib().quant_int8_fast_enabled())
+
+
+def should_use_prepacked_i8_b(m: int, k: int, n: int) -> bool:
+    return bool(lib().should_use_prepacked_i8_b(m, k, n))
+
+
+def should_prepack_i8_b(k: int, n: int) -> bool:
+    return bool(lib().should_prepack_i8_b(k, n))
+
+
+class PrepackedI8B:
+    """Load-time prepack of a weight initialiser given as an f32 carrier [k][n] (plan/build.rs:1367-1454)."""
+
+    def __init__(self, b):
+        b = _dev_f32(b, "b")
+        if b.dim() != 2:
+            raise ValueError("prepack takes a rank-2 weight")
+        self.k, self.n = int(b.shape[0]), int(b.shape[1])
+        h = C.c_void_p()
+        lib().i8_weight_from_f32(_p(b), _sz(self.k), _sz(self.n), _stream_ptr(), C.byref(h))
+        self._h = h
+
+    @property
+    def handle(self):
+        return self._h
+
+    def close(self):
+        if self._h:
+            lib().i8_weight_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def _matmul_operands(a, b, prepacked):
+    import torch
+
+    a = _dev_f32(a, "a")
+    if a.dim() != 2:
+        raise ValueError("a must be rank 2 (flatten leading dimensions into m)")
+    m, k = int(a.shape[0]), int(a.shape[1])
+    if b is not None:
+        b = _dev_f32(b, "b")
+        if b.dim() != 2 or int(b.shape[0]) != k:
+            raise ValueError("b must be [k][n] with k = a.shape[1]")
+        n = int(b.shape[1])
+    elif prepacked is not None:
+        n = prepacked.n
+    else:
+        raise ValueError("neither b nor a prepacked weight given")
+    out = torch.empty(m, n, device=a.device, dtype=torch.float32)
+    return a, b, m, k, n, out
+
+
+def exec_matmul_integer(a, b=None, a_zp: float = 0.0, b_zp: float = 0.0, prepacked: PrepackedI8B | None = None):
+    """linear.rs:648-737.  Returns (out [m][n] f32, path)."""
+    a, b, m, k, n, out = _matmul_operands(a, b, prepacked)
+    path = C.c_int32(-1)
+    lib().exec_matmul_integer(_p(a), _p(b), prepacked.handle if prepacked is not None else None, C.c_float(a_zp),
+                              C.c_float(b_zp), _sz(m), _sz(k), _sz(n), _p(out), C.byref(path), _stream_ptr())
+    return out, path.value
+
+
+def exec_qlinear_matmul(a, a_scale, a_zp, b, b_scale, b_zp, y_scale, y_zp, prepacked: PrepackedI8B | None = None):
+    """linear.rs:438-538.  Returns (out [m][n] f32 holding values in [-128, 127], path)."""
+    a, b, m, k, n, out = _matmul_operands(a, b, prepacked)
+    path = C.c_int32(-1)
+    lib().exec_qlinear_matmul(_p(a), C.c_float(a_scale), C.c_float(a_zp), _p(b),
+                              prepacked.handle if prepacked is not None else None, C.c_float(b_scale),
+                              C.c_float(b_zp), C.c_float(y_scale), C.c_float(y_zp), _sz(m), _sz(k), _sz(n), _p(out),
+                              C.byref(path), _stream_ptr())
+    return out, path.value
+
+
+def exec_quantize_linear(x, scale: float, zero_point: float = 0.0):
+    """misc.rs:42-80 (f32-carrier arm): clamp(round_ties_even(x / scale + zp), -128, 127) as f32."""
+    import torch
+
+    x = _dev_f32(x, "x")
+    out = torch.empty_like(x)
+    lib().exec_quantize_linear(_p(x), _sz(x.numel()), C.c_float(scale), C.c_float(zero_point), _p(out), _stream_ptr())
+    return out
+
+
+def exec_dequantize_linear(q, scale, zero_point=None, axis: int = 1):
+    """misc.rs:110-239: (q - zp) * scale, per tensor (one scale) or per channel along `axis`."""
+    import torch
+
+    q = _dev_f32(q, "q")
+    scale = _dev_f32(scale.reshape(-1) if hasattr(scale, "reshape") else torch.tensor([scale], device=q.device), "scale")
+    if zero_point is not None:
+        zero_point = _dev_f32(zero_point.reshape(-1) if hasattr(zero_point, "reshape")
+                              else torch.tensor([zero_point], device=q.device, dtype=torch.float32), "zero_point")
+    if scale.numel() == 1:
+        outer, chan, inner = 1, 1, q.numel()
+    else:
+        ax = axis + q.dim() if axis < 0 else axis
+        shape = list(q.shape)
+        outer = 1
+        for d in shape[:ax]:
+            outer *= d
+        chan = shape[ax]
+        inner = 1
+        for d in shape[ax + 1:]:
+            inner *= d
+    out = torch.empty_like(q)
+    lib().exec_dequantize_linear(_p(q), _sz(outer), _sz(chan), _sz(inner), _p(scale), _p(zero_point),
+                                 _sz(scale.numel()), _p(out), _stream_ptr())
+    return out
+
+
+def exec_dynamic_quantize_linear(x):
+    """misc.rs:241-289.  Returns (y f32 in [0, 255], y_scale [1], y_zp [1]) as device tensors."""
+    import torch
+
+    x = _dev_f32(x, "x")
+    y = torch.empty_like(x)
+    sz = torch.empty(2, device=x.device, dtype=torch.float32)
+    lib().exec_dynamic_quantize_linear(_p(x), _sz(x.numel()), _p(y), _p(sz[0:1]), _p(sz[1:2]), _stream_ptr())
+    return y, sz[0:1], sz[1:2]
