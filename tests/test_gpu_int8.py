@@ -83,6 +83,38 @@ def test_config2_full_size_bit_exact(oracle, K, torch_cuda):
     assert q.dtype == np.int8 and np.array_equal(q.astype(np.int32), q_exp)
 
 
+# k a multiple of 64: the LDS-ring kernel.  Row / column tails, column counts that are not multiples of 4 or 16,
+# several ring revolutions, and sizes on both sides of the 64x128 / 128x128 tile switch (256 big tiles).
+RING_SHAPES = [(1, 64, 1), (65, 256, 129), (70, 2048, 250), (130, 1024, 260), (257, 4096, 515), (33, 192, 1030),
+               (2048, 512, 2048), (2100, 320, 2050), (1999, 1088, 2500)]
+
+
+@pytest.mark.parametrize("m,k,n", RING_SHAPES)
+@pytest.mark.parametrize("signed", [False, True])
+def test_ring_kernel_shapes_bit_exact(oracle, K, torch_cuda, m, k, n, signed):
+    torch = torch_cuda
+    rng = np.random.default_rng(m * 31 + k * 7 + n + int(signed))
+    a = rng.integers(-128, 128, (m, k)).astype(np.int8) if signed else rng.integers(0, 256, (m, k)).astype(np.uint8)
+    b = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    zp = 0 if signed else int(rng.integers(0, 256))
+    # float64 holds these sums exactly (|sum| < 2^31 << 2^53), so BLAS gives the integer reference quickly
+    exp = ((a.astype(np.float64) - zp) @ b.astype(np.float64)).astype(np.int64)
+    rows = [0, m // 2, m - 1]
+    sub = (a[rows].astype(np.int64) - zp) @ b.astype(np.int64)  # the same rows in integer arithmetic
+    assert np.array_equal(exp[rows], sub)
+    packed = K.pack_i8_b_for_matmul(b, k, n)
+    a_dev = torch.from_numpy(a).cuda()
+    got = packed.matmul(a_dev, a_zp=zp).cpu().numpy()
+    assert np.array_equal(got, exp.astype(np.int32))
+    corr = rng.integers(-3000, 3000, n, dtype=np.int32)
+    comp = rng.uniform(2e-5, 4e-4, n).astype(np.float32)
+    lo, hi = (-128, 127) if signed else (0, 255)
+    q = packed.matmul_requant(a_dev, zp, torch.from_numpy(comp).cuda(), 7.0, K.ROUND_HALF_AWAY, lo, hi,
+                              corr=torch.from_numpy(corr).cuda()).cpu().numpy()
+    q_exp = oracle.requant_general(exp.astype(np.int32), n, corr, comp, 7.0, K.ROUND_HALF_AWAY, lo, hi)
+    assert np.array_equal(q.astype(np.int32), np.asarray(q_exp).reshape(m, n))
+
+
 @pytest.mark.parametrize("zp", [0, 3, 128, 255])
 def test_u8_zero_points(oracle, K, torch_cuda, zp):
     torch = torch_cuda

@@ -16,6 +16,9 @@
 // uint8 activations are fed to the signed MFMA as (a ^ 0x80) = a - 128, the same bias shift
 // the reference uses for VNNI (int8_matmul.rs:1866-1868); the epilogue adds
 // (128 - a_zp) * colsum(b), the algebra of runner/conv/quantized.rs:119-147.
+#include <mutex>
+#include <utility>
+
 #include "int4_common.hpp"
 #include "kernels.hpp"
 
@@ -227,6 +230,277 @@ __global__ void __launch_bounds__(I8_THREADS) i8_gemm_kernel(I8Args p) {
   }
 }
 
+// ---- ring kernel: both operands stream through an LDS ring filled by LDS-direct loads -----------------
+// Used when k is a multiple of 64 and A is 16-byte aligned.  A workgroup has four compute waves (2 x 2) and four
+// producer waves.  It owns a (32 MT) x (32 NT) tile of C, a compute wave MT x NT MFMA tiles of it.  A stage holds
+// KS k-steps of 64: the A part in fragment order [m-tile][ks][lane][16 B] (each lane fetches its own 16 bytes of a
+// row, so the row-major -> fragment transposition costs nothing), the B part [n-tile][ks][lane][16 B] copied as
+// it lies in memory.  S stages form a ring: while the MFMAs of stage i run, the producers have the loads of
+// stages i+1 .. i+S-1 in flight, track them with their own vmcnt and publish a landed stage with one s_barrier
+// per stage; the compute waves never issue a global load, so their MFMAs do not queue behind the address
+// processing of the loads.  The MFMA is issued with the operands swapped, D = Bfrag x Afrag, which yields the
+// transposed tile: a lane holds four consecutive columns of one row of C.  The finished tile goes through LDS so
+// that all eight waves store whole rows of it (512 contiguous bytes of int32, 128 of requantised bytes).
+// Workgroups are numbered so that the ones sharing an XCD (id mod 8) cover a contiguous range of n-tiles over
+// all m-tiles: an XCD's L2 holds its slice of B once.
+typedef __attribute__((address_space(3))) void lds_void;
+#define I8_AS1(ptr) ((const void __attribute__((address_space(1))) *)(ptr))
+constexpr int I8R_THREADS = 512;
+
+template <int N>
+__device__ __forceinline__ void i8_wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+// one fragment read; the value is valid only after i8_frags_wait
+template <int OFF>
+__device__ __forceinline__ void i8_ds_read(int4_t &v, uint32_t addr) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int MT, int NT>
+struct I8Frags {
+  int4_t a[MT], b[NT];
+};
+template <int KS, int MT, int NT, int... I, int... J>
+__device__ __forceinline__ void i8_frags_issue_impl(I8Frags<MT, NT> &f, uint32_t a_addr, uint32_t b_addr,
+                                                    std::integer_sequence<int, I...>, std::integer_sequence<int, J...>) {
+  (i8_ds_read<I * KS * 1024>(f.a[I], a_addr), ...);
+  (i8_ds_read<J * KS * 1024>(f.b[J], b_addr), ...);
+}
+template <int KS, int MT, int NT>
+__device__ __forceinline__ void i8_frags_issue(I8Frags<MT, NT> &f, uint32_t a_addr, uint32_t b_addr) {
+  i8_frags_issue_impl<KS>(f, a_addr, b_addr, std::make_integer_sequence<int, MT>{}, std::make_integer_sequence<int, NT>{});
+}
+template <int MT, int NT>
+__device__ __forceinline__ void i8_frags_wait(I8Frags<MT, NT> &f) {
+  if constexpr (MT == 2 && NT == 4) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]), "+v"(f.b[3])::"memory");
+  } else {
+    static_assert(MT == 4 && NT == 4, "add a wait for this fragment count");
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]),
+                   "+v"(f.b[3])::"memory");
+  }
+}
+
+template <int MT, int NT, int KS, int S>
+__global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int tiles_m, int tiles_n) {
+  constexpr int BM = 32 * MT, BN = 32 * NT;
+  constexpr int A_BYTES = 2 * MT * KS * 1024, STAGE = 2 * (MT + NT) * KS * 1024;
+  constexpr int PER_WAVE = (MT + NT) * KS / 2;  // 1 KiB chunks a producer wave fetches per stage
+  static_assert(((MT + NT) * KS) % 2 == 0 && S >= 2 && S <= 7 && (S - 1) * PER_WAVE < 64, "vmcnt budget");
+  constexpr int RS32 = BN * 4 + 16, RS8 = BN + 16;  // row strides of the C tile in LDS (odd multiples of 16 B)
+  static_assert(BM * RS32 <= S * STAGE, "the C tile reuses the ring");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t i8_ring[];
+  const uint32_t lds0 = (uint32_t)(size_t)i8_ring;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, c = lane >> 4;
+
+  // XCD-aware tile numbering: the grid of tiles is cut into super-blocks of 8 x 4 tiles; workgroup ids that share
+  // an XCD (id mod 8) walk through one super-block at a time, so the 32 workgroups an XCD runs together read
+  // 8 row panels of A and 4 column panels of B between them.
+  const int sb_m = (tiles_m + 7) / 8;
+  const int j_in_xcd = (int)(blockIdx.x >> 3);
+  const int sb = (j_in_xcd >> 5) * 8 + (int)(blockIdx.x & 7);
+  const int tm = (sb % sb_m) * 8 + (j_in_xcd & 7), tn = (sb / sb_m) * 4 + ((j_in_xcd >> 3) & 3);
+  if (tm >= tiles_m || tn >= tiles_n) return;
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int nt_total = (p.n + 15) / 16;
+  const int nstages = (p.ksteps + KS - 1) / KS;
+
+  int4_t acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; i++)
+#pragma unroll
+    for (int j = 0; j < NT; j++) acc[i][j] = int4_t{0, 0, 0, 0};
+  const int wm = (wave >> 1) & 1, wn = wave & 1;
+
+  if (wave >= 4) {
+    // ---- producer: per-lane source addresses of this wave's chunks at k = 0 (chunk q < 2 MT KS: A, else B)
+    const int pw = wave - 4;
+    const uint8_t *src[PER_WAVE];
+#pragma unroll
+    for (int j = 0; j < PER_WAVE; j++) {
+      const int q = pw * PER_WAVE + j;
+      if (q < 2 * MT * KS) {
+        const int row = min(m0 + (q / KS) * 16 + r, p.m - 1);
+        src[j] = p.a + (size_t)row * p.k + c * 16;
+      } else {
+        const int gnt = min(n0 / 16 + (q - 2 * MT * KS) / KS, nt_total - 1);
+        src[j] = reinterpret_cast<const uint8_t *>(p.frag) + (size_t)gnt * p.ksteps * 1024 + lane * 16;
+      }
+    }
+    uint32_t fill_slot = 0;  // ring slot the next issued stage goes to
+    auto issue_stage = [&](int st) {
+      const uint32_t dst = lds0 + fill_slot + (uint32_t)(pw * PER_WAVE * 1024);
+      fill_slot = fill_slot + STAGE == S * STAGE ? 0 : fill_slot + STAGE;
+#pragma unroll
+      for (int j = 0; j < PER_WAVE; j++) {
+        const int q = pw * PER_WAVE + j;                      // wave-uniform
+        const bool is_a = q < 2 * MT * KS;
+        const int ks = (is_a ? q : q - 2 * MT * KS) % KS;
+        const int gks = min(st * KS + ks, p.ksteps - 1);       // k-steps past the end re-read the last one
+        const uint8_t *g = src[j] + (size_t)gks * (is_a ? 64 : 1024);
+        __builtin_amdgcn_global_load_lds(I8_AS1(g), (lds_void *)(uintptr_t)(dst + j * 1024), 16, 0, 0);
+      }
+    };
+    // wait until this wave's part of a stage has landed, given how many later stages it has in flight
+    auto wait_landed = [&](int later) {
+      switch (later) {
+        case 0: i8_wait_vm<0>(); break;
+        case 1: i8_wait_vm<PER_WAVE>(); break;
+        case 2: i8_wait_vm<(S > 2 ? 2 : 0) * PER_WAVE>(); break;
+        case 3: i8_wait_vm<(S > 3 ? 3 : 0) * PER_WAVE>(); break;
+        case 4: i8_wait_vm<(S > 4 ? 4 : 0) * PER_WAVE>(); break;
+        case 5: i8_wait_vm<(S > 5 ? 5 : 0) * PER_WAVE>(); break;
+        default: i8_wait_vm<(S > 6 ? 6 : 0) * PER_WAVE>(); break;
+      }
+    };
+    for (int st = 0; st < S; st++)
+      if (st < nstages) issue_stage(st);
+    wait_landed(min(S - 1, nstages - 1));
+    __builtin_amdgcn_s_barrier();
+    for (int st = 0; st + 1 < nstages; st++) {
+      // stages st+1 .. st+S-1 are in flight; after the barrier every compute wave is done with stage st
+      wait_landed(min(S - 2, nstages - 2 - st));
+      __builtin_amdgcn_s_barrier();
+      if (st + S < nstages) issue_stage(st + S);
+    }
+  } else {
+    // ---- compute -------------------------------------------------------------------------------------
+    const uint32_t a_lane = lds0 + (uint32_t)(wm * MT * KS * 1024 + lane * 16);
+    const uint32_t b_lane = lds0 + (uint32_t)(A_BYTES + wn * NT * KS * 1024 + lane * 16);
+    const int4_t xr = {p.a_xor, p.a_xor, p.a_xor, p.a_xor};
+    I8Frags<MT, NT> f[2];
+    __builtin_amdgcn_s_barrier();
+    i8_frags_issue<KS>(f[0], a_lane, b_lane);
+    auto mfmas = [&](I8Frags<MT, NT> &cur, int i0, int i1) {
+#pragma unroll
+      for (int i = i0; i < i1; i++) {
+        const int4_t av = cur.a[i] ^ xr;
+#pragma unroll
+        for (int j = 0; j < NT; j++) acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.b[j], av, acc[i][j], 0, 0, 0);
+      }
+    };
+    uint32_t slot = 0;
+    for (int st = 0; st < nstages; st++) {
+      const uint32_t nslot = slot + STAGE == S * STAGE ? 0 : slot + STAGE;
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        I8Frags<MT, NT> &cur = f[ks & 1], &nxt = f[(ks + 1) & 1];
+        const bool live = st * KS + ks < p.ksteps;  // false only in the padding of the last stage
+        i8_frags_wait(cur);
+        if (ks + 1 < KS) {
+          i8_frags_issue<KS>(nxt, a_lane + slot + (ks + 1) * 1024, b_lane + slot + (ks + 1) * 1024);
+          if (live) mfmas(cur, 0, MT);
+        } else {
+          // the first half of the MFMAs runs while this wave waits at the barrier, the second half while the
+          // first fragments of the next stage arrive
+          if (live) mfmas(cur, 0, MT / 2);
+          if (st + 1 < nstages) {
+            // every read of stage st by this wave has returned: tell the producers, pick up stage st+1
+            __builtin_amdgcn_s_barrier();
+            i8_frags_issue<KS>(nxt, a_lane + nslot, b_lane + nslot);
+          }
+          if (live) mfmas(cur, MT / 2, MT);
+        }
+      }
+      slot = nslot;
+    }
+  }
+  static_assert(KS % 2 == 0, "the two fragment sets alternate per k-step");
+
+  // ---- epilogue: the tile goes to LDS (lane (c, r) holds C[16 i + r][16 j + 4 c + 0..3] of its wave's part),
+  // then all waves store whole rows ---------------------------------------------------------------------
+  __syncthreads();  // every wave is done with the ring
+  const float lo = (float)p.lo, hi = (float)p.hi;
+  if (wave < 4) {
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+      const int lcol = wn * NT * 16 + j * 16 + c * 4;
+      int32_t zc[4], corr[4];
+      float comp[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const int cc = min(n0 + lcol + e, p.n - 1);
+        zc[e] = p.zp_mul * p.col_sum[cc];
+        corr[e] = p.corr ? p.corr[cc] : 0;
+        comp[e] = p.composite_v ? p.composite_v[cc] : p.composite;
+      }
+#pragma unroll
+      for (int i = 0; i < MT; i++) {
+        const int lrow = wm * MT * 16 + i * 16 + r;
+        int32_t v[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = (int32_t)((uint32_t)acc[i][j][e] + (uint32_t)zc[e]);
+        if (p.mode == 0) {
+          *reinterpret_cast<int4_t *>(i8_ring + lrow * RS32 + lcol * 4) = int4_t{v[0], v[1], v[2], v[3]};
+        } else {
+          uint32_t packed = 0;
+#pragma unroll
+          for (int e = 0; e < 4; e++)
+            packed |= (uint32_t)(uint8_t)requant_one(v[e], corr[e], comp[e], p.y_zp, p.round_mode, lo, hi) << (8 * e);
+          *reinterpret_cast<uint32_t *>(i8_ring + lrow * RS8 + lcol) = packed;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  if (p.mode == 0) {
+    constexpr int CPR = BN / 4;  // 16-byte chunks per row
+    const bool vec = (p.n & 3) == 0;
+    for (int q = tid; q < BM * CPR; q += I8R_THREADS) {
+      const int lrow = q / CPR, ch = q % CPR;
+      const int row = m0 + lrow, col = n0 + ch * 4;
+      if (row >= p.m || col >= p.n) continue;
+      const int4_t v = *reinterpret_cast<const int4_t *>(i8_ring + lrow * RS32 + ch * 16);
+      int32_t *out = reinterpret_cast<int32_t *>(p.out) + (size_t)row * p.n + col;
+      if (vec) {
+        *reinterpret_cast<int4_t *>(out) = v;
+      } else {
+        for (int e = 0; e < 4; e++)
+          if (col + e < p.n) out[e] = v[e];
+      }
+    }
+  } else {
+    constexpr int CPR = BN / 16;
+    const bool vec = (p.n & 15) == 0;
+    for (int q = tid; q < BM * CPR; q += I8R_THREADS) {
+      const int lrow = q / CPR, ch = q % CPR;
+      const int row = m0 + lrow, col = n0 + ch * 16;
+      if (row >= p.m || col >= p.n) continue;
+      const uint4_t v = *reinterpret_cast<const uint4_t *>(i8_ring + lrow * RS8 + ch * 16);
+      uint8_t *out = reinterpret_cast<uint8_t *>(p.out) + (size_t)row * p.n + col;
+      if (vec) {
+        *reinterpret_cast<uint4_t *>(out) = v;
+      } else {
+        for (int e = 0; e < 16; e++)
+          if (col + e < p.n) out[e] = (uint8_t)(v[e >> 2] >> (8 * (e & 3)));
+      }
+    }
+  }
+}
+
+template <int MT, int NT, int KS, int S>
+int32_t launch_ring(const I8Args &p, size_t m, size_t n, hipStream_t s) {
+  constexpr int LDS = 2 * (MT + NT) * KS * 1024 * S;
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(once, [] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(i8_gemm_ring_kernel<MT, NT, KS, S>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+  });
+  if (attr_err != hipSuccess)
+    return set_error(YSCV_HIP_ERR_DEVICE, "cannot reserve %d bytes of LDS: %s", LDS, hipGetErrorString(attr_err));
+  const int tiles_m = (int)ceil_div(m, (size_t)(32 * MT)), tiles_n = (int)ceil_div(n, (size_t)(32 * NT));
+  const int super_blocks = ((tiles_m + 7) / 8) * ((tiles_n + 3) / 4);
+  const unsigned grid = (unsigned)((super_blocks + 7) / 8) * 8 * 32;
+  hipLaunchKernelGGL((i8_gemm_ring_kernel<MT, NT, KS, S>), dim3(grid), dim3(I8R_THREADS), LDS, s, p, tiles_m, tiles_n);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
 int32_t launch_i8_gemm(const void *a, int a_is_u8, int a_zp, const yscv_hip_i8_weight *b, size_t m,
                        void *out, const I8Epilogue &ep, hipStream_t s) {
   I8Args p;
@@ -248,6 +522,16 @@ int32_t launch_i8_gemm(const void *a, int a_is_u8, int a_zp, const yscv_hip_i8_w
   p.ksteps = (int)(b->kp / 64);
   p.a_xor = a_is_u8 ? (int)0x80808080u : 0;
   p.zp_mul = a_is_u8 ? (128 - a_zp) : -a_zp;
+  const bool aligned = (reinterpret_cast<uintptr_t>(a) & 15) == 0;
+  const bool out_ok = (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+  if (b->k % 64 == 0 && aligned && out_ok && m * b->k < ((size_t)1 << 31)) {
+    // 128 x 128 tiles halve the LDS fill per MFMA; 64 x 128 tiles are for shapes that would not fill the CUs otherwise
+    const Context *ctx = nullptr;
+    YSCV_TRY(ensure_context(&ctx));
+    const size_t big_tiles = ceil_div(m, (size_t)128) * ceil_div(b->n, (size_t)128);
+    if (big_tiles >= (size_t)ctx->num_cus) return launch_ring<4, 4, 2, 4>(p, m, b->n, s);
+    return launch_ring<2, 4, 4, 3>(p, m, b->n, s);
+  }
   dim3 grid((unsigned)ceil_div(b->n, (size_t)I8_BN), (unsigned)ceil_div(m, (size_t)I8_BM));
   const bool vec = (b->k % 16 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
   if (vec)
