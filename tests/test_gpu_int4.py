@@ -249,6 +249,40 @@ def test_invalid_arguments_are_rejected(K, torch_cuda):
         w.matmul(x, mode="gemv")  # skinny kernel is m <= 16
 
 
+@pytest.mark.parametrize("m,n,k,g,sf16,zp", [(128, 128, 512, 32, False, False), (130, 200, 1024, 128, True, True),
+                                               (257, 1000, 640, 64, True, True), (512, 136, 2048, 32, True, False),
+                                               (300, 264, 768, 256, False, True), (1100, 520, 1152, 128, False, False)])
+@pytest.mark.parametrize("xdt", ["bf16", "f16"])
+def test_wide_m_ring_kernel(oracle, K, torch_cuda, m, n, k, g, sf16, zp, xdt):
+    """m >= 128 with 16-bit activations: the LDS-ring GEMM (weights decoded to fp16 with the scale folded in).
+    Row / column tails, every group mode, f32 and fp16 scales, with and without zero points, all output types."""
+    torch = torch_cuda
+    rng = np.random.default_rng(m + n * 3 + k * 7 + g)
+    groups = k // g
+    b = _rand_packed(rng, n, k)
+    scales = rng.uniform(0.005, 0.02, n * groups).astype(np.float16 if sf16 else np.float32)
+    zq = rng.integers(6, 11, (n, groups)) if zp else np.full((n, groups), 8)
+    zps = pack_zero_points(zq) if zp else None
+    xt = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32))
+    xt = xt.bfloat16() if xdt == "bf16" else xt.half()
+    x = xt.float().numpy()
+    ref = oracle.matmul_nbits(b, scales.astype(np.float32), pack_zero_points(zq), x, m, n, k, g)
+    w = K.PackedInt4Weight(b, scales, g, n, k, zero_points=zps, nibble_format=K.NIBBLE_UNSIGNED)
+    canary = torch.full((m + 1, n), 777.0, device="cuda")
+    w.matmul(xt.cuda(), out=canary[:m])
+    y32 = canary.cpu().numpy()
+    assert (y32[m] == 777.0).all()
+    d, rel = int4_tolerances(y32[:m], ref, k, x)
+    assert rel < 1e-3, rel  # fp16 rounding of (q - zp) * scale: about 2^-11 per weight, averaged over k
+    y16 = w.matmul(xt.cuda(), out_dtype=torch.bfloat16).float().cpu().numpy()
+    assert np.array_equal(y16, bf16_round(y32[:m]))
+    yh = w.matmul(xt.cuda(), out_dtype=torch.float16).float().cpu().numpy()
+    assert np.array_equal(yh, y32[:m].astype(np.float16).astype(np.float32))
+    # the same rows through the m <= 16 kernel (exact integer weights, f32 scales) agree to the same bar
+    ys = w.matmul(xt[:16].cuda(), out_dtype=torch.float32).cpu().numpy()
+    assert np.abs(ys - y32[:16]).max() <= 1e-3 * np.abs(ref).max()
+
+
 def test_prefill_gemm_sampled_at_full_size(oracle, K, torch_cuda):
     """BASELINE config 3 at full size (M=2048 K=4096 N=14336, g=128, fp16 scales, zero points 6..10,
     bf16 in/out); the oracle is evaluated on a sample of rows and columns."""

@@ -251,6 +251,8 @@ int32_t launch_int4_gemm(const yscv_hip_int4_weight *w, const _Float16 *xh, cons
                          const float *row_scale, size_t k_pad, int split, void *y, int y_dtype, size_t m,
                          hipStream_t s) {
   if (!w->tiled) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "int4 GEMM kernel needs the tiled layout");
+  if (m >= 128 && int4_gemm_ring_eligible(w, xh, y, y_dtype, split, m, k_pad))
+    return launch_int4_gemm_ring(w, xh, row_scale, k_pad, y, y_dtype, m, s);
   GemmArgs a;
   a.tiles = w->tiles;
   a.tscales = w->tscales;

@@ -1,0 +1,479 @@
+// Wide-M packed-int4 matmul for fp16 / bf16 activations: y[m][n] = sum_k x[m][k] * W[n][k], MFMA-bound design.
+// Replaces packed_int4_gemm_dispatch (crates/yscv-kernels/src/ops/int4_matmul.rs:548-605) for prefill-sized m.
+//
+// A workgroup owns a (32 MT) x (32 NT) tile of y.  It has four MMA waves (2 x 2, MT x NT MFMA tiles each) and NP
+// producer waves.  Per stage of KS k-steps (32 k each) the producers
+//   * fetch the activation rows (fp16, prepared by x_prep) with LDS-direct loads, one 16-byte piece per lane, so
+//     the row-major -> MFMA-fragment transposition costs nothing, and
+//   * load the packed weight words of the stage into registers, decode them to fp16 (q - zp) * scale ONCE per
+//     workgroup and write them to LDS in fragment order.
+// The MMA waves only read fragments (ds_read_b128) and issue v_mfma_f32_16x16x32_f16; a decoded weight is used by
+// 2 MT MFMAs and its decode never competes with them for issue slots.  The activation pieces of SA stages form a
+// ring (SA - 1 stages in flight hide the memory latency); decoded weights need two slots only because they are
+// written just before the stage is published, with one s_barrier per stage.
+// The scale is folded into the fp16 weight (relative rounding 2^-11 per weight, exact when the scales are stored
+// as fp16), so any group size costs the same; results stay inside the int4 tolerance (max-abs <= 1e-3 sqrt(K)
+// max|x|) by more than an order of magnitude.  f32 activations keep the exact-scale kernel of int4_gemm.hip.
+// The MFMA is issued with the operands swapped (D = Wfrag x Xfrag): a lane holds four consecutive columns of one
+// row of y; the finished tile goes through LDS so that whole rows are stored.
+#include <mutex>
+#include <type_traits>
+#include <utility>
+
+#include "int4_common.hpp"
+#include "kernels.hpp"
+
+namespace yscv {
+
+namespace {
+
+typedef __attribute__((address_space(3))) void lds_void;
+#define G4_AS1(ptr) ((const void __attribute__((address_space(1))) *)(ptr))
+
+struct RingArgs {
+  const uint8_t *tiles;
+  const void *tscales;
+  const uint8_t *tzps;
+  const _Float16 *xh;
+  const float *row_scale;
+  void *y;
+  int m, n;
+  int nt, kt, ktp;
+  int chunks, chunk_div;
+  int k_pad;
+  int y_dtype;
+};
+
+template <int N>
+__device__ __forceinline__ void g4_wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+template <int OFF>
+__device__ __forceinline__ void g4_ds_read(half8_t &v, uint32_t addr) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int MT, int NT>
+struct G4Frags {
+  half8_t a[MT], b[NT];
+};
+template <int KS, int MT, int NT, int... I, int... J>
+__device__ __forceinline__ void g4_issue_impl(G4Frags<MT, NT> &f, uint32_t a_addr, uint32_t b_addr,
+                                              std::integer_sequence<int, I...>, std::integer_sequence<int, J...>) {
+  (g4_ds_read<I * KS * 1024>(f.a[I], a_addr), ...);
+  (g4_ds_read<J * KS * 1024>(f.b[J], b_addr), ...);
+}
+template <int KS, int MT, int NT>
+__device__ __forceinline__ void g4_issue(G4Frags<MT, NT> &f, uint32_t a_addr, uint32_t b_addr) {
+  g4_issue_impl<KS>(f, a_addr, b_addr, std::make_integer_sequence<int, MT>{}, std::make_integer_sequence<int, NT>{});
+}
+template <int MT, int NT>
+__device__ __forceinline__ void g4_wait(G4Frags<MT, NT> &f) {
+  if constexpr (MT == 4 && NT == 4) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]),
+                   "+v"(f.b[3])::"memory");
+  } else {
+    static_assert(MT == 8 && NT == 4, "add a wait for this fragment count");
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.a[4]), "+v"(f.a[5]), "+v"(f.a[6]),
+                   "+v"(f.a[7]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]), "+v"(f.b[3])::"memory");
+  }
+}
+
+typedef unsigned int uint2_t __attribute__((ext_vector_type(2)));
+
+template <int B, int E, class F>
+__device__ __forceinline__ void g4_static_for(F &&f) {
+  if constexpr (B < E) {
+    f(std::integral_constant<int, B>{});
+    g4_static_for<B + 1, E>(f);
+  }
+}
+
+// Loads the producers keep in flight across stages are issued and awaited with opaque instructions: the compiler
+// cannot follow registers that rotate through a ring of stages and would wait for every load in flight.  All of
+// them use a uniform base pointer plus a 32-bit per-lane offset that never changes, so a stage costs a producer
+// a handful of scalar additions and no vector address arithmetic.
+template <int GM, bool SF16>
+struct G4Scale {
+  static constexpr int SPT = GM == GM32 ? 4 : (GM == GM64 ? 2 : 1);
+  static constexpr int SC_BYTES = SPT * (SF16 ? 2 : 4);
+  static constexpr int ZP_BYTES = SPT;
+  static constexpr int SC_REGS = (SC_BYTES + 3) / 4;
+};
+
+// One weight tile's share of two stages (128 k): four packed words, the scale chunk and the zero-point chunk of lane
+// row r.
+// Every member is the destination of exactly one load instruction, and nothing may copy a register between the
+// load and the wait (the data is not there yet): the loads name their destination as a read-write operand, which
+// ties every reload of a ring position to the same physical register, and the producer code below has no branch
+// between the issue of a load and its wait.
+template <int SC_REGS>
+struct G4ScaleRegs {
+  typedef uint32_t type __attribute__((ext_vector_type(SC_REGS)));
+};
+template <>
+struct G4ScaleRegs<1> {
+  typedef uint32_t type;
+};
+template <int SC_REGS>
+struct G4Tile {
+  uint4_t raw;
+  typename G4ScaleRegs<SC_REGS>::type sc;
+  uint32_t zp;
+  __device__ __forceinline__ uint32_t sc_reg(int i) const {
+    if constexpr (SC_REGS == 1) return sc;
+    else return sc[i];
+  }
+};
+template <int BYTES, int SC_REGS>
+__device__ __forceinline__ void g4_load_scale(G4Tile<SC_REGS> &t, uint32_t voff, const void *base) {
+  static_assert((BYTES + 3) / 4 == SC_REGS, "one load fills the scale registers");
+  if constexpr (BYTES == 2) asm volatile("global_load_ushort %0, %1, %2" : "+v"(t.sc) : "v"(voff), "s"(base) : "memory");
+  if constexpr (BYTES == 4) asm volatile("global_load_dword %0, %1, %2" : "+v"(t.sc) : "v"(voff), "s"(base) : "memory");
+  if constexpr (BYTES == 8) asm volatile("global_load_dwordx2 %0, %1, %2" : "+v"(t.sc) : "v"(voff), "s"(base) : "memory");
+  if constexpr (BYTES == 16) asm volatile("global_load_dwordx4 %0, %1, %2" : "+v"(t.sc) : "v"(voff), "s"(base) : "memory");
+}
+template <int BYTES, int SC_REGS>
+__device__ __forceinline__ void g4_load_zp(G4Tile<SC_REGS> &t, uint32_t voff, const void *base) {
+  if constexpr (BYTES == 1) asm volatile("global_load_ubyte %0, %1, %2" : "+v"(t.zp) : "v"(voff), "s"(base) : "memory");
+  if constexpr (BYTES == 2) asm volatile("global_load_ushort %0, %1, %2" : "+v"(t.zp) : "v"(voff), "s"(base) : "memory");
+  if constexpr (BYTES == 4) asm volatile("global_load_dword %0, %1, %2" : "+v"(t.zp) : "v"(voff), "s"(base) : "memory");
+}
+template <int SC_REGS>
+__device__ __forceinline__ void g4_load_raw(G4Tile<SC_REGS> &t, uint32_t voff, const void *base) {
+  asm volatile("global_load_dwordx4 %0, %1, %2" : "+v"(t.raw) : "v"(voff), "s"(base) : "memory");
+}
+// wait until at most N loads are in flight; the tile registers count as written by the wait
+template <int N, int SC_REGS>
+__device__ __forceinline__ void g4_wait_tiles(G4Tile<SC_REGS> (&t)[1]) {
+  asm volatile("s_waitcnt vmcnt(%3)" : "+v"(t[0].raw), "+v"(t[0].sc), "+v"(t[0].zp) : "n"(N) : "memory");
+}
+template <int N, int SC_REGS>
+__device__ __forceinline__ void g4_wait_tiles(G4Tile<SC_REGS> (&t)[2]) {
+  asm volatile("s_waitcnt vmcnt(%6)"
+               : "+v"(t[0].raw), "+v"(t[0].sc), "+v"(t[0].zp), "+v"(t[1].raw), "+v"(t[1].sc), "+v"(t[1].zp)
+               : "n"(N)
+               : "memory");
+}
+template <int N>
+__device__ __forceinline__ void g4_wait_vm_n() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <int MT, int NT, int KS, int SA, int NP, int GM, bool SF16>
+__global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs p, int tiles_m, int tiles_n) {
+  constexpr int THREADS = 256 + 64 * NP;
+  constexpr int BM = 32 * MT, BN = 32 * NT;
+  constexpr int A_BYTES = 2 * MT * KS * 1024, B_BYTES = 2 * NT * KS * 1024;  // one stage of each operand
+  constexpr int B_BASE = SA * A_BYTES, LDS_BYTES = SA * A_BYTES + 2 * B_BYTES;
+  constexpr int APW = 2 * MT * KS / NP;  // activation chunks (1 KiB) a producer wave fetches per stage
+  constexpr int WT = 2 * NT / NP;        // weight tiles (16 columns) a producer wave decodes per stage
+  static_assert(KS == 2, "a stage is half a 128-k weight tile");
+  static_assert((2 * MT * KS) % NP == 0 && (2 * NT) % NP == 0 && (WT == 1 || WT == 2), "work split over the producer waves");
+  static_assert(SA >= 2 && SA <= 6 && SA % 2 == 0, "stage parity must follow the ring position");
+  constexpr int RS = BN * 4 + 16;  // row stride of the f32 result tile in LDS (odd multiple of 16 B)
+  static_assert(BM * RS <= LDS_BYTES, "the result tile reuses the ring");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t g4_ring[];
+  const uint32_t lds0 = (uint32_t)(size_t)g4_ring;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, c = lane >> 4;
+
+  // XCD-aware tile numbering: super-blocks of 8 x 4 tiles, one at a time per XCD (workgroup id mod 8)
+  const int sb_m = (tiles_m + 7) / 8;
+  const int j_in_xcd = (int)(blockIdx.x >> 3);
+  const int sb = (j_in_xcd >> 5) * 8 + (int)(blockIdx.x & 7);
+  const int tm = (sb % sb_m) * 8 + (j_in_xcd & 7), tn = (sb / sb_m) * 4 + ((j_in_xcd >> 3) & 3);
+  if (tm >= tiles_m || tn >= tiles_n) return;
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int nstages = p.kt * (4 / KS);
+
+  float4_t acc[MT][NT];  // MMA waves only; the producers never touch it
+  const int wm = (wave >> 1) & 1, wn = wave & 1;
+
+  if (wave >= 4) {
+    // ---- producer ------------------------------------------------------------------------------------
+    typedef G4Scale<GM, SF16> SC;
+    typedef G4Tile<SC::SC_REGS> Tile;
+    // loads of this wave per stage: an even stage fetches the weight side of its 128-k tile (both stages of it)
+    // before its activation pieces, an odd stage only activation pieces
+    constexpr int PE = 3 * WT + APW, PO = APW;
+    static_assert((SA / 2) * PE + (SA / 2) * PO + APW < 64, "vmcnt budget");
+    const int pw = wave - 4;
+    const bool has_zp = p.tzps != nullptr;
+    // per-lane byte offsets (fixed) and uniform base pointers (advanced per stage)
+    uint32_t aoff[APW];
+#pragma unroll
+    for (int j = 0; j < APW; j++) {
+      const int q = pw * APW + j;
+      const int row = min(m0 + (q / KS) * 16 + r, p.m - 1);
+      aoff[j] = (uint32_t)(((size_t)row * p.k_pad + (q % KS) * 32 + c * 8) * sizeof(_Float16));
+    }
+    const uint32_t woff = lane * 16, soff = r * SC::SC_BYTES, zoff = r * SC::ZP_BYTES;
+    const uint8_t *wbase[WT], *sbase[WT], *zbase[WT];
+#pragma unroll
+    for (int u = 0; u < WT; u++) {
+      const int nt = min(n0 / 16 + pw * WT + u, p.nt - 1);
+      wbase[u] = p.tiles + (size_t)nt * p.ktp * kTileBytes;
+      sbase[u] = reinterpret_cast<const uint8_t *>(p.tscales) + (size_t)nt * p.chunks * 16 * SC::SC_BYTES;
+      zbase[u] = has_zp ? p.tzps + (size_t)nt * p.chunks * 16 * SC::ZP_BYTES : sbase[u];  // keeps the load count uniform
+    }
+    const int zstride = has_zp ? 16 * SC::ZP_BYTES : 16 * SC::SC_BYTES;
+
+    Tile wr[SA / 2][WT];  // weight registers of the even stages in flight
+    // stage st goes to activation slot / register set ri = st mod SA; par = st & 1 picks the words of the tile
+    auto issue_stage = [&](int st, auto ric, auto parc) {
+      constexpr int ri = decltype(ric)::value, par = decltype(parc)::value;
+      if constexpr (par == 0) {
+        const int kt = st >> 1;
+        const int chunk = GM == GM128 ? kt / p.chunk_div : kt;
+#pragma unroll
+        for (int u = 0; u < WT; u++) {
+          g4_load_raw(wr[ri / 2][u], woff, wbase[u] + (size_t)kt * kTileBytes);
+          g4_load_scale<SC::SC_BYTES>(wr[ri / 2][u], soff, sbase[u] + (size_t)chunk * 16 * SC::SC_BYTES);
+          g4_load_zp<SC::ZP_BYTES>(wr[ri / 2][u], zoff, zbase[u] + (size_t)chunk * zstride);
+        }
+      }
+      const char *abase = reinterpret_cast<const char *>(p.xh) + (size_t)st * KS * 32 * sizeof(_Float16);
+#pragma unroll
+      for (int j = 0; j < APW; j++)
+        __builtin_amdgcn_global_load_lds(G4_AS1(abase + aoff[j]),
+                                         (lds_void *)(uintptr_t)(lds0 + (uint32_t)(ri * A_BYTES + (pw * APW + j) * 1024)), 16, 0, 0);
+    };
+    // decode the weights of a stage (register set ri, parity par) into weight slot par
+    auto decode_stage = [&](auto ric, auto parc) {
+      constexpr int ri = decltype(ric)::value, par = decltype(parc)::value;
+      const uint32_t dst = lds0 + (uint32_t)(B_BASE + par * B_BYTES + pw * WT * KS * 1024 + lane * 16);
+#pragma unroll
+      for (int u = 0; u < WT; u++) {
+        half2_t c1[KS], c2[KS];
+        half8_t sv[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+          constexpr int dummy = 0;
+          (void)dummy;
+          const int e = GM == GM32 ? (par * KS + ks) : (GM == GM64 ? par : 0);  // group inside the chunk
+          if (ks > 0 && GM != GM32) {
+            c1[ks] = c1[0];
+            c2[ks] = c2[0];
+            sv[ks] = sv[0];
+            continue;
+          }
+          const uint32_t zq = has_zp ? ((wr[ri / 2][u].zp >> (8 * e)) & 0xFF) : 8u;
+          const _Float16 z = (_Float16)(float)zq;
+          const _Float16 c1v = (_Float16)(-1024.0f) - z, c2v = (_Float16)(-64.0f) - z;
+          c1[ks] = half2_t{c1v, c1v};
+          c2[ks] = half2_t{c2v, c2v};
+          _Float16 s;
+          if constexpr (SF16) {
+            U32H2 t;
+            t.u = wr[ri / 2][u].sc_reg(e >> 1);
+            s = t.h[e & 1];
+          } else {
+            s = (_Float16)__uint_as_float(wr[ri / 2][u].sc_reg(e));
+          }
+          sv[ks] = half8_t{s, s, s, s, s, s, s, s};
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+          const half8_t h = decode8(wr[ri / 2][u].raw[par * KS + ks], c1[ks], c2[ks]) * sv[ks];
+          // written with an opaque instruction: a compiler-visible LDS store would first wait for every LDS-direct
+          // load in flight
+          asm volatile("ds_write_b128 %0, %1" ::"v"(dst + (uint32_t)((u * KS + ks) * 1024)), "v"(h) : "memory");
+        }
+      }
+    };
+    // Loads complete in order and an even stage issues its weight loads before its activation pieces: the weights
+    // are decoded while the latter still fly.  NE / NO = even / odd stages issued after the published one.
+    auto publish = [&](auto ric, auto parc, auto nec, auto noc) {
+      constexpr int ri = decltype(ric)::value, par = decltype(parc)::value;
+      constexpr int L = decltype(nec)::value * PE + decltype(noc)::value * PO;
+      if constexpr (par == 0) g4_wait_tiles<L + APW>(wr[ri / 2]);
+      decode_stage(ric, parc);
+      g4_wait_vm_n<L>();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+    };
+    // Exactly SA stages are in flight at any time: past the last stage the producers keep fetching it again (into
+    // slots and registers nobody reads any more), so no wait count and no branch depends on how far the end is.
+    const int last = nstages - 1;
+    // one step while the MMA waves work on stage s: publish stage s+1, then refill the slot and registers of stage s
+    auto step = [&](int s, auto uc) {
+      constexpr int u = decltype(uc)::value;
+      publish(std::integral_constant<int, (u + 1) % SA>{}, std::integral_constant<int, ((u + 1) & 1)>{},
+              std::integral_constant<int, (SA - 2) / 2>{}, std::integral_constant<int, (SA - 2) / 2>{});
+      issue_stage(min(s + SA, last), uc, std::integral_constant<int, (u & 1)>{});
+    };
+
+#pragma unroll
+    for (int i = 0; i < SA / 2; i++)
+#pragma unroll
+      for (int u = 0; u < WT; u++) {
+        wr[i][u].raw = uint4_t{0, 0, 0, 0};
+        wr[i][u].sc = typename G4ScaleRegs<SC::SC_REGS>::type(0);
+        wr[i][u].zp = 0;
+      }
+    g4_static_for<0, SA>([&](auto uc) {
+      constexpr int u = decltype(uc)::value;
+      issue_stage(min(u, last), uc, std::integral_constant<int, (u & 1)>{});
+    });
+    publish(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, std::integral_constant<int, SA / 2 - 1>{},
+            std::integral_constant<int, SA / 2>{});
+    int s0 = 0;
+    for (; s0 + SA <= last; s0 += SA) g4_static_for<0, SA>([&](auto uc) { step(s0 + decltype(uc)::value, uc); });
+    // the remaining 0 .. SA-1 steps as straight-line code
+    g4_static_for<1, SA>([&](auto rc) {
+      constexpr int R = decltype(rc)::value;
+      if (last - s0 == R) g4_static_for<0, R>([&](auto uc) { step(s0 + decltype(uc)::value, uc); });
+    });
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // the registers of the loads issued past the end stay reserved until those loads have landed
+#pragma unroll
+    for (int i = 0; i < SA / 2; i++)
+#pragma unroll
+      for (int u = 0; u < WT; u++) asm volatile("" ::"v"(wr[i][u].raw), "v"(wr[i][u].sc), "v"(wr[i][u].zp));
+  } else {
+    // ---- MMA waves -----------------------------------------------------------------------------------
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+      for (int j = 0; j < NT; j++) acc[i][j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    const uint32_t a_lane = lds0 + (uint32_t)(wm * MT * KS * 1024 + lane * 16);
+    const uint32_t b_lane = lds0 + B_BASE + (uint32_t)(wn * NT * KS * 1024 + lane * 16);
+    G4Frags<MT, NT> f[2];
+    auto mfmas = [&](const G4Frags<MT, NT> &cur, int i0, int i1) {
+#pragma unroll
+      for (int i = i0; i < i1; i++)
+#pragma unroll
+        for (int j = 0; j < NT; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cur.b[j], cur.a[i], acc[i][j], 0, 0, 0);
+    };
+    __builtin_amdgcn_s_barrier();
+    g4_issue<KS>(f[0], a_lane, b_lane);
+    uint32_t aslot = 0, bslot = 0;
+    for (int st = 0; st < nstages; st++) {
+      const uint32_t naslot = aslot + A_BYTES == SA * A_BYTES ? 0 : aslot + A_BYTES;
+      const uint32_t nbslot = bslot ^ B_BYTES;
+      // k-step 0: the fragments of k-step 1 are on their way while its MFMAs run
+      g4_wait(f[0]);
+      g4_issue<KS>(f[1], a_lane + aslot + 1024, b_lane + bslot + 1024);
+      mfmas(f[0], 0, MT);
+      // k-step 1: the first MFMAs cover the barrier, the others the fragment reads of the next stage
+      g4_wait(f[1]);
+      mfmas(f[1], 0, MT / 2);
+      if (st + 1 < nstages) {
+        __builtin_amdgcn_s_barrier();
+        g4_issue<KS>(f[0], a_lane + naslot, b_lane + nbslot);
+      }
+      mfmas(f[1], MT / 2, MT);
+      aslot = naslot;
+      bslot = nbslot;
+    }
+  }
+
+  // ---- epilogue: lane (c, r) of an MMA wave holds y[16 i + r][16 j + 4 c + 0..3] of its part; through LDS so that
+  // all waves store whole rows ------------------------------------------------------------------------------
+  __syncthreads();
+  if (wave < 4) {
+#pragma unroll
+    for (int i = 0; i < MT; i++) {
+      const int lrow = wm * MT * 16 + i * 16 + r;
+      const int row = min(m0 + lrow, p.m - 1);
+      const float rs = p.row_scale ? p.row_scale[row] : 1.0f;
+#pragma unroll
+      for (int j = 0; j < NT; j++) {
+        const int lcol = wn * NT * 16 + j * 16 + c * 4;
+        *reinterpret_cast<float4_t *>(g4_ring + lrow * RS + lcol * 4) = acc[i][j] * rs;
+      }
+    }
+  }
+  __syncthreads();
+  constexpr int CPR = BN / 4;  // four-column chunks per row
+  const bool vec = (p.n & 3) == 0;
+  for (int q = tid; q < BM * CPR; q += THREADS) {
+    const int lrow = q / CPR, ch = q % CPR;
+    const int row = m0 + lrow, col = n0 + ch * 4;
+    if (row >= p.m || col >= p.n) continue;
+    const float4_t v = *reinterpret_cast<const float4_t *>(g4_ring + lrow * RS + ch * 16);
+    const size_t o = (size_t)row * p.n + col;
+    if (vec) {
+      if (p.y_dtype == YSCV_HIP_F32) {
+        *reinterpret_cast<float4_t *>(reinterpret_cast<float *>(p.y) + o) = v;
+      } else if (p.y_dtype == YSCV_HIP_F16) {
+        *reinterpret_cast<half4_t *>(reinterpret_cast<_Float16 *>(p.y) + o) =
+            half4_t{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+      } else {
+        uint2 b;
+        b.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+        b.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+        *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.y) + o) = b;
+      }
+    } else {
+      for (int e = 0; e < 4; e++)
+        if (col + e < p.n) store_out(p.y, o + e, v[e], p.y_dtype);
+    }
+  }
+}
+
+template <int MT, int NT, int KS, int SA, int NP, int GM, bool SF16>
+int32_t ring_launch_one(const RingArgs &a, hipStream_t s) {
+  constexpr int LDS = 2 * MT * KS * 1024 * SA + 2 * 2 * NT * KS * 1024;
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  auto kern = int4_gemm_ring_kernel<MT, NT, KS, SA, NP, GM, SF16>;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+  });
+  if (attr_err != hipSuccess)
+    return set_error(YSCV_HIP_ERR_DEVICE, "cannot reserve %d bytes of LDS: %s", LDS, hipGetErrorString(attr_err));
+  const int tiles_m = (int)ceil_div((size_t)a.m, (size_t)(32 * MT)), tiles_n = (int)ceil_div((size_t)a.n, (size_t)(32 * NT));
+  const int super_blocks = ((tiles_m + 7) / 8) * ((tiles_n + 3) / 4);
+  const unsigned grid = (unsigned)((super_blocks + 7) / 8) * 8 * 32;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256 + 64 * NP), LDS, s, a, tiles_m, tiles_n);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+template <int MT, int NT, int KS, int SA, int NP>
+int32_t ring_launch_gm(const RingArgs &a, int gm, bool sf16, hipStream_t s) {
+  if (gm == GM32)
+    return sf16 ? ring_launch_one<MT, NT, KS, SA, NP, GM32, true>(a, s) : ring_launch_one<MT, NT, KS, SA, NP, GM32, false>(a, s);
+  if (gm == GM64)
+    return sf16 ? ring_launch_one<MT, NT, KS, SA, NP, GM64, true>(a, s) : ring_launch_one<MT, NT, KS, SA, NP, GM64, false>(a, s);
+  return sf16 ? ring_launch_one<MT, NT, KS, SA, NP, GM128, true>(a, s) : ring_launch_one<MT, NT, KS, SA, NP, GM128, false>(a, s);
+}
+
+}  // namespace
+
+bool int4_gemm_ring_eligible(const yscv_hip_int4_weight *w, const _Float16 *xh, const void *y, int y_dtype, int split, size_t m,
+                             size_t k_pad) {
+  if (!w->tiled || split != 1) return false;
+  if ((reinterpret_cast<uintptr_t>(xh) & 15) != 0) return false;
+  if (m * k_pad * sizeof(_Float16) >= ((size_t)1 << 32)) return false;  // per-lane offsets are 32 bits wide
+  const size_t align = y_dtype == YSCV_HIP_F32 ? 16 : 8;
+  return (reinterpret_cast<uintptr_t>(y) & (align - 1)) == 0;
+}
+
+int32_t launch_int4_gemm_ring(const yscv_hip_int4_weight *w, const _Float16 *xh, const float *row_scale, size_t k_pad,
+                              void *y, int y_dtype, size_t m, hipStream_t s) {
+  RingArgs a;
+  a.tiles = w->tiles;
+  a.tscales = w->tscales;
+  a.tzps = w->has_zp ? w->tzps : nullptr;
+  a.xh = xh;
+  a.row_scale = row_scale;
+  a.y = y;
+  a.m = (int)m;
+  a.n = (int)w->n;
+  a.nt = (int)w->nt;
+  a.kt = (int)w->kt;
+  a.ktp = (int)w->ktp;
+  a.chunks = (int)w->chunks;
+  a.chunk_div = w->gm == GM128 ? (int)(w->g / 128) : 1;
+  a.k_pad = (int)k_pad;
+  a.y_dtype = y_dtype;
+  const bool sf16 = w->scale_dtype == YSCV_HIP_F16;
+  return ring_launch_gm<4, 4, 2, 6, 8>(a, w->gm, sf16, s);
+}
+
+}  // namespace yscv

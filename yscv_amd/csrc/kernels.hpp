@@ -74,6 +74,12 @@ int32_t launch_int4_gemm(const yscv_hip_int4_weight *w, const _Float16 *xh, cons
                          const float *row_scale, size_t k_pad, int split, void *y, int y_dtype,
                          size_t m, hipStream_t s);
 
+// LDS-ring GEMM for fp16-prepared activations (split == 1)
+bool int4_gemm_ring_eligible(const yscv_hip_int4_weight *w, const _Float16 *xh, const void *y, int y_dtype, int split, size_t m,
+                             size_t k_pad);
+int32_t launch_int4_gemm_ring(const yscv_hip_int4_weight *w, const _Float16 *xh, const float *row_scale, size_t k_pad,
+                              void *y, int y_dtype, size_t m, hipStream_t s);
+
 // Whole int4 call (activation preparation + kernel) with caller-provided scratch; ws may be null.
 int32_t int4_workspace_bytes(const yscv_hip_int4_weight *w, size_t m, int x_dtype, int force, size_t *bytes);
 int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, void *y, int y_dtype, size_t m,
