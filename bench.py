@@ -140,19 +140,36 @@ def cpu_baseline(cfg, seconds_budget=20.0):
 
 
 def extra_kernels(torch, stream_ptr):
-    """Stand-alone kernels of BASELINE configs 1-3 (short runs; the parity tests cover correctness)."""
+    """Stand-alone kernels of BASELINE configs 1-3 and 5 (short runs; the parity tests cover correctness).
+    Each call sequence is captured into a HIP graph and replayed, so the figures are device time per call
+    without the Python / launch overhead of the caller."""
     import numpy as np
 
     from yscv_amd import kernels as K
 
     out = {}
     rng = np.random.default_rng(1)
+    side = torch.cuda.Stream()
 
-    def tavg(fn, iters, warm=3):
-        for _ in range(warm):
-            fn()
-        torch.cuda.synchronize()
-        return event_time_ms(lambda: [fn() for _ in range(iters)], torch) * 1e-3 / iters
+    def tavg(fn, calls_per_graph, replays=10):
+        """Average device time of one fn() call: calls_per_graph calls captured once, replayed `replays` times."""
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                fn()
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=side):
+                for _ in range(calls_per_graph):
+                    fn()
+            g.replay()
+            torch.cuda.synchronize()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            for _ in range(replays):
+                g.replay()
+            e.record()
+            torch.cuda.synchronize()
+        return s.elapsed_time(e) * 1e-3 / (replays * calls_per_graph)
 
     # config 1: GEMV M1 K4096 N4096 g32, f32 scales, f32 activations; ring of weight copies > 256 MB
     n = k = 4096
@@ -161,18 +178,21 @@ def extra_kernels(torch, stream_ptr):
         ring.append(K.PackedInt4Weight(rng.integers(0, 256, n * k // 2, dtype=np.uint8),
                                        rng.uniform(0.005, 0.02, n * (k // 32)).astype(np.float32), 32, n, k,
                                        nibble_format=K.NIBBLE_UNSIGNED))
-    x = torch.randn(1, k, device="cuda")
-    y = torch.empty(1, n, device="cuda")
     i = [0]
-
-    def gemv():
-        ring[i[0] % len(ring)].matmul(x, out=y)
-        i[0] += 1
-
-    t = tavg(gemv, 128)
     byt = n * k // 2 + n * (k // 32) * 4 + k * 4 + n * 4
-    out["config1_gemv_m1_k4096_n4096"] = {"us_per_call_whole_op": round(t * 1e6, 2), "GB/s_whole_op": round(byt / t / 1e9, 1),
-                                          "note": "x_prep + kernel, 32 rotating weight copies"}
+    c1 = {}
+    for name, dt in (("f32_activations", torch.float32), ("f16_activations", torch.float16)):
+        x = torch.randn(1, k, device="cuda").to(dt)
+        y = torch.empty(1, n, device="cuda", dtype=dt)
+
+        def gemv():
+            ring[i[0] % len(ring)].matmul(x, out=y)
+            i[0] += 1
+
+        t = tavg(gemv, 32)
+        c1[name] = {"us_per_call_whole_op": round(t * 1e6, 2), "GB/s_whole_op": round(byt / t / 1e9, 1)}
+    c1["note"] = "32 rotating weight copies (320 MB, beyond the 256 MB Infinity Cache); f32 input = activation pass + kernel"
+    out["config1_gemv_m1_k4096_n4096"] = c1
     del ring
     # config 2: int8 M512 K4096 N4096
     m, k, n = 512, 4096, 4096
@@ -180,12 +200,12 @@ def extra_kernels(torch, stream_ptr):
     a = torch.randint(0, 256, (m, k), device="cuda", dtype=torch.uint8)
     o32 = torch.empty(m, n, device="cuda", dtype=torch.int32)
     q8 = torch.empty(m, n, device="cuda", dtype=torch.uint8)
-    t = tavg(lambda: pb.matmul(a, a_zp=128, out=o32), 50)
-    t2 = tavg(lambda: pb.matmul_requant(a, 128, 1.0 / 4096, 128.0, K.ROUND_HALF_AWAY, 0, 255, out=q8), 50)
+    t = tavg(lambda: pb.matmul(a, a_zp=128, out=o32), 20)
+    t2 = tavg(lambda: pb.matmul_requant(a, 128, 1.0 / 4096, 128.0, K.ROUND_HALF_AWAY, 0, 255, out=q8), 20)
     ops = 2.0 * m * k * n
     out["config2_int8_m512_k4096_n4096"] = {"us_i32": round(t * 1e6, 2), "TOP/s_i32": round(ops / t / 1e12, 1),
                                             "us_fused_requant": round(t2 * 1e6, 2), "TOP/s_fused_requant": round(ops / t2 / 1e12, 1),
-                                            "frac_of_i8_mfma_peak": round(ops / t2 / 1e12 / MFMA_I8_PEAK, 4)}
+                                            "frac_of_i8_mfma_peak": round(ops / t / 1e12 / MFMA_I8_PEAK, 4)}
     del pb
     # config 3: int4 prefill M2048 K4096 N14336 g128, zero points 6..10, bf16
     m, k, n, g = 2048, 4096, 14336, 128
@@ -195,10 +215,29 @@ def extra_kernels(torch, stream_ptr):
                            g, n, k, zero_points=zp, nibble_format=K.NIBBLE_UNSIGNED)
     xb = torch.randn(m, k, device="cuda").bfloat16()
     yb = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
-    t = tavg(lambda: w.matmul(xb, out=yb), 10)
+    t = tavg(lambda: w.matmul(xb, out=yb), 4, replays=5)
     fl = 2.0 * m * k * n
     out["config3_int4_prefill_m2048_k4096_n14336"] = {"us_whole_op": round(t * 1e6, 1), "TFLOP/s": round(fl / t / 1e12, 1),
                                                       "frac_of_bf16_mfma_peak": round(fl / t / 1e12 / MFMA_BF16_PEAK, 4)}
+    w.close()
+    del w, xb, yb
+    # config 5: LM-head shape K4096 N128256 g32, bf16 activations, M = 1 .. 256
+    k, n, g = 4096, 128256, 32
+    w = K.PackedInt4Weight(rng.integers(0, 256, n * k // 2, dtype=np.uint8), rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float16),
+                           g, n, k, nibble_format=K.NIBBLE_UNSIGNED)
+    wbytes = n * k // 2 + n * (k // g) * 2
+    sweep = {}
+    for m in (1, 2, 4, 8, 16, 32, 64, 128, 256):
+        xb = torch.randn(m, k, device="cuda").bfloat16()
+        yb = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
+        t = tavg(lambda: w.matmul(xb, out=yb), 4, replays=4)
+        fl = 2.0 * m * k * n
+        sweep["m%d" % m] = {"us": round(t * 1e6, 1), "weight_GB/s": round(wbytes / t / 1e9, 0),
+                            "frac_of_hbm_peak": round(wbytes / t / 1e9 / HBM_PEAK_GBS, 3),
+                            "TFLOP/s": round(fl / t / 1e12, 1), "frac_of_mfma_peak": round(fl / t / 1e12 / MFMA_BF16_PEAK, 4),
+                            "kernel": "int4_skinny_kernel" if m <= 16 else "int4_gemm_ring_kernel"}
+    out["config5_lm_head_sweep_k4096_n128256"] = sweep
+    w.close()
     return out
 
 
@@ -210,6 +249,9 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-extra", action="store_true", help="skip the stand-alone kernels and the batch-16 run")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--extra-only", action="store_true",
+                    help="run only the stand-alone kernels of BASELINE configs 1, 2, 3 and 5 and print their figures "
+                         "(the run the rocprofv3 summaries of those kernels are taken from)")
     ap.add_argument("--graph-path", action="store_true",
                     help="time the multi-kernel path (one HIP-graph replay per step) instead of the single-launch kernel")
     ap.add_argument("--calib-copy", action="store_true",
@@ -233,6 +275,9 @@ def main():
         cfg["max_ctx"] = ((need + 127) // 128) * 128
     cfg["max_steps"] = max(cfg["max_steps"], args.steps + args.warmup)
     stream_ptr = torch.cuda.current_stream().cuda_stream
+    if args.extra_only:
+        print(json.dumps({"extra": extra_kernels(torch, stream_ptr)}))
+        return
 
     if args.calib_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)

@@ -187,7 +187,8 @@ def test_group_sizes_and_zero_points(oracle, K, torch_cuda, g, m):
     w = K.PackedInt4Weight(b, scales16, g, n, k, zero_points=zps, nibble_format=K.NIBBLE_UNSIGNED)
     y32 = w.matmul(xt.cuda(), out_dtype=torch.float32).cpu().numpy()
     d, rel = int4_tolerances(y32, ref, k, x)
-    assert rel < 5e-5, rel
+    # m <= 16: exact integer weights, f32 scales; above: weights decoded to fp16 with the scale folded in
+    assert rel < (5e-5 if m <= 16 else 1e-3), rel
     # bf16 output = RNE narrowing of the f32 result (crates/yscv-tensor/src/tensor.rs:764-769)
     ybf = w.matmul(xt.cuda()).float().cpu().numpy()
     assert np.array_equal(ybf, bf16_round(y32))
@@ -249,12 +250,13 @@ def test_invalid_arguments_are_rejected(K, torch_cuda):
         w.matmul(x, mode="gemv")  # skinny kernel is m <= 16
 
 
-@pytest.mark.parametrize("m,n,k,g,sf16,zp", [(128, 128, 512, 32, False, False), (130, 200, 1024, 128, True, True),
+@pytest.mark.parametrize("m,n,k,g,sf16,zp", [(17, 40, 128, 32, True, False), (33, 300, 256, 64, False, True), (100, 129, 1536, 128, True, True),
+                                               (128, 128, 512, 32, False, False), (130, 200, 1024, 128, True, True),
                                                (257, 1000, 640, 64, True, True), (512, 136, 2048, 32, True, False),
                                                (300, 264, 768, 256, False, True), (1100, 520, 1152, 128, False, False)])
 @pytest.mark.parametrize("xdt", ["bf16", "f16"])
 def test_wide_m_ring_kernel(oracle, K, torch_cuda, m, n, k, g, sf16, zp, xdt):
-    """m >= 128 with 16-bit activations: the LDS-ring GEMM (weights decoded to fp16 with the scale folded in).
+    """m > 16 with 16-bit activations: the LDS-ring GEMM (weights decoded to fp16 with the scale folded in).
     Row / column tails, every group mode, f32 and fp16 scales, with and without zero points, all output types."""
     torch = torch_cuda
     rng = np.random.default_rng(m + n * 3 + k * 7 + g)

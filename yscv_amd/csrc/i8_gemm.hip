@@ -284,7 +284,7 @@ __device__ __forceinline__ void i8_frags_wait(I8Frags<MT, NT> &f) {
 }
 
 template <int MT, int NT, int KS, int S>
-__global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int tiles_m, int tiles_n) {
+__global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int tiles_m, int tiles_n, int sbm_log2) {
   constexpr int BM = 32 * MT, BN = 32 * NT;
   constexpr int A_BYTES = 2 * MT * KS * 1024, STAGE = 2 * (MT + NT) * KS * 1024;
   constexpr int PER_WAVE = (MT + NT) * KS / 2;  // 1 KiB chunks a producer wave fetches per stage
@@ -297,13 +297,14 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, c = lane >> 4;
 
-  // XCD-aware tile numbering: the grid of tiles is cut into super-blocks of 8 x 4 tiles; workgroup ids that share
-  // an XCD (id mod 8) walk through one super-block at a time, so the 32 workgroups an XCD runs together read
-  // 8 row panels of A and 4 column panels of B between them.
-  const int sb_m = (tiles_m + 7) / 8;
+  // XCD-aware tile numbering: the grid of tiles is cut into super-blocks of 32 tiles, 2^sbm_log2 (at most 8) along
+  // m; workgroup ids that share an XCD (id mod 8) walk through one super-block at a time, so the 32 workgroups an
+  // XCD runs together share row panels of A and column panels of B in its L2.
+  const int sbm = 1 << sbm_log2, sbn = 32 >> sbm_log2;
+  const int sb_m = (tiles_m + sbm - 1) >> sbm_log2;
   const int j_in_xcd = (int)(blockIdx.x >> 3);
   const int sb = (j_in_xcd >> 5) * 8 + (int)(blockIdx.x & 7);
-  const int tm = (sb % sb_m) * 8 + (j_in_xcd & 7), tn = (sb / sb_m) * 4 + ((j_in_xcd >> 3) & 3);
+  const int tm = (sb % sb_m) * sbm + (j_in_xcd & (sbm - 1)), tn = (sb / sb_m) * sbn + ((j_in_xcd & 31) >> sbm_log2);
   if (tm >= tiles_m || tn >= tiles_n) return;
   const int m0 = tm * BM, n0 = tn * BN;
   const int nt_total = (p.n + 15) / 16;
@@ -494,9 +495,12 @@ int32_t launch_ring(const I8Args &p, size_t m, size_t n, hipStream_t s) {
   if (attr_err != hipSuccess)
     return set_error(YSCV_HIP_ERR_DEVICE, "cannot reserve %d bytes of LDS: %s", LDS, hipGetErrorString(attr_err));
   const int tiles_m = (int)ceil_div(m, (size_t)(32 * MT)), tiles_n = (int)ceil_div(n, (size_t)(32 * NT));
-  const int super_blocks = ((tiles_m + 7) / 8) * ((tiles_n + 3) / 4);
+  int sbm_log2 = 3;
+  while (sbm_log2 > 0 && (1 << sbm_log2) > tiles_m) sbm_log2--;
+  const int sbm = 1 << sbm_log2, sbn = 32 >> sbm_log2;
+  const int super_blocks = ((tiles_m + sbm - 1) / sbm) * ((tiles_n + sbn - 1) / sbn);
   const unsigned grid = (unsigned)((super_blocks + 7) / 8) * 8 * 32;
-  hipLaunchKernelGGL((i8_gemm_ring_kernel<MT, NT, KS, S>), dim3(grid), dim3(I8R_THREADS), LDS, s, p, tiles_m, tiles_n);
+  hipLaunchKernelGGL((i8_gemm_ring_kernel<MT, NT, KS, S>), dim3(grid), dim3(I8R_THREADS), LDS, s, p, tiles_m, tiles_n, sbm_log2);
   YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
 }

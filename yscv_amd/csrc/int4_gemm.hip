@@ -251,7 +251,9 @@ int32_t launch_int4_gemm(const yscv_hip_int4_weight *w, const _Float16 *xh, cons
                          const float *row_scale, size_t k_pad, int split, void *y, int y_dtype, size_t m,
                          hipStream_t s) {
   if (!w->tiled) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "int4 GEMM kernel needs the tiled layout");
-  if (m >= 128 && int4_gemm_ring_eligible(w, xh, y, y_dtype, split, m, k_pad))
+  // 16-bit activations: the LDS-ring kernel from the first row count the skinny kernel does not take (rows are
+  // padded to its 128-row tile; with few rows the weights are still streamed exactly once)
+  if (m > 16 && int4_gemm_ring_eligible(w, xh, y, y_dtype, split, m, k_pad))
     return launch_int4_gemm_ring(w, xh, row_scale, k_pad, y, y_dtype, m, s);
   GemmArgs a;
   a.tiles = w->tiles;
