@@ -282,6 +282,24 @@ int32_t yscv_hip_exec_dequantize_linear(const float *q_dev, size_t outer, size_t
 int32_t yscv_hip_exec_dynamic_quantize_linear(const float *x_dev, size_t len, float *y_dev,
                                               float *y_scale_dev, float *y_zp_dev, void *stream);
 
+/* quantize_matmul_weights_int4_packed (crates/yscv-onnx/src/quantize/packed_int4.rs:50-128) for one weight
+ * initialiser held as f32 on the device.  layout KN: shape [d0 = K][d1 = N] (MatMul, Gemm transB = 0), transposed
+ * before packing; layout NK: shape [d0 = N][d1 = K] (Gemm transB = 1), packed as it is.  Symmetric per-group
+ * packing (pack_int4_symmetric_per_group, int4_matmul.rs:611-646), f32 scales.  group_size 0 or odd is the
+ * reference's error; a weight the reference skips (K % group_size != 0 or K * N < 32) returns OK with *out = NULL. */
+#define YSCV_HIP_WEIGHT_KN 0
+#define YSCV_HIP_WEIGHT_NK 1
+int32_t yscv_hip_int4_weight_from_f32(const float *w_dev, size_t d0, size_t d1, int32_t layout, size_t group_size,
+                                      void *stream, yscv_hip_int4_weight **out);
+
+/* KvCache int8 storage (crates/yscv-onnx/src/runner/kv_cache.rs:45-61): per-row symmetric int8 of the rows being
+ * appended, src_dev[rows][kv_dim] f32 -> data_dev[rows][kv_dim] int8 + scales_dev[rows]; and the read side
+ * (dequantise_to_vec, kv_cache.rs:64-79). */
+int32_t yscv_hip_kv_i8_quantize_rows(const float *src_dev, size_t rows, size_t kv_dim, int8_t *data_dev,
+                                     float *scales_dev, void *stream);
+int32_t yscv_hip_kv_i8_dequantize_rows(const int8_t *data_dev, const float *scales_dev, size_t rows, size_t kv_dim,
+                                       float *out_dev, void *stream);
+
 /* ---- decode loop (Llama-style decoder, int4 projections, fp16 KV cache) ----------------- */
 
 /* GPU-resident counterpart of the llm-bench decode loop (apps/llm-bench/src/main.rs:403-561:

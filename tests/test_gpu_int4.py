@@ -311,3 +311,33 @@ def test_prefill_gemm_sampled_at_full_size(oracle, K, torch_cuda):
     int4_tolerances(got, bf16_round(ref), k, xs)
     # bf16 output: at most one bf16 ulp away from the rounded oracle
     assert np.abs(got - bf16_round(ref)).max() <= np.abs(ref).max() * 2.0 ** -7
+
+
+@pytest.mark.parametrize("layout", ["kn", "nk"])
+@pytest.mark.parametrize("g", [32, 128])
+def test_int4_weight_from_f32_matches_the_packing_pass(oracle, K, torch_cuda, layout, g):
+    """quantize_matmul_weights_int4_packed (packed_int4.rs:50-128) on one f32 initialiser: transposition for the
+    [K, N] layouts, symmetric per-group packing bit-exact with pack_int4_symmetric_per_group, skip rules."""
+    torch = torch_cuda
+    rng = np.random.default_rng(g + len(layout))
+    n, k = 48, 256
+    w_nk = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    w_nk[3, :g] = 0.0  # an all-zero group: scale 1.0
+    dev = torch.from_numpy(w_nk if layout == "nk" else np.ascontiguousarray(w_nk.T)).cuda()
+    w = K.PackedInt4Weight.from_f32(dev, g, transposed_nk=(layout == "nk"))
+    assert w is not None and (w.m_w, w.k) == (n, k)
+    packed, scales = oracle.pack_int4_symmetric_per_group(w_nk.ravel(), n, k, g)
+    x = rng.standard_normal((3, k)).astype(np.float32)
+    ref = oracle.packed_int4_gemm_scalar(packed, scales, x, 3, n, k, g)
+    y = w.matmul(torch.from_numpy(x).cuda()).cpu().numpy()
+    d, rel = int4_tolerances(y, ref, k, x)
+    assert rel < 2e-5, rel  # same packed nibbles and scales as the reference pass, exact-weight kernel
+    # skip rules and the group-size error
+    assert K.PackedInt4Weight.from_f32(torch.zeros(100, 8, device="cuda"), 32) is None          # K % group != 0
+    assert K.PackedInt4Weight.from_f32(torch.zeros(2, 8, device="cuda"), 2, transposed_nk=True) is None  # K * N < 32
+    import yscv_amd
+
+    for bad in (0, 7):
+        with pytest.raises(yscv_amd.YscvHipError) as ei:
+            K.PackedInt4Weight.from_f32(dev, bad, transposed_nk=(layout == "nk"))
+        assert ei.value.code == -1 and "group_size must be even" in ei.value.message

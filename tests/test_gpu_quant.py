@@ -80,3 +80,26 @@ def test_dynamic_quantize_linear(oracle, K):
         assert np.array_equal(y.astype(np.float32), np.nan_to_num(ye, nan=0.0))
     y, s, z = K.dynamic_quantize_linear(np.zeros(0, np.float32))
     assert y.size == 0 and s == 1.0 and z == 0.0
+
+
+def test_kv_cache_int8_rows_bit_exact(oracle, K):
+    """KvCache I8 append / read (kv_cache.rs:45-79): per-row scale abs_max / 127, f32::round, clamp [-127, 127]."""
+    import torch
+
+    rng = np.random.default_rng(21)
+    for rows, kv_dim in ((1, 1024), (7, 1024), (33, 96), (5, 1)):
+        src = (rng.standard_normal((rows, kv_dim)) * rng.uniform(0.01, 30, (rows, 1))).astype(np.float32)
+        src[0, : min(3, kv_dim)] = [0.5, -0.5, 1.5][: min(3, kv_dim)]
+        if rows > 2:
+            src[1] = 0.0          # abs_max <= EPSILON: scale 1
+            src[2, 0] = np.nan    # NaN does not enter the abs-max and quantises to 0
+        ed, es = oracle.kv_i8_quantize_rows(src, rows, kv_dim)
+        d, s = K.kv_i8_quantize_rows(torch.from_numpy(src).cuda())
+        assert np.array_equal(s.cpu().numpy(), es)
+        assert np.array_equal(d.cpu().numpy().ravel(), ed)
+        back = K.kv_i8_dequantize_rows(d, s).cpu().numpy()
+        assert np.array_equal(back, ed.reshape(rows, kv_dim).astype(np.float32) * es[:, None])
+    # ties: v * inv exactly on .5 rounds away from zero
+    src = np.array([[127.0, 0.5, -0.5, 1.5, -2.5, 63.5]], np.float32)
+    d, s = K.kv_i8_quantize_rows(torch.from_numpy(src).cuda())
+    assert float(s[0]) == 1.0 and d.cpu().numpy().ravel().tolist() == [127, 1, -1, 2, -3, 64]

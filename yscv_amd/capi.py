@@ -91,6 +91,9 @@ _SIGNATURES = {
     "yscv_hip_exec_quantize_linear": [_vp, _sz, _f32, _f32, _vp, _vp],
     "yscv_hip_exec_dequantize_linear": [_vp, _sz, _sz, _sz, _vp, _vp, _sz, _vp, _vp],
     "yscv_hip_exec_dynamic_quantize_linear": [_vp, _sz, _vp, _vp, _vp, _vp],
+    "yscv_hip_int4_weight_from_f32": [_vp, _sz, _sz, _i32, _sz, _vp, C.POINTER(_vp)],
+    "yscv_hip_kv_i8_quantize_rows": [_vp, _sz, _sz, _vp, _vp, _vp],
+    "yscv_hip_kv_i8_dequantize_rows": [_vp, _vp, _sz, _sz, _vp, _vp],
     "yscv_hip_decoder_create": [_vp, C.POINTER(_vp)],
     "yscv_hip_decoder_destroy": [_vp],
     "yscv_hip_decoder_set_linear": [_vp, _i32, _i32, _vp, _vp, _sz, _sz],

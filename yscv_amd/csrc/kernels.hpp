@@ -121,4 +121,8 @@ int32_t launch_requant(const int32_t *acc, size_t len, size_t c, const int32_t *
 int32_t launch_dynamic_quantize_linear(const float *x, size_t len, uint8_t *y, float *scale_zp,
                                        hipStream_t s);
 
+int32_t launch_kv_i8_quantize_rows(const float *src, size_t rows, size_t kv_dim, int8_t *data, float *scales, hipStream_t s);
+int32_t launch_kv_i8_dequantize_rows(const int8_t *data, const float *scales, size_t rows, size_t kv_dim, float *out,
+                                     hipStream_t s);
+
 }  // namespace yscv

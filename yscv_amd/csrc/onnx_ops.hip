@@ -181,6 +181,18 @@ __global__ void u8_to_f32_kernel(const uint8_t *__restrict__ q, size_t len, cons
   }
 }
 
+// [d0][d1] -> [d1][d0]
+__global__ void transpose_f32_kernel(const float *__restrict__ in, size_t d0, size_t d1, float *__restrict__ out) {
+  __shared__ float tile[32][33];
+  const size_t x = blockIdx.x * 32 + threadIdx.x, y0 = blockIdx.y * 32;
+  for (int j = threadIdx.y; j < 32; j += blockDim.y)
+    if (x < d1 && y0 + j < d0) tile[j][threadIdx.x] = in[(y0 + j) * d1 + x];
+  __syncthreads();
+  const size_t ox = blockIdx.y * 32 + threadIdx.x, oy0 = blockIdx.x * 32;
+  for (int j = threadIdx.y; j < 32; j += blockDim.y)
+    if (ox < d0 && oy0 + j < d1) out[(oy0 + j) * d0 + ox] = tile[threadIdx.x][j];
+}
+
 struct Operand8 {
   DevBuf buf;
   int shift = 0;    // added to every value
@@ -426,6 +438,53 @@ int32_t yscv_hip_i8_weight_from_f32(const float *b_dev, size_t k, size_t n, void
     return set_error(YSCV_HIP_ERR_DEVICE, "packing B failed: %s", hipGetErrorString(e));
   }
   return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_int4_weight_from_f32(const float *w_dev, size_t d0, size_t d1, int32_t layout, size_t group_size,
+                                      void *stream, yscv_hip_int4_weight **out) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(out != nullptr, "null output handle pointer");
+  *out = nullptr;
+  YSCV_REQUIRE(group_size != 0 && (group_size & 1) == 0, "group_size must be even and > 0, got %zu", group_size);
+  YSCV_REQUIRE(layout == YSCV_HIP_WEIGHT_KN || layout == YSCV_HIP_WEIGHT_NK, "unknown weight layout %d", layout);
+  YSCV_REQUIRE(w_dev != nullptr && d0 > 0 && d1 > 0, "null weight / empty shape");
+  const size_t m_w = layout == YSCV_HIP_WEIGHT_KN ? d1 : d0, k = layout == YSCV_HIP_WEIGHT_KN ? d0 : d1;
+  if (k % group_size != 0 || k * m_w < 32) return YSCV_HIP_OK;  // the reference skips these weights silently
+  if (!(group_size == 32 || group_size == 64 || group_size % 128 == 0))
+    return set_error(YSCV_HIP_ERR_UNSUPPORTED, "device-side packing needs group size 32, 64 or a multiple of 128, got %zu",
+                     group_size);
+  hipStream_t s = as_stream(stream);
+  DevBuf t, packed, scales;
+  const float *src = w_dev;
+  if (layout == YSCV_HIP_WEIGHT_KN) {
+    YSCV_TRY(t.alloc(d0 * d1 * sizeof(float)));
+    dim3 grid((unsigned)ceil_div(d1, (size_t)32), (unsigned)ceil_div(d0, (size_t)32));
+    YSCV_REQUIRE(grid.y <= 65535, "weight too tall to transpose in one launch");
+    hipLaunchKernelGGL(transpose_f32_kernel, grid, dim3(32, 8), 0, s, w_dev, d0, d1, t.as<float>());
+    YSCV_HIP_TRY(hipGetLastError());
+    src = t.as<float>();
+  }
+  YSCV_TRY(packed.alloc(m_w * k / 2));
+  YSCV_TRY(scales.alloc(m_w * (k / group_size) * sizeof(float)));
+  YSCV_TRY(launch_pack_int4_symmetric(src, m_w, k, group_size, packed.as<uint8_t>(), scales.as<float>(), s));
+  YSCV_HIP_TRY(hipStreamSynchronize(s));
+  return int4_create_from_device(packed.as<uint8_t>(), scales.p, YSCV_HIP_F32, YSCV_HIP_NIBBLE_SIGNED, m_w, k, group_size, out);
+}
+
+int32_t yscv_hip_kv_i8_quantize_rows(const float *src_dev, size_t rows, size_t kv_dim, int8_t *data_dev, float *scales_dev,
+                                     void *stream) {
+  YSCV_TRY(ensure_context(nullptr));
+  if (rows == 0) return YSCV_HIP_OK;
+  YSCV_REQUIRE(src_dev && data_dev && scales_dev && kv_dim > 0, "null pointer / empty row");
+  return launch_kv_i8_quantize_rows(src_dev, rows, kv_dim, data_dev, scales_dev, as_stream(stream));
+}
+
+int32_t yscv_hip_kv_i8_dequantize_rows(const int8_t *data_dev, const float *scales_dev, size_t rows, size_t kv_dim,
+                                       float *out_dev, void *stream) {
+  YSCV_TRY(ensure_context(nullptr));
+  if (rows == 0) return YSCV_HIP_OK;
+  YSCV_REQUIRE(data_dev && scales_dev && out_dev && kv_dim > 0, "null pointer / empty row");
+  return launch_kv_i8_dequantize_rows(data_dev, scales_dev, rows, kv_dim, out_dev, as_stream(stream));
 }
 
 int32_t yscv_hip_exec_matmul_integer(const float *a_dev, const float *b_dev, const yscv_hip_i8_weight *b_packed,

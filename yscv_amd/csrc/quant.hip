@@ -172,4 +172,47 @@ int32_t launch_dynamic_quantize_linear(const float *x, size_t len, uint8_t *y, f
   return YSCV_HIP_OK;
 }
 
+// ---- KV-cache int8 storage: per-row symmetric quantisation (crates/yscv-onnx/src/runner/kv_cache.rs:45-61) ----
+// One wavefront per appended row: abs-max (f32::max ignores NaN), scale = abs_max / 127 (1.0 when abs_max <=
+// EPSILON), q = clamp(round_half_away(v * (1 / scale)), -127, 127) as i8.
+__global__ void __launch_bounds__(256) kv_i8_quantize_rows_kernel(const float *__restrict__ src, size_t rows, size_t kv_dim,
+                                                                  int8_t *__restrict__ data, float *__restrict__ scales) {
+  const size_t row = blockIdx.x * (size_t)(blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int lane = threadIdx.x & 63;
+  const float *x = src + row * kv_dim;
+  float amax = 0.0f;
+  for (size_t i = lane; i < kv_dim; i += 64) amax = fmaxf(amax, fabsf(x[i]));  // fmaxf drops NaN like f32::max
+  for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+  const float scale = (amax <= 1.1920929e-7f) ? 1.0f : __fdiv_rn(amax, 127.0f);
+  const float inv = __fdiv_rn(1.0f, scale);
+  if (lane == 0) scales[row] = scale;
+  for (size_t i = lane; i < kv_dim; i += 64)
+    data[row * kv_dim + i] = (int8_t)clamp_cast(round_half_away_f(__fmul_rn(x[i], inv)), -127.0f, 127.0f);
+}
+
+// LayerStorage::dequantise_to_vec (kv_cache.rs:64-79): q as f32 * scale of its row
+__global__ void kv_i8_dequantize_rows_kernel(const int8_t *__restrict__ data, const float *__restrict__ scales, size_t rows,
+                                             size_t kv_dim, float *__restrict__ out) {
+  const size_t total = rows * kv_dim;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x)
+    out[i] = __fmul_rn((float)data[i], scales[i / kv_dim]);
+}
+
+int32_t launch_kv_i8_quantize_rows(const float *src, size_t rows, size_t kv_dim, int8_t *data, float *scales, hipStream_t s) {
+  hipLaunchKernelGGL(kv_i8_quantize_rows_kernel, dim3((unsigned)ceil_div(rows, (size_t)4)), dim3(256), 0, s, src, rows, kv_dim,
+                     data, scales);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_kv_i8_dequantize_rows(const int8_t *data, const float *scales, size_t rows, size_t kv_dim, float *out,
+                                     hipStream_t s) {
+  size_t blocks = ceil_div(rows * kv_dim, (size_t)256);
+  if (blocks > 16384) blocks = 16384;
+  hipLaunchKernelGGL(kv_i8_dequantize_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, s, data, scales, rows, kv_dim, out);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
 }  // namespace yscv

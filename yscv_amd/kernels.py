@@ -116,6 +116,32 @@ def dynamic_quantize_linear(x):
     return y, np.float32(s.value), np.float32(z.value)
 
 
+def kv_i8_quantize_rows(src):
+    """KvCache int8 append (runner/kv_cache.rs:45-61): src CUDA f32 [rows][kv_dim] -> (int8 [rows][kv_dim], f32 [rows])."""
+    import torch
+
+    assert src.is_cuda and src.dtype == torch.float32 and src.dim() == 2
+    src = src.contiguous()
+    rows, kv_dim = int(src.shape[0]), int(src.shape[1])
+    data = torch.empty(rows, kv_dim, device=src.device, dtype=torch.int8)
+    scales = torch.empty(rows, device=src.device, dtype=torch.float32)
+    lib().kv_i8_quantize_rows(C.c_void_p(src.data_ptr()), _sz(rows), _sz(kv_dim), C.c_void_p(data.data_ptr()),
+                              C.c_void_p(scales.data_ptr()), _stream_ptr())
+    return data, scales
+
+
+def kv_i8_dequantize_rows(data, scales):
+    """KvCache int8 read (runner/kv_cache.rs:64-79)."""
+    import torch
+
+    assert data.is_cuda and data.dtype == torch.int8 and data.dim() == 2 and scales.dtype == torch.float32
+    rows, kv_dim = int(data.shape[0]), int(data.shape[1])
+    out = torch.empty(rows, kv_dim, device=data.device, dtype=torch.float32)
+    lib().kv_i8_dequantize_rows(C.c_void_p(data.contiguous().data_ptr()), C.c_void_p(scales.contiguous().data_ptr()), _sz(rows),
+                                _sz(kv_dim), C.c_void_p(out.data_ptr()), _stream_ptr())
+    return out
+
+
 # ---- device handles ---------------------------------------------------------------------------
 
 class PackedInt4Weight:
@@ -139,6 +165,27 @@ class PackedInt4Weight:
                                  _sz(m_w), _sz(k), _sz(group_size), C.byref(h))
         self._h = h
         self.m_w, self.k, self.group_size = m_w, k, group_size
+
+    @classmethod
+    def from_f32(cls, weight, group_size, transposed_nk=False):
+        """quantize_matmul_weights_int4_packed (quantize/packed_int4.rs:50-128) for one initialiser: weight is a CUDA
+        f32 tensor of shape [K, N] (MatMul, Gemm transB=0) or, with transposed_nk, [N, K] (Gemm transB=1).
+        Returns None for a weight the reference skips (K % group_size != 0 or K * N < 32)."""
+        import torch
+
+        assert weight.is_cuda and weight.dtype == torch.float32 and weight.dim() == 2
+        weight = weight.contiguous()
+        d0, d1 = int(weight.shape[0]), int(weight.shape[1])
+        h = C.c_void_p()
+        lib().int4_weight_from_f32(C.c_void_p(weight.data_ptr()), _sz(d0), _sz(d1), 1 if transposed_nk else 0,
+                                   _sz(group_size), _stream_ptr(), C.byref(h))
+        if not h:
+            return None
+        self = cls.__new__(cls)
+        self._h = h
+        self.m_w, self.k = (d0, d1) if transposed_nk else (d1, d0)
+        self.group_size = group_size
+        return self
 
     @property
     def handle(self):
