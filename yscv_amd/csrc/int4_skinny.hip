@@ -41,6 +41,7 @@ struct SkinnyArgs {
   const uint8_t *tzps;  // null: zero point 8 everywhere
   const _Float16 *xh;
   const _Float16 *xl;
+  const float *xf;  // raw f32 activations (row stride k_pad) for the kernels that split them themselves, else null
   const float *row_scale;
   void *y;
   float *partial;  // [ksg][m][n] when ksg > 1
@@ -140,8 +141,9 @@ __device__ __forceinline__ void zp_consts(uint32_t zp, half2_t &c1, half2_t &c2)
   c2 = half2_t{b, b};
 }
 
-template <int SPLIT, int NI, int GM, bool SF16, bool HAS_ZP, int P>
+template <int SPLIT, int NI, int GM, bool SF16, bool HAS_ZP, int P, bool RAWX>
 __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
+  static_assert(!RAWX || SPLIT == 2, "raw f32 activations are split into hi + lo");
   // OFFSET mode: leave the 1024-offsets in the weights and cancel them per group (see file header)
   constexpr bool OFFSET = (SPLIT == 1) && !HAS_ZP && (NI == 1);
   constexpr int SPT = GM == GM32 ? 4 : (GM == GM64 ? 2 : 1);
@@ -161,28 +163,82 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
   // MFMA row `r` carries batch row m when r == 4*(m / NI) + (m % NI): the useful results then sit
   // in the first NI of the four accumulator registers of each lane.
   half8_t xa[TPW][4][SPLIT];
+  float slice_scale = 1.0f;  // RAWX: what this wave's products of the row it loads must be multiplied by
   {
     const int i = r & 3;
     const int mrow = (r >> 2) * NI + i;
     const bool valid = wave_active && (i < NI) && (mrow < a.m);
     const half8_t pre = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)0.0625f, (_Float16)0.0625f,
                          (_Float16)1.0f, (_Float16)1.0f, (_Float16)0.0625f, (_Float16)0.0625f};
+    if constexpr (RAWX) {
+      // f32 activations straight from the caller: the wave normalises its own 512-k slice of every row by a power
+      // of two (abs-max to [2^14, 2^15), as the separate activation pass does per row) and splits it into fp16
+      // hi + lo; the power of two is undone on the wave's partial sums before they meet the other slices.
+      const float *src = a.xf + (size_t)mrow * a.k_pad + (size_t)t0 * 128 + c * 8;
+      float amax = 0.0f;
+      if (valid) {
 #pragma unroll
-    for (int t = 0; t < TPW; t++) {
+        for (int t = 0; t < TPW; t++)
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        half8_t h = {0, 0, 0, 0, 0, 0, 0, 0}, l = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (valid) {
-          const size_t off = (size_t)mrow * a.k_pad + (size_t)(t0 + t) * 128 + j * 32 + c * 8;
-          h = *reinterpret_cast<const half8_t *>(a.xh + off);
-          if constexpr (SPLIT == 2) l = *reinterpret_cast<const half8_t *>(a.xl + off);
+          for (int j = 0; j < 4; j++) {
+            const float4_t v0 = *reinterpret_cast<const float4_t *>(src + t * 128 + j * 32);
+            const float4_t v1 = *reinterpret_cast<const float4_t *>(src + t * 128 + j * 32 + 4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) amax = fmaxf(amax, fmaxf(fabsf(v0[e]), fabsf(v1[e])));
+          }
+      }
+      amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+      amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+      int e2 = 14;
+      if (amax > 0.0f && amax < 3.0e38f) {
+        (void)frexpf(amax, &e2);
+        e2 -= 1;
+      }
+      int shift = 14 - e2;
+      shift = shift > 100 ? 100 : (shift < -100 ? -100 : shift);
+      const float up = ldexpf(1.0f, shift);
+      slice_scale = ldexpf(1.0f, -shift);
+#pragma unroll
+      for (int t = 0; t < TPW; t++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          half8_t h = {0, 0, 0, 0, 0, 0, 0, 0}, l = {0, 0, 0, 0, 0, 0, 0, 0};
+          if (valid) {
+            const float4_t v0 = *reinterpret_cast<const float4_t *>(src + t * 128 + j * 32);
+            const float4_t v1 = *reinterpret_cast<const float4_t *>(src + t * 128 + j * 32 + 4);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+              const float sv = (e < 4 ? v0[e] : v1[e - 4]) * up;
+              h[e] = (_Float16)sv;
+              l[e] = (_Float16)(sv - (float)h[e]);
+            }
+          }
+          xa[t][j][0] = h;
+          xa[t][j][1] = l;
         }
-        if constexpr (OFFSET) h = h * pre;  // slots that meet 1024 + 16 q carry x / 16 (a power of two)
-        xa[t][j][0] = h;
-        if constexpr (SPLIT == 2) xa[t][j][1] = l;
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < TPW; t++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          half8_t h = {0, 0, 0, 0, 0, 0, 0, 0}, l = {0, 0, 0, 0, 0, 0, 0, 0};
+          if (valid) {
+            const size_t off = (size_t)mrow * a.k_pad + (size_t)(t0 + t) * 128 + j * 32 + c * 8;
+            h = *reinterpret_cast<const half8_t *>(a.xh + off);
+            if constexpr (SPLIT == 2) l = *reinterpret_cast<const half8_t *>(a.xl + off);
+          }
+          if constexpr (OFFSET) h = h * pre;  // slots that meet 1024 + 16 q carry x / 16 (a power of two)
+          xa[t][j][0] = h;
+          if constexpr (SPLIT == 2) xa[t][j][1] = l;
+        }
       }
     }
   }
+  // RAWX: accumulator i of lane (c, .) belongs to row c * NI + i, which lanes 4 c + i (+16, +32, +48) loaded
+  float acc_scale[NI];
+#pragma unroll
+  for (int i = 0; i < NI; i++) acc_scale[i] = RAWX ? __shfl(slice_scale, 4 * c + i, 64) : 1.0f;
   // offset term of every 32-k block: sum_k x'_k * (1024 + 8 | 1024 + 128), same register layout as D
   float corr1[OFFSET ? TPW : 1][4];
   if constexpr (OFFSET) {
@@ -269,6 +325,10 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
           d = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
         }
       }
+    }
+    if constexpr (RAWX) {
+#pragma unroll
+      for (int i = 0; i < NI; i++) acc[i] *= acc_scale[i];
     }
   };
 
@@ -432,7 +492,15 @@ static int32_t launch_one(const SkinnyArgs &a, const SkinnyPlan &plan, hipStream
   // ring depth: bounded by the VGPR budget (activations: 64 per split, ring: ~26 per slot)
   constexpr int P = SPLIT == 2 ? (NI == 1 ? 2 : 1) : (NI == 1 ? 4 : 3);
   const size_t lds = (size_t)2 * plan.waves * NI * 64 * sizeof(float);
-  hipLaunchKernelGGL((int4_skinny_kernel<SPLIT, NI, GM, SF16, HAS_ZP, P>), dim3(plan.grid_x, plan.ksg),
+  if constexpr (SPLIT == 2) {
+    if (a.xf != nullptr) {
+      hipLaunchKernelGGL((int4_skinny_kernel<SPLIT, NI, GM, SF16, HAS_ZP, P, true>), dim3(plan.grid_x, plan.ksg),
+                         dim3(plan.waves * 64), lds, s, a);
+      YSCV_HIP_TRY(hipGetLastError());
+      return YSCV_HIP_OK;
+    }
+  }
+  hipLaunchKernelGGL((int4_skinny_kernel<SPLIT, NI, GM, SF16, HAS_ZP, P, false>), dim3(plan.grid_x, plan.ksg),
                      dim3(plan.waves * 64), lds, s, a);
   YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
@@ -453,7 +521,7 @@ static int32_t launch_gm(const SkinnyArgs &a, const SkinnyPlan &plan, int gm, bo
 }
 
 int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan, const _Float16 *xh,
-                           const _Float16 *xl, const float *row_scale, size_t k_pad, int split,
+                           const _Float16 *xl, const float *xf, const float *row_scale, size_t k_pad, int split,
                            void *y, int y_dtype, size_t m, float *partial, int epi, hipStream_t s) {
   if (!w->tiled) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "skinny int4 kernel needs the tiled layout");
   if (m == 0 || m > 16) return set_error(YSCV_HIP_ERR_INVALID_ARG, "skinny int4 kernel handles 1 <= m <= 16, got %zu", m);
@@ -466,6 +534,7 @@ int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan
   a.tzps = w->has_zp ? w->tzps : nullptr;
   a.xh = xh;
   a.xl = xl;
+  a.xf = split == 2 ? xf : nullptr;
   a.row_scale = row_scale;
   a.y = y;
   a.partial = partial;
