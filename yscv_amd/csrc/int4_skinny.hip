@@ -332,35 +332,35 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
     }
   };
 
-  // meet the other k slices in LDS; one wave (rotating) sums them and writes the 16 x m results
+  // meet the other k slices in LDS; the NI x 64 sums are shared out over the waves in half-wave pieces (piece q =
+  // accumulator q / 2, lanes 32 (q % 2) .. +31), so no single wave is late for the next block
   auto reduce_store = [&](const float acc[NI], int nt, int it) {
     float *buf = red + (size_t)(it & 1) * waves * NI * 64;
 #pragma unroll
     for (int i = 0; i < NI; i++) buf[(wave * NI + i) * 64 + lane] = acc[i];
     lds_barrier();
-    if (wave == (it % waves)) {
+    for (int q = (wave + it) % waves; q < NI * 2; q += waves) {
+      const int i = q >> 1;
+      if ((lane >> 5) != (q & 1)) continue;
       const int col = nt * 16 + r;
-#pragma unroll
-      for (int i = 0; i < NI; i++) {
-        float v = 0.0f;
-        for (int w = 0; w < waves; w++) v += buf[(w * NI + i) * 64 + lane];
-        const int mrow = c * NI + i;
-        const bool live = mrow < a.m && col < a.n;
-        if (a.ksg > 1) {
-          if (live) a.partial[((size_t)blockIdx.y * a.m + mrow) * a.n + col] = v;
-        } else {
-          if (a.row_scale && mrow < a.m) v *= a.row_scale[mrow];
-          if (a.epi == EPI_SWIGLU) {
-            // rows 2i / 2i+1 of the weight are gate_i / up_i: neighbours in the wave
-            const float up = __shfl_xor(v, 1, 64);
-            if (live && !(r & 1))
-              store_out(a.y, (size_t)mrow * (a.n >> 1) + (col >> 1), silu(v) * up, a.y_dtype);
-          } else if (a.epi == EPI_ADD_F32) {
-            // single writer per element: a returnless add keeps the residual update off the load queue
-            if (live) unsafeAtomicAdd(reinterpret_cast<float *>(a.y) + (size_t)mrow * a.n + col, v);
-          } else if (live) {
-            store_out(a.y, (size_t)mrow * a.n + col, v, a.y_dtype);
-          }
+      float v = 0.0f;
+      for (int w = 0; w < waves; w++) v += buf[(w * NI + i) * 64 + lane];
+      const int mrow = c * NI + i;
+      const bool live = mrow < a.m && col < a.n;
+      if (a.ksg > 1) {
+        if (live) a.partial[((size_t)blockIdx.y * a.m + mrow) * a.n + col] = v;
+      } else {
+        if (a.row_scale && mrow < a.m) v *= a.row_scale[mrow];
+        if (a.epi == EPI_SWIGLU) {
+          // rows 2i / 2i+1 of the weight are gate_i / up_i: neighbours in the wave
+          const float up = __shfl_xor(v, 1, 64);
+          if (live && !(r & 1))
+            store_out(a.y, (size_t)mrow * (a.n >> 1) + (col >> 1), silu(v) * up, a.y_dtype);
+        } else if (a.epi == EPI_ADD_F32) {
+          // single writer per element: a returnless add keeps the residual update off the load queue
+          if (live) unsafeAtomicAdd(reinterpret_cast<float *>(a.y) + (size_t)mrow * a.n + col, v);
+        } else if (live) {
+          store_out(a.y, (size_t)mrow * a.n + col, v, a.y_dtype);
         }
       }
     }
