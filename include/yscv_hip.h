@@ -381,6 +381,29 @@ int32_t yscv_hip_decoder_read_tokens(yscv_hip_decoder *d, int32_t first_step, in
 int32_t yscv_hip_decoder_read_logits(yscv_hip_decoder *d, float *out_host);
 /* Bytes of packed weights + scales one decode step streams through the projections. */
 int32_t yscv_hip_decoder_weight_bytes(const yscv_hip_decoder *d, size_t *bytes);
+int32_t yscv_hip_decoder_vocab(const yscv_hip_decoder *d, size_t *vocab);
+
+/* GenerateConfig (crates/yscv-onnx/src/generate.rs:9-35; its Default is 256, 1.0, 50, 0.9, no EOS, 1.0). */
+typedef struct yscv_hip_generate_config {
+  size_t max_tokens;
+  float temperature;        /* 1.0 = unchanged; values <= 0 are ignored like in the reference */
+  size_t top_k;             /* 0 = disabled; 1 = greedy */
+  float top_p;              /* 1.0 = disabled */
+  int32_t has_eos;          /* Option<u32>: 0 = None */
+  uint32_t eos_token_id;
+  float repetition_penalty; /* 1.0 = disabled */
+} yscv_hip_generate_config;
+/* sample_token (generate.rs:121-208) on host logits, in place: top-k threshold, softmax, top-p cut, xorshift64
+ * draw; *rng is the sampler state (generate() starts it at 0xdeadbeef). */
+int32_t yscv_hip_sample_token(float *logits, size_t vocab_size, size_t top_k, float top_p, uint64_t *rng,
+                              uint32_t *token_out);
+/* generate (generate.rs:58-118) with the decoder as the model: the prompt is fed through the KV cache one position
+ * at a time from position 0, then up to max_tokens tokens are sampled on the host from the logits of each decode
+ * step.  generated_out holds max_tokens entries; *n_generated tells how many were produced (EOS stops early and is
+ * not stored). */
+int32_t yscv_hip_decoder_generate(yscv_hip_decoder *d, const uint32_t *input_ids, size_t n_input,
+                                  const yscv_hip_generate_config *cfg, uint32_t *generated_out,
+                                  size_t *n_generated);
 
 #if defined(__GNUC__)
 #pragma GCC visibility pop

@@ -156,3 +156,39 @@ def test_persistent_decode_matches_numpy_and_graph_path(prefill):
     graph_logits = dec.logits()
     assert np.array_equal(dec.tokens(0, 5)[:, 0], first)
     assert np.abs(graph_logits - logits5).max() / np.abs(logits5).max() < 5e-3
+
+
+def test_generate_matches_device_greedy_and_stops_at_eos():
+    """generate() (generate.rs:58-118) with the decoder as the model: top_k = 1 reproduces the tokens the device picks
+    greedily; an EOS token ends the loop without being stored; the sampling path runs with the default configuration."""
+    import numpy as np
+
+    from yscv_amd.decoder import Decoder
+
+    cfg = dict(n_layers=2, d_model=512, n_heads=4, n_kv_heads=2, head_dim=128, d_ff=1024, vocab=320, group_size=32,
+               max_batch=1, max_ctx=256, max_steps=64, rope_theta=10000.0, rms_eps=1e-5)
+    dec = Decoder(**cfg)
+    dec.init_random(seed=5)
+    prompt = [7, 3, 11]
+    got = dec.generate(prompt, max_tokens=12, top_k=1, top_p=1.0)
+    # the same through the device-side greedy loop: feed the prompt, then let the decoder run on its own picks
+    dec.reset(np.array([prompt[0]], np.int32), 0)
+    dec.run(1, use_graph=False)
+    for p, t in enumerate(prompt[1:], start=1):
+        dec.reset(np.array([t], np.int32), p)
+        dec.run(1, use_graph=False)
+    first = int(dec.tokens(0, 1)[0, 0])
+    dec.reset(np.array([first], np.int32), len(prompt))
+    dec.run(11, use_graph=False)
+    want = [first] + dec.tokens(0, 11)[:, 0].tolist()
+    assert got.tolist() == want
+    # EOS: the third generated token as EOS stops after two
+    eos = int(got[2])
+    if eos not in got[:2].tolist():
+        short = dec.generate(prompt, max_tokens=12, top_k=1, top_p=1.0, eos_token_id=eos)
+        assert short.tolist() == got[:2].tolist()
+    # default configuration (top_k 50, top_p 0.9) with temperature and repetition penalty: valid tokens, reproducible
+    a = dec.generate(prompt, max_tokens=8, temperature=0.8, repetition_penalty=1.3)
+    b = dec.generate(prompt, max_tokens=8, temperature=0.8, repetition_penalty=1.3)
+    assert a.tolist() == b.tolist() and len(a) == 8 and (a < cfg["vocab"]).all()
+    dec.close()

@@ -22,6 +22,13 @@ class DecoderConfig(C.Structure):
                [("rope_theta", C.c_float), ("rms_eps", C.c_float)]
 
 
+class GenerateConfig(C.Structure):
+    """yscv_hip_generate_config (GenerateConfig, crates/yscv-onnx/src/generate.rs:9-35)."""
+
+    _fields_ = [("max_tokens", C.c_size_t), ("temperature", C.c_float), ("top_k", C.c_size_t), ("top_p", C.c_float),
+                ("has_eos", C.c_int32), ("eos_token_id", C.c_uint32), ("repetition_penalty", C.c_float)]
+
+
 class QuantStats(C.Structure):
     """yscv_hip_quant_stats."""
 
@@ -109,6 +116,9 @@ _SIGNATURES = {
     "yscv_hip_decoder_read_tokens": [_vp, _i32, _i32, _vp],
     "yscv_hip_decoder_read_logits": [_vp, _vp],
     "yscv_hip_decoder_weight_bytes": [_vp, C.POINTER(_sz)],
+    "yscv_hip_decoder_vocab": [_vp, C.POINTER(_sz)],
+    "yscv_hip_sample_token": [_vp, _sz, _sz, _f32, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32)],
+    "yscv_hip_decoder_generate": [_vp, _vp, _sz, _vp, _vp, C.POINTER(_sz)],
 }
 _SPECIAL = {
     "yscv_hip_abi_version": ([], C.c_uint32),

@@ -715,6 +715,12 @@ int32_t yscv_hip_decoder_read_logits(yscv_hip_decoder *d, float *out_host) {
   return YSCV_HIP_OK;
 }
 
+int32_t yscv_hip_decoder_vocab(const yscv_hip_decoder *d, size_t *vocab) {
+  YSCV_REQUIRE(d && vocab, "null argument");
+  *vocab = (size_t)d->cfg.vocab;
+  return YSCV_HIP_OK;
+}
+
 int32_t yscv_hip_decoder_weight_bytes(const yscv_hip_decoder *d, size_t *bytes) {
   YSCV_REQUIRE(d && bytes, "null argument");
   *bytes = d->weight_bytes;

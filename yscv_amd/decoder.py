@@ -5,6 +5,7 @@ import ctypes as C
 
 import numpy as np
 
+from . import capi
 from .capi import DecoderConfig, lib
 
 KINDS = {"q": 0, "k": 1, "v": 2, "o": 3, "gate": 4, "up": 5, "down": 6, "lm_head": 7}
@@ -77,6 +78,18 @@ class Decoder:
         out = np.empty((self.batch, self.cfg["vocab"]), np.float32)
         lib().decoder_read_logits(self._h, _p(out))
         return out
+
+    def generate(self, input_ids, max_tokens=256, temperature=1.0, top_k=50, top_p=0.9, eos_token_id=None,
+                 repetition_penalty=1.0):
+        """generate() of crates/yscv-onnx/src/generate.rs:58-118 with this decoder as the model (defaults = GenerateConfig
+        ::default()).  Returns the generated token ids (prompt not included)."""
+        ids = np.ascontiguousarray(input_ids, dtype=np.uint32)
+        cfg = capi.GenerateConfig(max_tokens, temperature, top_k, top_p, 0 if eos_token_id is None else 1,
+                                  0 if eos_token_id is None else int(eos_token_id), repetition_penalty)
+        out = np.zeros(max(max_tokens, 1), np.uint32)
+        n = C.c_size_t(0)
+        lib().decoder_generate(self._h, _p(ids), C.c_size_t(ids.size), C.byref(cfg), _p(out), C.byref(n))
+        return out[: n.value].copy()
 
     def weight_bytes(self) -> int:
         b = C.c_size_t()

@@ -302,3 +302,13 @@ def pack_i8_b_for_matmul(b, k, n) -> PackedI8B:
 def int8_matmul_prepacked_dispatch(a, b: PackedI8B, m, out) -> None:
     """int8_matmul.rs:2420."""
     b.matmul_host(a, m, out)
+
+
+def sample_token(logits, top_k, top_p, rng_state):
+    """sample_token (crates/yscv-onnx/src/generate.rs:121-208) on a host float32 array, modified in place like the
+    Rust `&mut [f32]`.  Returns (token, new_rng_state)."""
+    assert isinstance(logits, np.ndarray) and logits.dtype == np.float32 and logits.flags.c_contiguous
+    rng = C.c_uint64(rng_state)
+    tok = C.c_uint32(0)
+    lib().sample_token(_ptr(logits), _sz(logits.size), _sz(top_k), C.c_float(top_p), C.byref(rng), C.byref(tok))
+    return tok.value, rng.value
