@@ -267,6 +267,14 @@ int32_t yscv_hip_exec_qlinear_matmul(const float *a_dev, float a_scale, float a_
                                      const yscv_hip_i8_weight *b_packed, float b_scale, float b_zp,
                                      float y_scale, float y_zp, size_t m, size_t k, size_t n,
                                      float *out_dev, int32_t *path_out, void *stream);
+/* The triple the reference's rewriter emits for a quantised MatMul, QuantizeLinear -> QLinearMatMul ->
+ * DequantizeLinear with symmetric activations and weights (crates/yscv-onnx/src/quantize/rewriter.rs:586-673), as
+ * one call on f32 in / f32 out: a_q = clamp(round_ties_even(x / a_scale), -128, 127) (misc.rs:42-80), the int8
+ * product against the prepacked weight, q = clamp(round_half_away(acc * ((a_scale * b_scale) / y_scale) + y_zp),
+ * -128, 127) (linear.rs:481-485), y = (q - y_zp) * y_scale (misc.rs:124-128).  Bit-identical to running the three
+ * operators one after the other; counted as one qlinear_matmul_fast. */
+int32_t yscv_hip_exec_qdq_matmul(const float *x_dev, size_t m, float a_scale, const yscv_hip_i8_weight *b,
+                                 float b_scale, float y_scale, float y_zp, float *out_dev, void *stream);
 /* exec_quantize_linear, f32-carrier arm (crates/yscv-onnx/src/runner/misc.rs:42-80) =
  * quantize_linear_f32_to_f32_i8_scalar (crates/yscv-kernels/src/ops/quantize.rs:226-238). */
 int32_t yscv_hip_exec_quantize_linear(const float *x_dev, size_t len, float scale, float zero_point,

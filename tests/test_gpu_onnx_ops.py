@@ -253,3 +253,32 @@ def test_dynamic_quantize_linear_matches_checker(oracle, torch_cuda, ops):
     assert path == ops.PATH_FALLBACK_EXACT
     exact = (y.cpu().numpy().astype(np.int64) - int(float(z))) @ w.astype(np.int64)
     assert np.array_equal(out.cpu().numpy(), exact.astype(np.float32))
+
+
+@pytest.mark.parametrize("shape", [(5, 64, 48), (33, 200, 70), (130, 1024, 260), (512, 512, 1040)])
+def test_qdq_matmul_equals_the_three_operators(oracle, torch_cuda, ops, shape):
+    """The rewriter's QuantizeLinear -> QLinearMatMul -> DequantizeLinear triple (rewriter.rs:586-673) as one call:
+    bit-identical to the oracle's three operators chained, and to this library's three entry points chained."""
+    torch = torch_cuda
+    m, k, n = shape
+    rng = np.random.default_rng(m + k + n)
+    x = (rng.standard_normal((m, k)) * 2.0).astype(np.float32)
+    w = (rng.standard_normal((k, n)) * 0.1).astype(np.float32)
+    a_s = float(np.abs(x).max() / 127.0)
+    b_s = float(np.abs(w).max() / 127.0)
+    wq = np.clip(np.rint(w / np.float32(b_s)), -127, 127).astype(np.float32)
+    y_s, y_zp = 0.37, 3.0
+    aq = oracle.quantize_linear_f32_to_f32_i8(x.ravel(), a_s, 0.0)
+    q, fast = oracle.exec_qlinear_matmul(aq, a_s, 0.0, wq.ravel(), b_s, 0.0, y_s, y_zp, m, k, n)
+    want = oracle.dequantize_linear(q.ravel(), y_s, y_zp).reshape(m, n)
+    assert fast
+    pre = ops.PrepackedI8B(_dev(torch, wq))
+    ops.reset_quant_runtime_stats()
+    got = ops.exec_qdq_matmul(_dev(torch, x), a_s, pre, b_s, y_s, y_zp).cpu().numpy()
+    assert ops.quant_runtime_stats().qlinear_matmul_fast == 1
+    assert np.array_equal(got, want)
+    a_dev = ops.exec_quantize_linear(_dev(torch, x), a_s, 0.0)
+    q_dev, _ = ops.exec_qlinear_matmul(a_dev, a_s, 0.0, None, b_s, 0.0, y_s, y_zp, prepacked=pre)
+    chained = ops.exec_dequantize_linear(q_dev, torch.tensor([y_s], device="cuda"), torch.tensor([y_zp], device="cuda"))
+    assert np.array_equal(got, chained.cpu().numpy())
+    pre.close()

@@ -95,6 +95,7 @@ _SIGNATURES = {
     "yscv_hip_exec_matmul_integer": [_vp, _vp, _vp, _f32, _f32, _sz, _sz, _sz, _vp, C.POINTER(_i32), _vp],
     "yscv_hip_exec_qlinear_matmul": [_vp, _f32, _f32, _vp, _vp, _f32, _f32, _f32, _f32, _sz, _sz, _sz, _vp,
                                      C.POINTER(_i32), _vp],
+    "yscv_hip_exec_qdq_matmul": [_vp, _sz, _f32, _vp, _f32, _f32, _f32, _vp, _vp],
     "yscv_hip_exec_quantize_linear": [_vp, _sz, _f32, _f32, _vp, _vp],
     "yscv_hip_exec_dequantize_linear": [_vp, _sz, _sz, _sz, _vp, _vp, _sz, _vp, _vp],
     "yscv_hip_exec_dynamic_quantize_linear": [_vp, _sz, _vp, _vp, _vp, _vp],

@@ -88,6 +88,13 @@ __device__ __forceinline__ int requant_one(int32_t acc, int32_t corr, float comp
   return (int)r;
 }
 
+// requantise, then DequantizeLinear of the quantised value: (q - y_zp) * dq_scale (crates/yscv-onnx/src/runner/misc.rs:124-128)
+__device__ __forceinline__ int32_t requant_dequant_bits(int32_t acc, int32_t corr, float comp, float y_zp, int round_mode,
+                                                        float lo, float hi, float dq_scale) {
+  const int q = requant_one(acc, corr, comp, y_zp, round_mode, lo, hi);
+  return __float_as_int(__fmul_rn(__fsub_rn((float)q, y_zp), dq_scale));
+}
+
 struct I8Args {
   const uint8_t *a;   // [m][k]
   const int8_t *frag; // packed B
@@ -95,8 +102,8 @@ struct I8Args {
   void *out;
   const int32_t *corr;
   const float *composite_v;
-  float composite, y_zp;
-  int round_mode, lo, hi, mode;
+  float composite, y_zp, dq_scale;
+  int round_mode, lo, hi, mode;  // mode 0: int32 out, 1: requantised bytes, 2: requantise + dequantise to f32
   int m, n, k;
   int ksteps;       // kp / 64
   int a_xor;        // 0x80808080 for uint8 activations, 0 for int8
@@ -221,6 +228,8 @@ __global__ void __launch_bounds__(I8_THREADS) i8_gemm_kernel(I8Args p) {
         const size_t o = (size_t)row * p.n + col;
         if (p.mode == 0) {
           reinterpret_cast<int32_t *>(p.out)[o] = v;
+        } else if (p.mode == 2) {
+          reinterpret_cast<int32_t *>(p.out)[o] = requant_dequant_bits(v, corr, comp, p.y_zp, p.round_mode, lo, hi, p.dq_scale);
         } else {
           int q = requant_one(v, corr, comp, p.y_zp, p.round_mode, lo, hi);
           reinterpret_cast<uint8_t *>(p.out)[o] = (uint8_t)q;
@@ -437,6 +446,12 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
         for (int e = 0; e < 4; e++) v[e] = (int32_t)((uint32_t)acc[i][j][e] + (uint32_t)zc[e]);
         if (p.mode == 0) {
           *reinterpret_cast<int4_t *>(i8_ring + lrow * RS32 + lcol * 4) = int4_t{v[0], v[1], v[2], v[3]};
+        } else if (p.mode == 2) {
+          int4_t f;
+#pragma unroll
+          for (int e = 0; e < 4; e++)
+            f[e] = requant_dequant_bits(v[e], corr[e], comp[e], p.y_zp, p.round_mode, lo, hi, p.dq_scale);
+          *reinterpret_cast<int4_t *>(i8_ring + lrow * RS32 + lcol * 4) = f;
         } else {
           uint32_t packed = 0;
 #pragma unroll
@@ -448,7 +463,7 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
     }
   }
   __syncthreads();
-  if (p.mode == 0) {
+  if (p.mode != 1) {  // four-byte results: int32 sums or dequantised f32
     constexpr int CPR = BN / 4;  // 16-byte chunks per row
     const bool vec = (p.n & 3) == 0;
     for (int q = tid; q < BM * CPR; q += I8R_THREADS) {
@@ -520,6 +535,7 @@ int32_t launch_i8_gemm(const void *a, int a_is_u8, int a_zp, const yscv_hip_i8_w
   p.lo = ep.lo;
   p.hi = ep.hi;
   p.mode = ep.mode;
+  p.dq_scale = ep.dq_scale;
   p.m = (int)m;
   p.n = (int)b->n;
   p.k = (int)b->k;

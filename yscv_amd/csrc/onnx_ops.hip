@@ -504,6 +504,36 @@ int32_t yscv_hip_exec_qlinear_matmul(const float *a_dev, float a_scale, float a_
   return run_matmul(g, path_out);
 }
 
+int32_t yscv_hip_exec_qdq_matmul(const float *x_dev, size_t m, float a_scale, const yscv_hip_i8_weight *b, float b_scale,
+                                 float y_scale, float y_zp, float *out_dev, void *stream) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(b != nullptr, "null int8 weight handle");
+  if (m == 0) return YSCV_HIP_OK;
+  YSCV_REQUIRE(x_dev && out_dev, "null x / out pointer");
+  hipStream_t s = as_stream(stream);
+  // QuantizeLinear (zero point 0) into a scratch int8 matrix, then the GEMM whose epilogue requantises with the
+  // QLinearMatMul fast-path expression and dequantises again
+  int8_t *a8 = nullptr;
+  YSCV_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&a8), m * b->k, s));
+  int32_t st = launch_quantize_linear_i8(x_dev, m * b->k, a_scale, 0.0f, a8, s);
+  if (st == YSCV_HIP_OK) {
+    I8Epilogue ep{};
+    ep.mode = 2;
+    ep.composite = (a_scale * b_scale) / y_scale;
+    ep.y_zp = y_zp;
+    ep.round_mode = YSCV_HIP_ROUND_HALF_AWAY;
+    ep.lo = -128;
+    ep.hi = 127;
+    ep.dq_scale = y_scale;
+    st = launch_i8_gemm(a8, 0, 0, b, m, out_dev, ep, s);
+  }
+  const hipError_t fe = hipFreeAsync(a8, s);
+  YSCV_TRY(st);
+  YSCV_HIP_TRY(fe);
+  g_qlinear_fast.fetch_add(1, std::memory_order_relaxed);
+  return YSCV_HIP_OK;
+}
+
 int32_t yscv_hip_exec_quantize_linear(const float *x_dev, size_t len, float scale, float zero_point, float *out_dev,
                                       void *stream) {
   YSCV_TRY(ensure_context(nullptr));

@@ -136,6 +136,19 @@ def exec_qlinear_matmul(a, a_scale, a_zp, b, b_scale, b_zp, y_scale, y_zp, prepa
     return out, path.value
 
 
+def exec_qdq_matmul(x, a_scale, prepacked: PrepackedI8B, b_scale, y_scale, y_zp: float = 0.0):
+    """QuantizeLinear -> QLinearMatMul -> DequantizeLinear (quantize/rewriter.rs:586-673) in one call, f32 in / out."""
+    import torch
+
+    x = _dev_f32(x, "x")
+    if x.dim() != 2 or int(x.shape[1]) != prepacked.k:
+        raise ValueError("x must be [m][k] with k matching the prepacked weight")
+    out = torch.empty(int(x.shape[0]), prepacked.n, device=x.device, dtype=torch.float32)
+    lib().exec_qdq_matmul(_p(x), _sz(int(x.shape[0])), C.c_float(a_scale), prepacked.handle, C.c_float(b_scale),
+                          C.c_float(y_scale), C.c_float(y_zp), _p(out), _stream_ptr())
+    return out
+
+
 def exec_quantize_linear(x, scale: float, zero_point: float = 0.0):
     """misc.rs:42-80 (f32-carrier arm): clamp(round_ties_even(x / scale + zp), -128, 127) as f32."""
     import torch
