@@ -341,3 +341,29 @@ def test_int4_weight_from_f32_matches_the_packing_pass(oracle, K, torch_cuda, la
         with pytest.raises(yscv_amd.YscvHipError) as ei:
             K.PackedInt4Weight.from_f32(dev, bad, transposed_nk=(layout == "nk"))
         assert ei.value.code == -1 and "group_size must be even" in ei.value.message
+
+
+def test_lm_head_sweep_sampled_at_full_size(oracle, K, torch_cuda):
+    """BASELINE config 5 at full size (K=4096, N=128256, g=32, bf16 activations), M across the switch from the skinny
+    kernel (m <= 16) to the LDS-ring GEMM: the oracle is evaluated on a sample of columns, every row."""
+    torch = torch_cuda
+    rng = np.random.default_rng(55)
+    k, n, g = 4096, 128256, 32
+    groups = k // g
+    b = rng.integers(0, 256, n * k // 2, dtype=np.uint8)
+    scales16 = rng.uniform(0.005, 0.02, n * groups).astype(np.float16)
+    w = K.PackedInt4Weight(b, scales16, g, n, k, nibble_format=K.NIBBLE_UNSIGNED)
+    cols = np.sort(rng.choice(n, 80, replace=False))
+    cols[-1] = n - 1  # the last row of the weight: the column tail of the last tile
+    bs = b.reshape(n, k // 2)[cols]
+    ss = scales16.reshape(n, groups)[cols].astype(np.float32)
+    for m in (1, 5, 16, 17, 64, 256):
+        xt = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).bfloat16()
+        xs = xt.float().numpy()
+        ref = oracle.packed_int4_gemm_scalar(bs ^ 0x88, ss, xs, m, len(cols), k, g)
+        y = w.matmul(xt.cuda())
+        assert y.dtype == torch.bfloat16 and tuple(y.shape) == (m, n)
+        got = y.float().cpu().numpy()[:, cols]
+        int4_tolerances(got, bf16_round(ref), k, xs)
+        assert np.abs(got - bf16_round(ref)).max() <= np.abs(ref).max() * 2.0 ** -7, m
+    w.close()
