@@ -249,26 +249,50 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const _Float16 *__res
   }
 }
 
-// merge the per-chunk partials: one workgroup per (batch, head), 128 threads = one per d
+// merge the per-chunk partials: one workgroup per (batch, head), 128 threads = one per d.  The chunk maxima and
+// sums are fetched by one thread each (one memory round trip instead of one per chunk), the softmax weights of the
+// chunks go through LDS, and the weighted sum over the chunks keeps several loads in flight.
 __global__ void __launch_bounds__(128) attn_combine_kernel(const float *__restrict__ part,
                                                            const int32_t *__restrict__ pos_ptr, int hq,
                                                            int max_chunks, _Float16 *__restrict__ out) {
   constexpr int HD = 128;
-  const int head = blockIdx.x, b = blockIdx.y;
+  constexpr int CAP = 256;  // chunks whose weights fit the LDS table; longer contexts take the tail loop below
+  __shared__ float wgt[CAP];
+  __shared__ float red_m[2], red_l[2];
+  const int head = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
   const int n_ctx = *pos_ptr + 1;
   const int chunks = (n_ctx + ATT_CHUNK - 1) / ATT_CHUNK;
   const float *src = part + (((size_t)b * hq + head) * max_chunks) * (HD + 2);
+  // maximum over all chunks
   float mx = -INFINITY;
-  for (int ch = 0; ch < chunks; ch++) mx = fmaxf(mx, src[(size_t)ch * (HD + 2)]);
-  float l = 0.0f, o = 0.0f;
-  for (int ch = 0; ch < chunks; ch++) {
+  for (int ch = tid; ch < chunks; ch += 128) mx = fmaxf(mx, src[(size_t)ch * (HD + 2)]);
+  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+  if ((tid & 63) == 0) red_m[tid >> 6] = mx;
+  __syncthreads();
+  mx = fmaxf(red_m[0], red_m[1]);
+  // weights exp(m_ch - mx) and the normaliser
+  float l = 0.0f;
+  for (int ch = tid; ch < chunks; ch += 128) {
     const float *p = src + (size_t)ch * (HD + 2);
     const float f = (p[0] == -INFINITY) ? 0.0f : __expf(p[0] - mx);
+    if (ch < CAP) wgt[ch] = f;
     l += p[1] * f;
-    o += p[2 + threadIdx.x] * f;
+  }
+  for (int off = 32; off > 0; off >>= 1) l += __shfl_xor(l, off, 64);
+  if ((tid & 63) == 0) red_l[tid >> 6] = l;
+  __syncthreads();
+  l = red_l[0] + red_l[1];
+  float o = 0.0f;
+  const int fast = chunks < CAP ? chunks : CAP;
+#pragma unroll 8
+  for (int ch = 0; ch < fast; ch++) o += src[(size_t)ch * (HD + 2) + 2 + tid] * wgt[ch];
+  for (int ch = CAP; ch < chunks; ch++) {
+    const float *p = src + (size_t)ch * (HD + 2);
+    const float f = (p[0] == -INFINITY) ? 0.0f : __expf(p[0] - mx);
+    o += p[2 + tid] * f;
   }
   const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-  out[((size_t)b * hq + head) * HD + threadIdx.x] = (_Float16)(o * inv);
+  out[((size_t)b * hq + head) * HD + tid] = (_Float16)(o * inv);
 }
 
 // ---- greedy pick: last index among equal maxima; also records the token and advances the position ------
