@@ -143,7 +143,9 @@ def test_skinny_all_m_and_dtypes(oracle, K, torch_cuda, m, xdt):
     w = K.PackedInt4Weight(b, scales16, g, n, k, nibble_format=K.NIBBLE_UNSIGNED)
     y = w.matmul(xt.cuda(), out_dtype=torch.float32, mode="gemv").cpu().numpy()
     d, rel = int4_tolerances(y, ref, k, x)
-    assert rel < 2e-5, rel
+    # f32 input: hi + lo activations against exact weights.  fp16 / bf16 input with symmetric weights: the 1024-offsets
+    # stay in the weights and are cancelled per group in fp32, which costs a few units of 1e-5.
+    assert rel < (2e-5 if xdt == "f32" else 5e-5), rel
     # GEMM kernel on the same data agrees with the skinny kernel to fp32 rounding
     y2 = w.matmul(xt.cuda(), out_dtype=torch.float32, mode="gemm").cpu().numpy()
     int4_tolerances(y2, ref, k, x)

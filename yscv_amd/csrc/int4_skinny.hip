@@ -6,22 +6,29 @@
 // issue per byte streamed (about 80 VALU slots per KiB of weights at 8 TB/s), so everything in the
 // inner loop is there to keep that count low:
 //   * weights stream from HBM exactly once, as 1 KiB coalesced tiles (one 128-bit load per lane,
-//     layout in int4_common.hpp); a ring of P register slots keeps P-1 blocks in flight per wave;
-//     the steady-state loop has no conditional loads, so the compiler's s_waitcnt counts are exact;
+//     layout in int4_common.hpp); a ring of P register slots keeps P-1 blocks in flight per wave.
+//     Every iteration issues the same loads (requests past the last block repeat it, served by the
+//     caches), so the compiler's s_waitcnt counts are exact; the first P blocks are requested
+//     before the activations are fetched, and no load in the kernel sits behind a per-load branch
+//     (a guarded load costs one memory round trip each, under load more than a microsecond);
 //   * the activation rows sit in registers for the whole kernel, as fp16 hi (+ lo for f32 input),
 //     already in MFMA A-operand order: the inner loop reads neither LDS nor L2 for them;
 //   * v_mfma_f32_16x16x32_f16 does the dot products (A = up to 16 activation rows, B = 16 weight
 //     rows), one MFMA per 32-k block = one quantisation group when group_size is 32;
-//   * nibbles become fp16 with one bit-field insert each: 0x6400 | q = 1024 + q and
-//     0x6400 | (q << 4) = 1024 + 16 q.  For symmetric weights (zero point 8), fp16/bf16
-//     activations and m <= 4 the offsets are not subtracted per weight: the activation slots that meet the
+//   * nibbles become fp16 with one v_and_or_b32 per pair: 0x6400 | q = 1024 + q and
+//     0x6400 | (q << 4) = 1024 + 16 q.  For symmetric weights (zero point 8) and fp16/bf16
+//     activations the offsets are not subtracted per weight: the activation slots that meet the
 //     16 q form are pre-divided by 16, and the offset term sum_k x_k * (1024 + 8 or 1024 + 128)
 //     -- which does not depend on the weight row -- is computed once per kernel by the same MFMA
-//     against a constant operand and removed from each group's result.  With explicit zero points,
-//     f32 activations or m > 4 the offsets are subtracted exactly in fp16 before the MFMA;
+//     against a constant operand.  With m <= 4 it is subtracted from each group's result; with
+//     m > 4 (four useful accumulators per lane) the products -offset[row][block] * scale[n][block]
+//     of a whole 16-row block are added by four v_mfma_f32_16x16x4_f32 at the end of the block.
+//     With explicit zero points or f32 activations the offsets are subtracted exactly in fp16
+//     before the MFMA;
 //   * group scales are applied in fp32 to the MFMA result (acc += scale * D);
 //   * K is split across the wavefronts of a workgroup (each wave owns 512 k of the activations);
-//     the per-wave partial sums meet in LDS once per 16-row block behind an LDS-only barrier.
+//     the per-wave partial sums meet in LDS behind an LDS-only barrier, once per 16-row block
+//     (m <= 4) or once per two blocks (m > 4, where every wave has a share of the sums to add).
 //     When K is too long for one workgroup, a grid-level split writes fp32 partials that a second
 //     small kernel adds in a fixed order (no atomics on shared outputs: results are deterministic).
 #include <type_traits>
@@ -83,19 +90,28 @@ struct TileRegs {
   uint32_t z[HAS_ZP ? TPW : 1];
 };
 
-// (mask & s) | (~mask & magic): one v_bfi_b32
-__device__ __forceinline__ uint32_t bfi(uint32_t mask, uint32_t s, uint32_t magic) {
-  return (mask & s) | (~mask & magic);
-}
+// Constants of the nibble -> fp16 decode, held in registers whose contents the compiler cannot see.  Given literal
+// constants it emits v_and_b32 + v_or_b32 per pair of nibbles (a VOP3 encoding cannot hold a literal); with a mask in
+// an SGPR and the magic in a VGPR it selects one v_and_or_b32.  The empty asm statements emit no instruction, so
+// every real instruction stays visible to the compiler's MFMA hazard handling.
+struct NibbleConsts {
+  uint32_t lo, hi, magic;  // 0x000F000F, 0x00F000F0, 0x64006400
+  __device__ __forceinline__ void init() {
+    lo = 0x000F000Fu;
+    hi = 0x00F000F0u;
+    magic = 0x64006400u;
+    asm volatile("" : "+s"(lo), "+s"(hi), "+v"(magic));
+  }
+};
 
 // raw fp16 forms of the 8 weights of one word: {1024+q0, 1024+q1, 1024+16 q2, 1024+16 q3, ...}
-__device__ __forceinline__ half8_t extract8(uint32_t s, uint32_t magic) {
+__device__ __forceinline__ half8_t extract8(uint32_t s, const NibbleConsts &nc) {
   U32H2 r0, r1, r2, r3;
   const uint32_t s2 = s >> 8;
-  r0.u = bfi(0x000F000Fu, s, magic);
-  r1.u = bfi(0x00F000F0u, s, magic);
-  r2.u = bfi(0x000F000Fu, s2, magic);
-  r3.u = bfi(0x00F000F0u, s2, magic);
+  r0.u = (s & nc.lo) | nc.magic;
+  r1.u = (s & nc.hi) | nc.magic;
+  r2.u = (s2 & nc.lo) | nc.magic;
+  r3.u = (s2 & nc.hi) | nc.magic;
   half8_t out;
   out[0] = r0.h[0];
   out[1] = r0.h[1];
@@ -109,13 +125,13 @@ __device__ __forceinline__ half8_t extract8(uint32_t s, uint32_t magic) {
 }
 
 // exact (q - zp) in fp16: c1 = -(1024 + zp), c2 = -(64 + zp)
-__device__ __forceinline__ half8_t decode8_exact(uint32_t s, uint32_t magic, half2_t c1, half2_t c2) {
+__device__ __forceinline__ half8_t decode8_exact(uint32_t s, const NibbleConsts &nc, half2_t c1, half2_t c2) {
   U32H2 r0, r1, r2, r3;
   const uint32_t s2 = s >> 8;
-  r0.u = bfi(0x000F000Fu, s, magic);
-  r1.u = bfi(0x00F000F0u, s, magic);
-  r2.u = bfi(0x000F000Fu, s2, magic);
-  r3.u = bfi(0x00F000F0u, s2, magic);
+  r0.u = (s & nc.lo) | nc.magic;
+  r1.u = (s & nc.hi) | nc.magic;
+  r2.u = (s2 & nc.lo) | nc.magic;
+  r3.u = (s2 & nc.hi) | nc.magic;
   const half2_t sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
   const half2_t h0 = r0.h + c1;
   const half2_t h1 = r1.h * sixteenth + c2;
@@ -145,10 +161,13 @@ template <int SPLIT, int NI, int GM, bool SF16, bool HAS_ZP, int P, bool RAWX>
 __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
   static_assert(!RAWX || SPLIT == 2, "raw f32 activations are split into hi + lo");
   // OFFSET mode: leave the 1024-offsets in the weights and cancel them per group (see file header)
-  constexpr bool OFFSET = (SPLIT == 1) && !HAS_ZP && (NI == 1);
+  constexpr bool OFFSET = (SPLIT == 1) && !HAS_ZP;
+  constexpr int UB = (NI > 1 && P % 2 == 0) ? 2 : 1;  // 16-row blocks per cross-wave reduction
+  constexpr bool OFFSET1 = OFFSET && NI == 1;  // one useful accumulator: offset subtracted after the MFMA
+  constexpr bool OFFSETC = OFFSET && NI > 1;   // all four useful: minus-offset enters as the MFMA's C operand
   constexpr int SPT = GM == GM32 ? 4 : (GM == GM64 ? 2 : 1);
   constexpr int SC_BYTES = SPT * (SF16 ? 2 : 4);
-  extern __shared__ float red[];  // [2][waves][NI][64]
+  extern __shared__ float red[];  // [2][waves][UB][NI][64]
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int waves = blockDim.x >> 6;
@@ -157,103 +176,8 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
   const int slice = blockIdx.y * waves + wave;     // this wave's 512-k slice
   const bool wave_active = slice < a.slices;       // trailing waves of the last k-split may be idle
   const int t0 = (wave_active ? slice : 0) * TPW;  // first 128-k tile of the slice
-  const uint32_t magic = 0x64006400u;
-
-  // ---- activations -> registers, in A-operand order ------------------------------------------
-  // MFMA row `r` carries batch row m when r == 4*(m / NI) + (m % NI): the useful results then sit
-  // in the first NI of the four accumulator registers of each lane.
-  half8_t xa[TPW][4][SPLIT];
-  float slice_scale = 1.0f;  // RAWX: what this wave's products of the row it loads must be multiplied by
-  {
-    const int i = r & 3;
-    const int mrow = (r >> 2) * NI + i;
-    const bool valid = wave_active && (i < NI) && (mrow < a.m);
-    const half8_t pre = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)0.0625f, (_Float16)0.0625f,
-                         (_Float16)1.0f, (_Float16)1.0f, (_Float16)0.0625f, (_Float16)0.0625f};
-    if constexpr (RAWX) {
-      // f32 activations straight from the caller: the wave normalises its own 512-k slice of every row by a power
-      // of two (abs-max to [2^14, 2^15), as the separate activation pass does per row) and splits it into fp16
-      // hi + lo; the power of two is undone on the wave's partial sums before they meet the other slices.
-      const float *src = a.xf + (size_t)mrow * a.k_pad + (size_t)t0 * 128 + c * 8;
-      float amax = 0.0f;
-      if (valid) {
-#pragma unroll
-        for (int t = 0; t < TPW; t++)
-#pragma unroll
-          for (int j = 0; j < 4; j++) {
-            const float4_t v0 = *reinterpret_cast<const float4_t *>(src + t * 128 + j * 32);
-            const float4_t v1 = *reinterpret_cast<const float4_t *>(src + t * 128 + j * 32 + 4);
-#pragma unroll
-            for (int e = 0; e < 4; e++) amax = fmaxf(amax, fmaxf(fabsf(v0[e]), fabsf(v1[e])));
-          }
-      }
-      amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-      amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-      int e2 = 14;
-      if (amax > 0.0f && amax < 3.0e38f) {
-        (void)frexpf(amax, &e2);
-        e2 -= 1;
-      }
-      int shift = 14 - e2;
-      shift = shift > 100 ? 100 : (shift < -100 ? -100 : shift);
-      const float up = ldexpf(1.0f, shift);
-      slice_scale = ldexpf(1.0f, -shift);
-#pragma unroll
-      for (int t = 0; t < TPW; t++) {
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          half8_t h = {0, 0, 0, 0, 0, 0, 0, 0}, l = {0, 0, 0, 0, 0, 0, 0, 0};
-          if (valid) {
-            const float4_t v0 = *reinterpret_cast<const float4_t *>(src + t * 128 + j * 32);
-            const float4_t v1 = *reinterpret_cast<const float4_t *>(src + t * 128 + j * 32 + 4);
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-              const float sv = (e < 4 ? v0[e] : v1[e - 4]) * up;
-              h[e] = (_Float16)sv;
-              l[e] = (_Float16)(sv - (float)h[e]);
-            }
-          }
-          xa[t][j][0] = h;
-          xa[t][j][1] = l;
-        }
-      }
-    } else {
-#pragma unroll
-      for (int t = 0; t < TPW; t++) {
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          half8_t h = {0, 0, 0, 0, 0, 0, 0, 0}, l = {0, 0, 0, 0, 0, 0, 0, 0};
-          if (valid) {
-            const size_t off = (size_t)mrow * a.k_pad + (size_t)(t0 + t) * 128 + j * 32 + c * 8;
-            h = *reinterpret_cast<const half8_t *>(a.xh + off);
-            if constexpr (SPLIT == 2) l = *reinterpret_cast<const half8_t *>(a.xl + off);
-          }
-          if constexpr (OFFSET) h = h * pre;  // slots that meet 1024 + 16 q carry x / 16 (a power of two)
-          xa[t][j][0] = h;
-          if constexpr (SPLIT == 2) xa[t][j][1] = l;
-        }
-      }
-    }
-  }
-  // RAWX: accumulator i of lane (c, .) belongs to row c * NI + i, which lanes 4 c + i (+16, +32, +48) loaded
-  float acc_scale[NI];
-#pragma unroll
-  for (int i = 0; i < NI; i++) acc_scale[i] = RAWX ? __shfl(slice_scale, 4 * c + i, 64) : 1.0f;
-  // offset term of every 32-k block: sum_k x'_k * (1024 + 8 | 1024 + 128), same register layout as D
-  float corr1[OFFSET ? TPW : 1][4];
-  if constexpr (OFFSET) {
-    const half8_t bc = {(_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f,
-                        (_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f};
-#pragma unroll
-    for (int t = 0; t < TPW; t++) {
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        float4_t z = {0.0f, 0.0f, 0.0f, 0.0f};
-        z = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][j][0], bc, z, 0, 0, 0);
-        corr1[t][j] = z[0];
-      }
-    }
-  }
+  NibbleConsts nc;
+  nc.init();
 
   // ---- per-wave stream pointers (advance by one grid stride of 16-row blocks per iteration) ----
   const int stride = gridDim.x;
@@ -286,6 +210,139 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
     if constexpr (HAS_ZP) zp += z_step;
   };
 
+  // ---- the first P blocks are requested before the activation set-up (EARLY, where the registers allow it: their
+  // HBM latency then overlaps the set-up) or right after it ----
+  // Block `it` of this workgroup is 16-row block blockIdx.x + it * stride.  Requests past the last block are clamped
+  // to it (a repeat served by the caches) so that every iteration issues the same number of loads and the
+  // compiler's s_waitcnt counts stay exact.
+  constexpr bool EARLY = SPLIT == 1 && !HAS_ZP;
+  const int iters = (a.nt - (int)blockIdx.x + stride - 1) / stride;  // >= 1, uniform in the workgroup
+  Regs ring[P];
+  auto fill_ring = [&]() {
+    if (wave_active) {
+#pragma unroll
+      for (int sl = 0; sl < P; sl++) issue(ring[sl], sl < iters ? sl : iters - 1);
+    }
+  };
+  if constexpr (EARLY) fill_ring();
+
+  // ---- activations -> registers, in A-operand order ------------------------------------------
+  // MFMA row `r` carries batch row m when r == 4*(m / NI) + (m % NI): the useful results then sit
+  // in the first NI of the four accumulator registers of each lane.
+  half8_t xa[TPW][4][SPLIT];
+  float slice_scale = 1.0f;  // RAWX: what this wave's products of the row it loads must be multiplied by
+  {
+    const int i = r & 3;
+    const int mrow = (r >> 2) * NI + i;
+    const bool valid = wave_active && (i < NI) && (mrow < a.m);
+    const half8_t pre = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)0.0625f, (_Float16)0.0625f,
+                         (_Float16)1.0f, (_Float16)1.0f, (_Float16)0.0625f, (_Float16)0.0625f};
+    if constexpr (RAWX) {
+      // f32 activations straight from the caller: the wave normalises its own 512-k slice of every row by a power
+      // of two (abs-max to [2^14, 2^15), as the separate activation pass does per row) and splits it into fp16
+      // hi + lo; the power of two is undone on the wave's partial sums before they meet the other slices.
+      // Idle lanes read row 0 and discard it: every load is unconditional, so all of them are in flight together
+      // instead of one round trip per guarded load.
+      const float *src = a.xf + (size_t)(valid ? mrow : 0) * a.k_pad + (size_t)t0 * 128 + c * 8;
+      float amax = 0.0f;
+#pragma unroll
+      for (int t = 0; t < TPW; t++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const float4_t v0 = *reinterpret_cast<const float4_t *>(src + t * 128 + j * 32);
+          const float4_t v1 = *reinterpret_cast<const float4_t *>(src + t * 128 + j * 32 + 4);
+#pragma unroll
+          for (int e = 0; e < 4; e++) amax = fmaxf(amax, fmaxf(fabsf(v0[e]), fabsf(v1[e])));
+        }
+      if (!valid) amax = 0.0f;
+      amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+      amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+      int e2 = 14;
+      if (amax > 0.0f && amax < 3.0e38f) {
+        (void)frexpf(amax, &e2);
+        e2 -= 1;
+      }
+      int shift = 14 - e2;
+      shift = shift > 100 ? 100 : (shift < -100 ? -100 : shift);
+      const float up = valid ? ldexpf(1.0f, shift) : 0.0f;
+      slice_scale = ldexpf(1.0f, -shift);
+#pragma unroll
+      for (int t = 0; t < TPW; t++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          // second read of the slice: served by the caches
+          const float4_t v0 = *reinterpret_cast<const float4_t *>(src + t * 128 + j * 32);
+          const float4_t v1 = *reinterpret_cast<const float4_t *>(src + t * 128 + j * 32 + 4);
+          half8_t h, l;
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            const float sv = (e < 4 ? v0[e] : v1[e - 4]) * up;
+            h[e] = (_Float16)sv;
+            l[e] = (_Float16)(sv - (float)h[e]);
+          }
+          if (!valid) {
+            h = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            l = h;
+          }
+          xa[t][j][0] = h;
+          xa[t][j][1] = l;
+        }
+      }
+    } else {
+      const size_t row_off = (size_t)(valid ? mrow : 0) * a.k_pad;
+      const half8_t hz = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int t = 0; t < TPW; t++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const size_t off = row_off + (size_t)(t0 + t) * 128 + j * 32 + c * 8;
+          half8_t h = *reinterpret_cast<const half8_t *>(a.xh + off);
+          if (!valid) h = hz;
+          if constexpr (OFFSET) h = h * pre;  // slots that meet 1024 + 16 q carry x / 16 (a power of two)
+          xa[t][j][0] = h;
+          if constexpr (SPLIT == 2) {
+            half8_t l = *reinterpret_cast<const half8_t *>(a.xl + off);
+            xa[t][j][1] = valid ? l : hz;
+          }
+        }
+      }
+    }
+  }
+  // RAWX: accumulator i of lane (c, .) belongs to row c * NI + i, which lanes 4 c + i (+16, +32, +48) loaded
+  float acc_scale[NI];
+#pragma unroll
+  for (int i = 0; i < NI; i++) acc_scale[i] = RAWX ? __shfl(slice_scale, 4 * c + i, 64) : 1.0f;
+  // offset term of every 32-k block: sum_k x'_k * (1024 + 8 | 1024 + 128), same register layout as D
+  float corr1[OFFSET1 ? TPW : 1][4];
+  // OFFSETC: minus the offset term of MFMA row r and 32-k block (t, j = c), i.e. in the A-operand layout of
+  // v_mfma_f32_16x16x4_f32: at the end of a 16-row block, four of those MFMAs (one per tile, B = the scale that
+  // applies to weight row r in 32-k block c) add sum_blocks -offset * scale to all four accumulators at once.
+  float ncorr_a[OFFSETC ? TPW : 1];
+  if constexpr (OFFSET) {
+    const half8_t bc = {(_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f,
+                        (_Float16)1032.0f, (_Float16)1032.0f, (_Float16)1152.0f, (_Float16)1152.0f};
+#pragma unroll
+    for (int t = 0; t < TPW; t++) {
+      float sel = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        float4_t z = {0.0f, 0.0f, 0.0f, 0.0f};
+        if constexpr (OFFSET1) {
+          z = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][j][0], bc, z, 0, 0, 0);
+          corr1[t][j] = z[0];
+        } else {
+          // operands swapped: the activations are the B matrix, so column r of the result (every register of lanes
+          // (r, .)) is the offset term of MFMA row r
+          z = __builtin_amdgcn_mfma_f32_16x16x32_f16(bc, xa[t][j][0], z, 0, 0, 0);
+          if (c == j) sel = z[0];
+        }
+      }
+      if constexpr (OFFSETC) ncorr_a[t] = -sel;
+    }
+  }
+
+  if constexpr (!EARLY) fill_ring();
+
   // dot products of one 16-row block against this wave's k slice
   auto dots = [&](const Regs &tr, float acc[NI]) {
 #pragma unroll
@@ -300,8 +357,8 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
         const bool group_end = GM == GM32 || (GM == GM64 && (j & 1)) || (GM == GM128 && j == 3);
         half8_t b;
         if constexpr (OFFSET) {
-          b = extract8(tr.w[t][j], magic);
-          csum = group_start ? corr1[t][j] : csum + corr1[t][j];
+          b = extract8(tr.w[t][j], nc);
+          if constexpr (OFFSET1) csum = group_start ? corr1[t][j] : csum + corr1[t][j];
         } else {
           half2_t c1 = {(_Float16)(-1032.0f), (_Float16)(-1032.0f)};
           half2_t c2 = {(_Float16)(-72.0f), (_Float16)(-72.0f)};
@@ -310,13 +367,13 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
                                           : (GM == GM64 ? ((tr.z[t] >> (8 * (j >> 1))) & 0xFF) : (tr.z[t] & 0xFF));
             zp_consts(z, c1, c2);
           }
-          b = decode8_exact(tr.w[t][j], magic, c1, c2);
+          b = decode8_exact(tr.w[t][j], nc, c1, c2);
         }
         d = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][j][0], b, d, 0, 0, 0);
         if constexpr (SPLIT == 2) d = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][j][1], b, d, 0, 0, 0);
         if (group_end) {
           const float sc = tr.s[t].get(GM == GM32 ? j : (GM == GM64 ? (j >> 1) : 0));
-          if constexpr (OFFSET) {
+          if constexpr (OFFSET1) {
             acc[0] = fmaf(sc, d[0] - csum, acc[0]);
           } else {
 #pragma unroll
@@ -326,31 +383,60 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
         }
       }
     }
+    if constexpr (OFFSETC) {
+      float4_t av = {acc[0], NI > 1 ? acc[1 % NI] : 0.0f, NI > 2 ? acc[2 % NI] : 0.0f, NI > 3 ? acc[3 % NI] : 0.0f};
+#pragma unroll
+      for (int t = 0; t < TPW; t++) {
+        const float sb = tr.s[t].get(GM == GM32 ? c : (GM == GM64 ? (c >> 1) : 0));
+        av = __builtin_amdgcn_mfma_f32_16x16x4f32(ncorr_a[t], sb, av, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < NI; i++) acc[i] = av[i];
+    }
     if constexpr (RAWX) {
 #pragma unroll
       for (int i = 0; i < NI; i++) acc[i] *= acc_scale[i];
     }
   };
 
-  // meet the other k slices in LDS; the NI x 64 sums are shared out over the waves in half-wave pieces (piece q =
-  // accumulator q / 2, lanes 32 (q % 2) .. +31), so no single wave is late for the next block
-  auto reduce_store = [&](const float acc[NI], int nt, int it) {
-    float *buf = red + (size_t)(it & 1) * waves * NI * 64;
+  // row scales of the activation pass, one per accumulator of this lane (loaded once: a load inside the loop
+  // would make the compiler wait for every weight block in flight)
+  float rs[NI];
 #pragma unroll
-    for (int i = 0; i < NI; i++) buf[(wave * NI + i) * 64 + lane] = acc[i];
+  for (int i = 0; i < NI; i++) rs[i] = (a.row_scale && c * NI + i < a.m) ? a.row_scale[c * NI + i] : 1.0f;
+
+  // Meet the other k slices in LDS, once per UB blocks: every wave leaves its UB x NI x 64 partial sums, and after
+  // one barrier the sums are shared out over the waves in 64-lane pieces (piece q = block q / NI of the group,
+  // accumulator q % NI), rotating so that no wave is always the late one.
+  auto reduce_store = [&](const float (&accs)[UB][NI], int nt0, int ex) {
+    float *buf = red + (size_t)(ex & 1) * waves * (UB * NI) * 64;
+#pragma unroll
+    for (int u = 0; u < UB; u++)
+#pragma unroll
+      for (int i = 0; i < NI; i++) buf[((wave * UB + u) * NI + i) * 64 + lane] = accs[u][i];
     lds_barrier();
-    for (int q = (wave + it) % waves; q < NI * 2; q += waves) {
-      const int i = q >> 1;
-      if ((lane >> 5) != (q & 1)) continue;
-      const int col = nt * 16 + r;
+    for (int q = (wave + ex) % waves; q < UB * NI; q += waves) {
+      const int u = q / NI, i = q % NI;
+      const int col = (nt0 + u * stride) * 16 + r;
+      // the slices are fetched four at a time (two LDS round trips, few registers), then added in slice order
       float v = 0.0f;
-      for (int w = 0; w < waves; w++) v += buf[(w * NI + i) * 64 + lane];
+#pragma unroll
+      for (int w0 = 0; w0 < 8; w0 += 4) {
+        float part[4];
+#pragma unroll
+        for (int w = 0; w < 4; w++) part[w] = w0 + w < waves ? buf[(((w0 + w) * UB + u) * NI + i) * 64 + lane] : 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) v += part[w];
+      }
       const int mrow = c * NI + i;
       const bool live = mrow < a.m && col < a.n;
       if (a.ksg > 1) {
         if (live) a.partial[((size_t)blockIdx.y * a.m + mrow) * a.n + col] = v;
       } else {
-        if (a.row_scale && mrow < a.m) v *= a.row_scale[mrow];
+        float rsv = rs[0];
+#pragma unroll
+        for (int ii = 1; ii < NI; ii++) rsv = (i == ii) ? rs[ii] : rsv;
+        v *= rsv;
         if (a.epi == EPI_SWIGLU) {
           // rows 2i / 2i+1 of the weight are gate_i / up_i: neighbours in the wave
           const float up = __shfl_xor(v, 1, 64);
@@ -366,60 +452,51 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
     }
   };
 
-  // ---- main loop over this workgroup's 16-row blocks: nt = blockIdx.x + i * stride ----------------
-  const int iters = (a.nt - (int)blockIdx.x + stride - 1) / stride;  // >= 1, uniform in the workgroup
-  int nt = blockIdx.x;
-  int it = 0;
-  float acc[NI];
+  // ---- main loop: slot it % P holds block it; after its dot products the slot is refilled with block it + P ----
+  int nt = blockIdx.x;  // first block of the current group of UB
+  int it = 0, ex = 0;
+  float accs[UB][NI];
 
   if (!wave_active) {
     // an idle wave only takes part in the reductions
 #pragma unroll
-    for (int i = 0; i < NI; i++) acc[i] = 0.0f;
-    for (; it < iters; it++, nt += stride) reduce_store(acc, nt, it);
+    for (int u = 0; u < UB; u++)
+#pragma unroll
+      for (int i = 0; i < NI; i++) accs[u][i] = 0.0f;
+    for (; it < iters; it += UB, nt += UB * stride, ex++) reduce_store(accs, nt, ex);
     return;
   }
 
-  Regs ring[P];
-  // head: the iterations that do not fill whole groups of P are issued together, then consumed
-  const int head = iters < P ? iters : iters % P;
-  if (head > 0) {
-#pragma unroll
-    for (int sl = 0; sl < P - 1; sl++)
-      if (sl < head) issue(ring[sl], sl);
-#pragma unroll
-    for (int sl = 0; sl < P - 1; sl++) {
-      if (sl < head) {
-        dots(ring[sl], acc);
-        reduce_store(acc, nt, it);
-        advance();
-        nt += stride;
-        it++;
-      }
-    }
-  }
-  const int groups = (iters - head) / P;  // whole groups of P iterations left
-  if (groups > 0) {
-#pragma unroll
-    for (int sl = 0; sl < P; sl++) issue(ring[sl], sl);
-    for (int g = 0; g + 1 < groups; g++) {
-#pragma unroll
-      for (int sl = 0; sl < P; sl++) {
-        dots(ring[sl], acc);
-        issue(ring[sl], P);  // refill the slot just consumed: stays P-1 blocks ahead
-        reduce_store(acc, nt, it);
-        advance();
-        nt += stride;
-        it++;
-      }
-    }
+  const int steady = (iters + P - 1) / P - 1;  // groups of P iterations that refill; the last group only drains
+  for (int g = 0; g < steady; g++) {
 #pragma unroll
     for (int sl = 0; sl < P; sl++) {
-      dots(ring[sl], acc);
-      reduce_store(acc, nt, it);
-      nt += stride;
+      dots(ring[sl], accs[sl % UB]);
+      const int left = iters - 1 - it;  // blocks after this one (>= P - sl, as one more group follows)
+      issue(ring[sl], left < P ? left : P);
+      if (sl % UB == UB - 1) {
+        reduce_store(accs, nt, ex);
+        nt += UB * stride;
+        ex++;
+      }
+      advance();
       it++;
     }
+  }
+#pragma unroll
+  for (int sl = 0; sl < P; sl++) {
+    if (it < iters) {
+      dots(ring[sl], accs[sl % UB]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < NI; i++) accs[sl % UB][i] = 0.0f;
+    }
+    if (sl % UB == UB - 1) {
+      if (it - (UB - 1) < iters) reduce_store(accs, nt, ex);  // the group's first block exists
+      nt += UB * stride;
+      ex++;
+    }
+    it++;
   }
 }
 
@@ -490,8 +567,9 @@ SkinnyPlan plan_int4_skinny(const yscv_hip_int4_weight *w, size_t m, int split, 
 template <int SPLIT, int NI, int GM, bool SF16, bool HAS_ZP>
 static int32_t launch_one(const SkinnyArgs &a, const SkinnyPlan &plan, hipStream_t s) {
   // ring depth: bounded by the VGPR budget (activations: 64 per split, ring: ~26 per slot)
-  constexpr int P = SPLIT == 2 ? (NI == 1 ? 2 : 1) : (NI == 1 ? 4 : 3);
-  const size_t lds = (size_t)2 * plan.waves * NI * 64 * sizeof(float);
+  constexpr int P = SPLIT == 2 ? (NI == 1 ? 2 : 1) : (SF16 && !HAS_ZP ? 4 : 3);
+  constexpr int UB = (NI > 1 && P % 2 == 0) ? 2 : 1;  // as in the kernel
+  const size_t lds = (size_t)2 * plan.waves * UB * NI * 64 * sizeof(float);
   if constexpr (SPLIT == 2) {
     if (a.xf != nullptr) {
       hipLaunchKernelGGL((int4_skinny_kernel<SPLIT, NI, GM, SF16, HAS_ZP, P, true>), dim3(plan.grid_x, plan.ksg),
