@@ -75,7 +75,7 @@ static size_t dtype_size(int d) { return d == YSCV_HIP_F32 ? 4 : 2; }
 
 // Scratch layout of one int4 call: [xh][xl][row_scale][partial], each part rounded to 256 B.
 // A fp16 activation whose row stride already equals the padded K needs no preparation at all, and neither does an
-// f32 one on its way to the skinny kernel, which normalises and splits it on the fly.
+// f32 or bf16 one on its way to the skinny kernel, which normalises (and for f32 splits) it on the fly.
 struct Int4Scratch {
   bool direct;       // x is used in place as the fp16 `hi` operand
   bool skinny;
@@ -90,7 +90,7 @@ static Int4Scratch int4_scratch_layout(const yscv_hip_int4_weight *w, const void
   Int4Scratch L{};
   L.skinny = force == 1 || (force == 0 && m <= 16);
   L.k_pad = w->ktp * 128;
-  L.direct = (x_dtype == YSCV_HIP_F16 || (x_dtype == YSCV_HIP_F32 && L.skinny)) && L.k_pad == w->k &&
+  L.direct = (x_dtype == YSCV_HIP_F16 || L.skinny) && L.k_pad == w->k &&
              (reinterpret_cast<uintptr_t>(x) & 15) == 0;
   L.split = x_dtype == YSCV_HIP_F32 ? 2 : 1;
   if (L.skinny) L.plan = plan_int4_skinny(w, m, L.split, num_cus);
@@ -146,7 +146,7 @@ int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, v
       own = true;
     }
   }
-  const float *xf = (L.direct && x_dtype == YSCV_HIP_F32) ? static_cast<const float *>(x) : nullptr;
+  const void *xraw = (L.direct && x_dtype != YSCV_HIP_F16) ? x : nullptr;
   const _Float16 *xh = L.direct ? static_cast<const _Float16 *>(x) : reinterpret_cast<_Float16 *>(scratch);
   _Float16 *xl = (!L.direct && L.split == 2) ? reinterpret_cast<_Float16 *>(scratch + L.xh_bytes) : nullptr;
   float *row_scale = L.direct ? nullptr : reinterpret_cast<float *>(scratch + L.xh_bytes * L.split);
@@ -156,7 +156,7 @@ int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, v
     st = launch_x_prep(x, x_dtype, m, w->k, L.k_pad, L.split, const_cast<_Float16 *>(xh), xl, row_scale, s);
   if (st == YSCV_HIP_OK) {
     if (L.skinny)
-      st = launch_int4_skinny(w, L.plan, xh, xl, xf, row_scale, L.k_pad, L.split, y, y_dtype, m, partial, epi, s);
+      st = launch_int4_skinny(w, L.plan, xh, xl, xraw, row_scale, L.k_pad, L.split, y, y_dtype, m, partial, epi, s);
     else
       st = launch_int4_gemm(w, xh, xl, row_scale, L.k_pad, L.split, y, y_dtype, m, s);
   }

@@ -48,7 +48,8 @@ struct SkinnyArgs {
   const uint8_t *tzps;  // null: zero point 8 everywhere
   const _Float16 *xh;
   const _Float16 *xl;
-  const float *xf;  // raw f32 activations (row stride k_pad) for the kernels that split them themselves, else null
+  const float *xf;     // raw f32 activations (row stride k_pad) for the kernels that split them themselves, else null
+  const uint16_t *xb;  // raw bf16 activations (row stride k_pad), else null
   const float *row_scale;
   void *y;
   float *partial;  // [ksg][m][n] when ksg > 1
@@ -157,9 +158,12 @@ __device__ __forceinline__ void zp_consts(uint32_t zp, half2_t &c1, half2_t &c2)
   c2 = half2_t{b, b};
 }
 
-template <int SPLIT, int NI, int GM, bool SF16, bool HAS_ZP, int P, bool RAWX>
+// XM: where the activations come from -- 0 prepared fp16 (hi [+ lo]), 1 raw f32 (split into hi + lo here), 2 raw bf16
+template <int SPLIT, int NI, int GM, bool SF16, bool HAS_ZP, int P, int XM>
 __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
-  static_assert(!RAWX || SPLIT == 2, "raw f32 activations are split into hi + lo");
+  constexpr bool RAWX = XM != 0;
+  static_assert(XM != 1 || SPLIT == 2, "raw f32 activations are split into hi + lo");
+  static_assert(XM != 2 || SPLIT == 1, "bf16 activations fit one fp16 operand exactly");
   // OFFSET mode: leave the 1024-offsets in the weights and cancel them per group (see file header)
   constexpr bool OFFSET = (SPLIT == 1) && !HAS_ZP;
   constexpr int UB = (NI > 1 && P % 2 == 0) ? 2 : 1;  // 16-row blocks per cross-wave reduction
@@ -237,7 +241,56 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
     const bool valid = wave_active && (i < NI) && (mrow < a.m);
     const half8_t pre = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)0.0625f, (_Float16)0.0625f,
                          (_Float16)1.0f, (_Float16)1.0f, (_Float16)0.0625f, (_Float16)0.0625f};
-    if constexpr (RAWX) {
+    if constexpr (XM == 2) {
+      // bf16 activations straight from the caller: the wave scales its own 512-k slice of every row by a power of
+      // two (abs-max to [2^14, 2^15)), which makes every bf16 value an exact fp16 one (8 significant bits; only
+      // values below 2^-29 of the slice maximum are lost); the power of two is undone on the wave's partial sums.
+      const uint16_t *src = a.xb + (size_t)(valid ? mrow : 0) * a.k_pad + (size_t)t0 * 128 + c * 8;
+      uint4_t raw[TPW][4];
+#pragma unroll
+      for (int t = 0; t < TPW; t++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) raw[t][j] = *reinterpret_cast<const uint4_t *>(src + t * 128 + j * 32);
+      uint32_t amax_bits = 0;  // |bf16| orders like its bit pattern
+#pragma unroll
+      for (int t = 0; t < TPW; t++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const uint32_t wd = raw[t][j][e];
+            const uint32_t lo = wd & 0x7FFFu, hi = (wd >> 16) & 0x7FFFu;
+            amax_bits = max(amax_bits, max(lo, hi));
+          }
+      float amax = valid ? __uint_as_float(amax_bits << 16) : 0.0f;
+      amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+      amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+      int e2 = 14;
+      if (amax > 0.0f && amax < 3.0e38f) {
+        (void)frexpf(amax, &e2);
+        e2 -= 1;
+      }
+      int shift = 14 - e2;
+      shift = shift > 100 ? 100 : (shift < -100 ? -100 : shift);
+      const float up = valid ? ldexpf(1.0f, shift) : 0.0f;
+      slice_scale = ldexpf(1.0f, -shift);
+#pragma unroll
+      for (int t = 0; t < TPW; t++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          half8_t h;
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const uint32_t wd = raw[t][j][e];
+            h[2 * e] = (_Float16)(__uint_as_float(wd << 16) * up);
+            h[2 * e + 1] = (_Float16)(__uint_as_float(wd & 0xFFFF0000u) * up);
+          }
+          if (!valid) h = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+          if constexpr (OFFSET) h = h * pre;
+          xa[t][j][0] = h;
+        }
+      }
+    } else if constexpr (XM == 1) {
       // f32 activations straight from the caller: the wave normalises its own 512-k slice of every row by a power
       // of two (abs-max to [2^14, 2^15), as the separate activation pass does per row) and splits it into fp16
       // hi + lo; the power of two is undone on the wave's partial sums before they meet the other slices.
@@ -572,13 +625,20 @@ static int32_t launch_one(const SkinnyArgs &a, const SkinnyPlan &plan, hipStream
   const size_t lds = (size_t)2 * plan.waves * UB * NI * 64 * sizeof(float);
   if constexpr (SPLIT == 2) {
     if (a.xf != nullptr) {
-      hipLaunchKernelGGL((int4_skinny_kernel<SPLIT, NI, GM, SF16, HAS_ZP, P, true>), dim3(plan.grid_x, plan.ksg),
+      hipLaunchKernelGGL((int4_skinny_kernel<SPLIT, NI, GM, SF16, HAS_ZP, P, 1>), dim3(plan.grid_x, plan.ksg),
+                         dim3(plan.waves * 64), lds, s, a);
+      YSCV_HIP_TRY(hipGetLastError());
+      return YSCV_HIP_OK;
+    }
+  } else {
+    if (a.xb != nullptr) {
+      hipLaunchKernelGGL((int4_skinny_kernel<SPLIT, NI, GM, SF16, HAS_ZP, P, 2>), dim3(plan.grid_x, plan.ksg),
                          dim3(plan.waves * 64), lds, s, a);
       YSCV_HIP_TRY(hipGetLastError());
       return YSCV_HIP_OK;
     }
   }
-  hipLaunchKernelGGL((int4_skinny_kernel<SPLIT, NI, GM, SF16, HAS_ZP, P, false>), dim3(plan.grid_x, plan.ksg),
+  hipLaunchKernelGGL((int4_skinny_kernel<SPLIT, NI, GM, SF16, HAS_ZP, P, 0>), dim3(plan.grid_x, plan.ksg),
                      dim3(plan.waves * 64), lds, s, a);
   YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
@@ -599,7 +659,7 @@ static int32_t launch_gm(const SkinnyArgs &a, const SkinnyPlan &plan, int gm, bo
 }
 
 int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan, const _Float16 *xh,
-                           const _Float16 *xl, const float *xf, const float *row_scale, size_t k_pad, int split,
+                           const _Float16 *xl, const void *xraw, const float *row_scale, size_t k_pad, int split,
                            void *y, int y_dtype, size_t m, float *partial, int epi, hipStream_t s) {
   if (!w->tiled) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "skinny int4 kernel needs the tiled layout");
   if (m == 0 || m > 16) return set_error(YSCV_HIP_ERR_INVALID_ARG, "skinny int4 kernel handles 1 <= m <= 16, got %zu", m);
@@ -612,7 +672,8 @@ int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan
   a.tzps = w->has_zp ? w->tzps : nullptr;
   a.xh = xh;
   a.xl = xl;
-  a.xf = split == 2 ? xf : nullptr;
+  a.xf = split == 2 ? static_cast<const float *>(xraw) : nullptr;
+  a.xb = split == 1 ? static_cast<const uint16_t *>(xraw) : nullptr;
   a.row_scale = row_scale;
   a.y = y;
   a.partial = partial;

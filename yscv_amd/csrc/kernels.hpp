@@ -65,10 +65,10 @@ struct SkinnyPlan {
   size_t partial_bytes;
 };
 SkinnyPlan plan_int4_skinny(const yscv_hip_int4_weight *w, size_t m, int split, int num_cus);
-// xf != null (split == 2 only): raw f32 activations with row stride k_pad; the kernel splits them itself and xh,
-// xl, row_scale are not used
+// xraw != null: raw activations with row stride k_pad, f32 when split == 2 and bf16 when split == 1; the kernel
+// normalises (and for f32 splits) them itself and xh, xl, row_scale are not used
 int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan, const _Float16 *xh,
-                           const _Float16 *xl, const float *xf, const float *row_scale, size_t k_pad, int split,
+                           const _Float16 *xl, const void *xraw, const float *row_scale, size_t k_pad, int split,
                            void *y, int y_dtype, size_t m, float *partial, int epi, hipStream_t s);
 int32_t launch_int4_generic(const yscv_hip_int4_weight *w, const void *x, int x_dtype, void *y,
                             int y_dtype, size_t m, hipStream_t s);
