@@ -191,7 +191,7 @@ def extra_kernels(torch, stream_ptr):
 
         t = tavg(gemv, 32)
         c1[name] = {"us_per_call_whole_op": round(t * 1e6, 2), "GB/s_whole_op": round(byt / t / 1e9, 1)}
-    c1["note"] = "32 rotating weight copies (320 MB, beyond the 256 MB Infinity Cache); f32 input = activation pass + kernel"
+    c1["note"] = "32 rotating weight copies (320 MB, beyond the 256 MB Infinity Cache); one kernel per call, the f32 input is normalised and split inside it"
     out["config1_gemv_m1_k4096_n4096"] = c1
     del ring
     # config 2: int8 M512 K4096 N4096

@@ -1,7 +1,7 @@
 // Wide-M packed-int4 matmul for fp16 / bf16 activations: y[m][n] = sum_k x[m][k] * W[n][k], MFMA-bound design.
 // Replaces packed_int4_gemm_dispatch (crates/yscv-kernels/src/ops/int4_matmul.rs:548-605) for prefill-sized m.
 //
-// A workgroup owns a (32 MT) x (32 NT) tile of y.  It has four MMA waves (2 x 2, MT x NT MFMA tiles each) and NP
+// A workgroup owns a (32 MT) x (32 NT) tile of y (MT = 1, 2 or 4 by m).  It has four MMA waves (2 x 2, MT x NT MFMA tiles each) and NP
 // producer waves.  Per stage of KS k-steps (32 k each) the producers
 //   * fetch the activation rows (fp16, prepared by x_prep) with LDS-direct loads, one 16-byte piece per lane, so
 //     the row-major -> MFMA-fragment transposition costs nothing, and
@@ -72,11 +72,12 @@ __device__ __forceinline__ void g4_wait(G4Frags<MT, NT> &f) {
     asm volatile("s_waitcnt lgkmcnt(0)"
                  : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]),
                    "+v"(f.b[3])::"memory");
-  } else {
-    static_assert(MT == 8 && NT == 4, "add a wait for this fragment count");
+  } else if constexpr (MT == 2 && NT == 4) {
     asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.a[4]), "+v"(f.a[5]), "+v"(f.a[6]),
-                   "+v"(f.a[7]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]), "+v"(f.b[3])::"memory");
+                 : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]), "+v"(f.b[3])::"memory");
+  } else {
+    static_assert(MT == 1 && NT == 4, "add a wait for this fragment count");
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.a[0]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]), "+v"(f.b[3])::"memory");
   }
 }
 
@@ -479,6 +480,11 @@ int32_t launch_int4_gemm_ring(const yscv_hip_int4_weight *w, const _Float16 *xh,
   a.k_pad = (int)k_pad;
   a.y_dtype = y_dtype;
   const bool sf16 = w->scale_dtype == YSCV_HIP_F16;
+  // The tile height follows m: the MFMA work of a workgroup, and with it the time a weight tile stays in LDS, is
+  // proportional to the tile's rows whether they exist or not, so a short m streams the weights faster on a
+  // 32- or 64-row tile.
+  if (m <= 32) return ring_launch_gm<1, 4, 2, 6, 4>(a, w->gm, sf16, s);
+  if (m <= 64) return ring_launch_gm<2, 4, 2, 6, 8>(a, w->gm, sf16, s);
   return ring_launch_gm<4, 4, 2, 6, 8>(a, w->gm, sf16, s);
 }
 
