@@ -95,6 +95,29 @@ typedef struct yscv_hip_int4_weight yscv_hip_int4_weight;
 int32_t yscv_hip_int4_weight_create(const uint8_t *packed, const void *scales, int32_t scale_dtype,
                                     const uint8_t *zero_points, int32_t nibble_format, size_t n,
                                     size_t k, size_t group_size, yscv_hip_int4_weight **out);
+/* ---- packed int4 weight files -------------------------------------------------
+ * The reference keeps PackedInt4Weight in memory only (packed_int4.rs:29-39) and re-quantises the f32 initialisers
+ * on every model load (quantize_matmul_weights_int4_packed, packed_int4.rs:50-128); it has no on-disk form.  This
+ * one stores exactly the arguments of yscv_hip_int4_weight_create behind a 64-byte header (magic "YSCVI4W", version,
+ * dtypes, n, k, group size, FNV-1a 64 checksum; sections padded to 64 bytes), so a quantised weight is uploaded
+ * again without the f32 round trip.  write / read_header / read are host-only and need no GPU. */
+typedef struct yscv_hip_int4_file_header {
+  uint64_t n, k, group_size;
+  int32_t scale_dtype, nibble_format, has_zero_points;
+  uint64_t packed_bytes, scales_bytes, zero_points_bytes; /* payload sizes the read call expects */
+  uint64_t checksum;
+} yscv_hip_int4_file_header;
+int32_t yscv_hip_int4_file_write(const char *path, const uint8_t *packed, const void *scales, int32_t scale_dtype,
+                                 const uint8_t *zero_points, int32_t nibble_format, size_t n, size_t k,
+                                 size_t group_size);
+/* Validates magic, version, shape contract and that the file length is the one the header implies. */
+int32_t yscv_hip_int4_file_read_header(const char *path, yscv_hip_int4_file_header *header);
+/* Reads the payload into caller buffers of exactly the header's sizes and verifies the checksum. */
+int32_t yscv_hip_int4_file_read(const char *path, uint8_t *packed, size_t packed_bytes, void *scales,
+                                size_t scales_bytes, uint8_t *zero_points, size_t zero_points_bytes);
+/* read + yscv_hip_int4_weight_create */
+int32_t yscv_hip_int4_weight_load(const char *path, yscv_hip_int4_weight **out);
+
 int32_t yscv_hip_int4_weight_destroy(yscv_hip_int4_weight *w);
 int32_t yscv_hip_int4_weight_dims(const yscv_hip_int4_weight *w, size_t *n, size_t *k,
                                   size_t *group_size, size_t *device_bytes);

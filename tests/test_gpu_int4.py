@@ -369,3 +369,22 @@ def test_lm_head_sweep_sampled_at_full_size(oracle, K, torch_cuda):
         int4_tolerances(got, bf16_round(ref), k, xs)
         assert np.abs(got - bf16_round(ref)).max() <= np.abs(ref).max() * 2.0 ** -7, m
     w.close()
+
+
+def test_weight_loaded_from_a_file_equals_the_uploaded_one(K, torch_cuda, tmp_path):
+    """yscv_hip_int4_weight_load: the on-disk form carries exactly the arguments of the upload call."""
+    torch = torch_cuda
+    rng = np.random.default_rng(77)
+    n, k, g = 272, 768, 64
+    b = _rand_packed(rng, n, k)
+    scales = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float16)
+    zq = rng.integers(5, 12, (n, k // g))
+    zps = pack_zero_points(zq)
+    path = tmp_path / "w.yi4"
+    K.int4_file_write(path, b, scales, g, n, k, zero_points=zps, nibble_format=K.NIBBLE_UNSIGNED)
+    w0 = K.PackedInt4Weight(b, scales, g, n, k, zero_points=zps, nibble_format=K.NIBBLE_UNSIGNED)
+    w1 = K.PackedInt4Weight.load(path)
+    assert (w1.m_w, w1.k, w1.group_size) == (n, k, g) and w1.device_bytes() == w0.device_bytes()
+    for m in (1, 9, 40):
+        x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).half().cuda()
+        assert torch.equal(w0.matmul(x, out_dtype=torch.float32), w1.matmul(x, out_dtype=torch.float32))

@@ -29,6 +29,13 @@ class GenerateConfig(C.Structure):
                 ("has_eos", C.c_int32), ("eos_token_id", C.c_uint32), ("repetition_penalty", C.c_float)]
 
 
+class Int4FileHeader(C.Structure):
+    """yscv_hip_int4_file_header"""
+    _fields_ = [("n", C.c_uint64), ("k", C.c_uint64), ("group_size", C.c_uint64), ("scale_dtype", C.c_int32),
+                ("nibble_format", C.c_int32), ("has_zero_points", C.c_int32), ("packed_bytes", C.c_uint64),
+                ("scales_bytes", C.c_uint64), ("zero_points_bytes", C.c_uint64), ("checksum", C.c_uint64)]
+
+
 class QuantStats(C.Structure):
     """yscv_hip_quant_stats."""
 
@@ -64,6 +71,10 @@ _SIGNATURES = {
     "yscv_hip_stream_synchronize": [_vp],
     "yscv_hip_int4_weight_create": [_vp, _vp, _i32, _vp, _i32, _sz, _sz, _sz, C.POINTER(_vp)],
     "yscv_hip_int4_weight_destroy": [_vp],
+    "yscv_hip_int4_file_write": [C.c_char_p, _vp, _vp, _i32, _vp, _i32, _sz, _sz, _sz],
+    "yscv_hip_int4_file_read_header": [C.c_char_p, _vp],
+    "yscv_hip_int4_file_read": [C.c_char_p, _vp, _sz, _vp, _sz, _vp, _sz],
+    "yscv_hip_int4_weight_load": [C.c_char_p, C.POINTER(_vp)],
     "yscv_hip_int4_weight_dims": [_vp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)],
     "yscv_hip_int4_matmul": [_vp, _vp, _i32, _vp, _i32, _sz, _vp],
     "yscv_hip_int4_gemv": [_vp, _vp, _i32, _vp, _i32, _sz, _vp],

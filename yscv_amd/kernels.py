@@ -142,6 +142,39 @@ def kv_i8_dequantize_rows(data, scales):
     return out
 
 
+# ---- packed int4 weight files (host only; the reference has no on-disk form of PackedInt4Weight) ----------
+
+def int4_file_write(path, packed, scales, group_size, m_w, k, zero_points=None, nibble_format=NIBBLE_SIGNED) -> None:
+    """Stores the arguments of PackedInt4Weight(...) behind the 64-byte header of the packed-int4 file format."""
+    p = _np(packed, np.uint8)
+    s = np.ascontiguousarray(scales)
+    if s.dtype not in (np.float32, np.float16):
+        raise TypeError("scales must be float32 or float16")
+    zp = None if zero_points is None else _np(zero_points, np.uint8)
+    if group_size <= 0 or p.size != m_w * k // 2 or s.size != m_w * (k // group_size):
+        raise ValueError("slice lengths do not match m_w, k, group_size")
+    lib().int4_file_write(str(path).encode(), _ptr(p), _ptr(s), F32 if s.dtype == np.float32 else F16,
+                          _ptr(zp) if zp is not None else None, nibble_format, _sz(m_w), _sz(k), _sz(group_size))
+
+
+def int4_file_read_header(path):
+    h = capi.Int4FileHeader()
+    lib().int4_file_read_header(str(path).encode(), C.byref(h))
+    return h
+
+
+def int4_file_read(path):
+    """-> (packed u8, scales f32|f16, zero_points u8|None, header); the checksum is verified."""
+    h = int4_file_read_header(path)
+    packed = np.empty(h.packed_bytes, np.uint8)
+    sdt = np.float32 if h.scale_dtype == F32 else np.float16
+    scales = np.empty(h.scales_bytes // np.dtype(sdt).itemsize, sdt)
+    zps = np.empty(h.zero_points_bytes, np.uint8) if h.has_zero_points else None
+    lib().int4_file_read(str(path).encode(), _ptr(packed), _sz(packed.size), _ptr(scales), _sz(scales.nbytes),
+                         _ptr(zps) if zps is not None else None, _sz(0 if zps is None else zps.size))
+    return packed, scales, zps, h
+
+
 # ---- device handles ---------------------------------------------------------------------------
 
 class PackedInt4Weight:
@@ -185,6 +218,17 @@ class PackedInt4Weight:
         self._h = h
         self.m_w, self.k = (d0, d1) if transposed_nk else (d1, d0)
         self.group_size = group_size
+        return self
+
+    @classmethod
+    def load(cls, path):
+        """Reads a packed-int4 weight file (int4_file_write) and uploads it."""
+        hdr = int4_file_read_header(path)
+        h = C.c_void_p()
+        lib().int4_weight_load(str(path).encode(), C.byref(h))
+        self = cls.__new__(cls)
+        self._h = h
+        self.m_w, self.k, self.group_size = int(hdr.n), int(hdr.k), int(hdr.group_size)
         return self
 
     @property
