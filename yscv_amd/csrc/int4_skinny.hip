@@ -27,8 +27,8 @@
 //     before the MFMA;
 //   * group scales are applied in fp32 to the MFMA result (acc += scale * D);
 //   * K is split across the wavefronts of a workgroup (each wave owns 512 k of the activations);
-//     the per-wave partial sums meet in LDS behind an LDS-only barrier, once per 16-row block
-//     (m <= 4) or once per two blocks (m > 4, where every wave has a share of the sums to add).
+//     the per-wave partial sums meet in LDS behind an LDS-only barrier, once per four 16-row blocks
+//     where the ring depth allows (fewer barriers, and every wave has a share of the sums to add).
 //     When K is too long for one workgroup, a grid-level split writes fp32 partials that a second
 //     small kernel adds in a fixed order (no atomics on shared outputs: results are deterministic).
 #include <type_traits>
@@ -158,6 +158,10 @@ __device__ __forceinline__ void zp_consts(uint32_t zp, half2_t &c1, half2_t &c2)
   c2 = half2_t{b, b};
 }
 
+// 16-row blocks whose partial sums cross the waves together (must divide the ring depth).  Four at a time measured
+// best for every m; two at a time is slower than one for m <= 4, where only two waves would have a piece to add.
+constexpr int skinny_ub(int ni, int p) { return p % 4 == 0 ? 4 : (p % 2 == 0 && ni > 1 ? 2 : 1); }
+
 // XM: where the activations come from -- 0 prepared fp16 (hi [+ lo]), 1 raw f32 (split into hi + lo here), 2 raw bf16
 template <int SPLIT, int NI, int GM, bool SF16, bool HAS_ZP, int P, int XM>
 __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
@@ -166,7 +170,7 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
   static_assert(XM != 2 || SPLIT == 1, "bf16 activations fit one fp16 operand exactly");
   // OFFSET mode: leave the 1024-offsets in the weights and cancel them per group (see file header)
   constexpr bool OFFSET = (SPLIT == 1) && !HAS_ZP;
-  constexpr int UB = (NI > 1 && P % 2 == 0) ? 2 : 1;  // 16-row blocks per cross-wave reduction
+  constexpr int UB = skinny_ub(NI, P);  // 16-row blocks per cross-wave reduction
   constexpr bool OFFSET1 = OFFSET && NI == 1;  // one useful accumulator: offset subtracted after the MFMA
   constexpr bool OFFSETC = OFFSET && NI > 1;   // all four useful: minus-offset enters as the MFMA's C operand
   constexpr int SPT = GM == GM32 ? 4 : (GM == GM64 ? 2 : 1);
@@ -621,7 +625,7 @@ template <int SPLIT, int NI, int GM, bool SF16, bool HAS_ZP>
 static int32_t launch_one(const SkinnyArgs &a, const SkinnyPlan &plan, hipStream_t s) {
   // ring depth: bounded by the VGPR budget (activations: 64 per split, ring: ~26 per slot)
   constexpr int P = SPLIT == 2 ? (NI == 1 ? 2 : 1) : (SF16 && !HAS_ZP ? 4 : 3);
-  constexpr int UB = (NI > 1 && P % 2 == 0) ? 2 : 1;  // as in the kernel
+  constexpr int UB = skinny_ub(NI, P);
   const size_t lds = (size_t)2 * plan.waves * UB * NI * 64 * sizeof(float);
   if constexpr (SPLIT == 2) {
     if (a.xf != nullptr) {
