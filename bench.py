@@ -139,6 +139,22 @@ def cpu_baseline(cfg, seconds_budget=20.0):
     }
 
 
+def measured_peaks(torch):
+    """What this GPU sustains on a plain 1 GiB HBM read stream and on back-to-back MFMAs held in registers
+    (yscv_hip_measure_peaks).  The roofline fractions stay priced against the published peaks; these figures say how
+    much of a published peak is within reach of any kernel on this machine."""
+    import ctypes as C
+
+    from yscv_amd import capi
+
+    torch.cuda.synchronize()
+    r, f, i = C.c_double(), C.c_double(), C.c_double()
+    capi.lib().measure_peaks(C.byref(r), C.byref(f), C.byref(i))
+    return {"hbm_read_GB/s": round(r.value, 1), "frac_of_8TB/s": round(r.value / HBM_PEAK_GBS, 3),
+            "mfma_f16_TFLOP/s": round(f.value, 1), "frac_of_2.5PFLOP/s": round(f.value / 2500.0, 3),
+            "mfma_i8_TOP/s": round(i.value, 1), "frac_of_5POP/s": round(i.value / 5000.0, 3)}
+
+
 def extra_kernels(torch, stream_ptr):
     """Stand-alone kernels of BASELINE configs 1-3 and 5 (short runs; the parity tests cover correctness).
     Each call sequence is captured into a HIP graph and replayed, so the figures are device time per call
@@ -283,7 +299,9 @@ def main():
     cfg["max_steps"] = max(cfg["max_steps"], args.steps + args.warmup)
     stream_ptr = torch.cuda.current_stream().cuda_stream
     if args.extra_only:
-        print(json.dumps({"extra": extra_kernels(torch, stream_ptr)}))
+        extra = extra_kernels(torch, stream_ptr)
+        extra["measured_peaks"] = measured_peaks(torch)
+        print(json.dumps({"extra": extra}))
         return
 
     if args.calib_copy:
@@ -370,6 +388,7 @@ def main():
     torch.cuda.empty_cache()
     if not args.no_extra:
         extra.update(extra_kernels(torch, stream_ptr))
+        extra["measured_peaks"] = measured_peaks(torch)
         result["extra"] = extra
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(cfg)

@@ -73,6 +73,13 @@ const char *yscv_hip_last_error(void);
  * (crates/yscv-kernels/src/core.rs:79-121).  Writes a NUL-terminated string. */
 int32_t yscv_hip_device_info(char *buf, size_t buf_len);
 
+/* Calibration: what this GPU sustains on a plain HBM read stream (1 GiB, GB/s) and on back-to-back matrix
+ * instructions held in registers (v_mfma_f32_16x16x32_f16 in TFLOP/s, v_mfma_i32_16x16x64_i8 in TOP/s).  Takes a
+ * few milliseconds, allocates 1 GiB for its duration, runs on the default stream.  No counterpart in the reference:
+ * its microbenchmark relates the dispatch kernels to its own scalar loops ("SIMD speedup vs scalar",
+ * apps/llm-bench/src/bin/kernel_bench.rs:187), not to a machine peak. */
+int32_t yscv_hip_measure_peaks(double *hbm_read_gbs, double *mfma_f16_tflops, double *mfma_i8_tops);
+
 /* Device memory helpers for hosts without their own HIP binding. */
 int32_t yscv_hip_malloc(void **dev_ptr, size_t bytes);
 int32_t yscv_hip_free(void *dev_ptr);

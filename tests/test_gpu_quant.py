@@ -103,3 +103,17 @@ def test_kv_cache_int8_rows_bit_exact(oracle, K):
     src = np.array([[127.0, 0.5, -0.5, 1.5, -2.5, 63.5]], np.float32)
     d, s = K.kv_i8_quantize_rows(torch.from_numpy(src).cuda())
     assert float(s[0]) == 1.0 and d.cpu().numpy().ravel().tolist() == [127, 1, -1, 2, -3, 64]
+
+
+def test_measured_peaks_are_plausible(K):
+    """yscv_hip_measure_peaks: a sustained figure can neither exceed the published peak nor sit far below what this
+    class of GPU reaches (the probes are registers-only MFMA loops and a 1 GiB read stream)."""
+    import ctypes as C
+
+    from yscv_amd import capi
+
+    r, f, i = C.c_double(), C.c_double(), C.c_double()
+    capi.lib().measure_peaks(C.byref(r), C.byref(f), C.byref(i))
+    assert 3000.0 < r.value <= 8000.0, r.value
+    assert 1000.0 < f.value <= 2500.0, f.value
+    assert 2000.0 < i.value <= 5000.0, i.value

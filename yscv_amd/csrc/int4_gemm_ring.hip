@@ -3,8 +3,10 @@
 //
 // A workgroup owns a (32 MT) x (32 NT) tile of y (MT = 1, 2 or 4 by m).  It has four MMA waves (2 x 2, MT x NT MFMA tiles each) and NP
 // producer waves.  Per stage of KS k-steps (32 k each) the producers
-//   * fetch the activation rows (fp16, prepared by x_prep) with LDS-direct loads, one 16-byte piece per lane, so
-//     the row-major -> MFMA-fragment transposition costs nothing, and
+//   * fetch the activation rows (fp16, prepared by x_prep) with LDS-direct loads, one 16-byte piece per lane: an
+//     instruction takes eight whole 128-byte lines (eight rows x both k-steps of the stage), and a per-row XOR of
+//     the chunk index makes the later fragment reads conflict-free, so the row-major -> MFMA-fragment
+//     transposition costs nothing, and
 //   * load the packed weight words of the stage into registers, decode them to fp16 (q - zp) * scale ONCE per
 //     workgroup and write them to LDS in fragment order.
 // The MMA waves only read fragments (ds_read_b128) and issue v_mfma_f32_16x16x32_f16; a decoded weight is used by
@@ -26,6 +28,8 @@
 namespace yscv {
 
 namespace {
+
+__device__ const float kOne = 1.0f;  // stands in for an absent row-scale vector
 
 typedef __attribute__((address_space(3))) void lds_void;
 #define G4_AS1(ptr) ((const void __attribute__((address_space(1))) *)(ptr))
@@ -209,10 +213,16 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
     // per-lane byte offsets (fixed) and uniform base pointers (advanced per stage)
     uint32_t aoff[APW];
 #pragma unroll
+    // Piece q of a stage = rows 8 h .. 8 h + 7 (h = q & 1) of 16-row group q / 2, both k-steps: eight whole 128-byte
+    // lines per load instruction, eight neighbouring lanes per line.  Lane i fetches 16-byte chunk (i & 7) ^ g of
+    // row i / 8, g = 4 h + (i / 8) / 2: with this swizzle the 16 lanes that later read one k-chunk of 16 rows in
+    // one ds_read_b128 pass hit 16 different 16-byte slots (no bank conflict).
     for (int j = 0; j < APW; j++) {
       const int q = pw * APW + j;
-      const int row = min(m0 + (q / KS) * 16 + r, p.m - 1);
-      aoff[j] = (uint32_t)(((size_t)row * p.k_pad + (q % KS) * 32 + c * 8) * sizeof(_Float16));
+      const int h = q & 1, row8 = lane >> 3;
+      const int chunk = (lane & 7) ^ (4 * h + (row8 >> 1));
+      const int row = min(m0 + (q >> 1) * 16 + 8 * h + row8, p.m - 1);
+      aoff[j] = (uint32_t)(((size_t)row * p.k_pad + chunk * 8) * sizeof(_Float16));
     }
     const uint32_t woff = lane * 16, soff = r * SC::SC_BYTES, zoff = r * SC::ZP_BYTES;
     const uint8_t *wbase[WT], *sbase[WT], *zbase[WT];
@@ -343,7 +353,14 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
     for (int i = 0; i < MT; i++)
 #pragma unroll
       for (int j = 0; j < NT; j++) acc[i][j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-    const uint32_t a_lane = lds0 + (uint32_t)(wm * MT * KS * 1024 + lane * 16);
+    // k-step ks of 16-row group: lane (r, c) wants chunk 4 ks + c of row r, stored at slot (r % 8) * 8 + (chunk ^ g)
+    // of the half r / 8 (see the producer's swizzle)
+    uint32_t a_lane_ks[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      const int g = 4 * (r >> 3) + ((r & 7) >> 1);
+      a_lane_ks[ks] = lds0 + (uint32_t)(wm * MT * KS * 1024 + (r >> 3) * 1024 + (((r & 7) * 8 + ((4 * ks + c) ^ g)) * 16));
+    }
     const uint32_t b_lane = lds0 + B_BASE + (uint32_t)(wn * NT * KS * 1024 + lane * 16);
     G4Frags<MT, NT> f[2];
     auto mfmas = [&](const G4Frags<MT, NT> &cur, int i0, int i1) {
@@ -353,21 +370,21 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
         for (int j = 0; j < NT; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cur.b[j], cur.a[i], acc[i][j], 0, 0, 0);
     };
     __builtin_amdgcn_s_barrier();
-    g4_issue<KS>(f[0], a_lane, b_lane);
+    g4_issue<KS>(f[0], a_lane_ks[0], b_lane);
     uint32_t aslot = 0, bslot = 0;
     for (int st = 0; st < nstages; st++) {
       const uint32_t naslot = aslot + A_BYTES == SA * A_BYTES ? 0 : aslot + A_BYTES;
       const uint32_t nbslot = bslot ^ B_BYTES;
       // k-step 0: the fragments of k-step 1 are on their way while its MFMAs run
       g4_wait(f[0]);
-      g4_issue<KS>(f[1], a_lane + aslot + 1024, b_lane + bslot + 1024);
+      g4_issue<KS>(f[1], a_lane_ks[1] + aslot, b_lane + bslot + 1024);
       mfmas(f[0], 0, MT);
       // k-step 1: the first MFMAs cover the barrier, the others the fragment reads of the next stage
       g4_wait(f[1]);
       mfmas(f[1], 0, MT / 2);
       if (st + 1 < nstages) {
         __builtin_amdgcn_s_barrier();
-        g4_issue<KS>(f[0], a_lane + naslot, b_lane + nbslot);
+        g4_issue<KS>(f[0], a_lane_ks[0] + naslot, b_lane + nbslot);
       }
       mfmas(f[1], MT / 2, MT);
       aslot = naslot;
@@ -379,15 +396,21 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
   // all waves store whole rows ------------------------------------------------------------------------------
   __syncthreads();
   if (wave < 4) {
+    // all row scales are requested together (a load behind a branch of its own is waited for on its own)
+    float rs[MT];
+#pragma unroll
+    for (int i = 0; i < MT; i++) {
+      const int row = min(m0 + wm * MT * 16 + i * 16 + r, p.m - 1);
+      const float *src = p.row_scale ? p.row_scale + row : &kOne;
+      rs[i] = *src;
+    }
 #pragma unroll
     for (int i = 0; i < MT; i++) {
       const int lrow = wm * MT * 16 + i * 16 + r;
-      const int row = min(m0 + lrow, p.m - 1);
-      const float rs = p.row_scale ? p.row_scale[row] : 1.0f;
 #pragma unroll
       for (int j = 0; j < NT; j++) {
         const int lcol = wn * NT * 16 + j * 16 + c * 4;
-        *reinterpret_cast<float4_t *>(g4_ring + lrow * RS + lcol * 4) = acc[i][j] * rs;
+        *reinterpret_cast<float4_t *>(g4_ring + lrow * RS + lcol * 4) = acc[i][j] * rs[i];
       }
     }
   }

@@ -173,14 +173,26 @@ __global__ void __launch_bounds__(1024) x_prep_kernel(const void *__restrict__ x
   const size_t row = blockIdx.x;
   const size_t base = row * k;
   const size_t chunks = k_pad / 8;
-  // pass 1: abs-max of the row (values stay in registers when the row fits one sweep)
+  // pass 1: abs-max of the row.  The first sweep's values stay in registers for pass 2 (a row of up to 8 blockDim
+  // elements is read from memory once); longer rows re-read the rest.
   float amax = 0.0f;
-  for (size_t ch = threadIdx.x; ch < chunks; ch += blockDim.x) {
+  float v0[8];
+  const size_t ch0 = threadIdx.x;
+  const bool have0 = ch0 < chunks && ch0 * 8 < k;
+  if (have0) {
+    load8<VEC>(x, base + ch0 * 8, x_dtype, base + k, v0);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; i++) v0[i] = 0.0f;
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(v0[i]));  // NaN is ignored here, kept in the values
+  for (size_t ch = ch0 + blockDim.x; ch < chunks; ch += blockDim.x) {
     if (ch * 8 < k) {
       float v[8];
       load8<VEC>(x, base + ch * 8, x_dtype, base + k, v);
 #pragma unroll
-      for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(v[i]));  // NaN is ignored here, kept in the values
+      for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(v[i]));
     }
   }
   for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
@@ -198,9 +210,12 @@ __global__ void __launch_bounds__(1024) x_prep_kernel(const void *__restrict__ x
   const float up = ldexpf(1.0f, shift);
   if (threadIdx.x == 0) row_scale[row] = ldexpf(1.0f, -shift);
   const size_t obase = row * k_pad;
-  for (size_t ch = threadIdx.x; ch < chunks; ch += blockDim.x) {
+  for (size_t ch = ch0; ch < chunks; ch += blockDim.x) {
     float v[8];
-    if (ch * 8 < k) {
+    if (ch == ch0) {
+#pragma unroll
+      for (int i = 0; i < 8; i++) v[i] = v0[i];
+    } else if (ch * 8 < k) {
       load8<VEC>(x, base + ch * 8, x_dtype, base + k, v);
     } else {
 #pragma unroll

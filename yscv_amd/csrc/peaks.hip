@@ -1,0 +1,117 @@
+// Calibration probes: what this GPU sustains on a plain HBM read stream and on back-to-back matrix instructions held
+// in registers.  The rooflines in the benchmark are priced against the published peaks (8 TB/s, 2.5 PFLOP/s fp16,
+// 5 POP/s int8); these figures say how much of a published peak any kernel can reach on the machine at hand (the
+// clock under a full MFMA load is below the nominal one).  No counterpart in the reference.
+#include "common.hpp"
+#include "int4_common.hpp"
+
+namespace yscv {
+namespace {
+
+// every wave reads 4 KiB chunks (four 128-bit loads per lane), chunks interleaved over all waves of the grid
+__global__ void __launch_bounds__(512) peak_read_kernel(const uint4_t *__restrict__ p, size_t n_chunks, uint32_t *out) {
+  const size_t wave = (blockIdx.x * (size_t)blockDim.x + threadIdx.x) >> 6;
+  const size_t nwaves = ((size_t)gridDim.x * blockDim.x) >> 6;
+  const int lane = threadIdx.x & 63;
+  uint4_t acc = {0, 0, 0, 0};
+  for (size_t c = wave; c < n_chunks; c += nwaves) {
+    const uint4_t *q = p + c * 256 + lane;
+    uint4_t v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) v[u] = __builtin_nontemporal_load(q + u * 64);
+#pragma unroll
+    for (int u = 0; u < 4; u++) acc ^= v[u];
+  }
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345678u) out[0] = 1;  // keeps the loads alive
+}
+
+template <bool I8>
+__global__ void __launch_bounds__(512) peak_mfma_kernel(int iters, uint32_t *out) {
+  constexpr int NACC = 16;  // independent accumulators: the matrix pipe never waits for a result
+  float s = 0.0f;
+  if constexpr (I8) {
+    int4_t a = {(int)threadIdx.x, 1, 2, 3}, b = {3, 2, 1, (int)threadIdx.x};
+    int4_t acc[NACC];
+    for (int i = 0; i < NACC; i++) acc[i] = int4_t{0, 0, 0, 0};
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+      for (int i = 0; i < NACC; i++) acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[i], 0, 0, 0);
+    }
+    for (int i = 0; i < NACC; i++) s += (float)(acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3]);
+  } else {
+    half8_t a, b;
+    for (int e = 0; e < 8; e++) {
+      a[e] = (_Float16)(0.001f * (float)((threadIdx.x + e) & 63));
+      b[e] = (_Float16)(0.002f * (float)((threadIdx.x - e) & 63));
+    }
+    float4_t acc[NACC];
+    for (int i = 0; i < NACC; i++) acc[i] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+      for (int i = 0; i < NACC; i++) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[i], 0, 0, 0);
+    }
+    for (int i = 0; i < NACC; i++) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+  }
+  if (s == 123.456f) out[0] = 1;
+}
+
+struct Events {
+  hipEvent_t a = nullptr, b = nullptr;
+  ~Events() {
+    if (a) (void)hipEventDestroy(a);
+    if (b) (void)hipEventDestroy(b);
+  }
+};
+
+}  // namespace
+}  // namespace yscv
+
+using namespace yscv;
+
+extern "C" int32_t yscv_hip_measure_peaks(double *hbm_read_gbs, double *mfma_f16_tflops, double *mfma_i8_tops) {
+  const Context *ctx = nullptr;
+  YSCV_TRY(ensure_context(&ctx));
+  YSCV_REQUIRE(hbm_read_gbs && mfma_f16_tflops && mfma_i8_tops, "null argument");
+  Events ev;
+  YSCV_HIP_TRY(hipEventCreate(&ev.a));
+  YSCV_HIP_TRY(hipEventCreate(&ev.b));
+  DevBuf flag, buf;
+  YSCV_TRY(flag.alloc(64));
+  // 1 GiB: four times the Infinity Cache, so the stream comes from HBM
+  const size_t bytes = (size_t)1 << 30;
+  YSCV_TRY(buf.alloc(bytes));
+  YSCV_HIP_TRY(hipMemset(buf.p, 1, bytes));
+  float ms = 0.0f, best = 1e30f;
+  const int wgs = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  for (int rep = 0; rep < 5; rep++) {  // the first repetition warms up; the best of the others counts
+    YSCV_HIP_TRY(hipEventRecord(ev.a, nullptr));
+    hipLaunchKernelGGL(peak_read_kernel, dim3(wgs), dim3(512), 0, nullptr, buf.as<uint4_t>(), bytes / 4096, flag.as<uint32_t>());
+    YSCV_HIP_TRY(hipGetLastError());
+    YSCV_HIP_TRY(hipEventRecord(ev.b, nullptr));
+    YSCV_HIP_TRY(hipEventSynchronize(ev.b));
+    YSCV_HIP_TRY(hipEventElapsedTime(&ms, ev.a, ev.b));
+    if (rep > 0 && ms < best) best = ms;
+  }
+  *hbm_read_gbs = (double)bytes / (best * 1e-3) / 1e9;
+  const int iters = 8000;
+  const double mfmas = (double)iters * 16 * 4 * wgs;  // 4 waves (one per SIMD) per workgroup, one workgroup per CU
+  for (int kind = 0; kind < 2; kind++) {
+    best = 1e30f;
+    for (int rep = 0; rep < 8; rep++) {  // the clock takes a few launches to settle after the memory-bound probe
+      YSCV_HIP_TRY(hipEventRecord(ev.a, nullptr));
+      if (kind == 0)
+        hipLaunchKernelGGL(peak_mfma_kernel<false>, dim3(wgs), dim3(256), 0, nullptr, iters, flag.as<uint32_t>());
+      else
+        hipLaunchKernelGGL(peak_mfma_kernel<true>, dim3(wgs), dim3(256), 0, nullptr, iters, flag.as<uint32_t>());
+      YSCV_HIP_TRY(hipGetLastError());
+      YSCV_HIP_TRY(hipEventRecord(ev.b, nullptr));
+      YSCV_HIP_TRY(hipEventSynchronize(ev.b));
+      YSCV_HIP_TRY(hipEventElapsedTime(&ms, ev.a, ev.b));
+      if (rep > 0 && ms < best) best = ms;
+    }
+    // 16x16x32 f16: 16384 flop; 16x16x64 i8: 32768 op
+    if (kind == 0) *mfma_f16_tflops = mfmas * 16384.0 / (best * 1e-3) / 1e12;
+    else *mfma_i8_tops = mfmas * 32768.0 / (best * 1e-3) / 1e12;
+  }
+  return YSCV_HIP_OK;
+}
