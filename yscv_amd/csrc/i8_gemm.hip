@@ -292,7 +292,11 @@ __device__ __forceinline__ void i8_frags_wait(I8Frags<MT, NT> &f) {
   }
 }
 
-template <int MT, int NT, int KS, int S>
+// WIDE_A (k-steps come in pairs, i.e. k % 128 == 0): an A load instruction takes eight whole 128-byte lines (eight
+// rows x two k-steps, eight neighbouring lanes per line) instead of sixteen half lines; lane i fetches 16-byte chunk
+// (i & 7) ^ g of row i / 8 with g = 4 h + (i / 8) / 2 (h = which eight rows of the 16-row group), so that the sixteen
+// lanes which later read one k-chunk of sixteen rows in one ds_read_b128 pass hit sixteen different 16-byte slots.
+template <int MT, int NT, int KS, int S, bool WIDE_A>
 __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int tiles_m, int tiles_n, int sbm_log2) {
   constexpr int BM = 32 * MT, BN = 32 * NT;
   constexpr int A_BYTES = 2 * MT * KS * 1024, STAGE = 2 * (MT + NT) * KS * 1024;
@@ -334,8 +338,16 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
     for (int j = 0; j < PER_WAVE; j++) {
       const int q = pw * PER_WAVE + j;
       if (q < 2 * MT * KS) {
-        const int row = min(m0 + (q / KS) * 16 + r, p.m - 1);
-        src[j] = p.a + (size_t)row * p.k + c * 16;
+        if constexpr (WIDE_A) {
+          // piece (q % KS) of 16-row group q / KS: k-step pair (q % KS) / 2, rows 8 h .. 8 h + 7 with h = q % 2
+          const int h = q & 1, row8 = lane >> 3;
+          const int chunk = (lane & 7) ^ (4 * h + (row8 >> 1));
+          const int row = min(m0 + (q / KS) * 16 + 8 * h + row8, p.m - 1);
+          src[j] = p.a + (size_t)row * p.k + chunk * 16;
+        } else {
+          const int row = min(m0 + (q / KS) * 16 + r, p.m - 1);
+          src[j] = p.a + (size_t)row * p.k + c * 16;
+        }
       } else {
         const int gnt = min(n0 / 16 + (q - 2 * MT * KS) / KS, nt_total - 1);
         src[j] = reinterpret_cast<const uint8_t *>(p.frag) + (size_t)gnt * p.ksteps * 1024 + lane * 16;
@@ -350,7 +362,8 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
         const int q = pw * PER_WAVE + j;                      // wave-uniform
         const bool is_a = q < 2 * MT * KS;
         const int ks = (is_a ? q : q - 2 * MT * KS) % KS;
-        const int gks = min(st * KS + ks, p.ksteps - 1);       // k-steps past the end re-read the last one
+        // k-steps past the end re-read the last one (WIDE_A pieces: the last pair)
+        const int gks = (WIDE_A && is_a) ? min(st * KS + (ks & ~1), p.ksteps - 2) : min(st * KS + ks, p.ksteps - 1);
         const uint8_t *g = src[j] + (size_t)gks * (is_a ? 64 : 1024);
         __builtin_amdgcn_global_load_lds(I8_AS1(g), (lds_void *)(uintptr_t)(dst + j * 1024), 16, 0, 0);
       }
@@ -379,12 +392,24 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
     }
   } else {
     // ---- compute -------------------------------------------------------------------------------------
-    const uint32_t a_lane = lds0 + (uint32_t)(wm * MT * KS * 1024 + lane * 16);
+    // A fragment of k-step ks: lane (r, c) wants chunk 4 (ks % 2) + c of row r.  WIDE_A stores it at slot
+    // (r % 8) * 8 + (chunk ^ g) of piece 2 (ks / 2) + r / 8 of its 16-row group (see the producer's swizzle).
+    uint32_t a_lane_ks[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      if constexpr (WIDE_A) {
+        const int g = 4 * (r >> 3) + ((r & 7) >> 1);
+        a_lane_ks[ks] = lds0 + (uint32_t)(wm * MT * KS * 1024 + (2 * (ks >> 1) + (r >> 3)) * 1024 +
+                                          ((r & 7) * 8 + ((4 * (ks & 1) + c) ^ g)) * 16);
+      } else {
+        a_lane_ks[ks] = lds0 + (uint32_t)(wm * MT * KS * 1024 + ks * 1024 + lane * 16);
+      }
+    }
     const uint32_t b_lane = lds0 + (uint32_t)(A_BYTES + wn * NT * KS * 1024 + lane * 16);
     const int4_t xr = {p.a_xor, p.a_xor, p.a_xor, p.a_xor};
     I8Frags<MT, NT> f[2];
     __builtin_amdgcn_s_barrier();
-    i8_frags_issue<KS>(f[0], a_lane, b_lane);
+    i8_frags_issue<KS>(f[0], a_lane_ks[0], b_lane);
     auto mfmas = [&](I8Frags<MT, NT> &cur, int i0, int i1) {
 #pragma unroll
       for (int i = i0; i < i1; i++) {
@@ -402,7 +427,7 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
         const bool live = st * KS + ks < p.ksteps;  // false only in the padding of the last stage
         i8_frags_wait(cur);
         if (ks + 1 < KS) {
-          i8_frags_issue<KS>(nxt, a_lane + slot + (ks + 1) * 1024, b_lane + slot + (ks + 1) * 1024);
+          i8_frags_issue<KS>(nxt, a_lane_ks[(ks + 1) % KS] + slot, b_lane + slot + (ks + 1) * 1024);
           if (live) mfmas(cur, 0, MT);
         } else {
           // the first half of the MFMAs runs while this wave waits at the barrier, the second half while the
@@ -411,7 +436,7 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
           if (st + 1 < nstages) {
             // every read of stage st by this wave has returned: tell the producers, pick up stage st+1
             __builtin_amdgcn_s_barrier();
-            i8_frags_issue<KS>(nxt, a_lane + nslot, b_lane + nslot);
+            i8_frags_issue<KS>(nxt, a_lane_ks[0] + nslot, b_lane + nslot);
           }
           if (live) mfmas(cur, MT / 2, MT);
         }
@@ -498,13 +523,13 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
   }
 }
 
-template <int MT, int NT, int KS, int S>
+template <int MT, int NT, int KS, int S, bool WIDE_A>
 int32_t launch_ring(const I8Args &p, size_t m, size_t n, hipStream_t s) {
   constexpr int LDS = 2 * (MT + NT) * KS * 1024 * S;
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   std::call_once(once, [] {
-    attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(i8_gemm_ring_kernel<MT, NT, KS, S>),
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(i8_gemm_ring_kernel<MT, NT, KS, S, WIDE_A>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
   });
   if (attr_err != hipSuccess)
@@ -515,7 +540,7 @@ int32_t launch_ring(const I8Args &p, size_t m, size_t n, hipStream_t s) {
   const int sbm = 1 << sbm_log2, sbn = 32 >> sbm_log2;
   const int super_blocks = ((tiles_m + sbm - 1) / sbm) * ((tiles_n + sbn - 1) / sbn);
   const unsigned grid = (unsigned)((super_blocks + 7) / 8) * 8 * 32;
-  hipLaunchKernelGGL((i8_gemm_ring_kernel<MT, NT, KS, S>), dim3(grid), dim3(I8R_THREADS), LDS, s, p, tiles_m, tiles_n, sbm_log2);
+  hipLaunchKernelGGL((i8_gemm_ring_kernel<MT, NT, KS, S, WIDE_A>), dim3(grid), dim3(I8R_THREADS), LDS, s, p, tiles_m, tiles_n, sbm_log2);
   YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
 }
@@ -549,8 +574,10 @@ int32_t launch_i8_gemm(const void *a, int a_is_u8, int a_zp, const yscv_hip_i8_w
     const Context *ctx = nullptr;
     YSCV_TRY(ensure_context(&ctx));
     const size_t big_tiles = ceil_div(m, (size_t)128) * ceil_div(b->n, (size_t)128);
-    if (big_tiles >= (size_t)ctx->num_cus) return launch_ring<4, 4, 2, 4>(p, m, b->n, s);
-    return launch_ring<2, 4, 4, 3>(p, m, b->n, s);
+    const bool wide_a = b->k % 128 == 0;  // k-steps come in pairs: A is fetched as whole 128-byte lines
+    if (big_tiles >= (size_t)ctx->num_cus)
+      return wide_a ? launch_ring<4, 4, 2, 4, true>(p, m, b->n, s) : launch_ring<4, 4, 2, 4, false>(p, m, b->n, s);
+    return wide_a ? launch_ring<2, 4, 4, 3, true>(p, m, b->n, s) : launch_ring<2, 4, 4, 3, false>(p, m, b->n, s);
   }
   dim3 grid((unsigned)ceil_div(b->n, (size_t)I8_BN), (unsigned)ceil_div(m, (size_t)I8_BM));
   const bool vec = (b->k % 16 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
