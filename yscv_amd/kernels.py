@@ -240,9 +240,20 @@ class PackedInt4Weight:
         lib().int4_weight_dims(self._h, C.byref(n), C.byref(k), C.byref(g), C.byref(b))
         return b.value
 
-    def matmul(self, x, out=None, out_dtype=None, mode: str = "auto"):
+    def workspace_bytes(self, m: int, x_dtype) -> int:
+        """Scratch yscv_hip_int4_matmul_ws needs for m rows of activations of torch dtype x_dtype (0 = none)."""
+        import torch
+
+        code = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}[x_dtype]
+        b = _sz()
+        lib().int4_workspace_bytes(self._h, _sz(m), code, C.byref(b))
+        return b.value
+
+    def matmul(self, x, out=None, out_dtype=None, mode: str = "auto", workspace=None):
         """x: CUDA tensor [..., k] (f32/f16/bf16).  mode: auto | gemv | gemm.  Output shape is
-        x.shape[:-1] + [m_w], like exec_matmul's int4 branch (runner/linear.rs:269-270)."""
+        x.shape[:-1] + [m_w], like exec_matmul's int4 branch (runner/linear.rs:269-270).  With `workspace` (a CUDA
+        uint8 tensor of at least workspace_bytes(m, x.dtype), 256-byte aligned) the call allocates nothing
+        (yscv_hip_int4_matmul_ws, mode auto only)."""
         import torch
 
         assert x.is_cuda and x.shape[-1] == self.k
@@ -251,6 +262,12 @@ class PackedInt4Weight:
         odt = out_dtype or x.dtype
         if out is None:
             out = torch.empty(*x.shape[:-1], self.m_w, device=x.device, dtype=odt)
+        if workspace is not None:
+            assert mode == "auto" and workspace.is_cuda and workspace.dtype == torch.uint8
+            lib().int4_matmul_ws(self._h, C.c_void_p(x.data_ptr()), _torch_dtype_code(x), C.c_void_p(out.data_ptr()),
+                                 _torch_dtype_code(out), _sz(m), C.c_void_p(workspace.data_ptr()),
+                                 _sz(workspace.numel()), _stream_ptr())
+            return out
         fn = {"auto": lib().int4_matmul, "gemv": lib().int4_gemv, "gemm": lib().int4_gemm}[mode]
         fn(self._h, C.c_void_p(x.data_ptr()), _torch_dtype_code(x), C.c_void_p(out.data_ptr()),
            _torch_dtype_code(out), _sz(m), _stream_ptr())
