@@ -700,6 +700,8 @@ int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan
   int32_t st;
   if (split == 2)
     st = small ? launch_gm<2, 1>(a, plan, w->gm, sf16, w->has_zp, s) : launch_gm<2, 4>(a, plan, w->gm, sf16, w->has_zp, s);
+  else if (m > 4 && m <= 8)  // two accumulators per lane: half the scale FMAs and half the exchange of the 16-row form
+    st = launch_gm<1, 2>(a, plan, w->gm, sf16, w->has_zp, s);
   else
     st = small ? launch_gm<1, 1>(a, plan, w->gm, sf16, w->has_zp, s) : launch_gm<1, 4>(a, plan, w->gm, sf16, w->has_zp, s);
   YSCV_TRY(st);
