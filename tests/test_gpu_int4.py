@@ -388,3 +388,25 @@ def test_weight_loaded_from_a_file_equals_the_uploaded_one(K, torch_cuda, tmp_pa
     for m in (1, 9, 40):
         x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).half().cuda()
         assert torch.equal(w0.matmul(x, out_dtype=torch.float32), w1.matmul(x, out_dtype=torch.float32))
+
+
+@pytest.mark.parametrize("m,xdt", [(3, "bf16"), (3, "f32"), (40, "bf16"), (300, "f16")])
+def test_caller_workspace_gives_the_same_bits(K, torch_cuda, m, xdt):
+    """yscv_hip_int4_matmul_ws: scratch from the caller instead of the stream-ordered allocator, same result."""
+    torch = torch_cuda
+    rng = np.random.default_rng(91 + m)
+    n, k, g = 300, 1000 if xdt == "f32" else 1024, 8 if xdt == "f32" else 64   # k = 1000: padded K, activation pass needed
+    b = _rand_packed(rng, n, k)
+    scales = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float32)
+    w = K.PackedInt4Weight(b, scales, g, n, k, nibble_format=K.NIBBLE_UNSIGNED)
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[xdt]
+    x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).to(tdt).cuda()
+    need = w.workspace_bytes(m, tdt)
+    ws = torch.full((need + 256,), 0xA5, dtype=torch.uint8, device="cuda")
+    y0 = w.matmul(x, out_dtype=torch.float32)
+    y1 = w.matmul(x, out_dtype=torch.float32, workspace=ws[: max(need, 1)])
+    assert torch.equal(y0, y1)
+    assert bool((ws[need:] == 0xA5).all())  # nothing written past the announced size
+    if need > 0:
+        with pytest.raises(Exception, match="workspace too small"):
+            w.matmul(x, out_dtype=torch.float32, workspace=ws[: need - 1])
