@@ -57,8 +57,7 @@ __device__ __forceinline__ void gemm_zp_consts(uint32_t zp, half2_t &c1, half2_t
 }
 
 constexpr int G_NTW = 4;       // weight tiles (16 columns each) per wave
-constexpr int G_WAVES = 4;
-constexpr int G_BN = G_NTW * G_WAVES * 16;  // 256 columns per workgroup
+constexpr int G_WAVES = 4;      // G_NTW * G_WAVES * 16 = 256 columns per workgroup
 
 template <int MT, int SPLIT, int GM, bool SF16>
 __global__ void __launch_bounds__(256) int4_gemm_kernel(GemmArgs a) {
