@@ -460,7 +460,11 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
   // would make the compiler wait for every weight block in flight)
   float rs[NI];
 #pragma unroll
-  for (int i = 0; i < NI; i++) rs[i] = (a.row_scale && c * NI + i < a.m) ? a.row_scale[c * NI + i] : 1.0f;
+  for (int i = 0; i < NI; i++) rs[i] = 1.0f;
+  if (a.row_scale) {  // one branch around all of them: rows past m read the last row's scale and are never stored
+#pragma unroll
+    for (int i = 0; i < NI; i++) rs[i] = a.row_scale[min(c * NI + i, a.m - 1)];
+  }
 
   // Meet the other k slices in LDS, once per UB blocks: every wave leaves its UB x NI x 64 partial sums, and after
   // one barrier the sums are shared out over the waves in 64-lane pieces (piece q = block q / NI of the group,
