@@ -451,6 +451,30 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
   __syncthreads();  // every wave is done with the ring
   const float lo = (float)p.lo, hi = (float)p.hi;
   if (wave < 4) {
+    // the per-column terms of all NT column tiles are requested together: one memory round trip, not one per tile
+    int32_t zc_all[NT][4], corr_all[NT][4];
+    float comp_all[NT][4];
+#pragma unroll
+    for (int j = 0; j < NT; j++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const int cc = min(n0 + wn * NT * 16 + j * 16 + c * 4 + e, p.n - 1);
+        zc_all[j][e] = p.col_sum[cc];
+        corr_all[j][e] = 0;
+        comp_all[j][e] = p.composite;
+      }
+    if (p.corr) {
+#pragma unroll
+      for (int j = 0; j < NT; j++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) corr_all[j][e] = p.corr[min(n0 + wn * NT * 16 + j * 16 + c * 4 + e, p.n - 1)];
+    }
+    if (p.composite_v) {
+#pragma unroll
+      for (int j = 0; j < NT; j++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) comp_all[j][e] = p.composite_v[min(n0 + wn * NT * 16 + j * 16 + c * 4 + e, p.n - 1)];
+    }
 #pragma unroll
     for (int j = 0; j < NT; j++) {
       const int lcol = wn * NT * 16 + j * 16 + c * 4;
@@ -458,10 +482,9 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
       float comp[4];
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        const int cc = min(n0 + lcol + e, p.n - 1);
-        zc[e] = p.zp_mul * p.col_sum[cc];
-        corr[e] = p.corr ? p.corr[cc] : 0;
-        comp[e] = p.composite_v ? p.composite_v[cc] : p.composite;
+        zc[e] = p.zp_mul * zc_all[j][e];
+        corr[e] = corr_all[j][e];
+        comp[e] = comp_all[j][e];
       }
 #pragma unroll
       for (int i = 0; i < MT; i++) {
