@@ -256,9 +256,11 @@ def test_invalid_arguments_are_rejected(K, torch_cuda):
                                                (128, 128, 512, 32, False, False), (130, 200, 1024, 128, True, True),
                                                (257, 1000, 640, 64, True, True), (512, 136, 2048, 32, True, False),
                                                (300, 264, 768, 256, False, True), (1100, 520, 1152, 128, False, False)])
-@pytest.mark.parametrize("xdt", ["bf16", "f16"])
+@pytest.mark.parametrize("xdt", ["bf16", "f16", "f32"])
 def test_wide_m_ring_kernel(oracle, K, torch_cuda, m, n, k, g, sf16, zp, xdt):
-    """m > 16 with 16-bit activations: the LDS-ring GEMM (weights decoded to fp16 with the scale folded in).
+    """m > 16: the LDS-ring GEMM (weights decoded to fp16 with the scale folded in) for 16-bit activations and, when
+    the weight's scales are fp16, for f32 activations as well; f32 activations against f32 scales take the exact-scale
+    kernel and meet the same bars with room to spare.
     Row / column tails, every group mode, f32 and fp16 scales, with and without zero points, all output types."""
     torch = torch_cuda
     rng = np.random.default_rng(m + n * 3 + k * 7 + g)
@@ -268,7 +270,7 @@ def test_wide_m_ring_kernel(oracle, K, torch_cuda, m, n, k, g, sf16, zp, xdt):
     zq = rng.integers(6, 11, (n, groups)) if zp else np.full((n, groups), 8)
     zps = pack_zero_points(zq) if zp else None
     xt = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32))
-    xt = xt.bfloat16() if xdt == "bf16" else xt.half()
+    xt = xt.bfloat16() if xdt == "bf16" else (xt.half() if xdt == "f16" else xt)
     x = xt.float().numpy()
     ref = oracle.matmul_nbits(b, scales.astype(np.float32), pack_zero_points(zq), x, m, n, k, g)
     w = K.PackedInt4Weight(b, scales, g, n, k, zero_points=zps, nibble_format=K.NIBBLE_UNSIGNED)

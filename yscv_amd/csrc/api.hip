@@ -151,14 +151,26 @@ int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, v
   _Float16 *xl = (!L.direct && L.split == 2) ? reinterpret_cast<_Float16 *>(scratch + L.xh_bytes) : nullptr;
   float *row_scale = L.direct ? nullptr : reinterpret_cast<float *>(scratch + L.xh_bytes * L.split);
   float *partial = L.part_bytes ? reinterpret_cast<float *>(scratch + L.xh_bytes * L.split + L.rs_bytes) : nullptr;
+  // f32 activations with more than 16 rows against a weight whose scales are stored as fp16 (the MatMulNBits form) go
+  // to the LDS-ring GEMM as ONE fp16 operand: that kernel folds the group scale into fp16 weights (2^-11 relative per
+  // weight), which a lo half of the activations could not refine, and it is 3.5x (prefill shapes) to 14x (few rows,
+  // wide N) faster than the exact-scale kernel.  Weights with f32 scales -- what packed_int4_gemm_dispatch hands
+  // over -- keep the exact-scale kernel with hi + lo activations: the reference's own test holds that entry point
+  // to 1e-3 absolute (int4_matmul.rs:816-855).  The scratch keeps the size of the two-operand form.
+  int run_split = L.split;
+  if (!L.skinny && x_dtype == YSCV_HIP_F32 && m > 16 && w->scale_dtype == YSCV_HIP_F16 &&
+      int4_gemm_ring_eligible(w, xh, y, y_dtype, 1, m, L.k_pad)) {
+    run_split = 1;
+    xl = nullptr;
+  }
   int32_t st = YSCV_HIP_OK;
   if (!L.direct)
-    st = launch_x_prep(x, x_dtype, m, w->k, L.k_pad, L.split, const_cast<_Float16 *>(xh), xl, row_scale, s);
+    st = launch_x_prep(x, x_dtype, m, w->k, L.k_pad, run_split, const_cast<_Float16 *>(xh), xl, row_scale, s);
   if (st == YSCV_HIP_OK) {
     if (L.skinny)
       st = launch_int4_skinny(w, L.plan, xh, xl, xraw, row_scale, L.k_pad, L.split, y, y_dtype, m, partial, epi, s);
     else
-      st = launch_int4_gemm(w, xh, xl, row_scale, L.k_pad, L.split, y, y_dtype, m, s);
+      st = launch_int4_gemm(w, xh, xl, row_scale, L.k_pad, run_split, y, y_dtype, m, s);
   }
   if (own) {
     hipError_t fe = hipFreeAsync(scratch, s);
