@@ -412,3 +412,26 @@ def test_caller_workspace_gives_the_same_bits(K, torch_cuda, m, xdt):
     if need > 0:
         with pytest.raises(Exception, match="workspace too small"):
             w.matmul(x, out_dtype=torch.float32, workspace=ws[: need - 1])
+
+
+def test_f32_rows_beyond_16_run_as_skinny_passes(oracle, K, torch_cuda):
+    """f32 activations against f32 scales with 16 < m <= 128: 16-row passes of the exact skinny kernel (K-split and
+    caller workspace included) -- every row equals what a call with that row alone gives."""
+    torch = torch_cuda
+    rng = np.random.default_rng(123)
+    n, k, g, m = 272, 14336, 32, 40
+    b = _rand_packed(rng, n, k)
+    scales = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float32)
+    w = K.PackedInt4Weight(b, scales, g, n, k, nibble_format=K.NIBBLE_UNSIGNED)
+    x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).cuda()
+    ws = torch.empty(w.workspace_bytes(m, torch.float32), dtype=torch.uint8, device="cuda")
+    canary = torch.full((m + 1, n), 777.0, device="cuda")
+    w.matmul(x, out=canary[:m], workspace=ws)
+    y = canary[:m].clone()
+    assert bool((canary[m] == 777.0).all())
+    assert torch.equal(y, w.matmul(x))  # allocator-backed call: same bits
+    for r0 in (0, 16, 32):
+        assert torch.equal(y[r0:r0 + 16], w.matmul(x[r0:r0 + 16], mode="gemv"))
+    ref = oracle.packed_int4_gemm_scalar(b ^ 0x88, scales, x[:3].cpu().numpy(), 3, n, k, g)
+    d, rel = int4_tolerances(y[:3].cpu().numpy(), ref, k, x[:3].cpu().numpy())
+    assert rel < 5e-5, rel

@@ -85,6 +85,9 @@ struct Int4Scratch {
   size_t xh_bytes, rs_bytes, part_bytes, total;
 };
 
+// f32 activations on the exact-scale route with 16 < m <= this many rows run as 16-row skinny calls
+constexpr size_t kChunkedSkinnyMaxRows = 128;
+
 static Int4Scratch int4_scratch_layout(const yscv_hip_int4_weight *w, const void *x, int x_dtype, size_t m,
                                        int force, int num_cus) {
   Int4Scratch L{};
@@ -98,6 +101,11 @@ static Int4Scratch int4_scratch_layout(const yscv_hip_int4_weight *w, const void
   L.rs_bytes = L.direct ? 0 : round_up(m * sizeof(float), 256);
   L.part_bytes = L.skinny ? round_up(L.plan.partial_bytes, 256) : 0;
   L.total = L.xh_bytes * L.split + L.rs_bytes + L.part_bytes;
+  if (!L.skinny && force == 0 && x_dtype == YSCV_HIP_F32 && m <= kChunkedSkinnyMaxRows) {
+    // this call may run as 16-row skinny calls (see int4_run_ws): the scratch must cover one of those too
+    const Int4Scratch c = int4_scratch_layout(w, x, x_dtype, 16, 1, num_cus);
+    if (c.total > L.total) L.total = c.total;
+  }
   return L;
 }
 
@@ -135,6 +143,23 @@ int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, v
   note_int4_fast();
   Int4Scratch L = int4_scratch_layout(w, x, x_dtype, m, force, ctx->num_cus);
   if (!L.skinny && epi != EPI_STORE) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "fused epilogues exist for m <= 16 only");
+  // f32 activations that stay on the exact-scale route (f32 scales, or an output the ring GEMM cannot take): up to
+  // 128 rows go through the skinny kernel 16 rows at a time.  Each pass streams the weights again, which is still
+  // 5-10 x faster than the exact-scale GEMM kernel there: that one keeps a 64 x 256 tile per workgroup and cannot fill
+  // the GPU with so few rows (m = 64 against 14336 x 4096: 432 us; four skinny passes: about 60 us).
+  if (!L.skinny && force == 0 && x_dtype == YSCV_HIP_F32 && m <= kChunkedSkinnyMaxRows) {
+    const bool ring_ok = w->scale_dtype == YSCV_HIP_F16 &&
+                         int4_gemm_ring_eligible(w, reinterpret_cast<const _Float16 *>(uintptr_t(256)), y, y_dtype, 1, m, L.k_pad);
+    if (!ring_ok) {
+      const size_t ysz = dtype_size(y_dtype);
+      for (size_t r0 = 0; r0 < m; r0 += 16) {
+        const size_t rows = m - r0 < 16 ? m - r0 : 16;
+        YSCV_TRY(int4_run_ws(w, static_cast<const char *>(x) + r0 * w->k * sizeof(float), x_dtype,
+                             static_cast<char *>(y) + r0 * w->n * ysz, y_dtype, rows, 1, epi, ws, ws_bytes, s));
+      }
+      return YSCV_HIP_OK;
+    }
+  }
   char *scratch = static_cast<char *>(ws);
   bool own = false;
   if (L.total > 0) {

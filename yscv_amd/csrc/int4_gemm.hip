@@ -85,15 +85,13 @@ __global__ void __launch_bounds__(256) int4_gemm_kernel(GemmArgs a) {
     for (int p = 0; p < PASSES; p++) {
       const int row = p * 16 + (tid >> 4);
       const int chunk = tid & 15;
-      const int gm = m0 + row;
+      // rows past m repeat the last row (never stored): no load sits behind a branch of its own, so all loads of a
+      // slab are in flight together
+      const int gm = min(m0 + row, a.m - 1);
 #pragma unroll
       for (int sp = 0; sp < SPLIT; sp++) {
-        uint4_t v = {0, 0, 0, 0};
-        if (gm < a.m) {
-          const _Float16 *src = (sp == 0 ? a.xh : a.xl) + (size_t)gm * a.k_pad + (size_t)kt * 128 + chunk * 8;
-          v = *reinterpret_cast<const uint4_t *>(src);
-        }
-        sreg[sp][p] = v;
+        const _Float16 *src = (sp == 0 ? a.xh : a.xl) + (size_t)gm * a.k_pad + (size_t)kt * 128 + chunk * 8;
+        sreg[sp][p] = *reinterpret_cast<const uint4_t *>(src);
       }
     }
   };
@@ -115,25 +113,20 @@ __global__ void __launch_bounds__(256) int4_gemm_kernel(GemmArgs a) {
   uint4_t wraw[2][G_NTW];
   GScale<GM, SF16> wsc[2][G_NTW];
   uint32_t wzp[2][G_NTW];
+  // weight tiles past the last one repeat it (their columns are never stored); without zero points the zero-point
+  // load reads the scale chunk instead and its value is ignored, so the load count does not depend on the weight
+  const uint8_t *zsrc = has_zp ? a.tzps : reinterpret_cast<const uint8_t *>(a.tscales);
   auto w_load = [&](int kt, int slot) {
 #pragma unroll
     for (int t = 0; t < G_NTW; t++) {
-      const int nt = nt0 + t;
-      if (nt < a.nt) {
-        wraw[slot][t] = *(reinterpret_cast<const uint4_t *>(a.tiles + ((size_t)nt * a.ktp + kt) * kTileBytes) + lane);
-        const size_t chunk = (size_t)nt * a.chunks + (GM == GM128 ? kt / a.chunk_div : kt);
-        wsc[slot][t].load(a.tscales, chunk, r);
-        if (has_zp) {
-          constexpr int SPT = GScale<GM, SF16>::SPT;
-          const uint8_t *zp = a.tzps + (chunk * 16 + r) * SPT;
-          wzp[slot][t] = SPT == 4 ? *reinterpret_cast<const uint32_t *>(zp)
-                                  : (SPT == 2 ? (uint32_t) * reinterpret_cast<const uint16_t *>(zp) : (uint32_t)zp[0]);
-        }
-      } else {
-        wraw[slot][t] = uint4_t{0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u};
-        wsc[slot][t].v = 0;
-        wzp[slot][t] = 0x08080808u;
-      }
+      const int nt = min(nt0 + t, a.nt - 1);
+      wraw[slot][t] = *(reinterpret_cast<const uint4_t *>(a.tiles + ((size_t)nt * a.ktp + kt) * kTileBytes) + lane);
+      const size_t chunk = (size_t)nt * a.chunks + (GM == GM128 ? kt / a.chunk_div : kt);
+      wsc[slot][t].load(a.tscales, chunk, r);
+      constexpr int SPT = GScale<GM, SF16>::SPT;
+      const uint8_t *zp = zsrc + (chunk * 16 + r) * SPT;
+      wzp[slot][t] = SPT == 4 ? *reinterpret_cast<const uint32_t *>(zp)
+                              : (SPT == 2 ? (uint32_t) * reinterpret_cast<const uint16_t *>(zp) : (uint32_t)zp[0]);
     }
   };
 
@@ -210,13 +203,24 @@ __global__ void __launch_bounds__(256) int4_gemm_kernel(GemmArgs a) {
   }
 
   // ---- epilogue ---------------------------------------------------------------------------
+  float rsv[MT][4];
+#pragma unroll
+  for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) rsv[mt][i] = 1.0f;
+  if (a.row_scale) {  // one branch around all row scales
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) rsv[mt][i] = a.row_scale[min(m0 + mt * 16 + c * 4 + i, a.m - 1)];
+  }
 #pragma unroll
   for (int mt = 0; mt < MT; mt++) {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int row = m0 + mt * 16 + c * 4 + i;
       if (row >= a.m) continue;
-      const float rs = a.row_scale ? a.row_scale[row] : 1.0f;
+      const float rs = rsv[mt][i];
 #pragma unroll
       for (int t = 0; t < G_NTW; t++) {
         const int col = (nt0 + t) * 16 + r;
