@@ -406,6 +406,35 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
     for (int i = 0; i < NI; i++) acc[i] = 0.0f;
 #pragma unroll
     for (int t = 0; t < TPW; t++) {
+      if constexpr (GM == GM32 && SPLIT == 1) {
+        // one group per 32-k block: the four MFMAs of a tile are issued before the first result is consumed, so the
+        // scale FMAs of one block never wait for its own MFMA
+        float4_t dd[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          half8_t b;
+          if constexpr (OFFSET) {
+            b = extract8(tr.w[t][j], nc);
+          } else {
+            half2_t c1 = {(_Float16)(-1032.0f), (_Float16)(-1032.0f)};
+            half2_t c2 = {(_Float16)(-72.0f), (_Float16)(-72.0f)};
+            if constexpr (HAS_ZP) zp_consts((tr.z[t] >> (8 * j)) & 0xFF, c1, c2);
+            b = decode8_exact(tr.w[t][j], nc, c1, c2);
+          }
+          dd[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t][j][0], b, float4_t{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const float sc = tr.s[t].get(j);
+          if constexpr (OFFSET1) {
+            acc[0] = fmaf(sc, dd[j][0] - corr1[t][j], acc[0]);
+          } else {
+#pragma unroll
+            for (int i = 0; i < NI; i++) acc[i] = fmaf(sc, dd[j][i], acc[i]);
+          }
+        }
+        continue;
+      }
       float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
       float csum = 0.0f;
 #pragma unroll
