@@ -31,6 +31,7 @@
 //     where the ring depth allows (fewer barriers, and every wave has a share of the sums to add).
 //     When K is too long for one workgroup, a grid-level split writes fp32 partials that a second
 //     small kernel adds in a fixed order (no atomics on shared outputs: results are deterministic).
+#include <mutex>
 #include <type_traits>
 
 #include "int4_common.hpp"
@@ -160,6 +161,9 @@ __device__ __forceinline__ void zp_consts(uint32_t zp, half2_t &c1, half2_t &c2)
 
 // 16-row blocks whose partial sums cross the waves together (must divide the ring depth).  Four at a time measured
 // best for every m; two at a time is slower than one for m <= 4, where only two waves would have a piece to add.
+// LDS staging of the raw-f32 path for at most four rows: per wave, fp16 hi then lo parts of 4 rows x 512 k; rows are
+// 64 bytes apart modulo the bank cycle so the sixteen lanes that carry a row read conflict-free
+constexpr int kStageRow = 512 * 2 + 64, kStageWave = 2 * 4 * kStageRow;
 constexpr int skinny_ub(int ni, int p) { return p % 4 == 0 ? 4 : (p % 2 == 0 && ni > 1 ? 2 : 1); }
 
 // XM: where the activations come from -- 0 prepared fp16 (hi [+ lo]), 1 raw f32 (split into hi + lo here), 2 raw bf16
@@ -223,7 +227,7 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
   // Block `it` of this workgroup is 16-row block blockIdx.x + it * stride.  Requests past the last block are clamped
   // to it (a repeat served by the caches) so that every iteration issues the same number of loads and the
   // compiler's s_waitcnt counts stay exact.
-  constexpr bool EARLY = SPLIT == 1 && !HAS_ZP;
+  constexpr bool EARLY = (SPLIT == 1 || (XM == 1 && NI == 1)) && !HAS_ZP;
   const int iters = (a.nt - (int)blockIdx.x + stride - 1) / stride;  // >= 1, uniform in the workgroup
   Regs ring[P];
   auto fill_ring = [&]() {
@@ -292,6 +296,65 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
           if (!valid) h = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
           if constexpr (OFFSET) h = h * pre;
           xa[t][j][0] = h;
+        }
+      }
+    } else if constexpr (XM == 1 && NI == 1) {
+      // f32 activations straight from the caller, at most four rows: converting them in the operand layout would
+      // have every lane convert 128 values although only a quarter of the lanes carry a row.  Instead lane L converts
+      // 32 values (row L / 16, 32-k block L % 16) and the fp16 hi + lo parts change places through this wave's own
+      // piece of LDS.  As below, the wave normalises its 512-k slice of every row by a power of two, undone on its
+      // partial sums.  Lanes without a row read row 0 and discard it (unconditional loads: one round trip for all).
+      const int srow = lane >> 4, q = lane & 15;
+      const bool svalid = wave_active && srow < a.m;
+      const float *src = a.xf + (size_t)(svalid ? srow : 0) * a.k_pad + (size_t)t0 * 128 + q * 32;
+      float4_t raw[8];
+#pragma unroll
+      for (int e = 0; e < 8; e++) raw[e] = *reinterpret_cast<const float4_t *>(src + 4 * e);
+      float amax = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; e++)
+#pragma unroll
+        for (int u = 0; u < 4; u++) amax = fmaxf(amax, fabsf(raw[e][u]));
+      if (!svalid) amax = 0.0f;
+      amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+      amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+      amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+      amax = fmaxf(amax, __shfl_xor(amax, 8, 64));
+      int e2 = 14;
+      if (amax > 0.0f && amax < 3.0e38f) {
+        (void)frexpf(amax, &e2);
+        e2 -= 1;
+      }
+      int shift = 14 - e2;
+      shift = shift > 100 ? 100 : (shift < -100 ? -100 : shift);
+      const float up = svalid ? ldexpf(1.0f, shift) : 0.0f;
+      slice_scale = ldexpf(1.0f, -shift);
+      unsigned char *stage = reinterpret_cast<unsigned char *>(red) + (size_t)2 * waves * UB * NI * 64 * sizeof(float) +
+                             (size_t)wave * kStageWave;
+#pragma unroll
+      for (int cc = 0; cc < 4; cc++) {
+        half8_t h, l;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          const float sv = (e < 4 ? raw[2 * cc][e] : raw[2 * cc + 1][e - 4]) * up;
+          h[e] = (_Float16)sv;
+          l[e] = (_Float16)(sv - (float)h[e]);
+        }
+        *reinterpret_cast<half8_t *>(stage + srow * kStageRow + (q * 32 + cc * 8) * 2) = h;
+        *reinterpret_cast<half8_t *>(stage + 4 * kStageRow + srow * kStageRow + (q * 32 + cc * 8) * 2) = l;
+      }
+      // the wave reads what its own lanes wrote: LDS serves a wave's accesses in order, the compiler must not reorder
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      const half8_t hz = {0, 0, 0, 0, 0, 0, 0, 0};
+      const unsigned char *rd = stage + (r >> 2) * kStageRow + c * 16;  // lanes without a row share a neighbour's address
+#pragma unroll
+      for (int t = 0; t < TPW; t++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const half8_t h = *reinterpret_cast<const half8_t *>(rd + (t * 4 + j) * 64);
+          const half8_t l = *reinterpret_cast<const half8_t *>(rd + 4 * kStageRow + (t * 4 + j) * 64);
+          xa[t][j][0] = valid ? h : hz;
+          xa[t][j][1] = valid ? l : hz;
         }
       }
     } else if constexpr (XM == 1) {
@@ -368,7 +431,8 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
   // RAWX: accumulator i of lane (c, .) belongs to row c * NI + i, which lanes 4 c + i (+16, +32, +48) loaded
   float acc_scale[NI];
 #pragma unroll
-  for (int i = 0; i < NI; i++) acc_scale[i] = RAWX ? __shfl(slice_scale, 4 * c + i, 64) : 1.0f;
+  for (int i = 0; i < NI; i++)
+    acc_scale[i] = RAWX ? __shfl(slice_scale, (XM == 1 && NI == 1) ? 16 * c : 4 * c + i, 64) : 1.0f;
   // offset term of every 32-k block: sum_k x'_k * (1024 + 8 | 1024 + 128), same register layout as D
   float corr1[OFFSET1 ? TPW : 1][4];
   // OFFSETC: minus the offset term of MFMA row r and 32-k block (t, j = c), i.e. in the A-operand layout of
@@ -654,16 +718,25 @@ SkinnyPlan plan_int4_skinny(const yscv_hip_int4_weight *w, size_t m, int split, 
   return p;
 }
 
-template <int SPLIT, int NI, int GM, bool SF16, bool HAS_ZP>
-static int32_t launch_one(const SkinnyArgs &a, const SkinnyPlan &plan, hipStream_t s) {
-  // ring depth: bounded by the VGPR budget (activations: 64 per split, ring: ~26 per slot)
-  constexpr int P = SPLIT == 2 ? (NI == 1 ? 2 : 1) : (SF16 && !HAS_ZP ? 4 : 3);
+template <int SPLIT, int NI, int GM, bool SF16, bool HAS_ZP, int P>
+static int32_t launch_p(const SkinnyArgs &a, const SkinnyPlan &plan, hipStream_t s) {
   constexpr int UB = skinny_ub(NI, P);
   const size_t lds = (size_t)2 * plan.waves * UB * NI * 64 * sizeof(float);
   if constexpr (SPLIT == 2) {
     if (a.xf != nullptr) {
+      const size_t stage = NI == 1 ? (size_t)plan.waves * kStageWave : 0;
+      if (stage > 0) {  // 8 waves: 68 KB, above the default dynamic-LDS limit
+        static std::once_flag once;
+        static hipError_t attr_err = hipSuccess;
+        std::call_once(once, [] {
+          attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(int4_skinny_kernel<SPLIT, NI, GM, SF16, HAS_ZP, P, 1>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 8 * (2 * UB * NI * 64 * 4 + kStageWave));
+        });
+        if (attr_err != hipSuccess)
+          return set_error(YSCV_HIP_ERR_DEVICE, "cannot reserve LDS for the activation staging: %s", hipGetErrorString(attr_err));
+      }
       hipLaunchKernelGGL((int4_skinny_kernel<SPLIT, NI, GM, SF16, HAS_ZP, P, 1>), dim3(plan.grid_x, plan.ksg),
-                         dim3(plan.waves * 64), lds, s, a);
+                         dim3(plan.waves * 64), lds + stage, s, a);
       YSCV_HIP_TRY(hipGetLastError());
       return YSCV_HIP_OK;
     }
@@ -679,6 +752,20 @@ static int32_t launch_one(const SkinnyArgs &a, const SkinnyPlan &plan, hipStream
                      dim3(plan.waves * 64), lds, s, a);
   YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
+}
+
+template <int SPLIT, int NI, int GM, bool SF16, bool HAS_ZP>
+static int32_t launch_one(const SkinnyArgs &a, const SkinnyPlan &plan, hipStream_t s) {
+  // ring depth: bounded by the VGPR budget (activations: 64 per split, ring: ~26 per slot)
+  if constexpr (SPLIT == 2 && NI == 1) {
+    // two slots fit only with a few spilled registers, whose cost a workgroup recovers over sixteen or more blocks
+    const int blocks_per_wg = (a.nt + plan.grid_x - 1) / plan.grid_x;
+    if (blocks_per_wg < 16) return launch_p<SPLIT, NI, GM, SF16, HAS_ZP, 1>(a, plan, s);
+    return launch_p<SPLIT, NI, GM, SF16, HAS_ZP, 2>(a, plan, s);
+  } else {
+    constexpr int P = SPLIT == 2 ? 1 : (SF16 && !HAS_ZP ? 4 : 3);
+    return launch_p<SPLIT, NI, GM, SF16, HAS_ZP, P>(a, plan, s);
+  }
 }
 
 template <int SPLIT, int NI, int GM>
