@@ -330,6 +330,26 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
     for (int j = 0; j < NT; j++) acc[i][j] = int4_t{0, 0, 0, 0};
   const int wm = (wave >> 1) & 1, wn = wave & 1;
 
+  // The per-column terms of the epilogue are requested before the main loop (compute waves issue no other global
+  // load, so nothing in the loop waits for them): their round trip is over long before the tile is finished.
+  int32_t zc_all[NT][4], corr_all[NT][4];
+  float comp_all[NT][4];
+  if (wave < 4) {
+    // absent tables are read from the column sums instead and ignored later: the loads stay unconditional and no
+    // instruction consumes them before the epilogue
+    const int32_t *corr_src = p.corr ? p.corr : p.col_sum;
+    const float *comp_src = p.composite_v ? p.composite_v : reinterpret_cast<const float *>(p.col_sum);
+#pragma unroll
+    for (int j = 0; j < NT; j++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const int cc = min(n0 + wn * NT * 16 + j * 16 + c * 4 + e, p.n - 1);
+        zc_all[j][e] = p.col_sum[cc];
+        corr_all[j][e] = corr_src[cc];
+        comp_all[j][e] = comp_src[cc];
+      }
+  }
+
   if (wave >= 4) {
     // ---- producer: per-lane source addresses of this wave's chunks at k = 0 (chunk q < 2 MT KS: A, else B)
     const int pw = wave - 4;
@@ -451,30 +471,6 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
   __syncthreads();  // every wave is done with the ring
   const float lo = (float)p.lo, hi = (float)p.hi;
   if (wave < 4) {
-    // the per-column terms of all NT column tiles are requested together: one memory round trip, not one per tile
-    int32_t zc_all[NT][4], corr_all[NT][4];
-    float comp_all[NT][4];
-#pragma unroll
-    for (int j = 0; j < NT; j++)
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        const int cc = min(n0 + wn * NT * 16 + j * 16 + c * 4 + e, p.n - 1);
-        zc_all[j][e] = p.col_sum[cc];
-        corr_all[j][e] = 0;
-        comp_all[j][e] = p.composite;
-      }
-    if (p.corr) {
-#pragma unroll
-      for (int j = 0; j < NT; j++)
-#pragma unroll
-        for (int e = 0; e < 4; e++) corr_all[j][e] = p.corr[min(n0 + wn * NT * 16 + j * 16 + c * 4 + e, p.n - 1)];
-    }
-    if (p.composite_v) {
-#pragma unroll
-      for (int j = 0; j < NT; j++)
-#pragma unroll
-        for (int e = 0; e < 4; e++) comp_all[j][e] = p.composite_v[min(n0 + wn * NT * 16 + j * 16 + c * 4 + e, p.n - 1)];
-    }
 #pragma unroll
     for (int j = 0; j < NT; j++) {
       const int lcol = wn * NT * 16 + j * 16 + c * 4;
@@ -483,8 +479,8 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
 #pragma unroll
       for (int e = 0; e < 4; e++) {
         zc[e] = p.zp_mul * zc_all[j][e];
-        corr[e] = corr_all[j][e];
-        comp[e] = comp_all[j][e];
+        corr[e] = p.corr ? corr_all[j][e] : 0;
+        comp[e] = p.composite_v ? comp_all[j][e] : p.composite;
       }
 #pragma unroll
       for (int i = 0; i < MT; i++) {
