@@ -697,11 +697,6 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
 
   // ---- producer waves: stream the weight records of their compute waves into the LDS rings -------------
   // A producer issues a record (3 direct global->LDS loads) whenever a ring of one of its waves has a free
-  // slot, and publishes how many records have landed from its own outstanding-load counter (loads return in
-  // order).  Compute waves never have a weight load of their own in flight, so their polls are not queued
-  // behind the stream.
-  // ---- producer waves: stream the weight records of their compute waves into the LDS rings -------------
-  // A producer issues a record (3 direct global->LDS loads) whenever a ring of one of its waves has a free
   // slot, and publishes how many records have landed, which it reads from its own outstanding-load counter
   // (loads return in order).  Compute waves never have a weight load of their own in flight, so their polls
   // are not queued behind the stream.  The LDS words shared with the compute waves are accessed with explicit
