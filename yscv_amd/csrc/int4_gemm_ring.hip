@@ -1,8 +1,8 @@
 // Wide-M packed-int4 matmul for fp16 / bf16 activations: y[m][n] = sum_k x[m][k] * W[n][k], MFMA-bound design.
 // Replaces packed_int4_gemm_dispatch (crates/yscv-kernels/src/ops/int4_matmul.rs:548-605) for prefill-sized m.
 //
-// A workgroup owns a (32 MT) x (32 NT) tile of y (MT = 1, 2 or 4 by m).  It has four MMA waves (2 x 2, MT x NT MFMA tiles each) and NP
-// producer waves.  Per stage of KS k-steps (32 k each) the producers
+// A workgroup owns a (32 MT) x (32 NT) tile of y (MT = 1, 2 or 4 by m; NT = 4, or 8 where 128 x 256 tiles still fill
+// the CUs in whole rounds).  It has four MMA waves (2 x 2, MT x NT MFMA tiles each) and NP producer waves.  Per stage of KS k-steps (32 k each) the producers
 //   * fetch the activation rows (fp16, prepared by x_prep) with LDS-direct loads, one 16-byte piece per lane: an
 //     instruction takes eight whole 128-byte lines (eight rows x both k-steps of the stage), and a per-row XOR of
 //     the chunk index makes the later fragment reads conflict-free, so the row-major -> MFMA-fragment
@@ -76,6 +76,10 @@ __device__ __forceinline__ void g4_wait(G4Frags<MT, NT> &f) {
     asm volatile("s_waitcnt lgkmcnt(0)"
                  : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]),
                    "+v"(f.b[3])::"memory");
+  } else if constexpr (MT == 4 && NT == 8) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]),
+                   "+v"(f.b[3]), "+v"(f.b[4]), "+v"(f.b[5]), "+v"(f.b[6]), "+v"(f.b[7])::"memory");
   } else if constexpr (MT == 2 && NT == 4) {
     asm volatile("s_waitcnt lgkmcnt(0)"
                  : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]), "+v"(f.b[3])::"memory");
@@ -161,6 +165,14 @@ __device__ __forceinline__ void g4_wait_tiles(G4Tile<SC_REGS> (&t)[2]) {
                : "n"(N)
                : "memory");
 }
+template <int N, int SC_REGS>
+__device__ __forceinline__ void g4_wait_tiles(G4Tile<SC_REGS> (&t)[4]) {
+  asm volatile("s_waitcnt vmcnt(%12)"
+               : "+v"(t[0].raw), "+v"(t[0].sc), "+v"(t[0].zp), "+v"(t[1].raw), "+v"(t[1].sc), "+v"(t[1].zp), "+v"(t[2].raw),
+                 "+v"(t[2].sc), "+v"(t[2].zp), "+v"(t[3].raw), "+v"(t[3].sc), "+v"(t[3].zp)
+               : "n"(N)
+               : "memory");
+}
 template <int N>
 __device__ __forceinline__ void g4_wait_vm_n() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
@@ -175,10 +187,13 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
   constexpr int APW = 2 * MT * KS / NP;  // activation chunks (1 KiB) a producer wave fetches per stage
   constexpr int WT = 2 * NT / NP;        // weight tiles (16 columns) a producer wave decodes per stage
   static_assert(KS == 2, "a stage is half a 128-k weight tile");
-  static_assert((2 * MT * KS) % NP == 0 && (2 * NT) % NP == 0 && (WT == 1 || WT == 2), "work split over the producer waves");
+  static_assert((2 * MT * KS) % NP == 0 && (2 * NT) % NP == 0 && (WT == 1 || WT == 2 || WT == 4), "work split over the producer waves");
   static_assert(SA >= 2 && SA <= 6 && SA % 2 == 0, "stage parity must follow the ring position");
   constexpr int RS = BN * 4 + 16;  // row stride of the f32 result tile in LDS (odd multiple of 16 B)
-  static_assert(BM * RS <= LDS_BYTES, "the result tile reuses the ring");
+  // the result tile reuses the ring: whole when it fits, else the rows of the upper and the lower MMA waves in turn
+  constexpr int EPI_PASSES = BM * RS <= LDS_BYTES ? 1 : 2;
+  constexpr int EPI_ROWS = BM / EPI_PASSES;
+  static_assert(EPI_ROWS * RS <= LDS_BYTES && (EPI_PASSES == 1 || EPI_ROWS == MT * 16), "the result tile reuses the ring");
   extern __shared__ __attribute__((aligned(1024))) uint8_t g4_ring[];
   const uint32_t lds0 = (uint32_t)(size_t)g4_ring;
   const int tid = threadIdx.x;
@@ -395,49 +410,55 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
   // ---- epilogue: lane (c, r) of an MMA wave holds y[16 i + r][16 j + 4 c + 0..3] of its part; through LDS so that
   // all waves store whole rows ------------------------------------------------------------------------------
   __syncthreads();
+  // all row scales are requested together (a load behind a branch of its own is waited for on its own)
+  float rs[MT];
   if (wave < 4) {
-    // all row scales are requested together (a load behind a branch of its own is waited for on its own)
-    float rs[MT];
 #pragma unroll
     for (int i = 0; i < MT; i++) {
       const int row = min(m0 + wm * MT * 16 + i * 16 + r, p.m - 1);
       const float *src = p.row_scale ? p.row_scale + row : &kOne;
       rs[i] = *src;
     }
-#pragma unroll
-    for (int i = 0; i < MT; i++) {
-      const int lrow = wm * MT * 16 + i * 16 + r;
-#pragma unroll
-      for (int j = 0; j < NT; j++) {
-        const int lcol = wn * NT * 16 + j * 16 + c * 4;
-        *reinterpret_cast<float4_t *>(g4_ring + lrow * RS + lcol * 4) = acc[i][j] * rs[i];
-      }
-    }
   }
-  __syncthreads();
   constexpr int CPR = BN / 4;  // four-column chunks per row
   const bool vec = (p.n & 3) == 0;
-  for (int q = tid; q < BM * CPR; q += THREADS) {
-    const int lrow = q / CPR, ch = q % CPR;
-    const int row = m0 + lrow, col = n0 + ch * 4;
-    if (row >= p.m || col >= p.n) continue;
-    const float4_t v = *reinterpret_cast<const float4_t *>(g4_ring + lrow * RS + ch * 16);
-    const size_t o = (size_t)row * p.n + col;
-    if (vec) {
-      if (p.y_dtype == YSCV_HIP_F32) {
-        *reinterpret_cast<float4_t *>(reinterpret_cast<float *>(p.y) + o) = v;
-      } else if (p.y_dtype == YSCV_HIP_F16) {
-        *reinterpret_cast<half4_t *>(reinterpret_cast<_Float16 *>(p.y) + o) =
-            half4_t{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-      } else {
-        uint2 b;
-        b.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
-        b.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
-        *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.y) + o) = b;
+#pragma unroll
+  for (int hp = 0; hp < EPI_PASSES; hp++) {
+    if (hp > 0) __syncthreads();  // the stores of the previous pass have read their rows
+    if (wave < 4 && (EPI_PASSES == 1 || wm == hp)) {
+#pragma unroll
+      for (int i = 0; i < MT; i++) {
+        const int lrow = wm * MT * 16 + i * 16 + r - hp * EPI_ROWS;
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+          const int lcol = wn * NT * 16 + j * 16 + c * 4;
+          *reinterpret_cast<float4_t *>(g4_ring + lrow * RS + lcol * 4) = acc[i][j] * rs[i];
+        }
       }
-    } else {
-      for (int e = 0; e < 4; e++)
-        if (col + e < p.n) store_out(p.y, o + e, v[e], p.y_dtype);
+    }
+    __syncthreads();
+    for (int q = tid; q < EPI_ROWS * CPR; q += THREADS) {
+      const int lrow = q / CPR, ch = q % CPR;
+      const int row = m0 + hp * EPI_ROWS + lrow, col = n0 + ch * 4;
+      if (row >= p.m || col >= p.n) continue;
+      const float4_t v = *reinterpret_cast<const float4_t *>(g4_ring + lrow * RS + ch * 16);
+      const size_t o = (size_t)row * p.n + col;
+      if (vec) {
+        if (p.y_dtype == YSCV_HIP_F32) {
+          *reinterpret_cast<float4_t *>(reinterpret_cast<float *>(p.y) + o) = v;
+        } else if (p.y_dtype == YSCV_HIP_F16) {
+          *reinterpret_cast<half4_t *>(reinterpret_cast<_Float16 *>(p.y) + o) =
+              half4_t{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+        } else {
+          uint2 b;
+          b.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+          b.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+          *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.y) + o) = b;
+        }
+      } else {
+        for (int e = 0; e < 4; e++)
+          if (col + e < p.n) store_out(p.y, o + e, v[e], p.y_dtype);
+      }
     }
   }
 }
@@ -508,6 +529,16 @@ int32_t launch_int4_gemm_ring(const yscv_hip_int4_weight *w, const _Float16 *xh,
   // 32- or 64-row tile.
   if (m <= 32) return ring_launch_gm<1, 4, 2, 6, 4>(a, w->gm, sf16, s);
   if (m <= 64) return ring_launch_gm<2, 4, 2, 6, 8>(a, w->gm, sf16, s);
+  // 128 x 256 tiles (two 64 x 128 parts per MMA wave: a third fewer fragment reads per MFMA) take about 1.72 times
+  // as long as 128 x 128 ones; they pay when the tiles come in rounds over the CUs and the wide ones need at most
+  // half as many rounds.
+  const Context *ctx = nullptr;
+  YSCV_TRY(ensure_context(&ctx));
+  const size_t cus = (size_t)(ctx->num_cus > 0 ? ctx->num_cus : 256);
+  const size_t tiles_m = ceil_div(m, (size_t)128);
+  const size_t rounds_sq = ceil_div(tiles_m * ceil_div((size_t)w->n, (size_t)128), cus);
+  const size_t rounds_wide = ceil_div(tiles_m * ceil_div((size_t)w->n, (size_t)256), cus);
+  if (rounds_wide * 172 < rounds_sq * 100) return ring_launch_gm<4, 8, 2, 4, 4>(a, w->gm, sf16, s);
   return ring_launch_gm<4, 4, 2, 6, 8>(a, w->gm, sf16, s);
 }
 
