@@ -1,8 +1,8 @@
 // Wide-M packed-int4 matmul for fp16 / bf16 activations: y[m][n] = sum_k x[m][k] * W[n][k], MFMA-bound design.
 // Replaces packed_int4_gemm_dispatch (crates/yscv-kernels/src/ops/int4_matmul.rs:548-605) for prefill-sized m.
 //
-// A workgroup owns a (32 MT) x (32 NT) tile of y (MT = 1, 2 or 4 by m; NT = 4, or 8 where 128 x 256 tiles still fill
-// the CUs in whole rounds).  It has four MMA waves (2 x 2, MT x NT MFMA tiles each) and NP producer waves.  Per stage of KS k-steps (32 k each) the producers
+// A workgroup owns a (32 MT) x (32 NT) tile of y: 32, 64 or 128 rows by 128 columns by m, or 128 x 256 / 256 x 128
+// where such tiles still fill the CUs in whole rounds.  It has four MMA waves (2 x 2, MT x NT MFMA tiles each) and NP producer waves.  Per stage of KS k-steps (32 k each) the producers
 //   * fetch the activation rows (fp16, prepared by x_prep) with LDS-direct loads, one 16-byte piece per lane: an
 //     instruction takes eight whole 128-byte lines (eight rows x both k-steps of the stage), and a per-row XOR of
 //     the chunk index makes the later fragment reads conflict-free, so the row-major -> MFMA-fragment
@@ -80,6 +80,10 @@ __device__ __forceinline__ void g4_wait(G4Frags<MT, NT> &f) {
     asm volatile("s_waitcnt lgkmcnt(0)"
                  : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]),
                    "+v"(f.b[3]), "+v"(f.b[4]), "+v"(f.b[5]), "+v"(f.b[6]), "+v"(f.b[7])::"memory");
+  } else if constexpr (MT == 8 && NT == 4) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.a[4]), "+v"(f.a[5]), "+v"(f.a[6]),
+                   "+v"(f.a[7]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]), "+v"(f.b[3])::"memory");
   } else if constexpr (MT == 2 && NT == 4) {
     asm volatile("s_waitcnt lgkmcnt(0)"
                  : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]), "+v"(f.b[3])::"memory");
@@ -529,16 +533,19 @@ int32_t launch_int4_gemm_ring(const yscv_hip_int4_weight *w, const _Float16 *xh,
   // 32- or 64-row tile.
   if (m <= 32) return ring_launch_gm<1, 4, 2, 6, 4>(a, w->gm, sf16, s);
   if (m <= 64) return ring_launch_gm<2, 4, 2, 6, 8>(a, w->gm, sf16, s);
-  // 128 x 256 tiles (two 64 x 128 parts per MMA wave: a third fewer fragment reads per MFMA) take about 1.72 times
-  // as long as 128 x 128 ones; they pay when the tiles come in rounds over the CUs and the wide ones need at most
-  // half as many rounds.
+  // Larger tiles: 128 x 256 (a third fewer fragment reads per MFMA) and 256 x 128 (the same, and every decoded
+  // weight feeds twice as many MFMAs, so the producers' decode instructions take half as many issue slots from the
+  // MFMAs of their SIMD).  A workgroup needs about 1.72 / 1.63 times as long for them as for a 128 x 128 tile; they
+  // pay when the tiles come in rounds over the CUs and the larger ones need sufficiently fewer rounds.
   const Context *ctx = nullptr;
   YSCV_TRY(ensure_context(&ctx));
   const size_t cus = (size_t)(ctx->num_cus > 0 ? ctx->num_cus : 256);
-  const size_t tiles_m = ceil_div(m, (size_t)128);
-  const size_t rounds_sq = ceil_div(tiles_m * ceil_div((size_t)w->n, (size_t)128), cus);
-  const size_t rounds_wide = ceil_div(tiles_m * ceil_div((size_t)w->n, (size_t)256), cus);
-  if (rounds_wide * 172 < rounds_sq * 100) return ring_launch_gm<4, 8, 2, 4, 4>(a, w->gm, sf16, s);
+  const size_t tn128 = ceil_div((size_t)w->n, (size_t)128), tn256 = ceil_div((size_t)w->n, (size_t)256);
+  const size_t cost_sq = ceil_div(ceil_div(m, (size_t)128) * tn128, cus) * 100;
+  const size_t cost_wide = ceil_div(ceil_div(m, (size_t)128) * tn256, cus) * 172;
+  const size_t cost_tall = m > 128 ? ceil_div(ceil_div(m, (size_t)256) * tn128, cus) * 163 : (size_t)-1;
+  if (cost_tall < cost_sq && cost_tall <= cost_wide) return ring_launch_gm<8, 4, 2, 4, 4>(a, w->gm, sf16, s);
+  if (cost_wide < cost_sq) return ring_launch_gm<4, 8, 2, 4, 4>(a, w->gm, sf16, s);
   return ring_launch_gm<4, 4, 2, 6, 8>(a, w->gm, sf16, s);
 }
 
