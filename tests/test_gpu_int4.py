@@ -256,7 +256,9 @@ def test_invalid_arguments_are_rejected(K, torch_cuda):
                                                (128, 128, 512, 32, False, False), (130, 200, 1024, 128, True, True),
                                                (257, 1000, 640, 64, True, True), (512, 136, 2048, 32, True, False),
                                                (300, 264, 768, 256, False, True), (1100, 520, 1152, 128, False, False),
-                                               (200, 24011, 256, 32, True, True), (250, 16499, 256, 64, True, True)])  # the last two: 128 x 256 and 256 x 128 tiles
+                                               (200, 24011, 256, 32, True, True), (250, 16499, 256, 64, True, True),
+                                               (250, 40997, 128, 32, True, False)])  # the last three: 128 x 256 tiles, 256 x 128 tiles, and one round of
+                                                                                      # 256 x 128 tiles followed by a second launch with 128 x 128 tiles
 @pytest.mark.parametrize("xdt", ["bf16", "f16", "f32"])
 def test_wide_m_ring_kernel(oracle, K, torch_cuda, m, n, k, g, sf16, zp, xdt):
     """m > 16: the LDS-ring GEMM (weights decoded to fp16 with the scale folded in) for 16-bit activations and, when

@@ -41,7 +41,8 @@ struct RingArgs {
   const _Float16 *xh;
   const float *row_scale;
   void *y;
-  int m, n;
+  int m, n;        // rows; end of the column range of this launch
+  int col0, ldy;   // first column of this launch (a multiple of the tile width); row stride of y
   int nt, kt, ktp;
   int chunks, chunk_div;
   int k_pad;
@@ -213,7 +214,7 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
   const int sb = (j_in_xcd >> 5) * 8 + (int)(blockIdx.x & 7);
   const int tm = (sb % sb_m) * sbm + (j_in_xcd & (sbm - 1)), tn = (sb / sb_m) * sbn + ((j_in_xcd & 31) >> sbm_log2);
   if (tm >= tiles_m || tn >= tiles_n) return;
-  const int m0 = tm * BM, n0 = tn * BN;
+  const int m0 = tm * BM, n0 = p.col0 + tn * BN;
   const int nstages = p.kt * (4 / KS);
 
   float4_t acc[MT][NT];  // MMA waves only; the producers never touch it
@@ -229,6 +230,8 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
     static_assert((SA / 2) * PE + (SA / 2) * PO + APW < 64, "vmcnt budget");
     const int pw = wave - 4;
     const bool has_zp = p.tzps != nullptr;
+    NibbleConsts nc;  // one v_and_or_b32 per pair of nibbles: the decode shares the SIMD's issue port with the MFMAs
+    nc.init();
     // per-lane byte offsets (fixed) and uniform base pointers (advanced per stage)
     uint32_t aoff[APW];
 #pragma unroll
@@ -270,9 +273,14 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
       }
       const char *abase = reinterpret_cast<const char *>(p.xh) + (size_t)st * KS * 32 * sizeof(_Float16);
 #pragma unroll
-      for (int j = 0; j < APW; j++)
-        __builtin_amdgcn_global_load_lds(G4_AS1(abase + aoff[j]),
-                                         (lds_void *)(uintptr_t)(lds0 + (uint32_t)(ri * A_BYTES + (pw * APW + j) * 1024)), 16, 0, 0);
+      for (int j = 0; j < APW; j++) {
+        // uniform base + per-lane 32-bit offset, written out: left to the compiler, the loads inside the loop take
+        // 64-bit per-lane addresses, one more vector instruction each next to the MFMAs
+        const uint32_t dst = lds0 + (uint32_t)(ri * A_BYTES + (pw * APW + j) * 1024);
+        const uint32_t off = aoff[j];
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(abase)
+                     : "memory");  // m0: reserved, never allocated by the compiler; nothing else in this kernel reads it
+      }
     };
     // decode the weights of a stage (register set ri, parity par) into weight slot par
     auto decode_stage = [&](auto ric, auto parc) {
@@ -310,7 +318,7 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
         }
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
-          const half8_t h = decode8(wr[ri / 2][u].raw[par * KS + ks], c1[ks], c2[ks]) * sv[ks];
+          const half8_t h = decode8_exact(wr[ri / 2][u].raw[par * KS + ks], nc, c1[ks], c2[ks]) * sv[ks];
           // written with an opaque instruction: a compiler-visible LDS store would first wait for every LDS-direct
           // load in flight
           asm volatile("ds_write_b128 %0, %1" ::"v"(dst + (uint32_t)((u * KS + ks) * 1024)), "v"(h) : "memory");
@@ -425,7 +433,7 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
     }
   }
   constexpr int CPR = BN / 4;  // four-column chunks per row
-  const bool vec = (p.n & 3) == 0;
+  const bool vec = ((p.n | p.ldy) & 3) == 0;
 #pragma unroll
   for (int hp = 0; hp < EPI_PASSES; hp++) {
     if (hp > 0) __syncthreads();  // the stores of the previous pass have read their rows
@@ -446,7 +454,7 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
       const int row = m0 + hp * EPI_ROWS + lrow, col = n0 + ch * 4;
       if (row >= p.m || col >= p.n) continue;
       const float4_t v = *reinterpret_cast<const float4_t *>(g4_ring + lrow * RS + ch * 16);
-      const size_t o = (size_t)row * p.n + col;
+      const size_t o = (size_t)row * p.ldy + col;
       if (vec) {
         if (p.y_dtype == YSCV_HIP_F32) {
           *reinterpret_cast<float4_t *>(reinterpret_cast<float *>(p.y) + o) = v;
@@ -478,7 +486,7 @@ int32_t ring_launch_one(const RingArgs &a, hipStream_t s) {
   });
   if (attr_err != hipSuccess)
     return set_error(YSCV_HIP_ERR_DEVICE, "cannot reserve %d bytes of LDS: %s", LDS, hipGetErrorString(attr_err));
-  const int tiles_m = (int)ceil_div((size_t)a.m, (size_t)(32 * MT)), tiles_n = (int)ceil_div((size_t)a.n, (size_t)(32 * NT));
+  const int tiles_m = (int)ceil_div((size_t)a.m, (size_t)(32 * MT)), tiles_n = (int)ceil_div((size_t)(a.n - a.col0), (size_t)(32 * NT));
   int sbm_log2 = 3;
   while (sbm_log2 > 0 && (1 << sbm_log2) > tiles_m) sbm_log2--;
   const int sbm = 1 << sbm_log2, sbn = 32 >> sbm_log2;
@@ -520,6 +528,8 @@ int32_t launch_int4_gemm_ring(const yscv_hip_int4_weight *w, const _Float16 *xh,
   a.y = y;
   a.m = (int)m;
   a.n = (int)w->n;
+  a.col0 = 0;
+  a.ldy = (int)w->n;
   a.nt = (int)w->nt;
   a.kt = (int)w->kt;
   a.ktp = (int)w->ktp;
@@ -534,19 +544,63 @@ int32_t launch_int4_gemm_ring(const yscv_hip_int4_weight *w, const _Float16 *xh,
   if (m <= 32) return ring_launch_gm<1, 4, 2, 6, 4>(a, w->gm, sf16, s);
   if (m <= 64) return ring_launch_gm<2, 4, 2, 6, 8>(a, w->gm, sf16, s);
   // Larger tiles: 128 x 256 (a third fewer fragment reads per MFMA) and 256 x 128 (the same, and every decoded
-  // weight feeds twice as many MFMAs, so the producers' decode instructions take half as many issue slots from the
-  // MFMAs of their SIMD).  A workgroup needs about 1.72 / 1.63 times as long for them as for a 128 x 128 tile; they
-  // pay when the tiles come in rounds over the CUs and the larger ones need sufficiently fewer rounds.
+  // weight feeds twice as many MFMAs).  A workgroup needs about 1.72 / 1.63 times as long for them as for a
+  // 128 x 128 tile; they pay when the tiles come in rounds over the CUs and the larger ones need sufficiently fewer
+  // rounds.  When the last round of the best shape would leave most CUs idle, the columns of its whole rounds go to
+  // one launch and the rest to a second one with the shape that suits the rest (config 3: three rounds of
+  // 256 x 128 tiles, then one round of 128 x 128 tiles, instead of three and a half rounds).
   const Context *ctx = nullptr;
   YSCV_TRY(ensure_context(&ctx));
   const size_t cus = (size_t)(ctx->num_cus > 0 ? ctx->num_cus : 256);
-  const size_t tn128 = ceil_div((size_t)w->n, (size_t)128), tn256 = ceil_div((size_t)w->n, (size_t)256);
-  const size_t cost_sq = ceil_div(ceil_div(m, (size_t)128) * tn128, cus) * 100;
-  const size_t cost_wide = ceil_div(ceil_div(m, (size_t)128) * tn256, cus) * 172;
-  const size_t cost_tall = m > 128 ? ceil_div(ceil_div(m, (size_t)256) * tn128, cus) * 163 : (size_t)-1;
-  if (cost_tall < cost_sq && cost_tall <= cost_wide) return ring_launch_gm<8, 4, 2, 4, 4>(a, w->gm, sf16, s);
-  if (cost_wide < cost_sq) return ring_launch_gm<4, 8, 2, 4, 4>(a, w->gm, sf16, s);
-  return ring_launch_gm<4, 4, 2, 6, 8>(a, w->gm, sf16, s);
+  struct Shape {
+    size_t bm, bn, cost;
+  };
+  const Shape shapes[3] = {{128, 128, 100}, {128, 256, 172}, {256, 128, 163}};
+  auto launch_shape = [&](int which, RingArgs r) {
+    if (which == 2) return ring_launch_gm<8, 4, 2, 4, 4>(r, w->gm, sf16, s);
+    if (which == 1) return ring_launch_gm<4, 8, 2, 4, 4>(r, w->gm, sf16, s);
+    return ring_launch_gm<4, 4, 2, 6, 8>(r, w->gm, sf16, s);
+  };
+  // best single shape for columns [c0, n): cost in hundredths of a 128 x 128 tile time
+  auto best_single = [&](size_t c0, int *which) {
+    size_t best = (size_t)-1;
+    for (int i = 0; i < 3; i++) {
+      if (i == 2 && m <= 128) continue;
+      const size_t tiles = ceil_div(m, shapes[i].bm) * ceil_div((size_t)w->n - c0, shapes[i].bn);
+      const size_t cost = ceil_div(tiles, cus) * shapes[i].cost;
+      if (cost < best) {
+        best = cost;
+        *which = i;
+      }
+    }
+    return best;
+  };
+  int one = 0;
+  size_t best = best_single(0, &one);
+  int first = -1, second = 0;
+  size_t split_col = 0;
+  const size_t launch_cost = 10;  // a second launch: about a tenth of a tile time
+  for (int i = 0; i < 3; i++) {
+    if (i == 2 && m <= 128) continue;
+    const size_t tm = ceil_div(m, shapes[i].bm), tn = ceil_div((size_t)w->n, shapes[i].bn);
+    const size_t rounds = tm * tn / cus;                // whole rounds
+    const size_t cols = rounds * cus / tm;              // whole tile columns inside them
+    if (rounds == 0 || cols == 0 || cols >= tn) continue;
+    int rest = 0;
+    const size_t cost = ceil_div(tm * cols, cus) * shapes[i].cost + best_single(cols * shapes[i].bn, &rest) + launch_cost;
+    if (cost < best) {
+      best = cost;
+      first = i;
+      second = rest;
+      split_col = cols * shapes[i].bn;
+    }
+  }
+  if (first < 0) return launch_shape(one, a);
+  RingArgs a1 = a, a2 = a;
+  a1.n = (int)split_col;
+  a2.col0 = (int)split_col;
+  YSCV_TRY(launch_shape(first, a1));
+  return launch_shape(second, a2);
 }
 
 }  // namespace yscv

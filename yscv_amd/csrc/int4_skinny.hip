@@ -92,64 +92,6 @@ struct TileRegs {
   uint32_t z[HAS_ZP ? TPW : 1];
 };
 
-// Constants of the nibble -> fp16 decode, held in registers whose contents the compiler cannot see.  Given literal
-// constants it emits v_and_b32 + v_or_b32 per pair of nibbles (a VOP3 encoding cannot hold a literal); with a mask in
-// an SGPR and the magic in a VGPR it selects one v_and_or_b32.  The empty asm statements emit no instruction, so
-// every real instruction stays visible to the compiler's MFMA hazard handling.
-struct NibbleConsts {
-  uint32_t lo, hi, magic;  // 0x000F000F, 0x00F000F0, 0x64006400
-  __device__ __forceinline__ void init() {
-    lo = 0x000F000Fu;
-    hi = 0x00F000F0u;
-    magic = 0x64006400u;
-    asm volatile("" : "+s"(lo), "+s"(hi), "+v"(magic));
-  }
-};
-
-// raw fp16 forms of the 8 weights of one word: {1024+q0, 1024+q1, 1024+16 q2, 1024+16 q3, ...}
-__device__ __forceinline__ half8_t extract8(uint32_t s, const NibbleConsts &nc) {
-  U32H2 r0, r1, r2, r3;
-  const uint32_t s2 = s >> 8;
-  r0.u = (s & nc.lo) | nc.magic;
-  r1.u = (s & nc.hi) | nc.magic;
-  r2.u = (s2 & nc.lo) | nc.magic;
-  r3.u = (s2 & nc.hi) | nc.magic;
-  half8_t out;
-  out[0] = r0.h[0];
-  out[1] = r0.h[1];
-  out[2] = r1.h[0];
-  out[3] = r1.h[1];
-  out[4] = r2.h[0];
-  out[5] = r2.h[1];
-  out[6] = r3.h[0];
-  out[7] = r3.h[1];
-  return out;
-}
-
-// exact (q - zp) in fp16: c1 = -(1024 + zp), c2 = -(64 + zp)
-__device__ __forceinline__ half8_t decode8_exact(uint32_t s, const NibbleConsts &nc, half2_t c1, half2_t c2) {
-  U32H2 r0, r1, r2, r3;
-  const uint32_t s2 = s >> 8;
-  r0.u = (s & nc.lo) | nc.magic;
-  r1.u = (s & nc.hi) | nc.magic;
-  r2.u = (s2 & nc.lo) | nc.magic;
-  r3.u = (s2 & nc.hi) | nc.magic;
-  const half2_t sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
-  const half2_t h0 = r0.h + c1;
-  const half2_t h1 = r1.h * sixteenth + c2;
-  const half2_t h2 = r2.h + c1;
-  const half2_t h3 = r3.h * sixteenth + c2;
-  half8_t out;
-  out[0] = h0[0];
-  out[1] = h0[1];
-  out[2] = h1[0];
-  out[3] = h1[1];
-  out[4] = h2[0];
-  out[5] = h2[1];
-  out[6] = h3[0];
-  out[7] = h3[1];
-  return out;
-}
 
 __device__ __forceinline__ void zp_consts(uint32_t zp, half2_t &c1, half2_t &c2) {
   const _Float16 z = (_Float16)(float)zp;
