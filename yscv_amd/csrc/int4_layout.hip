@@ -233,10 +233,77 @@ __global__ void __launch_bounds__(1024) x_prep_kernel(const void *__restrict__ x
   }
 }
 
+// Rows of at most 4096 padded elements, aligned: one wavefront per row, eight 8-element chunks per lane held in
+// registers from the abs-max sweep to the conversion; no LDS, no barrier, and every load is unconditional (lanes
+// past the end of the row re-read its last chunk and drop it), so a row costs one memory round trip.
+template <int DT>
+__global__ void __launch_bounds__(256) x_prep_wave_kernel(const void *__restrict__ x, size_t m, size_t k, size_t k_pad,
+                                                          int split, _Float16 *__restrict__ xh,
+                                                          _Float16 *__restrict__ xl, float *__restrict__ row_scale) {
+  const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= m) return;
+  const int lane = threadIdx.x & 63;
+  const size_t base = row * k;
+  const int chunks = (int)(k_pad / 8), data_chunks = (int)(k / 8);  // k % 8 == 0 on this path
+  float v[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int ch = lane + 64 * i;
+    load8<true>(x, base + (size_t)min(ch, data_chunks - 1) * 8, DT, base + k, v[i]);
+  }
+  float amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const bool have = lane + 64 * i < data_chunks;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      v[i][e] = have ? v[i][e] : 0.0f;
+      amax = fmaxf(amax, fabsf(v[i][e]));  // NaN is ignored here, kept in the values
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+  int e2 = 14;
+  if (amax > 0.0f && amax < 3.0e38f) {
+    (void)frexpf(amax, &e2);
+    e2 -= 1;
+  }
+  int shift = 14 - e2;
+  shift = shift > 100 ? 100 : (shift < -100 ? -100 : shift);
+  const float up = ldexpf(1.0f, shift);
+  if (lane == 0) row_scale[row] = ldexpf(1.0f, -shift);
+  const size_t obase = row * k_pad;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int ch = lane + 64 * i;
+    if (ch < chunks) {
+      half8_t h, l;
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const float sv = v[i][e] * up;
+        h[e] = (_Float16)sv;
+        l[e] = (_Float16)(sv - (float)h[e]);
+      }
+      *reinterpret_cast<half8_t *>(xh + obase + (size_t)ch * 8) = h;
+      if (split == 2) *reinterpret_cast<half8_t *>(xl + obase + (size_t)ch * 8) = l;
+    }
+  }
+}
+
 int32_t launch_x_prep(const void *x, int x_dtype, size_t m, size_t k, size_t k_pad, int split,
                       _Float16 *xh, _Float16 *xl, float *row_scale, hipStream_t s) {
   const size_t esz = x_dtype == YSCV_HIP_F32 ? 4 : 2;
   const bool vec = (k % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) && ((k * esz) % 16 == 0);
+  if (vec && k >= 8 && k_pad <= 4096) {
+    const dim3 grid((unsigned)ceil_div(m, (size_t)4));
+    if (x_dtype == YSCV_HIP_F32)
+      hipLaunchKernelGGL(x_prep_wave_kernel<YSCV_HIP_F32>, grid, dim3(256), 0, s, x, m, k, k_pad, split, xh, xl, row_scale);
+    else if (x_dtype == YSCV_HIP_F16)
+      hipLaunchKernelGGL(x_prep_wave_kernel<YSCV_HIP_F16>, grid, dim3(256), 0, s, x, m, k, k_pad, split, xh, xl, row_scale);
+    else
+      hipLaunchKernelGGL(x_prep_wave_kernel<YSCV_HIP_BF16>, grid, dim3(256), 0, s, x, m, k, k_pad, split, xh, xl, row_scale);
+    YSCV_HIP_TRY(hipGetLastError());
+    return YSCV_HIP_OK;
+  }
   size_t chunks = k_pad / 8;
   unsigned threads = chunks >= 1024 ? 1024 : (unsigned)round_up(chunks < 64 ? 64 : chunks, 64);
   if (vec)
