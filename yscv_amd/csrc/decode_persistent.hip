@@ -586,10 +586,12 @@ __device__ GEMV_INL GemvState gemv_stage(GemvArgs a, GemvState st) {
 
   // ---- one record: 8 rows x 512 k against fragment xa ------------------------------------------------------
   unsigned crec = st.crec;
+  unsigned landed_seen = st.crec;  // the producer's count as last read: while it is ahead, no record waits for a poll
   auto consume = [&](bool single, const half8_t &xf, const float4_t &zf, float &acc) {
-    {
+    if ((int)(landed_seen - (crec + 1)) < 0) {
       unsigned spins = 0;
-      while ((int)(__hip_atomic_load(sync + wave, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) - (crec + 1)) < 0) {
+      while ((int)((landed_seen = __hip_atomic_load(sync + wave, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) -
+                   (crec + 1)) < 0) {
         __builtin_amdgcn_s_sleep(0);
         if (++spins > 40000000u) {  // the stream stalled: never expected, but no wait here is unbounded
           __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
