@@ -721,13 +721,13 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
     const unsigned total = per_step * (unsigned)n_steps;  // records per compute wave in this launch
     const unsigned char *base[SERVED], *ptr[SERVED];
     int kind[SERVED], layer[SERVED], blk[SERVED], pair[SERVED];
-    unsigned issued[SERVED], landed_cnt[SERVED];
+    unsigned issued[SERVED], landed_cnt[SERVED], consumed_seen[SERVED];
 #pragma unroll
     for (int j = 0; j < SERVED; j++) {
       const int w = p * SERVED + j;
       base[j] = ptr[j] = m.stream + m.wg_off[wg] + (size_t)w * m.wave_bytes[wg];
       kind[j] = layer[j] = blk[j] = pair[j] = 0;
-      issued[j] = landed_cnt[j] = 0;
+      issued[j] = landed_cnt[j] = consumed_seen[j] = 0;
     }
     unsigned long long fifo = 0;  // bit (i & 63): which served wave the i-th issued record belongs to
     unsigned n_issued = 0, n_retired = 0;
@@ -740,8 +740,10 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
 #pragma unroll
         for (int j = 0; j < SERVED; j++) {
           const int w = p * SERVED + j;
-          if (issued[j] < total && n_issued - n_retired < INFLIGHT_CAP &&
-              issued[j] - lds_peek(sync_lds + 4 * (8 + w)) < RING) {
+          // the consumer's count is read again only when the last value read leaves no free slot
+          if (issued[j] < total && n_issued - n_retired < INFLIGHT_CAP && issued[j] - consumed_seen[j] >= RING)
+            consumed_seen[j] = lds_peek(sync_lds + 4 * (8 + w));
+          if (issued[j] < total && n_issued - n_retired < INFLIGHT_CAP && issued[j] - consumed_seen[j] < RING) {
             while (kv(nb_k, kind[j]) == 0) {  // kinds this workgroup has no rows of
               if (kind[j] == PK_DOWN) { layer[j]++; kind[j] = layer[j] == L ? PK_LM : PK_QKV; }
               else if (kind[j] == PK_LM) { layer[j] = 0; kind[j] = PK_QKV; ptr[j] = base[j]; }
