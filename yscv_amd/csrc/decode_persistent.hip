@@ -41,6 +41,12 @@ typedef unsigned long long u64;
 #ifndef YSCV_PERSIST_TRACE
 #define YSCV_PERSIST_TRACE 0
 #endif
+// records a producer may issue per served wave between two looks at its outstanding-load counter (measured:
+// 1 -> 584, 2 -> 589, 3 -> 594, 5 -> 583, 8 -> 569 tokens/s: more amortises the bookkeeping, too many delay the
+// publication of landed records)
+#ifndef ISSUE_PER_ITER
+#define ISSUE_PER_ITER 3
+#endif
 #ifndef INFLIGHT_CAP
 #define INFLIGHT_CAP 20
 #endif
@@ -738,7 +744,8 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
       while (n_retired < total * SERVED) {
         bool did = false;
 #pragma unroll
-        for (int j = 0; j < SERVED; j++) {
+        for (int jj = 0; jj < SERVED * ISSUE_PER_ITER; jj++) {
+          const int j = jj % SERVED;
           const int w = p * SERVED + j;
           // the consumer's count is read again only when the last value read leaves no free slot
           if (issued[j] < total && n_issued - n_retired < INFLIGHT_CAP && issued[j] - consumed_seen[j] >= RING)
