@@ -596,7 +596,8 @@ __device__ GEMV_INL GemvState gemv_stage(GemvArgs a, GemvState st) {
   auto consume = [&](bool single, const half8_t &xf, const float4_t &zf, float &acc) {
     if ((int)(landed_seen - (crec + 1)) < 0) {
       unsigned spins = 0;
-      while ((int)((landed_seen = __hip_atomic_load(sync + wave, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) -
+      while ((int)((landed_seen = __builtin_amdgcn_readfirstlane(
+                        __hip_atomic_load(sync + wave, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP))) -
                    (crec + 1)) < 0) {
         __builtin_amdgcn_s_sleep(0);
         if (++spins > 40000000u) {  // the stream stalled: never expected, but no wait here is unbounded
@@ -749,7 +750,7 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
           const int w = p * SERVED + j;
           // the consumer's count is read again only when the last value read leaves no free slot
           if (issued[j] < total && n_issued - n_retired < INFLIGHT_CAP && issued[j] - consumed_seen[j] >= RING)
-            consumed_seen[j] = lds_peek(sync_lds + 4 * (8 + w));
+            consumed_seen[j] = __builtin_amdgcn_readfirstlane(lds_peek(sync_lds + 4 * (8 + w)));  // uniform: keeps the state machine scalar
           if (issued[j] < total && n_issued - n_retired < INFLIGHT_CAP && issued[j] - consumed_seen[j] < RING) {
             while (kv(nb_k, kind[j]) == 0) {  // kinds this workgroup has no rows of
               if (kind[j] == PK_DOWN) { layer[j]++; kind[j] = layer[j] == L ? PK_LM : PK_QKV; }
