@@ -41,11 +41,11 @@ typedef unsigned long long u64;
 #ifndef YSCV_PERSIST_TRACE
 #define YSCV_PERSIST_TRACE 0
 #endif
-// records a producer may issue per served wave between two looks at its outstanding-load counter (measured:
-// 1 -> 584, 2 -> 589, 3 -> 594, 5 -> 583, 8 -> 569 tokens/s: more amortises the bookkeeping, too many delay the
-// publication of landed records)
+// records a producer may issue per served wave between two looks at its outstanding-load counter (measured with the
+// scalar state machine: 1 -> 626, 2 -> 638, 3 -> 643, 4 -> 645, 5 -> 647, 7 -> 647, 10 -> 637 tokens/s: more amortises
+// the bookkeeping, too many delay the publication of landed records)
 #ifndef ISSUE_PER_ITER
-#define ISSUE_PER_ITER 3
+#define ISSUE_PER_ITER 5
 #endif
 #ifndef INFLIGHT_CAP
 #define INFLIGHT_CAP 20
