@@ -146,11 +146,50 @@ __device__ __forceinline__ int xidx(int i, int ks, int frags) {
   const int r = k2 >> 5, c = (k2 >> 3) & 3, q = (k2 & 7) >> 1;
   return ((v * frags + f) << 8) + ((q >> 1) << 7) + 2 * (16 * c + r) + (q & 1);
 }
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+// Cross-lane moves without LDS: __shfl_* compiles to ds_bpermute_b32, about a hundred cycles each when one depends
+// on the other, and a layer has some ninety of them on its critical path.  Within a row of 16 lanes DPP does the
+// same in one vector instruction; v_permlane16_swap / v_permlane32_swap exchange rows and halves of the wave.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
+}
+constexpr int DPP_XOR1 = 0xB1, DPP_XOR2 = 0x4E;         // quad_perm [1,0,3,2], [2,3,0,1]
+constexpr int DPP_NEXT1 = 0xF5, DPP_NEXT2 = 0xEE;       // quad_perm [1,1,3,3], [2,3,2,3]: lane + 1 / lane + 2 inside a quad
+constexpr int DPP_ROR4 = 0x124, DPP_ROR8 = 0x128;       // row_ror:4, row_ror:8 (= lane ^ 8 inside a row)
+constexpr int DPP_HALF_MIRROR = 0x141;                  // lane -> 7 - lane inside each group of 8
+typedef uint32_t swap_pair_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void xor16_pair(float v, float &x, float &y) {  // {x, y} = {v[lane & ~16], v[lane | 16]}
+  const swap_pair_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  x = __uint_as_float(r[0]);
+  y = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ void xor32_pair(float v, float &x, float &y) {  // {x, y} = {v[lane & ~32], v[lane | 32]}
+  const swap_pair_t r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  x = __uint_as_float(r[0]);
+  y = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float sum_xor16_xor32(float v) {  // v + v[lane ^ 16], then the same over lane ^ 32
+  float x, y;
+  xor16_pair(v, x, y);
+  v = x + y;
+  xor32_pair(v, x, y);
+  return x + y;
+}
+__device__ __forceinline__ float row_sum16(float v) {  // sum over the 16 lanes of a row, in every lane
+  v += dpp_move<DPP_XOR1>(v);
+  v += dpp_move<DPP_XOR2>(v);
+  v += dpp_move<DPP_ROR4>(v);
+  v += dpp_move<DPP_ROR8>(v);
   return v;
 }
+__device__ __forceinline__ float row_max16(float v) {
+  v = fmaxf(v, dpp_move<DPP_XOR1>(v));
+  v = fmaxf(v, dpp_move<DPP_XOR2>(v));
+  v = fmaxf(v, dpp_move<DPP_HALF_MIRROR>(v));
+  v = fmaxf(v, dpp_move<DPP_ROR8>(v));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) { return sum_xor16_xor32(row_sum16(v)); }
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + __expf(-g)); }
 // order of the greedy pick: higher value wins, equal (or unordered) values -> larger index
 __device__ __forceinline__ bool better(float va, int ia, float vb, int ib) {
@@ -306,13 +345,11 @@ __device__ ATTN_INL WaitState attn_items(AttnArgs a, WaitState ws) {
         sc2[pbk] = (p < pos) ? d[0] * scale : -INFINITY;
       }
       float mx = fmaxf(sc2[0], sc2[1]);
-#pragma unroll
-      for (int off = 8; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+      mx = row_max16(mx);
       const float e0 = (sc2[0] == -INFINITY) ? 0.0f : __expf(sc2[0] - mx);
       const float e1 = (sc2[1] == -INFINITY) ? 0.0f : __expf(sc2[1] - mx);
       float sum = e0 + e1;
-#pragma unroll
-      for (int off = 8; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+      sum = row_sum16(sum);
       m_h = mx;
       l_h = sum;
       lds_f16 *pw = p_lds + (size_t)wave * 4 * 32;
@@ -666,9 +703,8 @@ __device__ GEMV_INL GemvState gemv_stage(GemvArgs a, GemvState st) {
     for (int p = 0; p < MAXF; p++)
       if (p < a.pairs) consume(a.odd && p == a.pairs - 1, xa[p], z[p], acc);
     acc = useful ? acc : 0.0f;
-    acc += __shfl_xor(acc, 8, 64);
-    acc += __shfl_xor(acc, 16, 64);
-    acc += __shfl_xor(acc, 32, 64);
+    acc += dpp_move<DPP_ROR8>(acc);
+    acc = sum_xor16_xor32(acc);
     if (lane < 8) dst[blk * 8 + lane] = acc;
   }
   if (YSCV_PERSIST_TRACE && a.dbg_t && threadIdx.x == 0) a.dbg_t[1] = wall_clock64();
@@ -854,13 +890,13 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
     if (tid < 64) {
       const float xs = own ? h * gamma : 0.0f;
       float mx = fabsf(xs);
-      mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
+      mx = fmaxf(mx, dpp_move<DPP_XOR1>(mx));
+      mx = fmaxf(mx, dpp_move<DPP_XOR2>(mx));
+      mx = fmaxf(mx, dpp_move<DPP_HALF_MIRROR>(mx));
       int e = (mx > 0.0f && mx < INFINITY) ? ilogbf(mx) + 1 : 0;
       e = e < -100 ? -100 : (e > 100 ? 100 : e);
       const float sc = ldexpf(xs, -e);
-      const float nxt = __shfl_down(sc, 1, 64);
+      const float nxt = dpp_move<DPP_NEXT1>(sc);  // used by even lanes only
       if (own && !(tid & 1))
         st_entry(buf + xidx(own_row, m.ph[PK_QKV].ks, m.ph[PK_QKV].frags), pack_h2(sc, nxt), tag | ((uint32_t)(e + 128) << 24));
       const float ss = wave_sum(own ? h * h : 0.0f);
@@ -902,13 +938,13 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
         }
         gemv(PK_QKV, m.xn, tag, true, 1);
         const float val = act ? row_sum(tid) : 0.0f;
-        const float partner = __shfl_xor(val, 1, 64);
+        const float partner = dpp_move<DPP_XOR1>(val);
         const int which = pr & 1;
         const float x0 = which ? partner : val, x1 = which ? val : partner;
         const float rotated = which ? x0 * sn + x1 * cs : x0 * cs - x1 * sn;
         const float out = rot ? rotated : val;
-        const float out2 = __shfl_down(out, 2, 64);  // same member of the next rotary pair
-        const float out1 = __shfl_down(out, 1, 64);  // next row (v rows are in natural order)
+        const float out2 = dpp_move<DPP_NEXT2>(out);  // same member of the next rotary pair (read by lanes 0, 1 of a quad)
+        const float out1 = dpp_move<DPP_NEXT1>(out);  // next row (v rows are in natural order; read by even lanes)
         if (act) {
           if (rot) {
             if (!(tid & 2)) {
@@ -955,9 +991,9 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
         const bool act = tid < 8 * nb;
         const int pr = 8 * (wg + G * (tid >> 3)) + (tid & 7);
         const float val = act ? row_sum(tid) : 0.0f;
-        const float up = __shfl_down(val, 1, 64);
+        const float up = dpp_move<DPP_NEXT1>(val);
         const float a = silu_f(val) * up;          // meaningful in even threads
-        const float a2 = __shfl_down(a, 2, 64);    // act value of the next pair of rows
+        const float a2 = dpp_move<DPP_NEXT2>(a);   // act value of the next pair of rows (read by lane 0 of a quad)
         if (act && !(tid & 3)) st_entry(m.act + xidx(pr / 2, m.ph[PK_DOWN].ks, m.ph[PK_DOWN].frags), pack_h2(a, a2), tag);
         pb ^= 1;
         mark(10);
