@@ -53,8 +53,11 @@ typedef unsigned long long u64;
 #ifndef GEMV_INL
 #define GEMV_INL __noinline__
 #endif
+// (the attention stages are inlined: as functions their argument structure travels through scratch memory, a memory
+// round trip in front of each of them -- 668 -> 693 tokens/s; the projection stage stays a function: inlined at its
+// five call sites, or with its arguments passed one by one in registers, the kernel is slower, 688 and 663)
 #ifndef ATTN_INL
-#define ATTN_INL __noinline__
+#define ATTN_INL __forceinline__
 #endif
 
 constexpr int CW = PS_WAVES;                   // compute waves per workgroup (waves 0 .. CW-1)
