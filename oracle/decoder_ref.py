@@ -8,6 +8,10 @@ Tolerance-checked glue (libm-dependent, not bit-pinned), following the reference
   greedy    apps/llm-bench/src/main.rs:538-543 (last index among equal maxima)
 and the int4 projection definition of packed_int4_gemm_scalar (int4_matmul.rs:387-435) through
 dequantised weights.  Activations are rounded to fp16 where the GPU decoder stores fp16.
+
+The glue functions (rmsnorm, rope, gqa_attend, swiglu, greedy_pick) are module-level and work in f32, so
+that tests/test_oracle_decoder.py can pin each of them to the reference's own unit-test vectors and to
+closed forms; RefDecoder only strings them together and adds the fp16 roundings.
 """
 from __future__ import annotations
 
@@ -26,6 +30,53 @@ def dequant_uint4(packed, scales16, n, k, g):
     q[:, 1::2] = (pb >> 4).astype(np.float32) - 8.0
     s = np.asarray(scales16).reshape(n, k // g).astype(np.float32)
     return q * np.repeat(s, g, axis=1)
+
+
+def rmsnorm(h, gamma, eps):
+    """y = x * (1 / sqrt(mean(x^2) + eps)) * gamma over the last axis (ops/norm.rs:1497-1518)."""
+    h = np.asarray(h, np.float32)
+    inv = np.float32(1.0) / np.sqrt((h * h).mean(-1, keepdims=True, dtype=np.float32) + np.float32(eps))
+    return (h * inv.astype(np.float32) * np.asarray(gamma, np.float32)).astype(np.float32)
+
+
+def rope(x, pos, theta):
+    """Rotate-half RoPE of x [..., d] at absolute position pos (ops/rope.rs:24-117): inv_freq[i] = 1/theta^(2i/d),
+    pair (x[i], x[i + d/2]), x0' = x0 cos - x1 sin, x1' = x0 sin + x1 cos, angle = inv_freq[i] * pos in f32."""
+    x = np.asarray(x, np.float32)
+    d = x.shape[-1]
+    i = np.arange(d // 2, dtype=np.float32)
+    inv_freq = (np.float32(1.0) / np.power(np.float32(theta), np.float32(2.0) * i / np.float32(d))).astype(np.float32)
+    ang = (inv_freq * np.float32(pos)).astype(np.float32)
+    cs, sn = np.cos(ang), np.sin(ang)
+    x0, x1 = x[..., : d // 2], x[..., d // 2:]
+    return np.concatenate([x0 * cs - x1 * sn, x0 * sn + x1 * cs], -1).astype(np.float32)
+
+
+def gqa_attend(q, kc, vc, groups):
+    """One query position against a cache: q [heads][d], kc / vc [positions][kv_heads][d] ->
+    [heads][d] (runner/linear.rs:552-646: kv_h = qh / groups, scores * 1/sqrt(d), max-subtracted softmax)."""
+    q = np.asarray(q, np.float32)
+    nh, hd = q.shape
+    out = np.zeros((nh, hd), np.float32)
+    scale = np.float32(1.0 / np.sqrt(hd))
+    for qh in range(nh):
+        kvh = qh // groups
+        s = (kc[:, kvh, :] @ q[qh]) * scale
+        p = np.exp(s - s.max())
+        p /= p.sum()
+        out[qh] = p @ vc[:, kvh, :]
+    return out
+
+
+def swiglu(gate, up):
+    gate = np.asarray(gate, np.float32)
+    return (gate / (np.float32(1.0) + np.exp(-gate)) * np.asarray(up, np.float32)).astype(np.float32)
+
+
+def greedy_pick(row):
+    """Last index among equal maxima (Iterator::max_by, apps/llm-bench/src/main.rs:538-543)."""
+    row = np.asarray(row)
+    return int(np.flatnonzero(row == row.max())[-1])
 
 
 class RefDecoder:
@@ -54,18 +105,11 @@ class RefDecoder:
             self.vc[layer][b] = np.array(v_nat[b], np.float32)
 
     def _rmsnorm(self, h, gamma):
-        inv = 1.0 / np.sqrt((h.astype(np.float32) ** 2).mean(-1, keepdims=True) + np.float32(self.c["rms_eps"]))
-        return f16(h * inv.astype(np.float32) * gamma)
+        return f16(rmsnorm(h, gamma, self.c["rms_eps"]))
 
     def _rope(self, x, pos):
         """x: [heads][d]."""
-        d = x.shape[-1]
-        i = np.arange(d // 2, dtype=np.float32)
-        inv_freq = (1.0 / np.power(np.float32(self.c["rope_theta"]), 2 * i / np.float32(d))).astype(np.float32)
-        ang = inv_freq * np.float32(pos)
-        cs, sn = np.cos(ang), np.sin(ang)
-        x0, x1 = x[..., : d // 2], x[..., d // 2:]
-        return f16(np.concatenate([x0 * cs - x1 * sn, x0 * sn + x1 * cs], -1))
+        return f16(rope(x, pos, self.c["rope_theta"]))
 
     def step(self, tokens, pos):
         """tokens: int [batch]; pos: position the new token is written at.  Returns logits f32 [batch][vocab]."""
@@ -84,18 +128,13 @@ class RefDecoder:
                 qr, kr = self._rope(q[b], pos), self._rope(k[b], pos)
                 self.kc[l][b] = np.concatenate([self.kc[l][b][:pos], kr[None]], 0)
                 self.vc[l][b] = np.concatenate([self.vc[l][b][:pos], v[b][None]], 0)
-                for qh in range(nh):
-                    kvh = qh // groups
-                    s = (self.kc[l][b][:, kvh, :] @ qr[qh]) * np.float32(1.0 / np.sqrt(hd))
-                    p = np.exp(s - s.max())
-                    p /= p.sum()
-                    ao[b, qh] = p @ self.vc[l][b][:, kvh, :]
+                ao[b] = gqa_attend(qr, self.kc[l][b], self.vc[l][b], groups)
             ao = f16(ao.reshape(B, nh * hd))
             h = h + ao @ self.w[(l, "o")].T
             xn = self._rmsnorm(h, self.norms[(l, "ffn")])
             gt = xn @ self.w[(l, "gate")].T
             up = xn @ self.w[(l, "up")].T
-            act = f16(gt / (1.0 + np.exp(-gt)) * up)
+            act = f16(swiglu(gt, up))
             h = h + act @ self.w[(l, "down")].T
         xn = self._rmsnorm(h, self.norms[("final",)])
         return (xn @ self.w[("lm_head",)].T).astype(np.float32)

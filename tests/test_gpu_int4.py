@@ -364,7 +364,7 @@ def test_lm_head_sweep_sampled_at_full_size(oracle, K, torch_cuda):
     cols[-1] = n - 1  # the last row of the weight: the column tail of the last tile
     bs = b.reshape(n, k // 2)[cols]
     ss = scales16.reshape(n, groups)[cols].astype(np.float32)
-    for m in (1, 5, 16, 17, 64, 256):
+    for m in (1, 2, 4, 5, 8, 16, 17, 32, 64, 128, 256):  # every M of the BASELINE sweep + both sides of the switch
         xt = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).bfloat16()
         xs = xt.float().numpy()
         ref = oracle.packed_int4_gemm_scalar(bs ^ 0x88, ss, xs, m, len(cols), k, g)
@@ -438,3 +438,48 @@ def test_f32_rows_beyond_16_run_as_skinny_passes(oracle, K, torch_cuda):
     ref = oracle.packed_int4_gemm_scalar(b ^ 0x88, scales, x[:3].cpu().numpy(), 3, n, k, g)
     d, rel = int4_tolerances(y[:3].cpu().numpy(), ref, k, x[:3].cpu().numpy())
     assert rel < 5e-5, rel
+
+
+@pytest.mark.parametrize("n,k", [(4096, 14336), (4096, 4096), (28672, 4096)])
+@pytest.mark.parametrize("m", [1, 3, 16])
+def test_fused_epilogues_at_decoder_shapes(oracle, K, torch_cuda, n, k, m):
+    """yscv_hip_int4_matmul_fused at the projection shapes of the 7B-shape decoder: the down projection (K = 14336, grid
+    K split with the second-pass kernel) adding into an f32 residual, and the gate / up projection (rows interleaved)
+    with SwiGLU, against the scalar oracle on a sample of output rows; fp16 activations and scales like the decoder."""
+    torch = torch_cuda
+    rng = np.random.default_rng(1000 + n + k + m)
+    g = 32
+    b = _rand_packed(rng, n, k)
+    scales16 = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float16)
+    w = K.PackedInt4Weight(b, scales16, g, n, k, nibble_format=K.NIBBLE_UNSIGNED)
+    xt = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).half()
+    xs = xt.float().numpy()
+    pairs = np.sort(rng.choice(n // 2, 48, replace=False))
+    pairs[-1] = n // 2 - 1
+    rows = np.stack([2 * pairs, 2 * pairs + 1], 1).reshape(-1)  # gate_i, up_i of the sampled pairs
+    bs = b.reshape(n, k // 2)[rows]
+    ss = scales16.reshape(n, k // g)[rows].astype(np.float32)
+    ref = oracle.packed_int4_gemm_scalar(bs ^ 0x88, ss, xs, m, len(rows), k, g).reshape(m, len(rows))
+    # store
+    y = torch.full((m, n), 7.0, device="cuda")
+    w.matmul_fused(xt.cuda(), y, K.EPILOGUE_STORE)
+    int4_tolerances(y.cpu().numpy()[:, rows], ref, k, xs)
+    assert torch.equal(y, w.matmul(xt.cuda(), out_dtype=torch.float32, mode="gemv"))
+    # residual add: y += x W^T on an f32 residual
+    resid = rng.standard_normal((m, n)).astype(np.float32) * 10
+    y = torch.from_numpy(resid).cuda()
+    w.matmul_fused(xt.cuda(), y, K.EPILOGUE_ADD_F32)
+    got = y.cpu().numpy()
+    int4_tolerances(got[:, rows] - resid[:, rows], ref, k, xs)  # f32 add of the two: one rounding of |resid + y| on top
+    # SwiGLU: out[i] = silu(gate_i) * up_i, fp16 out like the decoder and f32 out
+    gate, up = ref[:, 0::2].astype(np.float64), ref[:, 1::2].astype(np.float64)
+    want = gate / (1.0 + np.exp(-gate)) * up
+    for odt in (torch.float16, torch.float32):
+        act = torch.full((m, n // 2), 7.0, device="cuda", dtype=odt)
+        w.matmul_fused(xt.cuda(), act, K.EPILOGUE_SWIGLU)
+        ga = act.float().cpu().numpy()[:, pairs]
+        err = np.abs(ga - want).max() / np.abs(want).max()
+        assert err < (2e-3 if odt == torch.float16 else 1e-3), (odt, err)
+    with pytest.raises(Exception, match="m <= 16"):
+        w.matmul_fused(torch.zeros(17, k, device="cuda", dtype=torch.float16), torch.zeros(17, n, device="cuda"), K.EPILOGUE_STORE)
+    w.close()

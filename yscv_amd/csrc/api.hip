@@ -469,6 +469,15 @@ int32_t yscv_hip_int4_gemm(const yscv_hip_int4_weight *w, const void *x_dev, int
   return int4_run(w, x_dev, x_dtype, y_dev, y_dtype, m, 2, as_stream(stream));
 }
 
+int32_t yscv_hip_int4_matmul_fused(const yscv_hip_int4_weight *w, const void *x_dev, int32_t x_dtype, void *y_dev,
+                                   int32_t y_dtype, size_t m, int32_t epilogue, void *stream) {
+  YSCV_REQUIRE(epilogue == YSCV_HIP_EPILOGUE_STORE || epilogue == YSCV_HIP_EPILOGUE_ADD_F32 ||
+                   epilogue == YSCV_HIP_EPILOGUE_SWIGLU,
+               "unknown epilogue %d", epilogue);
+  YSCV_REQUIRE(m <= 16, "fused epilogues run on the skinny kernel: m <= 16, got %zu", m);
+  return int4_run_ws(w, x_dev, x_dtype, y_dev, y_dtype, m, 1, epilogue, nullptr, 0, as_stream(stream));
+}
+
 int32_t yscv_hip_int4_workspace_bytes(const yscv_hip_int4_weight *w, size_t m, int32_t x_dtype, size_t *bytes) {
   return int4_workspace_bytes(w, m, x_dtype, 0, bytes);
 }

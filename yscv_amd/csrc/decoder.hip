@@ -122,10 +122,19 @@ struct yscv_hip_decoder {
   uint32_t epoch = 1;          // tag epoch of the next persistent step; never reused
 };
 
-static void decoder_free(yscv_hip_decoder *d) {
-  if (!d) return;
+// A captured step holds the addresses of the weights and of the workspace as they were at capture time: whatever
+// frees or replaces one of them drops the graph, and the next graph run captures again.
+static void drop_graph(yscv_hip_decoder *d) {
   if (d->graph_exec) (void)hipGraphExecDestroy(d->graph_exec);
   if (d->graph) (void)hipGraphDestroy(d->graph);
+  d->graph_exec = nullptr;
+  d->graph = nullptr;
+  d->graph_batch = 0;
+}
+
+static void decoder_free(yscv_hip_decoder *d) {
+  if (!d) return;
+  drop_graph(d);
   for (auto &L : d->layers) {
     destroy_int4(L.wqkv);
     destroy_int4(L.wo);
@@ -318,6 +327,7 @@ static int32_t alloc_runtime(yscv_hip_decoder *d) {
 }
 
 static int32_t finish_setup(yscv_hip_decoder *d) {
+  drop_graph(d);
   // workspace: the largest any projection needs at the maximum batch
   size_t need = 0;
   auto upd = [&](const yscv_hip_int4_weight *w) -> int32_t {
@@ -470,6 +480,7 @@ int32_t yscv_hip_decoder_set_linear(yscv_hip_decoder *d, int32_t layer, int32_t 
   YSCV_REQUIRE(n == exp_n[kind] && k == exp_k[kind], "projection %d must be [%zu][%zu], got [%zu][%zu]", kind,
                exp_n[kind], exp_k[kind], n, k);
   d->finalized = false;
+  drop_graph(d);
   if (kind == YSCV_HIP_DEC_LM_HEAD) {
     destroy_int4(d->lm_head);
     d->lm_head = nullptr;
@@ -547,6 +558,8 @@ int32_t yscv_hip_decoder_init_random(yscv_hip_decoder *d, uint64_t seed) {
   const size_t g = c.group_size, D = c.d_model;
   const size_t qkv_n = (size_t)(c.n_heads + 2 * c.n_kv_heads) * c.head_dim;
   uint64_t sd = seed * 0x100000001B3ull + 1;
+  d->finalized = false;
+  drop_graph(d);
   // one raw buffer, sized for the largest projection, reused for every weight
   const size_t max_elems = std::max(std::max(qkv_n, 2 * (size_t)c.d_ff) * D, std::max((size_t)c.vocab * D, D * (size_t)c.d_ff));
   DevBuf raw, rsc;
@@ -656,10 +669,7 @@ int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_g
     return YSCV_HIP_OK;
   }
   if (!d->graph_exec || d->graph_batch != d->batch) {
-    if (d->graph_exec) (void)hipGraphExecDestroy(d->graph_exec);
-    if (d->graph) (void)hipGraphDestroy(d->graph);
-    d->graph_exec = nullptr;
-    d->graph = nullptr;
+    drop_graph(d);
     hipStream_t cs = nullptr;
     DEC_HIP(hipStreamCreateWithFlags(&cs, hipStreamNonBlocking));
     hipError_t e = hipStreamBeginCapture(cs, hipStreamCaptureModeThreadLocal);

@@ -12,7 +12,8 @@ import ctypes as C
 import numpy as np
 
 from . import capi
-from .capi import BF16, F16, F32, NIBBLE_SIGNED, NIBBLE_UNSIGNED, ROUND_HALF_AWAY, ROUND_TIES_EVEN, lib
+from .capi import (BF16, EPILOGUE_ADD_F32, EPILOGUE_STORE, EPILOGUE_SWIGLU, F16, F32, NIBBLE_SIGNED, NIBBLE_UNSIGNED,
+                   ROUND_HALF_AWAY, ROUND_TIES_EVEN, lib)
 
 _sz = C.c_size_t
 
@@ -271,6 +272,17 @@ class PackedInt4Weight:
         fn = {"auto": lib().int4_matmul, "gemv": lib().int4_gemv, "gemm": lib().int4_gemm}[mode]
         fn(self._h, C.c_void_p(x.data_ptr()), _torch_dtype_code(x), C.c_void_p(out.data_ptr()),
            _torch_dtype_code(out), _sz(m), _stream_ptr())
+        return out
+
+    def matmul_fused(self, x, out, epilogue: int):
+        """yscv_hip_int4_matmul_fused: skinny kernel (m <= 16) with the epilogue fused.  EPILOGUE_ADD_F32 adds into the
+        f32 tensor `out` [m, m_w]; EPILOGUE_SWIGLU writes silu(gate) * up into `out` [m, m_w / 2]."""
+        assert x.is_cuda and out.is_cuda and x.shape[-1] == self.k
+        x = x.contiguous()
+        m = x.numel() // self.k
+        assert out.is_contiguous() and out.numel() == m * (self.m_w // 2 if epilogue == 2 else self.m_w)
+        lib().int4_matmul_fused(self._h, C.c_void_p(x.data_ptr()), _torch_dtype_code(x), C.c_void_p(out.data_ptr()),
+                                _torch_dtype_code(out), _sz(m), int(epilogue), _stream_ptr())
         return out
 
     def close(self):
