@@ -405,11 +405,21 @@ int32_t yscv_hip_decoder_finalize(yscv_hip_decoder *d);
  * device (uniform nibbles, scales ~U(0.005,0.02), embedding ~N(0,1)), and a KV cache filled with
  * ~N(0,1) values.  No reference counterpart (llm-bench loads an ONNX file). */
 int32_t yscv_hip_decoder_init_random(yscv_hip_decoder *d, uint64_t seed);
+/* The same with the nibbles uniform over nibble_lo .. nibble_hi.  0 .. 15 has mean -0.5 after the zero point 8,
+ * which gives every projection output a common offset and makes a deep random model ill-conditioned (all logits
+ * nearly equal); 1 .. 15 is symmetric about the zero point and yields a model whose greedy tokens vary. */
+int32_t yscv_hip_decoder_init_random_range(yscv_hip_decoder *d, uint64_t seed, int32_t nibble_lo,
+                                           int32_t nibble_hi);
 int32_t yscv_hip_decoder_fill_kv_random(yscv_hip_decoder *d, uint64_t seed);
 /* Load cache positions [0, n_positions) of one layer from host arrays laid out
  * [batch][position][kv_head][head_dim] fp16 (keys already rotated). */
 int32_t yscv_hip_decoder_set_kv(yscv_hip_decoder *d, int32_t layer, const uint16_t *k_f16,
                                 const uint16_t *v_f16, int32_t batch, int32_t n_positions);
+/* The read side of the cache (KvCache::get, crates/yscv-onnx/src/runner/kv_cache.rs:207-241): positions
+ * [first_pos, first_pos + n_positions) of one layer into host arrays laid out like yscv_hip_decoder_set_kv's,
+ * [batch][position][kv_head][head_dim] fp16, keys as stored (rotated). */
+int32_t yscv_hip_decoder_get_kv(yscv_hip_decoder *d, int32_t layer, uint16_t *k_f16, uint16_t *v_f16,
+                                int32_t batch, int32_t first_pos, int32_t n_positions);
 /* Start a generation: batch rows, the position the next token is written at, one input token per row. */
 int32_t yscv_hip_decoder_reset(yscv_hip_decoder *d, int32_t batch, int32_t start_pos,
                                const int32_t *tokens_host);
@@ -429,6 +439,17 @@ int32_t yscv_hip_decoder_read_tokens(yscv_hip_decoder *d, int32_t first_step, in
                                      int32_t *out_host);
 /* Logits of the last step, [batch][vocab] f32. */
 int32_t yscv_hip_decoder_read_logits(yscv_hip_decoder *d, float *out_host);
+/* Inspection aid for parity tests: the activation buffers of the multi-kernel path (use_graph 0 or 1) as the last
+ * step left them, widened to f32, [batch][width]: the residual stream after the last layer, the final RMSNorm's
+ * output (the LM head's input), and the last layer's q|k|v (q and k rotated), attention output and SwiGLU output.
+ * The single-launch path keeps these in registers and exchange records and does not fill them.  No counterpart in
+ * the reference (its runner keeps every intermediate tensor in the TensorEnv by name). */
+#define YSCV_HIP_DEC_ACT_RESIDUAL 0 /* [batch][d_model] */
+#define YSCV_HIP_DEC_ACT_NORMED 1   /* [batch][d_model] */
+#define YSCV_HIP_DEC_ACT_QKV 2      /* [batch][(n_heads + 2 n_kv_heads) * head_dim] */
+#define YSCV_HIP_DEC_ACT_ATTN_OUT 3 /* [batch][n_heads * head_dim] */
+#define YSCV_HIP_DEC_ACT_FFN 4      /* [batch][d_ff] */
+int32_t yscv_hip_decoder_read_activation(yscv_hip_decoder *d, int32_t which, float *out_host, size_t capacity);
 /* Bytes of packed weights + scales one decode step streams through the projections. */
 int32_t yscv_hip_decoder_weight_bytes(const yscv_hip_decoder *d, size_t *bytes);
 int32_t yscv_hip_decoder_vocab(const yscv_hip_decoder *d, size_t *vocab);

@@ -112,7 +112,9 @@ class RefDecoder:
         return f16(rope(x, pos, self.c["rope_theta"]))
 
     def step(self, tokens, pos):
-        """tokens: int [batch]; pos: position the new token is written at.  Returns logits f32 [batch][vocab]."""
+        """tokens: int [batch]; pos: position the new token is written at.  Returns logits f32 [batch][vocab].
+        self.trace keeps the last layer's intermediates (q|k|v with q and k rotated, attention output, SwiGLU
+        output), the residual stream after the last layer and the LM head's input, each [batch][width]."""
         c = self.c
         hd, nh, nkv = c["head_dim"], c["n_heads"], c["n_kv_heads"]
         groups = nh // nkv
@@ -124,8 +126,10 @@ class RefDecoder:
             k = f16(xn @ self.w[(l, "k")].T).reshape(B, nkv, hd)
             v = f16(xn @ self.w[(l, "v")].T).reshape(B, nkv, hd)
             ao = np.zeros((B, nh, hd), np.float32)
+            qkv = np.zeros((B, (nh + 2 * nkv) * hd), np.float32)
             for b in range(B):
                 qr, kr = self._rope(q[b], pos), self._rope(k[b], pos)
+                qkv[b] = np.concatenate([qr.reshape(-1), kr.reshape(-1), v[b].reshape(-1)])
                 self.kc[l][b] = np.concatenate([self.kc[l][b][:pos], kr[None]], 0)
                 self.vc[l][b] = np.concatenate([self.vc[l][b][:pos], v[b][None]], 0)
                 ao[b] = gqa_attend(qr, self.kc[l][b], self.vc[l][b], groups)
@@ -137,4 +141,5 @@ class RefDecoder:
             act = f16(swiglu(gt, up))
             h = h + act @ self.w[(l, "down")].T
         xn = self._rmsnorm(h, self.norms[("final",)])
+        self.trace = {"qkv": qkv, "attn_out": ao, "ffn": act, "residual": h.astype(np.float32), "normed": xn}
         return (xn @ self.w[("lm_head",)].T).astype(np.float32)

@@ -123,13 +123,16 @@ _SIGNATURES = {
     "yscv_hip_decoder_set_embedding": [_vp, _vp],
     "yscv_hip_decoder_finalize": [_vp],
     "yscv_hip_decoder_init_random": [_vp, C.c_uint64],
+    "yscv_hip_decoder_init_random_range": [_vp, C.c_uint64, _i32, _i32],
     "yscv_hip_decoder_fill_kv_random": [_vp, C.c_uint64],
     "yscv_hip_decoder_set_kv": [_vp, _i32, _vp, _vp, _i32, _i32],
+    "yscv_hip_decoder_get_kv": [_vp, _i32, _vp, _vp, _i32, _i32, _i32],
     "yscv_hip_decoder_reset": [_vp, _i32, _i32, _vp],
     "yscv_hip_decoder_run": [_vp, _i32, _i32, _vp],
     "yscv_hip_decoder_run_projections": [_vp, _i32, _vp],
     "yscv_hip_decoder_read_tokens": [_vp, _i32, _i32, _vp],
     "yscv_hip_decoder_read_logits": [_vp, _vp],
+    "yscv_hip_decoder_read_activation": [_vp, _i32, _vp, _sz],
     "yscv_hip_decoder_weight_bytes": [_vp, C.POINTER(_sz)],
     "yscv_hip_decoder_vocab": [_vp, C.POINTER(_sz)],
     "yscv_hip_sample_token": [_vp, _sz, _sz, _f32, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32)],

@@ -26,6 +26,7 @@ static std::mutex g_ctx_mutex;
 static Context g_ctx;
 static bool g_ctx_ready = false;
 
+
 int32_t init_context(int device) {
   std::lock_guard<std::mutex> lock(g_ctx_mutex);
   if (g_ctx_ready && g_ctx.device == device) return YSCV_HIP_OK;

@@ -16,12 +16,20 @@ namespace yscv {
 // ---- random-initialised tiled weights (benchmark setup) -------------------------------------------
 // Uniform nibbles and scales ~U(0.005, 0.02) written straight into the tiled layout: for random data
 // the tiling is just another arrangement of the same distribution, so no host round trip is needed.
-__global__ void random_tiles_kernel(uint32_t *__restrict__ words, size_t n_words, uint64_t seed) {
+// eight nibbles per word, each uniform over lo .. hi (0 .. 15: the random bits as they come)
+__global__ void random_tiles_kernel(uint32_t *__restrict__ words, size_t n_words, uint64_t seed, int lo, int hi) {
+  const uint32_t span = (uint32_t)(hi - lo + 1);
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n_words; i += (size_t)gridDim.x * blockDim.x) {
     uint64_t z = (i + 1) * 0x9E3779B97F4A7C15ull + seed;
     z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
     z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
-    words[i] = (uint32_t)(z ^ (z >> 31));
+    z ^= z >> 31;
+    uint32_t w = (uint32_t)z;
+    if (span != 16) {
+      w = 0;
+      for (int e = 0; e < 8; e++) w |= ((uint32_t)lo + (uint32_t)((z >> (8 * e)) & 0xFFu) * span / 256u) << (4 * e);
+    }
+    words[i] = w;
   }
 }
 __global__ void random_scales_kernel(_Float16 *__restrict__ sc, size_t n, uint64_t seed, float lo, float hi) {
@@ -53,10 +61,11 @@ static unsigned grid_for(size_t n) {
 
 // Random raw weight on the device: [n][k/2] uniform nibble bytes and fp16 scales ~U(0.005, 0.02) in natural
 // order, so that every layout built from it (tiled, persistent stream) holds the same logical matrix.
-static int32_t random_raw_weight(size_t n, size_t k, size_t g, uint64_t seed, uint8_t *raw, _Float16 *scales) {
+static int32_t random_raw_weight(size_t n, size_t k, size_t g, uint64_t seed, int lo, int hi, uint8_t *raw,
+                                 _Float16 *scales) {
   const size_t words = n * k / 8, sc = n * (k / g);
   hipLaunchKernelGGL(random_tiles_kernel, dim3(grid_for(words)), dim3(256), 0, nullptr, reinterpret_cast<uint32_t *>(raw),
-                     words, seed);
+                     words, seed, lo, hi);
   hipLaunchKernelGGL(random_scales_kernel, dim3(grid_for(sc)), dim3(256), 0, nullptr, scales, sc, seed ^ 0x5ca1e5ull, 0.005f,
                      0.02f);
   YSCV_HIP_TRY(hipGetLastError());
@@ -553,7 +562,12 @@ int32_t yscv_hip_decoder_finalize(yscv_hip_decoder *d) {
 }
 
 int32_t yscv_hip_decoder_init_random(yscv_hip_decoder *d, uint64_t seed) {
+  return yscv_hip_decoder_init_random_range(d, seed, 0, 15);
+}
+
+int32_t yscv_hip_decoder_init_random_range(yscv_hip_decoder *d, uint64_t seed, int32_t nibble_lo, int32_t nibble_hi) {
   YSCV_REQUIRE(d != nullptr, "null decoder");
+  YSCV_REQUIRE(nibble_lo >= 0 && nibble_lo <= nibble_hi && nibble_hi <= 15, "nibble range must lie in 0..15");
   const auto &c = d->cfg;
   const size_t g = c.group_size, D = c.d_model;
   const size_t qkv_n = (size_t)(c.n_heads + 2 * c.n_kv_heads) * c.head_dim;
@@ -567,7 +581,7 @@ int32_t yscv_hip_decoder_init_random(yscv_hip_decoder *d, uint64_t seed) {
   YSCV_TRY(rsc.alloc(max_elems / g * 2));
   auto make = [&](int layer, int pkind, size_t n, size_t k, yscv_hip_int4_weight **out) -> int32_t {
     YSCV_REQUIRE(g == 32 || g == 64 || g % 128 == 0, "random weights need a tiled group size");
-    YSCV_TRY(random_raw_weight(n, k, g, sd++, raw.as<uint8_t>(), rsc.as<_Float16>()));
+    YSCV_TRY(random_raw_weight(n, k, g, sd++, nibble_lo, nibble_hi, raw.as<uint8_t>(), rsc.as<_Float16>()));
     YSCV_TRY(int4_create_from_device(raw.as<uint8_t>(), rsc.p, YSCV_HIP_F16, YSCV_HIP_NIBBLE_UNSIGNED, n, k, g, out));
     if (d->persist_ok) YSCV_TRY(launch_persist_pack(d->pm, layer, pkind, raw.as<uint8_t>(), rsc.as<_Float16>(), d->p_stream, nullptr));
     DEC_HIP(hipDeviceSynchronize());  // the raw buffer is reused by the next weight
@@ -621,6 +635,36 @@ int32_t yscv_hip_decoder_set_kv(yscv_hip_decoder *d, int32_t layer, const uint16
   YSCV_TRY(launch_kv_relayout(dk.as<_Float16>(), dv.as<_Float16>(), batch, n_positions, c.n_kv_heads, c.head_dim,
                               c.max_ctx, L.kc, L.vc, nullptr));
   DEC_HIP(hipDeviceSynchronize());
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_get_kv(yscv_hip_decoder *d, int32_t layer, uint16_t *k_f16, uint16_t *v_f16, int32_t batch,
+                                int32_t first_pos, int32_t n_positions) {
+  YSCV_REQUIRE(d && k_f16 && v_f16, "null argument");
+  const auto &c = d->cfg;
+  YSCV_REQUIRE(layer >= 0 && layer < c.n_layers, "layer %d out of range", layer);
+  YSCV_REQUIRE(batch >= 1 && batch <= c.max_batch && first_pos >= 0 && n_positions >= 0 &&
+                   first_pos + n_positions <= c.max_ctx,
+               "bad batch / position range");
+  if (n_positions == 0) return YSCV_HIP_OK;
+  DEC_HIP(hipDeviceSynchronize());
+  const int hd = c.head_dim, hkv = c.n_kv_heads;
+  const int s0 = first_pos / 8, s1 = (first_pos + n_positions + 7) / 8;  // 8-position slabs of the V layout
+  std::vector<uint16_t> kt((size_t)n_positions * hd), vt((size_t)(s1 - s0) * hd * 8);
+  const auto &L = d->layers[layer];
+  for (int b = 0; b < batch; b++)
+    for (int h = 0; h < hkv; h++) {
+      const size_t row = (size_t)b * hkv + h;
+      DEC_HIP(hipMemcpy(kt.data(), L.kc + (row * c.max_ctx + first_pos) * hd, kt.size() * 2, hipMemcpyDeviceToHost));
+      DEC_HIP(hipMemcpy(vt.data(), L.vc + ((row * (c.max_ctx / 8) + s0) * hd) * 8, vt.size() * 2, hipMemcpyDeviceToHost));
+      for (int p = 0; p < n_positions; p++) {
+        uint16_t *kd = k_f16 + (((size_t)b * n_positions + p) * hkv + h) * hd;
+        uint16_t *vd = v_f16 + (((size_t)b * n_positions + p) * hkv + h) * hd;
+        memcpy(kd, &kt[(size_t)p * hd], (size_t)hd * 2);
+        const int ap = first_pos + p;
+        for (int i = 0; i < hd; i++) vd[i] = vt[((size_t)(ap / 8 - s0) * hd + i) * 8 + (ap & 7)];
+      }
+    }
   return YSCV_HIP_OK;
 }
 
@@ -722,6 +766,35 @@ int32_t yscv_hip_decoder_read_logits(yscv_hip_decoder *d, float *out_host) {
   DEC_HIP(hipDeviceSynchronize());
   YSCV_TRY(check_persist_abort(d));
   DEC_HIP(hipMemcpy(out_host, d->logits, (size_t)d->batch * d->cfg.vocab * 4, hipMemcpyDeviceToHost));
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_read_activation(yscv_hip_decoder *d, int32_t which, float *out_host, size_t capacity) {
+  YSCV_REQUIRE(d && out_host, "null argument");
+  YSCV_REQUIRE(d->batch >= 1, "call yscv_hip_decoder_reset first");
+  const auto &c = d->cfg;
+  const size_t B = (size_t)d->batch;
+  const size_t qkv_n = (size_t)(c.n_heads + 2 * c.n_kv_heads) * c.head_dim;
+  const void *src = nullptr;
+  size_t elems = 0;
+  bool half = true;
+  switch (which) {
+    case YSCV_HIP_DEC_ACT_RESIDUAL: src = d->h; elems = B * c.d_model; half = false; break;
+    case YSCV_HIP_DEC_ACT_NORMED: src = d->xn; elems = B * c.d_model; break;
+    case YSCV_HIP_DEC_ACT_QKV: src = d->qkv; elems = B * qkv_n; break;
+    case YSCV_HIP_DEC_ACT_ATTN_OUT: src = d->ao; elems = B * (size_t)c.n_heads * c.head_dim; break;
+    case YSCV_HIP_DEC_ACT_FFN: src = d->act; elems = B * (size_t)c.d_ff; break;
+    default: return set_error(YSCV_HIP_ERR_INVALID_ARG, "unknown activation buffer %d", which);
+  }
+  YSCV_REQUIRE(capacity >= elems, "output holds %zu values, the buffer has %zu", capacity, elems);
+  DEC_HIP(hipDeviceSynchronize());
+  if (!half) {
+    DEC_HIP(hipMemcpy(out_host, src, elems * 4, hipMemcpyDeviceToHost));
+    return YSCV_HIP_OK;
+  }
+  std::vector<_Float16> tmp(elems);
+  DEC_HIP(hipMemcpy(tmp.data(), src, elems * 2, hipMemcpyDeviceToHost));
+  for (size_t i = 0; i < elems; i++) out_host[i] = (float)tmp[i];
   return YSCV_HIP_OK;
 }
 

@@ -43,8 +43,8 @@ class Decoder:
     def finalize(self):
         lib().decoder_finalize(self._h)
 
-    def init_random(self, seed=0):
-        lib().decoder_init_random(self._h, C.c_uint64(seed))
+    def init_random(self, seed=0, nibbles=(0, 15)):
+        lib().decoder_init_random_range(self._h, C.c_uint64(seed), int(nibbles[0]), int(nibbles[1]))
 
     def fill_kv_random(self, seed=0):
         lib().decoder_fill_kv_random(self._h, C.c_uint64(seed))
@@ -54,6 +54,13 @@ class Decoder:
         v = np.ascontiguousarray(v16)
         assert k.dtype == np.float16 and v.dtype == np.float16 and k.shape == v.shape and k.ndim == 4
         lib().decoder_set_kv(self._h, int(layer), _p(k), _p(v), int(k.shape[0]), int(k.shape[1]))
+
+    def get_kv(self, layer, batch, first_pos, n_positions):
+        """(k, v) fp16 arrays [batch][n_positions][kv_head][head_dim] of cache positions first_pos .. (keys rotated)."""
+        shape = (batch, n_positions, self.cfg["n_kv_heads"], self.cfg["head_dim"])
+        k, v = np.empty(shape, np.float16), np.empty(shape, np.float16)
+        lib().decoder_get_kv(self._h, int(layer), _p(k), _p(v), int(batch), int(first_pos), int(n_positions))
+        return k, v
 
     def reset(self, tokens, start_pos):
         t = np.ascontiguousarray(tokens, np.int32)
@@ -77,6 +84,16 @@ class Decoder:
     def logits(self):
         out = np.empty((self.batch, self.cfg["vocab"]), np.float32)
         lib().decoder_read_logits(self._h, _p(out))
+        return out
+
+    def activation(self, which):
+        """yscv_hip_decoder_read_activation: 'residual' | 'normed' | 'qkv' | 'attn_out' | 'ffn' of the last multi-kernel step."""
+        c = self.cfg
+        width = {"residual": c["d_model"], "normed": c["d_model"], "qkv": (c["n_heads"] + 2 * c["n_kv_heads"]) * c["head_dim"],
+                 "attn_out": c["n_heads"] * c["head_dim"], "ffn": c["d_ff"]}[which]
+        code = ["residual", "normed", "qkv", "attn_out", "ffn"].index(which)
+        out = np.empty((self.batch, width), np.float32)
+        lib().decoder_read_activation(self._h, code, _p(out), C.c_size_t(out.size))
         return out
 
     def generate(self, input_ids, max_tokens=256, temperature=1.0, top_k=50, top_p=0.9, eos_token_id=None,
