@@ -166,6 +166,20 @@ int32_t yscv_hip_int4_matmul_ws(const yscv_hip_int4_weight *w, const void *x_dev
                                 void *y_dev, int32_t y_dtype, size_t m, void *workspace_dev,
                                 size_t workspace_bytes, void *stream);
 
+/* yscv_hip_int4_matmul for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its kernels need no scratch).  The
+ * scratch -- prepared activations and the partial sums of a grid-level K split -- lives in a device array that is
+ * part of the library's code object, YSCV_HIP_STATIC_SCRATCH_BYTES per GPU, held until the process ends; the call
+ * allocates and frees nothing and enqueues only kernels.  A call whose scratch would exceed that size
+ * (yscv_hip_int4_workspace_bytes tells) is YSCV_HIP_ERR_INVALID_ARG; every m <= 16 call fits, and so does a
+ * bf16 / fp16 prefill of 2048 x 4096.  All calls on one GPU share the one array: calls that overlap in time (two
+ * streams, two threads) race on it -- serialise them, or use yscv_hip_int4_matmul_ws with a workspace per stream.
+ * Nothing in the array has to start at zero: every byte a kernel reads was written earlier in the same call.
+ * Results are bit-identical to yscv_hip_int4_matmul. */
+#define YSCV_HIP_STATIC_SCRATCH_BYTES (32u << 20)
+int32_t yscv_hip_int4_matmul_static(const yscv_hip_int4_weight *w, const void *x_dev, int32_t x_dtype,
+                                    void *y_dev, int32_t y_dtype, size_t m, void *stream);
+
 /* Exact argument lists of the Rust functions (host slices -> host pointers):
  * packed_int4_gemv_dispatch  int4_matmul.rs:310-318
  * packed_int4_gemm_dispatch  int4_matmul.rs:548-557

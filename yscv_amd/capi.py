@@ -8,6 +8,7 @@ F32, F16, BF16 = 0, 1, 2
 NIBBLE_SIGNED, NIBBLE_UNSIGNED = 0, 1
 ROUND_HALF_AWAY, ROUND_TIES_EVEN = 0, 1
 EPILOGUE_STORE, EPILOGUE_ADD_F32, EPILOGUE_SWIGLU = 0, 1, 2
+STATIC_SCRATCH_BYTES = 32 << 20
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "lib", "libyscv_hip.so")
@@ -82,6 +83,7 @@ _SIGNATURES = {
     "yscv_hip_int4_gemv": [_vp, _vp, _i32, _vp, _i32, _sz, _vp],
     "yscv_hip_int4_gemm": [_vp, _vp, _i32, _vp, _i32, _sz, _vp],
     "yscv_hip_int4_matmul_fused": [_vp, _vp, _i32, _vp, _i32, _sz, _i32, _vp],
+    "yscv_hip_int4_matmul_static": [_vp, _vp, _i32, _vp, _i32, _sz, _vp],
     "yscv_hip_int4_workspace_bytes": [_vp, _sz, _i32, C.POINTER(_sz)],
     "yscv_hip_int4_matmul_ws": [_vp, _vp, _i32, _vp, _i32, _sz, _vp, _sz, _vp],
     "yscv_hip_packed_int4_gemv_dispatch": [_vp, _vp, _vp, _vp, _sz, _sz, _sz],

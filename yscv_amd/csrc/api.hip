@@ -26,6 +26,12 @@ static std::mutex g_ctx_mutex;
 static Context g_ctx;
 static bool g_ctx_ready = false;
 
+// Scratch of yscv_hip_int4_matmul_static: device memory that exists from the moment the code object is loaded, so
+// that entry point never allocates.  Every GPU holds its own copy at its own address; the name below is only the
+// host-side handle of the symbol, the address a kernel can use is looked up once per device in init_context().
+static __device__ __align__(256) unsigned char scratch[YSCV_HIP_STATIC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+static void *g_scratch_ptr[kMaxDevices] = {};
 
 int32_t init_context(int device) {
   std::lock_guard<std::mutex> lock(g_ctx_mutex);
@@ -42,6 +48,11 @@ int32_t init_context(int device) {
     return set_error(YSCV_HIP_ERR_NO_DEVICE, "device %d is %s; this library is built for gfx950 only", device,
                      prop.gcnArchName);
   YSCV_HIP_TRY(hipSetDevice(device));
+  if (device < kMaxDevices && g_scratch_ptr[device] == nullptr) {
+    void *p = nullptr;
+    YSCV_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    g_scratch_ptr[device] = p;
+  }
   // Calls without a caller-provided workspace take their scratch from the stream-ordered allocator; keeping freed
   // blocks in its pool makes that a sub-microsecond operation instead of a trip to the driver per call.
   hipMemPool_t pool = nullptr;
@@ -477,6 +488,25 @@ int32_t yscv_hip_int4_matmul_fused(const yscv_hip_int4_weight *w, const void *x_
                "unknown epilogue %d", epilogue);
   YSCV_REQUIRE(m <= 16, "fused epilogues run on the skinny kernel: m <= 16, got %zu", m);
   return int4_run_ws(w, x_dev, x_dtype, y_dev, y_dtype, m, 1, epilogue, nullptr, 0, as_stream(stream));
+}
+
+int32_t yscv_hip_int4_matmul_static(const yscv_hip_int4_weight *w, const void *x_dev, int32_t x_dtype, void *y_dev,
+                                    int32_t y_dtype, size_t m, void *stream) {
+  const Context *ctx = nullptr;
+  YSCV_TRY(ensure_context(&ctx));
+  YSCV_REQUIRE(w != nullptr && x_dev != nullptr && y_dev != nullptr, "null argument");
+  YSCV_REQUIRE(valid_act_dtype(x_dtype) && valid_act_dtype(y_dtype), "unknown dtype code");
+  if (m == 0) return YSCV_HIP_OK;
+  void *ws = ctx->device < kMaxDevices ? g_scratch_ptr[ctx->device] : nullptr;
+  if (ws == nullptr) return set_error(YSCV_HIP_ERR_DEVICE, "the static scratch of device %d was never resolved", ctx->device);
+  if (w->tiled) {
+    const Int4Scratch L = int4_scratch_layout(w, x_dev, x_dtype, m, 0, ctx->num_cus);
+    if (L.total > (size_t)YSCV_HIP_STATIC_SCRATCH_BYTES)
+      return set_error(YSCV_HIP_ERR_INVALID_ARG,
+                       "this call needs %zu bytes of scratch, the static scratch holds %zu: use yscv_hip_int4_matmul_ws",
+                       L.total, (size_t)YSCV_HIP_STATIC_SCRATCH_BYTES);
+  }
+  return int4_run_ws(w, x_dev, x_dtype, y_dev, y_dtype, m, 0, EPI_STORE, ws, YSCV_HIP_STATIC_SCRATCH_BYTES, as_stream(stream));
 }
 
 int32_t yscv_hip_int4_workspace_bytes(const yscv_hip_int4_weight *w, size_t m, int32_t x_dtype, size_t *bytes) {

@@ -274,6 +274,16 @@ class PackedInt4Weight:
            _torch_dtype_code(out), _sz(m), _stream_ptr())
         return out
 
+    def matmul_static(self, x, out):
+        """yscv_hip_int4_matmul_static: scratch in the library's static device array, nothing allocated by the call
+        (`out` comes from the caller for the same reason)."""
+        assert x.is_cuda and out.is_cuda and x.is_contiguous() and out.is_contiguous() and x.shape[-1] == self.k
+        m = x.numel() // self.k
+        assert out.numel() == m * self.m_w
+        lib().int4_matmul_static(self._h, C.c_void_p(x.data_ptr()), _torch_dtype_code(x), C.c_void_p(out.data_ptr()),
+                                 _torch_dtype_code(out), _sz(m), _stream_ptr())
+        return out
+
     def matmul_fused(self, x, out, epilogue: int):
         """yscv_hip_int4_matmul_fused: skinny kernel (m <= 16) with the epilogue fused.  EPILOGUE_ADD_F32 adds into the
         f32 tensor `out` [m, m_w]; EPILOGUE_SWIGLU writes silu(gate) * up into `out` [m, m_w / 2]."""
