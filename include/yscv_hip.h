@@ -185,7 +185,10 @@ int32_t yscv_hip_int4_matmul_static(const yscv_hip_int4_weight *w, const void *x
  * packed_int4_gemm_dispatch  int4_matmul.rs:548-557
  * pack_int4_symmetric_per_group  int4_matmul.rs:611-616 (returns into caller buffers
  *   packed_out[m_w*k/2], scales_out[m_w*k/group_size])
- * dequantize_int4_to_f32     ops/quantize.rs:18 (output[2*n_bytes]) */
+ * dequantize_int4_to_f32     ops/quantize.rs:18 (output[2*n_bytes])
+ * quantize_f32_to_int4       ops/quantize.rs:69 (output[(len+1)/2]: q = clamp(round_ties_even(x / scale) + zp, -8, 7),
+ *   element 2i in the low nibble, |scale| <= f32::EPSILON quantises everything to zp); `_dev` is the same on device
+ *   pointers, asynchronous on `stream` */
 int32_t yscv_hip_packed_int4_gemv_dispatch(const uint8_t *weight_packed, const float *scales,
                                            const float *activation, float *output, size_t m_w,
                                            size_t k, size_t group_size);
@@ -197,6 +200,10 @@ int32_t yscv_hip_pack_int4_symmetric_per_group(const float *weights, size_t m_w,
                                                float *scales_out);
 int32_t yscv_hip_dequantize_int4_to_f32(const uint8_t *packed, size_t n_bytes, float scale,
                                         int8_t zero_point, float *output);
+int32_t yscv_hip_quantize_f32_to_int4(const float *data, size_t len, float scale, int8_t zero_point,
+                                      uint8_t *output);
+int32_t yscv_hip_quantize_f32_to_int4_dev(const float *data_dev, size_t len, float scale, int8_t zero_point,
+                                          uint8_t *out_dev, void *stream);
 
 /* ---- int8 GEMM ------------------------------------------------------------------ */
 
@@ -331,6 +338,29 @@ int32_t yscv_hip_exec_qlinear_matmul(const float *a_dev, float a_scale, float a_
  * operators one after the other; counted as one qlinear_matmul_fast. */
 int32_t yscv_hip_exec_qdq_matmul(const float *x_dev, size_t m, float a_scale, const yscv_hip_i8_weight *b,
                                  float b_scale, float y_scale, float y_zp, float *out_dev, void *stream);
+/* MatMulNBits (com.microsoft), the operator ONNX exporters emit for 4-bit weights: Y = A x dequant(B)^T + bias.  The
+ * reference's dispatcher has no such operator (crates/yscv-onnx/src/runner/dispatch.rs:191-322), so its int4 branch
+ * only ever sees weights it packed itself; here the initialisers of the node -- B [N][K/block][block/2] bytes, element
+ * 2i in the low nibble (the byte order of PackedInt4Weight, int4_matmul.rs:12-14), scales [N*K/block] f32 or f16,
+ * optional packed uint4 zero_points [N][ceil(K/block/2)], default 8 -- are uploaded once with
+ * yscv_hip_int4_weight_create(B, scales, dtype, zero_points, YSCV_HIP_NIBBLE_UNSIGNED, N, K, block) at load time, and
+ * the executor passes the node's attributes, which must agree with the handle (a mismatch is the runner's ShapeMismatch
+ * error; bits other than 4 is unsupported; g_idx is not supported).  a_dev is [m][K] with the leading dimensions of A
+ * flattened into m, bias_dev is null or [N] f32; with a bias the f32 product plus bias is rounded once to y_dtype.
+ * Kernel choice by m as in yscv_hip_int4_matmul; counted in int4_fast / int4_fallback. */
+int32_t yscv_hip_exec_matmul_nbits(const void *a_dev, int32_t a_dtype, size_t m, const yscv_hip_int4_weight *b,
+                                   const float *bias_dev, int64_t attr_k, int64_t attr_n, int64_t attr_bits,
+                                   int64_t attr_block_size, void *y_dev, int32_t y_dtype, void *stream);
+/* Gemm whose weight the int4 packing pass quantised (quantize_matmul_weights_int4_packed packs Gemm weights for both
+ * transB values, crates/yscv-onnx/src/quantize/packed_int4.rs:155-168, but exec_gemm never reads them,
+ * runner/linear.rs:5,228): Y = alpha * (A x W^T) + beta * C on f32 carriers with the int4 product in place of the f32
+ * one.  W is the handle yscv_hip_int4_weight_from_f32 made from the Gemm's B (either layout), a_dev is [m][K] (a transA
+ * node is transposed by the caller, as exec_gemm does first), c_dev is null (c_rows 0), one row of N values broadcast over
+ * the rows (c_rows 1) or [m][N] (c_rows m).  alpha and beta are applied only when they differ from 1 by more than
+ * f32::EPSILON, each as its own rounded multiply before the rounded add, like Tensor::scale + kernel_add
+ * (linear.rs:54-66). */
+int32_t yscv_hip_exec_gemm_int4(const float *a_dev, size_t m, const yscv_hip_int4_weight *b, const float *c_dev,
+                                size_t c_rows, float alpha, float beta, float *y_dev, void *stream);
 /* exec_quantize_linear, f32-carrier arm (crates/yscv-onnx/src/runner/misc.rs:42-80) =
  * quantize_linear_f32_to_f32_i8_scalar (crates/yscv-kernels/src/ops/quantize.rs:226-238). */
 int32_t yscv_hip_exec_quantize_linear(const float *x_dev, size_t len, float scale, float zero_point,

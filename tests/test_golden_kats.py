@@ -33,6 +33,7 @@ def test_oracle_nibbles_and_dequant(oracle):
         assert np.abs(out - np.array(c["expected"], np.float32)).max() <= c.get("tol", 0.0)
     for c in KATS["quantize_f32_to_int4"]["cases"]:
         packed = oracle.quantize_f32_to_int4(c["data"], c["scale"], c["zero_point"])
+        assert packed.size == (len(c["data"]) + 1) // 2
         assert oracle.dequantize_int4_to_f32(packed, 1.0, 0).tolist() == [float(v) for v in c["expected_nibbles"]]
 
 
@@ -88,6 +89,12 @@ def test_hip_library_matches_reference_kats():
         out = np.empty(2 * len(c["packed"]), np.float32)
         K.dequantize_int4_to_f32(np.array(c["packed"], np.uint8), c["scale"], c["zero_point"], out)
         assert np.abs(out - np.array(c["expected"], np.float32)).max() <= c.get("tol", 0.0)
+    for c in KATS["quantize_f32_to_int4"]["cases"]:
+        packed = np.full((len(c["data"]) + 1) // 2, 0xEE, np.uint8)
+        K.quantize_f32_to_int4(np.array(c["data"], np.float32), c["scale"], c["zero_point"], packed)
+        out = np.empty(2 * packed.size, np.float32)
+        K.dequantize_int4_to_f32(packed, 1.0, 0, out)
+        assert out.tolist() == [float(v) for v in c["expected_nibbles"]]
     for c in KATS["int4_gemv_hand"]["cases"]:
         out = np.zeros(c["m_w"], np.float32)
         K.packed_int4_gemv_dispatch(np.array(c["packed"], np.uint8), np.array(c["scales"], np.float32),

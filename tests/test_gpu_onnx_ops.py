@@ -282,3 +282,96 @@ def test_qdq_matmul_equals_the_three_operators(oracle, torch_cuda, ops, shape):
     chained = ops.exec_dequantize_linear(q_dev, torch.tensor([y_s], device="cuda"), torch.tensor([y_zp], device="cuda"))
     assert np.array_equal(got, chained.cpu().numpy())
     pre.close()
+
+
+# ---- MatMulNBits and the int4 Gemm ------------------------------------------------------------------------------
+@pytest.mark.parametrize("m,k,n,g,with_zp,sdt", [(1, 4096, 512, 32, False, "f32"), (5, 256, 48, 32, True, "f16"),
+                                                   (16, 1024, 300, 128, True, "f16"), (40, 512, 272, 64, False, "f32"),
+                                                   (3, 96, 20, 16, True, "f32"), (200, 1024, 256, 128, True, "f16")])
+def test_matmul_nbits_operator(oracle, torch_cuda, ops, m, k, n, g, with_zp, sdt):
+    """MatMulNBits = A x dequant(B)^T + bias on the node's initialisers (uint4 nibbles, per-block scales, optional
+    packed uint4 zero points), against the checker's dequantise-then-dot definition, within the int4 float bar."""
+    from gpu_util import int4_tolerances, pack_zero_points
+
+    torch = torch_cuda
+    rng = np.random.default_rng(m * 1000 + k + n)
+    b = rng.integers(0, 256, n * k // 2, dtype=np.uint8)
+    scales = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float16 if sdt == "f16" else np.float32)
+    zps = pack_zero_points(rng.integers(6, 11, (n, k // g))) if with_zp else None
+    w = ops.MatMulNBitsWeight(b, scales, zps, K=k, N=n, bits=4, block_size=g)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    ref = oracle.matmul_nbits(b, scales.astype(np.float32), zps, x, m, n, k, g)
+    bias = rng.standard_normal(n).astype(np.float32)
+    y = ops.exec_matmul_nbits(_dev(torch, x), w)
+    assert tuple(y.shape) == (m, n) and y.dtype == torch.float32
+    int4_tolerances(y.cpu().numpy(), ref, k, x)
+    yb = ops.exec_matmul_nbits(_dev(torch, x), w, bias=_dev(torch, bias))
+    assert np.array_equal(yb.cpu().numpy(), y.cpu().numpy() + bias[None, :])  # one f32 add on top of the product
+    # rank-3 activations, 16-bit types: [2][m][k] -> [2][m][n], rounded once after the bias
+    x3 = torch.from_numpy(np.stack([x, -x])).bfloat16().cuda()
+    y3 = ops.exec_matmul_nbits(x3, w, bias=_dev(torch, bias))
+    assert tuple(y3.shape) == (2, m, n) and y3.dtype == torch.bfloat16
+    xs = x3.float().cpu().numpy().reshape(2 * m, k)
+    ref3 = oracle.matmul_nbits(b, scales.astype(np.float32), zps, xs, 2 * m, n, k, g) + bias[None, :]
+    from gpu_util import bf16_round
+    got3 = y3.float().cpu().numpy().reshape(2 * m, n)
+    assert np.abs(got3 - bf16_round(ref3)).max() <= np.abs(ref3).max() * 2.0 ** -7
+    w.close()
+
+
+def test_matmul_nbits_attribute_errors(torch_cuda, ops):
+    import yscv_amd
+
+    torch = torch_cuda
+    rng = np.random.default_rng(3)
+    k, n, g = 128, 16, 32
+    w = ops.MatMulNBitsWeight(rng.integers(0, 256, n * k // 2, dtype=np.uint8), rng.uniform(0.01, 0.02, n * (k // g)).astype(np.float32),
+                              None, K=k, N=n, block_size=g)
+    x = torch.zeros(2, k, device="cuda")
+    for kw, frag in [(dict(K=256), "attributes K=256"), (dict(N=8), "N=8"), (dict(block_size=64), "block_size=64")]:
+        with pytest.raises(yscv_amd.YscvHipError, match=frag) as ei:
+            ops.exec_matmul_nbits(x, w, **kw)
+        assert ei.value.code == -1
+    with pytest.raises(yscv_amd.YscvHipError, match="only 4 is supported") as ei:
+        ops.exec_matmul_nbits(x, w, bits=8)
+    assert ei.value.code == -4
+    with pytest.raises(ValueError):
+        ops.MatMulNBitsWeight(np.zeros(8, np.uint8), np.zeros(1, np.float32), None, K=16, N=1, bits=2, block_size=16)
+    w.close()
+
+
+@pytest.mark.parametrize("m,k,n,g,nk", [(1, 256, 64, 32, True), (7, 512, 40, 64, False), (32, 1024, 128, 128, True)])
+def test_gemm_through_the_int4_branch(oracle, torch_cuda, ops, m, k, n, g, nk):
+    """Gemm(alpha, beta, C) whose B the int4 packing pass quantised (packed_int4.rs:155-168): the weight is packed on the
+    device from the f32 initialiser in either layout, the product equals the int4 matmul of the same weight, and alpha /
+    beta / C follow exec_gemm's order of operations (linear.rs:54-66) bit for bit."""
+    from gpu_util import int4_tolerances
+    from yscv_amd import kernels as K
+
+    torch = torch_cuda
+    rng = np.random.default_rng(m + k + n)
+    w_nk = rng.standard_normal((n, k)).astype(np.float32)
+    wt = _dev(torch, w_nk if nk else np.ascontiguousarray(w_nk.T))
+    w = K.PackedInt4Weight.from_f32(wt, g, transposed_nk=nk)
+    packed, scales = oracle.pack_int4_symmetric_per_group(w_nk.ravel(), n, k, g)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    ref = oracle.packed_int4_gemm_scalar(packed, scales, x, m, n, k, g).reshape(m, n)
+    a = _dev(torch, x)
+    prod = ops.exec_gemm_int4(a, w)
+    int4_tolerances(prod.cpu().numpy(), ref, k, x)
+    assert torch.equal(prod, w.matmul(a))
+    p = prod.cpu().numpy()
+    c_row = rng.standard_normal(n).astype(np.float32)
+    c_full = rng.standard_normal((m, n)).astype(np.float32)
+    for alpha, beta, c in [(1.0, 1.0, c_row), (0.5, 1.0, c_row), (1.0, 2.5, c_full), (-1.25, 0.3, c_full), (3.0, 1.0, None),
+                           (1.0 + 1e-8, 1.0, c_row)]:
+        got = ops.exec_gemm_int4(a, w, c=None if c is None else _dev(torch, c), alpha=alpha, beta=beta).cpu().numpy()
+        want = p.copy()
+        if abs(np.float32(alpha) - np.float32(1.0)) > np.finfo(np.float32).eps:
+            want = want * np.float32(alpha)
+        if c is not None:
+            add = c * np.float32(beta) if abs(np.float32(beta) - np.float32(1.0)) > np.finfo(np.float32).eps else c
+            want = want + (add[None, :] if add.ndim == 1 else add)
+        assert np.array_equal(got, want.astype(np.float32)), (alpha, beta)
+    with pytest.raises(ValueError):
+        ops.exec_gemm_int4(a, w, c=_dev(torch, np.zeros(n + 1, np.float32)))

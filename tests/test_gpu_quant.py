@@ -117,3 +117,35 @@ def test_measured_peaks_are_plausible(K):
     assert 3000.0 < r.value <= 8000.0, r.value
     assert 1000.0 < f.value <= 2500.0, f.value
     assert 2000.0 < i.value <= 5000.0, i.value
+
+
+def test_quantize_f32_to_int4_bit_exact(oracle, K):
+    """quantize_f32_to_int4 (ops/quantize.rs:69-95): ties-even rounding, clamp after the zero point, low nibble first,
+    odd tails, the epsilon-scale rule, NaN / inf -- host-pointer form and device-pointer form."""
+    import ctypes as C
+
+    import torch
+
+    from yscv_amd import lib
+
+    rng = np.random.default_rng(43)
+    base = np.concatenate([rng.uniform(-6, 6, 100001), np.arange(-9, 9) + 0.5, [np.nan, np.inf, -np.inf, 0.0, -0.0, 3e38, -3e38]])
+    for scale, zp in [(1.0, 0), (0.5, 3), (0.37, -4), (-0.8, 1), (1e-8, -2), (0.0, 5), (1e-30, 0)]:
+        v = base.astype(np.float32)
+        want = oracle.quantize_f32_to_int4(v, scale, zp)
+        got = np.full((v.size + 1) // 2, 0xEE, np.uint8)
+        K.quantize_f32_to_int4(v, scale, zp, got)
+        assert np.array_equal(got, want), (scale, zp)
+        x = torch.from_numpy(v).cuda()
+        out = torch.full(((v.size + 1) // 2 + 1,), 0xEE, dtype=torch.uint8, device="cuda")
+        lib().quantize_f32_to_int4_dev(C.c_void_p(x.data_ptr()), C.c_size_t(v.size), C.c_float(scale), C.c_int8(zp),
+                                       C.c_void_p(out.data_ptr()), None)
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy()[:-1], want) and int(out[-1]) == 0xEE
+    # round trip through dequantize_int4_to_f32 stays within one step (quantize.rs:739-757)
+    original = (np.arange(-8, 8) * 0.5).astype(np.float32)
+    packed = np.zeros(8, np.uint8)
+    K.quantize_f32_to_int4(original, 0.5, 0, packed)
+    rec = np.zeros(16, np.float32)
+    K.dequantize_int4_to_f32(packed, 0.5, 0, rec)
+    assert np.abs(rec - original).max() <= 0.5 + 1e-6

@@ -215,3 +215,39 @@ def test_fp16_bf16_bit_goldens(oracle):
     assert np.float16(v).view(np.uint16) == 0x3C01
     # f32 -> bf16 is RNE (tensor.rs:764-769): 1 + 2^-8 is a tie -> even (1.0); 1 + 3*2^-8 -> 1 + 2^-6
     assert oracle.f32_to_bf16_bits([1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8]).tolist() == [0x3F80, 0x3F82]
+
+
+def test_matmul_nbits_bridge_hand_vectors_and_default_zero_point(oracle):
+    """The MatMulNBits definition the checker composes from dequantize_int4_to_f32 (quantize.rs:215-222) and an f32 dot:
+    unsigned nibbles, value (q - zp) * scale, zero point 8 when none is given, group 2j in the low nibble of a
+    zero-point byte."""
+    # bytes [0xA9, 0x70]: nibbles 9, 10 | 0, 7; K = 4, block 2, scales 0.5 / 0.25, x = 1 2 3 4
+    b = np.array([0xA9, 0x70], np.uint8)
+    s = np.array([0.5, 0.25], np.float32)
+    x = np.array([[1.0, 2.0, 3.0, 4.0]], np.float32)
+    assert oracle.matmul_nbits(b, s, None, x, 1, 1, 4, 2).tolist() == [[-4.5]]        # zp 8: (1*1 + 2*2)/2 + (-8*3 - 1*4)/4
+    zps = np.array([0x79], np.uint8)                                                   # block 0: zp 9, block 1: zp 7
+    assert oracle.matmul_nbits(b, s, zps, x, 1, 1, 4, 2).tolist() == [[-4.25]]         # (0*1 + 1*2)/2 + (-7*3 + 0*4)/4
+    # zero point 8 everywhere = the reference kernel on byte ^ 0x88, up to the order of the scale multiplication
+    rng = np.random.default_rng(11)
+    m, n, k, g = 3, 10, 128, 32
+    bb = rng.integers(0, 256, n * k // 2, dtype=np.uint8)
+    sc = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float32)
+    xx = rng.standard_normal((m, k)).astype(np.float32)
+    ref = oracle.packed_int4_gemm_scalar(bb ^ 0x88, sc, xx, m, n, k, g).reshape(m, n)
+    got = oracle.matmul_nbits(bb, sc, None, xx, m, n, k, g)
+    assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max()
+    explicit = np.full((n, (k // g + 1) // 2), 0x88, np.uint8)
+    assert np.array_equal(oracle.matmul_nbits(bb, sc, explicit, xx, m, n, k, g), got)
+    # float64 definition with random zero points
+    zq = rng.integers(0, 16, (n, k // g))
+    zp = np.zeros((n, (k // g + 1) // 2), np.uint8)
+    for j in range(k // g):
+        zp[:, j // 2] |= (zq[:, j] << (4 * (j & 1))).astype(np.uint8)
+    q = np.empty((n, k))
+    pb = bb.reshape(n, k // 2)
+    q[:, 0::2], q[:, 1::2] = pb & 15, pb >> 4
+    w = (q - np.repeat(zq, g, axis=1)) * np.repeat(sc.reshape(n, k // g).astype(np.float64), g, axis=1)
+    want = xx.astype(np.float64) @ w.T
+    got = oracle.matmul_nbits(bb, sc, zp, xx, m, n, k, g)
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()

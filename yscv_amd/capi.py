@@ -90,6 +90,8 @@ _SIGNATURES = {
     "yscv_hip_packed_int4_gemm_dispatch": [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz],
     "yscv_hip_pack_int4_symmetric_per_group": [_vp, _sz, _sz, _sz, _vp, _vp],
     "yscv_hip_dequantize_int4_to_f32": [_vp, _sz, _f32, C.c_int8, _vp],
+    "yscv_hip_quantize_f32_to_int4": [_vp, _sz, _f32, C.c_int8, _vp],
+    "yscv_hip_quantize_f32_to_int4_dev": [_vp, _sz, _f32, C.c_int8, _vp, _vp],
     "yscv_hip_pack_i8_b_for_matmul": [_vp, _sz, _sz, C.POINTER(_vp)],
     "yscv_hip_i8_weight_destroy": [_vp],
     "yscv_hip_i8_weight_dims": [_vp, C.POINTER(_sz), C.POINTER(_sz)],
@@ -112,6 +114,8 @@ _SIGNATURES = {
     "yscv_hip_exec_qlinear_matmul": [_vp, _f32, _f32, _vp, _vp, _f32, _f32, _f32, _f32, _sz, _sz, _sz, _vp,
                                      C.POINTER(_i32), _vp],
     "yscv_hip_exec_qdq_matmul": [_vp, _sz, _f32, _vp, _f32, _f32, _f32, _vp, _vp],
+    "yscv_hip_exec_matmul_nbits": [_vp, _i32, _sz, _vp, _vp, C.c_int64, C.c_int64, C.c_int64, C.c_int64, _vp, _i32, _vp],
+    "yscv_hip_exec_gemm_int4": [_vp, _sz, _vp, _vp, _sz, _f32, _f32, _vp, _vp],
     "yscv_hip_exec_quantize_linear": [_vp, _sz, _f32, _f32, _vp, _vp],
     "yscv_hip_exec_dequantize_linear": [_vp, _sz, _sz, _sz, _vp, _vp, _sz, _vp, _vp],
     "yscv_hip_exec_dynamic_quantize_linear": [_vp, _sz, _vp, _vp, _vp, _vp],

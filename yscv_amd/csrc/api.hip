@@ -574,6 +574,26 @@ int32_t yscv_hip_pack_int4_symmetric_per_group(const float *weights, size_t m_w,
   return YSCV_HIP_OK;
 }
 
+int32_t yscv_hip_quantize_f32_to_int4_dev(const float *data_dev, size_t len, float scale, int8_t zero_point,
+                                          uint8_t *out_dev, void *stream) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(len == 0 || (data_dev && out_dev), "null argument");
+  return launch_quantize_f32_to_int4(data_dev, len, scale, (int)zero_point, out_dev, as_stream(stream));
+}
+
+int32_t yscv_hip_quantize_f32_to_int4(const float *data, size_t len, float scale, int8_t zero_point, uint8_t *output) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(len == 0 || (data && output), "null argument");
+  if (len == 0) return YSCV_HIP_OK;
+  DevBuf dx, dq;
+  YSCV_TRY(dx.alloc(len * sizeof(float)));
+  YSCV_TRY(dq.alloc((len + 1) / 2));
+  YSCV_HIP_TRY(hipMemcpy(dx.p, data, len * sizeof(float), hipMemcpyHostToDevice));
+  YSCV_TRY(launch_quantize_f32_to_int4(dx.as<float>(), len, scale, (int)zero_point, dq.as<uint8_t>(), nullptr));
+  YSCV_HIP_TRY(hipMemcpy(output, dq.p, (len + 1) / 2, hipMemcpyDeviceToHost));
+  return YSCV_HIP_OK;
+}
+
 int32_t yscv_hip_dequantize_int4_to_f32(const uint8_t *packed, size_t n_bytes, float scale, int8_t zero_point,
                                         float *output) {
   YSCV_TRY(ensure_context(nullptr));

@@ -118,6 +118,7 @@ int32_t launch_i8_gemm(const void *a, int a_is_u8, int a_zp, const yscv_hip_i8_w
 // ---- elementwise ---------------------------------------------------------------------
 int32_t launch_quantize_linear_i8(const float *x, size_t len, float scale, float zp, int8_t *out,
                                   hipStream_t s);
+int32_t launch_quantize_f32_to_int4(const float *x, size_t len, float scale, int zp, uint8_t *out, hipStream_t s);
 int32_t launch_requant(const int32_t *acc, size_t len, size_t c, const int32_t *corr,
                        const float *composite_v, float composite, float y_zp, int round_mode,
                        int lo, int hi, int relu, void *out, hipStream_t s);

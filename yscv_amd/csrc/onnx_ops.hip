@@ -201,6 +201,35 @@ struct Operand8 {
 
 bool is_int_in(float v, int lo, int hi) { return v == (float)(int)v && (int)v >= lo && (int)v <= hi; }
 
+// y[m][n] (f32) = (alpha != 1 ? y * alpha : y) + (beta != 1 ? c * beta : c), each multiply and add rounded on its own
+// like Tensor::scale followed by kernel_add in exec_gemm (crates/yscv-onnx/src/runner/linear.rs:54-66); c is null,
+// one row [n] broadcast over the rows, or [m][n].  c_rows: 0 none, 1 broadcast, m full.
+__global__ void gemm_post_kernel(float *__restrict__ y, size_t m, size_t n, const float *__restrict__ c, size_t c_rows,
+                                 float alpha, int use_alpha, float beta, int use_beta) {
+  const size_t total = m * n;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    float v = y[i];
+    if (use_alpha) v = __fmul_rn(v, alpha);
+    if (c) {
+      float a = c[c_rows == 1 ? i % n : i];
+      if (use_beta) a = __fmul_rn(a, beta);
+      v = __fadd_rn(v, a);
+    }
+    y[i] = v;
+  }
+}
+// out[m][n] (f32 / f16 / bf16) = acc[m][n] (f32) + bias[n]: the f32 sum is rounded once to the output type
+__global__ void bias_cast_kernel(const float *__restrict__ acc, size_t m, size_t n, const float *__restrict__ bias,
+                                 void *__restrict__ out, int out_dtype) {
+  const size_t total = m * n;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    const float v = __fadd_rn(acc[i], bias[i % n]);
+    if (out_dtype == YSCV_HIP_F32) static_cast<float *>(out)[i] = v;
+    else if (out_dtype == YSCV_HIP_F16) static_cast<_Float16 *>(out)[i] = (_Float16)v;
+    else static_cast<uint16_t *>(out)[i] = float_to_bf16_bits(v);
+  }
+}
+
 int32_t free_weight(yscv_hip_i8_weight *w) {
   if (!w) return YSCV_HIP_OK;
   if (w->frag) (void)hipFree(w->frag);
@@ -531,6 +560,61 @@ int32_t yscv_hip_exec_qdq_matmul(const float *x_dev, size_t m, float a_scale, co
   YSCV_TRY(st);
   YSCV_HIP_TRY(fe);
   g_qlinear_fast.fetch_add(1, std::memory_order_relaxed);
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_exec_matmul_nbits(const void *a_dev, int32_t a_dtype, size_t m, const yscv_hip_int4_weight *b,
+                                   const float *bias_dev, int64_t attr_k, int64_t attr_n, int64_t attr_bits,
+                                   int64_t attr_block_size, void *y_dev, int32_t y_dtype, void *stream) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(b != nullptr, "MatMulNBits: null weight handle");
+  if (attr_bits != 4) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "MatMulNBits: bits=%lld, only 4 is supported", (long long)attr_bits);
+  size_t n = 0, k = 0, g = 0;
+  YSCV_TRY(yscv_hip_int4_weight_dims(b, &n, &k, &g, nullptr));
+  YSCV_REQUIRE(attr_k > 0 && attr_n > 0 && (size_t)attr_k == k && (size_t)attr_n == n,
+               "MatMulNBits: attributes K=%lld N=%lld but the packed weight is [N=%zu][K=%zu]", (long long)attr_k,
+               (long long)attr_n, n, k);
+  YSCV_REQUIRE(attr_block_size > 0 && (size_t)attr_block_size == g,
+               "MatMulNBits: block_size=%lld but the packed weight has group size %zu", (long long)attr_block_size, g);
+  if (m == 0) return YSCV_HIP_OK;
+  YSCV_REQUIRE(a_dev && y_dev, "MatMulNBits: null A / Y pointer");
+  hipStream_t s = as_stream(stream);
+  if (bias_dev == nullptr) return yscv_hip_int4_matmul(b, a_dev, a_dtype, y_dev, y_dtype, m, stream);
+  // with a bias the product is kept in f32 until the bias is added, then rounded once to the output type
+  float *acc = nullptr;
+  const bool in_place = y_dtype == YSCV_HIP_F32;
+  if (in_place) acc = static_cast<float *>(y_dev);
+  else YSCV_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&acc), m * n * sizeof(float), s));
+  int32_t st = yscv_hip_int4_matmul(b, a_dev, a_dtype, acc, YSCV_HIP_F32, m, stream);
+  if (st == YSCV_HIP_OK) {
+    hipLaunchKernelGGL(bias_cast_kernel, dim3(grid_for(m * n)), dim3(256), 0, s, acc, m, n, bias_dev, y_dev, y_dtype);
+    if (hipGetLastError() != hipSuccess) st = set_error(YSCV_HIP_ERR_DEVICE, "MatMulNBits: bias kernel launch failed");
+  }
+  if (!in_place) {
+    const hipError_t fe = hipFreeAsync(acc, s);
+    YSCV_TRY(st);
+    YSCV_HIP_TRY(fe);
+  }
+  return st;
+}
+
+int32_t yscv_hip_exec_gemm_int4(const float *a_dev, size_t m, const yscv_hip_int4_weight *b, const float *c_dev,
+                                size_t c_rows, float alpha, float beta, float *y_dev, void *stream) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(b != nullptr, "Gemm: null weight handle");
+  size_t n = 0, k = 0, g = 0;
+  YSCV_TRY(yscv_hip_int4_weight_dims(b, &n, &k, &g, nullptr));
+  YSCV_REQUIRE(c_dev == nullptr ? c_rows == 0 : (c_rows == 1 || c_rows == m),
+               "Gemm: C must be absent, one row of N values or [M][N] (c_rows = %zu, m = %zu)", c_rows, m);
+  if (m == 0) return YSCV_HIP_OK;
+  YSCV_REQUIRE(a_dev && y_dev, "Gemm: null A / Y pointer");
+  YSCV_TRY(yscv_hip_int4_matmul(b, a_dev, YSCV_HIP_F32, y_dev, YSCV_HIP_F32, m, stream));
+  // exec_gemm scales only when |alpha - 1| (|beta - 1|) exceeds f32::EPSILON (linear.rs:54,58)
+  const int use_alpha = fabsf(alpha - 1.0f) > 1.1920929e-7f, use_beta = fabsf(beta - 1.0f) > 1.1920929e-7f;
+  if (!use_alpha && c_dev == nullptr) return YSCV_HIP_OK;
+  hipLaunchKernelGGL(gemm_post_kernel, dim3(grid_for(m * n)), dim3(256), 0, as_stream(stream), y_dev, m, n, c_dev, c_rows,
+                     alpha, use_alpha, beta, use_beta);
+  YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
 }
 

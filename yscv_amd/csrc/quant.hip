@@ -42,6 +42,39 @@ int32_t launch_quantize_linear_i8(const float *x, size_t len, float scale, float
   return YSCV_HIP_OK;
 }
 
+// quantize_f32_to_int4 (crates/yscv-kernels/src/ops/quantize.rs:69-95): q = clamp(round_ties_even(x * inv_scale) as
+// i32 + zp, -8, 7) with inv_scale = 1 / scale, or 0 when |scale| <= f32::EPSILON; element 2i in the low nibble, the
+// high nibble of an odd tail is 0.  `as i32` saturates and maps NaN to 0; the addition of zp wraps.
+__device__ __forceinline__ int quant_int4_one(float x, float inv_scale, int zp) {
+  const float r = rintf(__fmul_rn(x, inv_scale));
+  int32_t q;
+  if (r != r) q = 0;
+  else if (r >= 2147483648.0f) q = INT32_MAX;
+  else if (r <= -2147483648.0f) q = INT32_MIN;
+  else q = (int32_t)r;
+  q = (int32_t)((uint32_t)q + (uint32_t)zp);
+  return q < -8 ? -8 : (q > 7 ? 7 : q);
+}
+__global__ void quantize_int4_kernel(const float *__restrict__ x, size_t len, float inv_scale, int zp,
+                                     uint8_t *__restrict__ out) {
+  const size_t n_out = (len + 1) / 2;
+  for (size_t o = blockIdx.x * (size_t)blockDim.x + threadIdx.x; o < n_out; o += (size_t)gridDim.x * blockDim.x) {
+    const int q0 = quant_int4_one(x[2 * o], inv_scale, zp);
+    const int q1 = (2 * o + 1 < len) ? quant_int4_one(x[2 * o + 1], inv_scale, zp) : 0;
+    out[o] = (uint8_t)((q0 & 0x0F) | ((q1 & 0x0F) << 4));
+  }
+}
+
+int32_t launch_quantize_f32_to_int4(const float *x, size_t len, float scale, int zp, uint8_t *out, hipStream_t s) {
+  if (len == 0) return YSCV_HIP_OK;
+  const float inv_scale = fabsf(scale) > 1.1920929e-7f ? 1.0f / scale : 0.0f;  // host IEEE division, as the reference's
+  size_t blocks = ceil_div((len + 1) / 2, (size_t)256);
+  if (blocks > 16384) blocks = 16384;
+  hipLaunchKernelGGL(quantize_int4_kernel, dim3((unsigned)blocks), dim3(256), 0, s, x, len, inv_scale, zp, out);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
 __global__ void requant_kernel(const int32_t *__restrict__ acc, size_t len, size_t c,
                                const int32_t *__restrict__ corr, const float *__restrict__ composite_v,
                                float composite, float y_zp, int round_mode, float lo, float hi, int relu,

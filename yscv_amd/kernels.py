@@ -76,6 +76,13 @@ def dequantize_int4_to_f32(packed, scale, zero_point, output) -> None:
     lib().dequantize_int4_to_f32(_ptr(p), _sz(p.size), C.c_float(scale), C.c_int8(zero_point), _ptr(output))
 
 
+def quantize_f32_to_int4(data, scale, zero_point, output) -> None:
+    """ops/quantize.rs:69 -- output holds (len + 1) / 2 bytes."""
+    d = _np(data, np.float32)
+    assert output.dtype == np.uint8 and output.size >= (d.size + 1) // 2
+    lib().quantize_f32_to_int4(_ptr(d), _sz(d.size), C.c_float(scale), C.c_int8(zero_point), _ptr(output))
+
+
 def int8_matmul_dispatch(a, b, m, k, n, out) -> None:
     """int8_matmul.rs:2407 -- b is row-major [k][n]."""
     aa, bb = _np(a, np.int8), _np(b, np.int8)

@@ -149,6 +149,70 @@ def exec_qdq_matmul(x, a_scale, prepacked: PrepackedI8B, b_scale, y_scale, y_zp:
     return out
 
 
+class MatMulNBitsWeight:
+    """The initialisers of one MatMulNBits node (com.microsoft) uploaded once: B [N][K/block][block/2] uint8 (element 2i
+    in the low nibble), scales [N * K/block] float32 or float16, optional packed uint4 zero_points [N][ceil(K/block/2)]
+    (default 8).  Same byte order as the reference's PackedInt4Weight (int4_matmul.rs:12-14) with unsigned nibbles."""
+
+    def __init__(self, b, scales, zero_points, K: int, N: int, bits: int = 4, block_size: int = 32):
+        from .kernels import NIBBLE_UNSIGNED, PackedInt4Weight
+
+        if bits != 4:
+            raise ValueError("MatMulNBits: only bits = 4 is supported")
+        self.K, self.N, self.bits, self.block_size = int(K), int(N), int(bits), int(block_size)
+        self.weight = PackedInt4Weight(b, scales, block_size, N, K, zero_points=zero_points, nibble_format=NIBBLE_UNSIGNED)
+
+    def close(self):
+        self.weight.close()
+
+
+def exec_matmul_nbits(a, w: MatMulNBitsWeight, bias=None, out_dtype=None, *, K=None, N=None, bits=None, block_size=None):
+    """MatMulNBits executor: Y = A x dequant(B)^T (+ bias).  a: CUDA tensor [..., K] f32 / f16 / bf16; the attributes
+    default to the ones the weight was built with (a graph executor passes the node's own).  Output [..., N]."""
+    import torch
+
+    from .kernels import _torch_dtype_code
+
+    if not a.is_cuda or a.shape[-1] != w.K:
+        raise ValueError("a must be a CUDA tensor whose last dimension is K")
+    a = a.contiguous()
+    m = a.numel() // w.K
+    out = torch.empty(*a.shape[:-1], w.N, device=a.device, dtype=out_dtype or a.dtype)
+    if bias is not None:
+        bias = _dev_f32(bias, "bias")
+        if bias.numel() != w.N:
+            raise ValueError("bias must hold N values")
+    lib().exec_matmul_nbits(_p(a), _torch_dtype_code(a), _sz(m), w.weight.handle, _p(bias),
+                            C.c_int64(w.K if K is None else K), C.c_int64(w.N if N is None else N),
+                            C.c_int64(w.bits if bits is None else bits),
+                            C.c_int64(w.block_size if block_size is None else block_size), _p(out), _torch_dtype_code(out),
+                            _stream_ptr())
+    return out
+
+
+def exec_gemm_int4(a, w, c=None, alpha: float = 1.0, beta: float = 1.0):
+    """Gemm (transA = 0) whose weight the int4 packing pass quantised: alpha * (a x W^T) + beta * c on f32 carriers.
+    w: kernels.PackedInt4Weight (from_f32 of the Gemm's B in either layout); c: None, [N], [1][N] or [M][N]."""
+    import torch
+
+    a = _dev_f32(a, "a")
+    if a.dim() != 2 or int(a.shape[1]) != w.k:
+        raise ValueError("a must be [m][K]")
+    m = int(a.shape[0])
+    c_rows = 0
+    if c is not None:
+        c = _dev_f32(c, "c")
+        if c.numel() == w.m_w:
+            c_rows = 1
+        elif c.numel() == m * w.m_w:
+            c_rows = m
+        else:
+            raise ValueError("c must hold N or M * N values")
+    out = torch.empty(m, w.m_w, device=a.device, dtype=torch.float32)
+    lib().exec_gemm_int4(_p(a), _sz(m), w.handle, _p(c), _sz(c_rows), C.c_float(alpha), C.c_float(beta), _p(out), _stream_ptr())
+    return out
+
+
 def exec_quantize_linear(x, scale: float, zero_point: float = 0.0):
     """misc.rs:42-80 (f32-carrier arm): clamp(round_ties_even(x / scale + zp), -128, 127) as f32."""
     import torch
