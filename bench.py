@@ -78,6 +78,26 @@ def bench_decode(dec, torch, batch, steps, warmup, stream_ptr, persistent=False)
     return dt, s_ev.elapsed_time(e_ev) * 1e-3
 
 
+def check_single_launch(dec, torch, steps=8):
+    """The single-launch kernel against the multi-kernel path from the benchmark's own start state: the last step's
+    logits agree to 2e-2 of max|logit| (two implementations with different fp16 rounding points) and a token differs
+    only where the other path's logits of the two picks are within that difference.  Raises if not."""
+    import numpy as np
+
+    start = np.arange(1, 2, dtype=np.int32)
+    dec.reset(start, PREFILL)
+    dec.run(steps, use_graph=True)
+    tg, lg = dec.tokens(0, steps)[:, 0].copy(), dec.logits()[0].copy()
+    dec.reset(start, PREFILL)
+    dec.run(steps, persistent=True)
+    tp, lp = dec.tokens(0, steps)[:, 0].copy(), dec.logits()[0].copy()
+    same = bool(np.array_equal(tg, tp))
+    rel = float(np.abs(lg - lp).max() / np.abs(lg).max())
+    assert np.isfinite(lp).all() and (same or rel < 2e-2), "single-launch decode disagrees with the multi-kernel path"
+    assert not same or rel < 2e-2, "same tokens but logits differ by %g of max|logit|" % rel
+    return {"steps": steps, "tokens_equal_multi_kernel_path": same, "max_rel_logit_diff_last_step": round(rel, 6)}
+
+
 def bench_projections(dec, torch, batch, stream_ptr, reps=6):
     """Average duration of one skinny-kernel launch over the projections of whole decode steps."""
     import numpy as np
@@ -124,8 +144,7 @@ def cpu_baseline(cfg, seconds_budget=20.0):
     while len(times) < 3 or (time.perf_counter() - t_start < seconds_budget / 2 and len(times) < 15):
         times.append(one_pass(1))
     t1 = sorted(times)[len(times) // 2]
-    cores = os.cpu_count() or 1
-    nthreads = min(cores, 64)
+    model, usable, nthreads = host_cpu()
     one_pass(nthreads)
     tm = sorted(one_pass(nthreads) for _ in range(3))[1]
     paths = orc.simd_paths(g)
@@ -134,9 +153,137 @@ def cpu_baseline(cfg, seconds_budget=20.0):
         "sample": "projections of 1 of 32 layers + 1/8 of lm_head at batch 1, median of %d, extrapolated to a "
                   "full step; attention/norm glue not included (favours the CPU)" % len(times),
         "kernel": "restated packed_int4_gemv_dispatch -> " + paths["int4_gemv"],
-        "all_cores": {"value": round(1.0 / tm, 3), "threads": nthreads,
-                      "note": "N-row partition; not present in the reference for MatMul"},
+        "cpu_model": model,
+        "all_cores": {"value": round(1.0 / tm, 3), "threads": nthreads, "usable_logical_cpus": usable,
+                      "note": "one thread per physical core, N-row partition; not present in the reference for MatMul"},
+        "other_configs": cpu_baseline_kernels(),
     }
+
+
+def lcg_states(seed, n):
+    """s_1 .. s_n of s <- s * 6364136223846793005 + 1442695040888963407 (mod 2^64), the generator of the reference's
+    micro-benchmark (apps/llm-bench/src/bin/kernel_bench.rs:28-50), vectorised: s_i = a^i s_0 + c (1 + a + .. + a^(i-1))."""
+    import numpy as np
+
+    a, c = np.uint64(6364136223846793005), np.uint64(1442695040888963407)
+    with np.errstate(over="ignore"):
+        pw = np.multiply.accumulate(np.full(n, a, np.uint64))            # a^1 .. a^n (wraps mod 2^64)
+        geo = np.cumsum(np.concatenate([np.ones(1, np.uint64), pw[:-1]]))  # 1 + a + .. + a^(i-1)
+        return pw * np.uint64(seed) + c * geo
+
+
+def lcg_i8(seed, n):
+    import numpy as np
+
+    return ((lcg_states(seed, n) >> np.uint64(33)).astype(np.int64) % 256 - 128).astype(np.int8)
+
+
+def lcg_f32(seed, n):
+    import numpy as np
+
+    return ((lcg_states(seed, n) >> np.uint64(33)).astype(np.int64) % 2001 - 1000).astype(np.float32) * np.float32(0.001)
+
+
+def host_cpu():
+    """(model name, logical CPUs this process may use, physical cores among them)."""
+    model, cores = "unknown", set()
+    try:
+        phys = core = None
+        for line in open("/proc/cpuinfo"):
+            key, _, val = line.partition(":")
+            key, val = key.strip(), val.strip()
+            if key == "model name":
+                model = val
+            elif key == "physical id":
+                phys = val
+            elif key == "core id":
+                core = val
+            elif key == "processor":
+                cur = int(val)
+            if not line.strip() and phys is not None and core is not None:
+                cores.add((phys, core))
+                phys = core = None
+    except OSError:
+        pass
+    usable = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    physical = min(usable, len(cores)) if cores else usable
+    return model, usable, max(1, physical)
+
+
+def cpu_baseline_kernels(budget_s=12.0):
+    """The restated reference CPU kernels (runtime-dispatched AVX-512 / AVX2 / VNNI, oracle/yscv_cpu_simd.c) on the
+    stand-alone BASELINE configs, inputs from the reference micro-benchmark's generator and seeds
+    (kernel_bench.rs:159-160, 304-306, 343-345); one thread (what the reference runs) and all physical cores."""
+    import numpy as np
+
+    from oracle import oracle as orc
+
+    orc.build()
+    model, usable, physical = host_cpu()
+    out = {"cpu_model": model, "usable_logical_cpus": usable, "physical_cores_used": physical,
+           "kernels": orc.simd_paths(32)}
+
+    def med(fn, iters, warm=1):
+        for _ in range(warm):
+            fn()
+        ts = []
+        for _ in range(iters):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return sorted(ts)[len(ts) // 2]
+
+    # config 1: int4 GEMV 4096 x 4096, group 32 (kernel_bench bench_int4_gemv: weights 0x100, activation 0x200)
+    n = k = 4096
+    packed, scales = orc.pack_int4_symmetric_per_group(lcg_f32(0x100, n * k), n, k, 32)
+    x = lcg_f32(0x200, k)
+    byt = n * k // 2 + n * (k // 32) * 4 + k * 4 + n * 4
+    t1 = med(lambda: orc.simd_packed_int4_gemv_dispatch(packed, scales, x, n, k, 32), 20, 2)
+    tm = med(lambda: orc.simd_packed_int4_gemv_dispatch(packed, scales, x, n, k, 32, threads=physical), 20, 2)
+    out["config1_gemv_m1_k4096_n4096"] = {"us_1_thread": round(t1 * 1e6, 1), "GB/s_1_thread": round(byt / t1 / 1e9, 2),
+                                          "us_all_cores": round(tm * 1e6, 1), "GB/s_all_cores": round(byt / tm / 1e9, 2)}
+    # config 2: int8 GEMM 512 x 4096 x 4096 (bench_int8_gemm: A 0xAA, B 0xBB), prepacked dispatch
+    m, k, n = 512, 4096, 4096
+    a, b = lcg_i8(0xAA, m * k), lcg_i8(0xBB, k * n)
+    pb = orc.SimdPackedI8B(b, k, n)
+    ops = 2.0 * m * k * n
+    t1 = med(lambda: pb.matmul(a, m), 3)
+    tm = med(lambda: pb.matmul(a, m, threads=physical), 3)
+    out["config2_int8_m512_k4096_n4096"] = {"ms_1_thread": round(t1 * 1e3, 2), "GOP/s_1_thread": round(ops / t1 / 1e9, 1),
+                                            "ms_all_cores": round(tm * 1e3, 2), "GOP/s_all_cores": round(ops / tm / 1e9, 1),
+                                            "note": "M-row blocks over the cores (the split of runner/conv/quantized.rs:410-445; "
+                                                    "the reference's MatMul runs one thread)"}
+    del pb, a, b
+    # config 3: int4 GEMM 2048 x 4096 -> 14336, group 128: a 64-row sample of the 2048 rows (the kernel unpacks a group once
+    # and loops over the rows, so time grows linearly in M), symmetric weights (the reference kernel has no zero points)
+    m_full, m, k, n, g = 2048, 64, 4096, 14336, 128
+    rng = np.random.default_rng(3)
+    packed = rng.integers(0, 256, n * k // 2, dtype=np.uint8)
+    scales = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float32)
+    x = lcg_f32(0x300 + m, m * k)
+    fl = 2.0 * m * k * n
+    t1 = med(lambda: orc.simd_packed_int4_gemm_dispatch(packed, scales, x, m, n, k, g), 1, 0)
+    tm = med(lambda: orc.simd_packed_int4_gemm_dispatch(packed, scales, x, m, n, k, g, threads=physical), 2, 0)
+    out["config3_int4_prefill_m2048_k4096_n14336"] = {
+        "sample": "64 of the 2048 rows, full weight", "GFLOP/s_1_thread": round(fl / t1 / 1e9, 1),
+        "GFLOP/s_all_cores": round(fl / tm / 1e9, 1), "s_full_shape_1_thread_extrapolated": round(t1 * m_full / m, 2),
+        "s_full_shape_all_cores_extrapolated": round(tm * m_full / m, 2)}
+    # config 5: LM-head shape 4096 -> 128256, group 32: m = 1 (GEMV) and m = 16 (GEMM, the reference switches at m >= 8)
+    k, n, g = 4096, 128256, 32
+    packed = rng.integers(0, 256, n * k // 2, dtype=np.uint8)
+    scales = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float32)
+    wbytes = n * k // 2 + n * (k // g) * 4
+    x1, x16 = lcg_f32(0x200, k), lcg_f32(0x300 + 16, 16 * k)
+    t1 = med(lambda: orc.simd_packed_int4_gemv_dispatch(packed, scales, x1, n, k, g), 3)
+    tm = med(lambda: orc.simd_packed_int4_gemv_dispatch(packed, scales, x1, n, k, g, threads=physical), 3)
+    t16 = med(lambda: orc.simd_packed_int4_gemm_dispatch(packed, scales, x16, 16, n, k, g), 1, 0)
+    t16m = med(lambda: orc.simd_packed_int4_gemm_dispatch(packed, scales, x16, 16, n, k, g, threads=physical), 1, 0)
+    out["config5_lm_head_k4096_n128256"] = {
+        "m1": {"ms_1_thread": round(t1 * 1e3, 2), "weight_GB/s_1_thread": round(wbytes / t1 / 1e9, 2),
+               "ms_all_cores": round(tm * 1e3, 2), "weight_GB/s_all_cores": round(wbytes / tm / 1e9, 2)},
+        "m16": {"ms_1_thread": round(t16 * 1e3, 1), "GFLOP/s_1_thread": round(2.0 * 16 * k * n / t16 / 1e9, 1),
+                "ms_all_cores": round(t16m * 1e3, 1), "GFLOP/s_all_cores": round(2.0 * 16 * k * n / t16m / 1e9, 1)}}
+    return out
 
 
 def measured_peaks(torch):
@@ -324,6 +471,7 @@ def main():
     assert dec.weight_bytes() >= w_bytes
 
     persistent = args.batch == 1 and not args.graph_path
+    check = check_single_launch(dec, torch) if persistent else None
     dt, dt_events = bench_decode(dec, torch, args.batch, args.steps, args.warmup, stream_ptr, persistent=persistent)
     tok_s = args.batch * args.steps / dt
     kv_row_bytes = 2 * cfg["n_layers"] * cfg["n_kv_heads"] * cfg["head_dim"] * 2  # K + V bytes one cached position adds
@@ -367,12 +515,16 @@ def main():
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this benchmark (profiles/), scaled to this "
+                              "run's launch; not re-measured in this run",
             "kernel": kernel, "bytes_per_launch": int(bytes_per_launch), "avg_launch_us": round(launch_s * 1e6, 3),
             "launches_timed": launches,
         },
         "hbm_roofline_whole_step": {"ideal_ms": round(ideal_step_s * 1e3, 4), "frac": round(ideal_step_s / (dt / args.steps), 4),
                                     "bytes_weights": w_bytes, "bytes_kv_per_seq": kv_bytes_per_seq},
     }
+    if check is not None:
+        result["config"]["checked_before_timing"] = check
     extra = {}
     if not args.no_extra:
         n_proj = 4 * cfg["n_layers"] + 1

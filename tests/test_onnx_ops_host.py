@@ -42,3 +42,18 @@ def test_fast_switch_reads_the_environment():
         out = subprocess.run([sys.executable, "-c", code], cwd=ROOT, env=env, capture_output=True, text=True, timeout=300)
         assert out.returncode == 0, out.stderr
         assert out.stdout.strip().splitlines()[-1] == want, (val, out.stdout)
+
+
+def test_bench_lcg_equals_the_reference_generator(oracle):
+    """bench.py draws the stand-alone kernels' inputs from the reference micro-benchmark's generator
+    (apps/llm-bench/src/bin/kernel_bench.rs:28-50), vectorised; it must equal the sequential restatement."""
+    import numpy as np
+
+    import bench
+
+    for seed in (0xAA, 0xBB, 0x100, 0x200, 0x300 + 64, 7):
+        assert np.array_equal(bench.lcg_i8(seed, 5000), oracle.lcg_i8(seed, 5000))
+        assert np.array_equal(bench.lcg_f32(seed, 5000), oracle.lcg_f32(seed, 5000))
+    # first values by hand: s1 = seed * a + c (mod 2^64)
+    s1 = (0xAA * 6364136223846793005 + 1442695040888963407) % (1 << 64)
+    assert int(bench.lcg_i8(0xAA, 1)[0]) == ((s1 >> 33) % 256) - 128
