@@ -543,6 +543,17 @@ def main():
                                        "skinny_kernel_GB/s": round(w_bytes / n_proj / avg16 / 1e9, 1)}
     del dec
     torch.cuda.empty_cache()
+    if not args.no_extra and args.batch != 16:
+        # the same batch-16 run with the int8 KV cache (llm-bench --kv-dtype i8): half the cache bytes per step
+        dec8 = Decoder(kv_dtype="i8", **cfg)
+        dec8.init_random(seed=1)
+        dec8.fill_kv_random(seed=2)
+        dt8, _ = bench_decode(dec8, torch, 16, min(args.steps, 64), 4, stream_ptr)
+        extra["decode_batch16_kv_i8"] = {"tok/s": round(16 * min(args.steps, 64) / dt8, 1),
+                                         "ms_per_step": round(dt8 / min(args.steps, 64) * 1e3, 4),
+                                         "path": "one HIP-graph replay per step, int8 KV cache with one scale per position"}
+        del dec8
+        torch.cuda.empty_cache()
     if not args.no_extra:
         extra.update(extra_kernels(torch, stream_ptr))
         extra["measured_peaks"] = measured_peaks(torch)

@@ -434,6 +434,15 @@ typedef struct yscv_hip_decoder_config {
 #define YSCV_HIP_DEC_FINAL_NORM 2
 
 int32_t yscv_hip_decoder_create(const yscv_hip_decoder_config *cfg, yscv_hip_decoder **out);
+/* The same with the storage type of the KV cache chosen (llm-bench --kv-dtype, apps/llm-bench/src/main.rs:232-265;
+ * KvCache::with_dtype, crates/yscv-onnx/src/runner/kv_cache.rs:14-61).  I8: every appended K row and V row (the
+ * kv_dim = n_kv_heads * head_dim values of one position) is stored as int8 with one f32 scale, scale = absmax / 127
+ * (1.0 when absmax <= f32::EPSILON), q = clamp(round_half_away(v / scale), -127, 127), and attention reads q * scale;
+ * the current token attends to its own quantised row, as the reference's loop appends before it reads.  Half the
+ * cache bytes of fp16 per step.  Multi-kernel path only (use_graph 0 or 1). */
+#define YSCV_HIP_KV_F16 0
+#define YSCV_HIP_KV_I8 1
+int32_t yscv_hip_decoder_create_kv(const yscv_hip_decoder_config *cfg, int32_t kv_dtype, yscv_hip_decoder **out);
 int32_t yscv_hip_decoder_destroy(yscv_hip_decoder *d);
 /* Host inputs, borrowed: packed [n][k/2] uint4 nibbles (zero point 8, MatMulNBits order),
  * scales_f16 [n][k/group_size] fp16 bit patterns.  `layer` is ignored for LM_HEAD. */

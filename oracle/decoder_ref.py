@@ -79,11 +79,25 @@ def greedy_pick(row):
     return int(np.flatnonzero(row == row.max())[-1])
 
 
+def kv_i8_roundtrip(rows):
+    """rows [n][kv_dim] f32 -> what an int8 cache returns for them: per-row scale = absmax / 127, q = round half away
+    of v / scale clamped to +-127, value q * scale (LayerStorage::append / dequantise_to_vec,
+    crates/yscv-onnx/src/runner/kv_cache.rs:45-79), through the C restatement."""
+    from . import oracle as orc
+
+    rows = np.ascontiguousarray(rows, np.float32)
+    data, scales = orc.kv_i8_quantize_rows(rows, rows.shape[0], rows.shape[1])
+    return (data.reshape(rows.shape).astype(np.float32) * scales.reshape(-1, 1).astype(np.float32)).astype(np.float32)
+
+
 class RefDecoder:
-    def __init__(self, cfg: dict, linears: dict, norms: dict, emb16):
+    def __init__(self, cfg: dict, linears: dict, norms: dict, emb16, kv_i8: bool = False):
         """linears[(layer, kind)] = (packed, scales16) with kind in q k v o gate up down, and
-        linears[('lm_head',)]; norms[(layer, 'attn'|'ffn')], norms[('final',)] f32 gamma."""
+        linears[('lm_head',)]; norms[(layer, 'attn'|'ffn')], norms[('final',)] f32 gamma.
+        kv_i8: the cache stores per-row int8 (KvDtype::I8); the rotated key of a new token is then quantised from its f32
+        value, not from an fp16 rounding of it."""
         self.c = cfg
+        self.kv_i8 = kv_i8
         g = cfg["group_size"]
         D, hd = cfg["d_model"], cfg["head_dim"]
         hq, hkv, ff = cfg["n_heads"] * hd, cfg["n_kv_heads"] * hd, cfg["d_ff"]
@@ -101,8 +115,11 @@ class RefDecoder:
     def set_kv(self, layer, k_nat, v_nat):
         """k_nat / v_nat: f32 [batch][pos][kv_head][d] (keys already rotated)."""
         for b in range(k_nat.shape[0]):
-            self.kc[layer][b] = np.array(k_nat[b], np.float32)
-            self.vc[layer][b] = np.array(v_nat[b], np.float32)
+            kb, vb = np.array(k_nat[b], np.float32), np.array(v_nat[b], np.float32)
+            if self.kv_i8:
+                kb = kv_i8_roundtrip(kb.reshape(kb.shape[0], -1)).reshape(kb.shape)
+                vb = kv_i8_roundtrip(vb.reshape(vb.shape[0], -1)).reshape(vb.shape)
+            self.kc[layer][b], self.vc[layer][b] = kb, vb
 
     def _rmsnorm(self, h, gamma):
         return f16(rmsnorm(h, gamma, self.c["rms_eps"]))
@@ -129,9 +146,13 @@ class RefDecoder:
             qkv = np.zeros((B, (nh + 2 * nkv) * hd), np.float32)
             for b in range(B):
                 qr, kr = self._rope(q[b], pos), self._rope(k[b], pos)
-                qkv[b] = np.concatenate([qr.reshape(-1), kr.reshape(-1), v[b].reshape(-1)])
-                self.kc[l][b] = np.concatenate([self.kc[l][b][:pos], kr[None]], 0)
-                self.vc[l][b] = np.concatenate([self.vc[l][b][:pos], v[b][None]], 0)
+                k_row, v_row = kr, v[b]
+                if self.kv_i8:
+                    k_row = kv_i8_roundtrip(rope(k[b], pos, self.c["rope_theta"]).reshape(1, -1)).reshape(kr.shape)
+                    v_row = kv_i8_roundtrip(v[b].reshape(1, -1)).reshape(v[b].shape)
+                qkv[b] = np.concatenate([qr.reshape(-1), k_row.reshape(-1), v_row.reshape(-1)])
+                self.kc[l][b] = np.concatenate([self.kc[l][b][:pos], k_row[None]], 0)
+                self.vc[l][b] = np.concatenate([self.vc[l][b][:pos], v_row[None]], 0)
                 ao[b] = gqa_attend(qr, self.kc[l][b], self.vc[l][b], groups)
             ao = f16(ao.reshape(B, nh * hd))
             h = h + ao @ self.w[(l, "o")].T

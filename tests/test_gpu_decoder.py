@@ -9,14 +9,14 @@ CFG = dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, head_dim=128, d_ff=
            max_batch=3, max_ctx=256, max_steps=16, rope_theta=10000.0, rms_eps=1e-5)
 
 
-def _build(rng, cfg):
+def _build(rng, cfg, kv_dtype="f16"):
     from oracle.decoder_ref import RefDecoder
     from yscv_amd.decoder import Decoder
 
     D, hd, g = cfg["d_model"], cfg["head_dim"], cfg["group_size"]
     hq, hkv, ff = cfg["n_heads"] * hd, cfg["n_kv_heads"] * hd, cfg["d_ff"]
     shapes = {"q": (hq, D), "k": (hkv, D), "v": (hkv, D), "o": (D, hq), "gate": (ff, D), "up": (ff, D), "down": (D, ff)}
-    dec = Decoder(**cfg)
+    dec = Decoder(kv_dtype=kv_dtype, **cfg)
     linears, norms = {}, {}
     for l in range(cfg["n_layers"]):
         for kind, (n, k) in shapes.items():
@@ -38,7 +38,7 @@ def _build(rng, cfg):
     emb = rng.standard_normal((cfg["vocab"], D)).astype(np.float16)
     dec.set_embedding(emb)
     dec.finalize()
-    ref = RefDecoder(cfg, linears, norms, emb)
+    ref = RefDecoder(cfg, linears, norms, emb, kv_i8=kv_dtype == "i8")
     return dec, ref
 
 
@@ -72,6 +72,59 @@ def test_decode_steps_match_numpy(use_graph):
             row = got_logits[b]
             assert got_tok[b] == np.flatnonzero(row == row.max())[-1]
         cur = got_tok.copy()  # teacher-force the restatement with the GPU's picks
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_decode_with_int8_kv_cache_matches_numpy(use_graph):
+    """--kv-dtype i8 (apps/llm-bench/src/main.rs:232-265; KvCache I8 storage, kv_cache.rs:45-79): rows quantised on
+    append with one scale per position over all kv heads, attention over q * scale, against the checker in the same
+    mode.  The cache read back from the GPU holds exactly the checker's rows up to the rounding of the new keys."""
+    import torch
+
+    import yscv_amd
+
+    assert torch.cuda.is_available()
+    rng = np.random.default_rng(4300)
+    cfg = dict(CFG)
+    dec, ref = _build(rng, cfg, kv_dtype="i8")
+    B, prefill = 3, 133
+    for l in range(cfg["n_layers"]):
+        k = (rng.standard_normal((B, prefill, cfg["n_kv_heads"], cfg["head_dim"])) * 1.7).astype(np.float16)
+        v = rng.standard_normal((B, prefill, cfg["n_kv_heads"], cfg["head_dim"])).astype(np.float16)
+        dec.set_kv(l, k, v)
+        ref.set_kv(l, k.astype(np.float32), v.astype(np.float32))
+        gk, gv = dec.get_kv(l, B, 0, prefill)   # q * scale narrowed to fp16
+        for b in range(B):
+            assert np.abs(gk[b].astype(np.float32) - ref.kc[l][b]).max() <= 2.0 ** -10 * np.abs(ref.kc[l][b]).max()
+            assert np.abs(gv[b].astype(np.float32) - ref.vc[l][b]).max() <= 2.0 ** -10 * np.abs(ref.vc[l][b]).max()
+    tokens = np.array([5, 17, 300], np.int32)
+    dec.reset(tokens, prefill)
+    cur = tokens.copy()
+    for step in range(6):
+        dec.run(1, use_graph=use_graph)
+        got_logits = dec.logits()
+        got_tok = dec.tokens(step, 1)[0]
+        exp_logits = ref.step(cur, prefill + step)
+        err = np.abs(got_logits - exp_logits).max() / np.abs(exp_logits).max()
+        assert err < 2e-2, (step, err)
+        for b in range(B):
+            row = got_logits[b]
+            assert got_tok[b] == np.flatnonzero(row == row.max())[-1]
+        cur = got_tok.copy()
+    # appended rows: the GPU's cache against the checker's (a one-step difference of a quantised value at most, where
+    # sincosf and numpy disagree in the last bit of a rotated key)
+    L = cfg["n_layers"] - 1
+    gk, gv = dec.get_kv(L, B, prefill, 6)
+    for b in range(B):
+        rk, rv = ref.kc[L][b][prefill:], ref.vc[L][b][prefill:]
+        step_k = np.abs(rk).reshape(6, -1).max(1) / 127.0
+        assert (np.abs(gk[b].astype(np.float32) - rk).reshape(6, -1).max(1) <= 1.01 * step_k + 2.0 ** -10 * np.abs(rk).max()).all()
+        step_v = np.abs(rv).reshape(6, -1).max(1) / 127.0
+        assert (np.abs(gv[b].astype(np.float32) - rv).reshape(6, -1).max(1) <= 1.01 * step_v + 2.0 ** -10 * np.abs(rv).max()).all()
+    # the single-launch kernel reads an fp16 cache only
+    dec.reset(tokens[:1], prefill)
+    with pytest.raises(yscv_amd.YscvHipError, match="fp16 KV cache only"):
+        dec.run(1, persistent=True)
 
 
 def test_graph_replay_equals_eager():

@@ -182,6 +182,49 @@ def test_multi_kernel_batch16_at_7b_widths_matches_numpy(two_layers, oracle):
     assert np.array_equal(dec.logits(), graph_logits)
 
 
+def test_multi_kernel_int8_cache_at_7b_widths_matches_numpy(two_layers):
+    """The int8 KV cache (--kv-dtype i8) at the 7B-shape widths, four sequences beyond 2048 cached positions, against
+    the checker in its int8 mode; the weights are the fixture's."""
+    from oracle.decoder_ref import RefDecoder
+    from yscv_amd.decoder import Decoder
+
+    cfg, _, ref16, linears = two_layers
+    cfg = dict(cfg, max_batch=4)
+    D, hd = cfg["d_model"], cfg["head_dim"]
+    hq, hkv, ff = cfg["n_heads"] * hd, cfg["n_kv_heads"] * hd, cfg["d_ff"]
+    shapes = {"q": (hq, D), "k": (hkv, D), "v": (hkv, D), "o": (D, hq), "gate": (ff, D), "up": (ff, D), "down": (D, ff)}
+    dec = Decoder(kv_dtype="i8", **cfg)
+    for (key, (p, s)) in linears.items():
+        if key == ("lm_head",):
+            dec.set_linear(0, "lm_head", p, s, cfg["vocab"], D)
+        else:
+            dec.set_linear(key[0], key[1], p, s, *shapes[key[1]])
+    for key, g in ref16.norms.items():
+        dec.set_norm(0 if key == ("final",) else key[0], "final" if key == ("final",) else key[1], g)
+    emb16 = ref16.emb.astype(np.float16)
+    dec.set_embedding(emb16)
+    dec.finalize()
+    ref = RefDecoder(cfg, linears, ref16.norms, emb16, kv_i8=True)
+    rng = np.random.default_rng(7100)
+    B = cfg["max_batch"]
+    for l in range(cfg["n_layers"]):
+        k = (rng.standard_normal((B, PREFILL, cfg["n_kv_heads"], hd), dtype=np.float32) * 1.5).astype(np.float16)
+        v = rng.standard_normal((B, PREFILL, cfg["n_kv_heads"], hd), dtype=np.float32).astype(np.float16)
+        dec.set_kv(l, k, v)
+        ref.set_kv(l, k.astype(np.float32), v.astype(np.float32))
+    tokens = np.array([11, 2222, 13333, 31999], np.int32)
+    dec.reset(tokens, PREFILL)
+    cur = tokens.copy()
+    for step in range(3):
+        dec.run(1, use_graph=True)
+        got_logits, got_tok = dec.logits(), dec.tokens(step, 1)[0]
+        exp = ref.step(cur, PREFILL + step)
+        worst = _check_rows(got_logits, got_tok, exp, f"int8 cache step {step}")
+        print(f"[7b widths, int8 cache] step {step}: worst row rel err {worst:.2e}", flush=True)
+        cur = got_tok.copy()
+    dec.close()
+
+
 @pytest.mark.parametrize("nibbles", [(0, 15), (1, 15)], ids=["benchmark-init", "symmetric-init"])
 def test_full_depth_single_launch_agrees_with_multi_kernel_path(nibbles):
     """32 layers, random init, cache filled to beyond 2000 positions: 16 steps.  The benchmark's init (nibbles 0..15)

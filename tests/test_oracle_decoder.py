@@ -292,3 +292,41 @@ def test_ref_decoder_set_kv_and_overwrite_at_pos():
     la2 = a.step(np.array([toks[2]]), 2)  # position 2 again: the old entry is replaced, not appended to
     np.testing.assert_array_equal(la2, la)
     assert a.kc[0][0].shape[0] == 3
+
+
+# ---- int8 cache mode of the checker (KvCache with KvDtype::I8, crates/yscv-onnx/src/runner/kv_cache.rs:45-79) ---------
+def test_kv_i8_roundtrip_hand_vector_and_bounds(oracle):
+    # kv_cache.rs:321-358 holds a bound test (|error| <= scale); a hand vector on top: absmax 2.54 -> scale 0.02,
+    # 1.27 -> 63.5 -> 64 (half away from zero, round_ties_even would give 64 too), 0.25 -> 12.5 -> 13, -0.01 -> -0.5 -> -1
+    row = np.array([[2.54, 1.27, 0.25, -0.01, 0.0, -2.54]], np.float32)
+    got = R.kv_i8_roundtrip(row)
+    scale = np.float32(2.54) / np.float32(127.0)
+    np.testing.assert_allclose(got[0], np.array([127, 64, 13, -1, 0, -127], np.float32) * scale, rtol=1e-6)
+    rng = np.random.default_rng(9)
+    rows = (rng.standard_normal((7, 256)) * rng.uniform(0.1, 30, (7, 1))).astype(np.float32)
+    back = R.kv_i8_roundtrip(rows)
+    step = np.abs(rows).max(1, keepdims=True) / 127.0
+    assert (np.abs(back - rows) <= step * 0.5 * (1 + 1e-5)).all()      # the scale is per row, not per tensor or per head
+    assert np.array_equal(R.kv_i8_roundtrip(np.zeros((2, 8), np.float32)), np.zeros((2, 8), np.float32))
+
+
+def test_ref_decoder_kv_i8_quantises_rows_over_all_kv_heads():
+    rng = np.random.default_rng(10)
+    cfg = dict(CFG)
+    lin, norms, emb, _ = _tiny_model(rng, cfg)
+    a = R.RefDecoder(cfg, lin, norms, emb, kv_i8=True)
+    f = R.RefDecoder(cfg, lin, norms, emb)
+    la, lf = a.step(np.array([5]), 0), f.step(np.array([5]), 0)
+    for l in range(cfg["n_layers"]):
+        for cache in (a.kc[l][0], a.vc[l][0]):
+            row = cache[0].reshape(-1)                                   # one position, both kv heads: one scale
+            scale = np.abs(row).max() / 127.0
+            q = row / scale
+            assert np.abs(q - np.round(q)).max() < 1e-3 and np.abs(q).max() <= 127.0 + 1e-3
+    # quantisation noise of a few 1e-3 of the value range, not a different computation
+    assert 0 < np.abs(la - lf).max() < 0.05 * np.abs(lf).max()
+    # a cache loaded with set_kv is quantised the same way
+    b = R.RefDecoder(cfg, lin, norms, emb, kv_i8=True)
+    k = rng.standard_normal((1, 3, cfg["n_kv_heads"], cfg["head_dim"])).astype(np.float32)
+    b.set_kv(0, k, k)
+    np.testing.assert_array_equal(b.kc[0][0].reshape(3, -1), R.kv_i8_roundtrip(k[0].reshape(3, -1)))

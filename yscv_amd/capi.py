@@ -123,6 +123,7 @@ _SIGNATURES = {
     "yscv_hip_kv_i8_quantize_rows": [_vp, _sz, _sz, _vp, _vp, _vp],
     "yscv_hip_kv_i8_dequantize_rows": [_vp, _vp, _sz, _sz, _vp, _vp],
     "yscv_hip_decoder_create": [_vp, C.POINTER(_vp)],
+    "yscv_hip_decoder_create_kv": [_vp, _i32, C.POINTER(_vp)],
     "yscv_hip_decoder_destroy": [_vp],
     "yscv_hip_decoder_set_linear": [_vp, _i32, _i32, _vp, _vp, _sz, _sz],
     "yscv_hip_decoder_set_norm": [_vp, _i32, _i32, _vp],

@@ -98,7 +98,9 @@ struct yscv_hip_decoder {
   struct Layer {
     yscv_hip_int4_weight *wqkv = nullptr, *wo = nullptr, *wgu = nullptr, *wdown = nullptr;
     float *attn_norm = nullptr, *ffn_norm = nullptr;
-    _Float16 *kc = nullptr, *vc = nullptr;
+    _Float16 *kc = nullptr, *vc = nullptr;   // fp16 cache
+    int8_t *kc8 = nullptr, *vc8 = nullptr;   // int8 cache (kv_dtype I8) ...
+    float *ks = nullptr, *vs = nullptr;      // ... with one scale per (batch row, position)
     HostLinear stage[7];  // q k v o gate up down, kept until finalize
   };
   std::vector<Layer> layers;
@@ -112,6 +114,7 @@ struct yscv_hip_decoder {
   size_t ws_bytes = 0;
   int32_t *tokens = nullptr, *history = nullptr, *pos = nullptr, *step = nullptr;
   int batch = 0;
+  int kv_dtype = YSCV_HIP_KV_F16;
   bool finalized = false;
   hipGraph_t graph = nullptr;
   hipGraphExec_t graph_exec = nullptr;
@@ -153,6 +156,10 @@ static void decoder_free(yscv_hip_decoder *d) {
     (void)hipFree(L.ffn_norm);
     (void)hipFree(L.kc);
     (void)hipFree(L.vc);
+    (void)hipFree(L.kc8);
+    (void)hipFree(L.vc8);
+    (void)hipFree(L.ks);
+    (void)hipFree(L.vs);
   }
   destroy_int4(d->lm_head);
   (void)hipFree(d->final_norm);
@@ -198,6 +205,7 @@ static int32_t persist_setup(yscv_hip_decoder *d) {
   YSCV_TRY(ensure_context(&ctx));
   const auto &c = d->cfg;
   const char *why = "";
+  if (d->kv_dtype != YSCV_HIP_KV_F16) return YSCV_HIP_OK;  // the single-launch kernel reads an fp16 cache only
   if (!persist_supported(c, ctx->num_cus, &why)) return YSCV_HIP_OK;  // the multi-kernel path remains
   PersistModel &m = d->pm;
   persist_fill_phases(c, ctx->num_cus, &m);
@@ -382,10 +390,17 @@ static int32_t enqueue_step(yscv_hip_decoder *d, int batch, hipStream_t s) {
   for (auto &L : d->layers) {
     YSCV_TRY(launch_rmsnorm(d->h, L.attn_norm, batch, D, c.rms_eps, d->xn, s));
     YSCV_TRY(int4_run_ws(L.wqkv, d->xn, YSCV_HIP_F16, d->qkv, YSCV_HIP_F16, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s));
-    YSCV_TRY(launch_rope_append(d->qkv, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_theta, c.max_ctx,
-                                L.kc, L.vc, s));
-    YSCV_TRY(launch_attention(d->qkv, L.kc, L.vc, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim, c.max_ctx,
-                              d->attn_part, d->ao, s));
+    if (d->kv_dtype == YSCV_HIP_KV_I8) {
+      YSCV_TRY(launch_rope_append_i8(d->qkv, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_theta, c.max_ctx,
+                                     L.kc8, L.ks, L.vc8, L.vs, s));
+      YSCV_TRY(launch_attention_i8(d->qkv, L.kc8, L.ks, L.vc8, L.vs, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim,
+                                   c.max_ctx, d->attn_part, d->ao, s));
+    } else {
+      YSCV_TRY(launch_rope_append(d->qkv, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_theta, c.max_ctx,
+                                  L.kc, L.vc, s));
+      YSCV_TRY(launch_attention(d->qkv, L.kc, L.vc, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim, c.max_ctx,
+                                d->attn_part, d->ao, s));
+    }
     YSCV_TRY(int4_run_ws(L.wo, d->ao, YSCV_HIP_F16, d->h, YSCV_HIP_F32, batch, 1, EPI_ADD_F32, d->ws, d->ws_bytes, s));
     YSCV_TRY(launch_rmsnorm(d->h, L.ffn_norm, batch, D, c.rms_eps, d->xn, s));
     YSCV_TRY(int4_run_ws(L.wgu, d->xn, YSCV_HIP_F16, d->act, YSCV_HIP_F16, batch, 1, EPI_SWIGLU, d->ws, d->ws_bytes, s));
@@ -412,8 +427,13 @@ static int32_t check_persist_abort(yscv_hip_decoder *d) {
 extern "C" {
 
 int32_t yscv_hip_decoder_create(const yscv_hip_decoder_config *cfg, yscv_hip_decoder **out) {
+  return yscv_hip_decoder_create_kv(cfg, YSCV_HIP_KV_F16, out);
+}
+
+int32_t yscv_hip_decoder_create_kv(const yscv_hip_decoder_config *cfg, int32_t kv_dtype, yscv_hip_decoder **out) {
   YSCV_TRY(ensure_context(nullptr));
   YSCV_REQUIRE(cfg && out, "null argument");
+  YSCV_REQUIRE(kv_dtype == YSCV_HIP_KV_F16 || kv_dtype == YSCV_HIP_KV_I8, "unknown KV cache dtype %d", kv_dtype);
   *out = nullptr;
   const auto &c = *cfg;
   YSCV_REQUIRE(c.n_layers > 0 && c.d_model > 0 && c.n_heads > 0 && c.n_kv_heads > 0 && c.d_ff > 0 && c.vocab > 0,
@@ -429,6 +449,7 @@ int32_t yscv_hip_decoder_create(const yscv_hip_decoder_config *cfg, yscv_hip_dec
   YSCV_REQUIRE(c.rms_eps > 0.0f, "rms_eps must be finite and > 0 (ops/norm.rs:1471)");
   auto *d = new yscv_hip_decoder();
   d->cfg = c;
+  d->kv_dtype = kv_dtype;
   d->layers.resize(c.n_layers);
   int32_t st = alloc_runtime(d);
   const size_t D = c.d_model;
@@ -436,10 +457,22 @@ int32_t yscv_hip_decoder_create(const yscv_hip_decoder_config *cfg, yscv_hip_dec
     if (st != YSCV_HIP_OK) break;
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&L.attn_norm), D * 4);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&L.ffn_norm), D * 4);
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&L.kc), kv_elems(c) * 2);
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&L.vc), kv_elems(c) * 2);
-    if (e == hipSuccess) e = hipMemset(L.kc, 0, kv_elems(c) * 2);
-    if (e == hipSuccess) e = hipMemset(L.vc, 0, kv_elems(c) * 2);
+    if (kv_dtype == YSCV_HIP_KV_I8) {
+      const size_t rows = (size_t)c.max_batch * c.max_ctx;
+      if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&L.kc8), kv_elems(c));
+      if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&L.vc8), kv_elems(c));
+      if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&L.ks), rows * 4);
+      if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&L.vs), rows * 4);
+      if (e == hipSuccess) e = hipMemset(L.kc8, 0, kv_elems(c));
+      if (e == hipSuccess) e = hipMemset(L.vc8, 0, kv_elems(c));
+      if (e == hipSuccess) e = hipMemset(L.ks, 0, rows * 4);
+      if (e == hipSuccess) e = hipMemset(L.vs, 0, rows * 4);
+    } else {
+      if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&L.kc), kv_elems(c) * 2);
+      if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&L.vc), kv_elems(c) * 2);
+      if (e == hipSuccess) e = hipMemset(L.kc, 0, kv_elems(c) * 2);
+      if (e == hipSuccess) e = hipMemset(L.vc, 0, kv_elems(c) * 2);
+    }
     if (e != hipSuccess)
       st = set_error(e == hipErrorOutOfMemory ? YSCV_HIP_ERR_OOM : YSCV_HIP_ERR_DEVICE, "layer allocation failed: %s",
                      hipGetErrorString(e));
@@ -610,9 +643,15 @@ int32_t yscv_hip_decoder_init_random_range(yscv_hip_decoder *d, uint64_t seed, i
 int32_t yscv_hip_decoder_fill_kv_random(yscv_hip_decoder *d, uint64_t seed) {
   YSCV_REQUIRE(d != nullptr, "null decoder");
   uint64_t sd = seed * 0x9E3779B1ull + 7;
+  const size_t rows = (size_t)d->cfg.max_batch * d->cfg.max_ctx;
   for (auto &L : d->layers) {
-    YSCV_TRY(launch_kv_random_fill(L.kc, kv_elems(d->cfg), sd++, nullptr));
-    YSCV_TRY(launch_kv_random_fill(L.vc, kv_elems(d->cfg), sd++, nullptr));
+    if (d->kv_dtype == YSCV_HIP_KV_I8) {  // bytes uniform in [-127, 127], scale 3.5 / 127: values span about +-3.5
+      YSCV_TRY(launch_kv_random_fill_i8(L.kc8, kv_elems(d->cfg), L.ks, rows, 3.5f / 127.0f, sd++, nullptr));
+      YSCV_TRY(launch_kv_random_fill_i8(L.vc8, kv_elems(d->cfg), L.vs, rows, 3.5f / 127.0f, sd++, nullptr));
+    } else {
+      YSCV_TRY(launch_kv_random_fill(L.kc, kv_elems(d->cfg), sd++, nullptr));
+      YSCV_TRY(launch_kv_random_fill(L.vc, kv_elems(d->cfg), sd++, nullptr));
+    }
   }
   DEC_HIP(hipDeviceSynchronize());
   return YSCV_HIP_OK;
@@ -632,8 +671,12 @@ int32_t yscv_hip_decoder_set_kv(yscv_hip_decoder *d, int32_t layer, const uint16
   DEC_HIP(hipMemcpy(dk.p, k_f16, elems * 2, hipMemcpyHostToDevice));
   DEC_HIP(hipMemcpy(dv.p, v_f16, elems * 2, hipMemcpyHostToDevice));
   auto &L = d->layers[layer];
-  YSCV_TRY(launch_kv_relayout(dk.as<_Float16>(), dv.as<_Float16>(), batch, n_positions, c.n_kv_heads, c.head_dim,
-                              c.max_ctx, L.kc, L.vc, nullptr));
+  if (d->kv_dtype == YSCV_HIP_KV_I8)
+    YSCV_TRY(launch_kv_relayout_i8(dk.as<_Float16>(), dv.as<_Float16>(), batch, n_positions, c.n_kv_heads, c.head_dim,
+                                   c.max_ctx, L.kc8, L.ks, L.vc8, L.vs, nullptr));
+  else
+    YSCV_TRY(launch_kv_relayout(dk.as<_Float16>(), dv.as<_Float16>(), batch, n_positions, c.n_kv_heads, c.head_dim,
+                                c.max_ctx, L.kc, L.vc, nullptr));
   DEC_HIP(hipDeviceSynchronize());
   return YSCV_HIP_OK;
 }
@@ -650,8 +693,31 @@ int32_t yscv_hip_decoder_get_kv(yscv_hip_decoder *d, int32_t layer, uint16_t *k_
   DEC_HIP(hipDeviceSynchronize());
   const int hd = c.head_dim, hkv = c.n_kv_heads;
   const int s0 = first_pos / 8, s1 = (first_pos + n_positions + 7) / 8;  // 8-position slabs of the V layout
-  std::vector<uint16_t> kt((size_t)n_positions * hd), vt((size_t)(s1 - s0) * hd * 8);
   const auto &L = d->layers[layer];
+  if (d->kv_dtype == YSCV_HIP_KV_I8) {  // q * scale of its row (dequantise_to_vec, kv_cache.rs:64-79), narrowed to fp16
+    std::vector<int8_t> k8((size_t)n_positions * hd), v8((size_t)(s1 - s0) * hd * 8);
+    std::vector<float> ksc(n_positions), vsc(n_positions);
+    for (int b = 0; b < batch; b++) {
+      DEC_HIP(hipMemcpy(ksc.data(), L.ks + (size_t)b * c.max_ctx + first_pos, (size_t)n_positions * 4, hipMemcpyDeviceToHost));
+      DEC_HIP(hipMemcpy(vsc.data(), L.vs + (size_t)b * c.max_ctx + first_pos, (size_t)n_positions * 4, hipMemcpyDeviceToHost));
+      for (int h = 0; h < hkv; h++) {
+        const size_t row = (size_t)b * hkv + h;
+        DEC_HIP(hipMemcpy(k8.data(), L.kc8 + (row * c.max_ctx + first_pos) * hd, k8.size(), hipMemcpyDeviceToHost));
+        DEC_HIP(hipMemcpy(v8.data(), L.vc8 + ((row * (c.max_ctx / 8) + s0) * hd) * 8, v8.size(), hipMemcpyDeviceToHost));
+        for (int p = 0; p < n_positions; p++) {
+          _Float16 *kd = reinterpret_cast<_Float16 *>(k_f16) + (((size_t)b * n_positions + p) * hkv + h) * hd;
+          _Float16 *vd = reinterpret_cast<_Float16 *>(v_f16) + (((size_t)b * n_positions + p) * hkv + h) * hd;
+          const int ap = first_pos + p;
+          for (int i = 0; i < hd; i++) {
+            kd[i] = (_Float16)((float)k8[(size_t)p * hd + i] * ksc[p]);
+            vd[i] = (_Float16)((float)v8[((size_t)(ap / 8 - s0) * hd + i) * 8 + (ap & 7)] * vsc[p]);
+          }
+        }
+      }
+    }
+    return YSCV_HIP_OK;
+  }
+  std::vector<uint16_t> kt((size_t)n_positions * hd), vt((size_t)(s1 - s0) * hd * 8);
   for (int b = 0; b < batch; b++)
     for (int h = 0; h < hkv; h++) {
       const size_t row = (size_t)b * hkv + h;
@@ -697,6 +763,8 @@ int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_g
   YSCV_REQUIRE(step + n_steps <= d->cfg.max_steps, "token history overflow: %d + %d > max_steps %d", step, n_steps,
                d->cfg.max_steps);
   if (use_graph == 2) {
+    if (d->kv_dtype != YSCV_HIP_KV_F16)
+      return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the single-launch decode path reads an fp16 KV cache only");
     if (!d->persist_ok)
       return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the single-launch decode path does not support this model shape");
     if (d->batch != 1) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the single-launch decode path runs batch 1 only");

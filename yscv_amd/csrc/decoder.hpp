@@ -16,6 +16,16 @@ int32_t launch_kv_relayout(const _Float16 *k_nat, const _Float16 *v_nat, int bat
 int32_t launch_attention(const _Float16 *qkv, const _Float16 *kc, const _Float16 *vc, const int32_t *pos_ptr,
                          int batch, int hq, int hkv, int hd, int max_ctx, float *part, _Float16 *out,
                          hipStream_t s);
+// int8 cache (KvCache with KvDtype::I8): K int8 [batch][kv_head][max_ctx][128], V int8 [batch][kv_head][max_ctx/8][128][8],
+// one f32 scale per (batch row, position) for each of them
+int32_t launch_rope_append_i8(_Float16 *qkv, const int32_t *pos_ptr, int batch, int hq, int hkv, int hd, float theta,
+                              int max_ctx, int8_t *kc, float *ks, int8_t *vc, float *vs, hipStream_t s);
+int32_t launch_kv_relayout_i8(const _Float16 *k_nat, const _Float16 *v_nat, int batch, int npos, int hkv, int hd, int max_ctx,
+                              int8_t *kc, float *ks, int8_t *vc, float *vs, hipStream_t s);
+int32_t launch_attention_i8(const _Float16 *qkv, const int8_t *kc, const float *ks, const int8_t *vc, const float *vs,
+                            const int32_t *pos_ptr, int batch, int hq, int hkv, int hd, int max_ctx, float *part,
+                            _Float16 *out, hipStream_t s);
+int32_t launch_kv_random_fill_i8(int8_t *buf, size_t n, float *scales, size_t n_scales, float scale, uint64_t seed, hipStream_t s);
 int32_t launch_argmax(const float *logits, int batch, int vocab, int32_t *tokens, int32_t *history,
                       int32_t *step_ptr, int max_steps, hipStream_t s);
 int32_t launch_advance(int32_t *pos_ptr, int32_t *step_ptr, hipStream_t s);

@@ -121,9 +121,23 @@ constexpr int ATT_WAVES = 4;
 constexpr int ATT_POS_PER_WAVE = 32;
 constexpr int ATT_CHUNK = ATT_WAVES * ATT_POS_PER_WAVE;  // 128 positions per workgroup
 
+// KV8: the cache holds int8 rows with one f32 scale per (batch row, position) for K and for V (KvCache with
+// KvDtype::I8, crates/yscv-onnx/src/runner/kv_cache.rs:45-79: values read back as q * scale).  int8 values are exact in
+// fp16, so the K scale multiplies the finished score and the V scale is folded into the fp16 operand.
+__device__ __forceinline__ half8_t i8x8_to_half8(const int8_t *p, const float *sc8) {
+  typedef int8_t char8_t __attribute__((ext_vector_type(8)));
+  const char8_t v = *reinterpret_cast<const char8_t *>(p);
+  half8_t h;
+#pragma unroll
+  for (int e = 0; e < 8; e++) h[e] = sc8 ? (_Float16)((float)v[e] * sc8[e]) : (_Float16)(float)v[e];
+  return h;
+}
+
+template <bool KV8>
 __global__ void __launch_bounds__(256) attn_partial_kernel(const _Float16 *__restrict__ qkv,
-                                                           const _Float16 *__restrict__ kc,
-                                                           const _Float16 *__restrict__ vc,
+                                                           const void *__restrict__ kc_v,
+                                                           const void *__restrict__ vc_v,
+                                                           const float *__restrict__ ks, const float *__restrict__ vs,
                                                            const int32_t *__restrict__ pos_ptr, int hq, int hkv,
                                                            int max_ctx, int max_chunks, float scale,
                                                            float *__restrict__ part) {
@@ -158,18 +172,37 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const _Float16 *__res
         qa[j] = valid ? *reinterpret_cast<const half8_t *>(qsrc + 8 * j) : z;
       }
     }
-    const _Float16 *kbase = kc + (((size_t)b * hkv + kvh) * max_ctx + p0) * HD;
-    const _Float16 *vbase = vc + ((((size_t)b * hkv + kvh) * (max_ctx / 8) + p0 / 8) * HD) * 8;
-    // issue every load of this wave up front: 8 KiB of K, 8 KiB of V
+    const size_t k_off = (((size_t)b * hkv + kvh) * max_ctx + p0) * HD;
+    const size_t v_off = ((((size_t)b * hkv + kvh) * (max_ctx / 8) + p0 / 8) * HD) * 8;
+    // issue every load of this wave up front: 8 KiB of K, 8 KiB of V (half of that from an int8 cache)
     half8_t kf[2][4], vf[8];
+    float k_scale[2] = {1.0f, 1.0f};
+    if constexpr (KV8) {
+      const int8_t *kbase = static_cast<const int8_t *>(kc_v) + k_off;
+      const int8_t *vbase = static_cast<const int8_t *>(vc_v) + v_off;
+      float v_scale[8];
 #pragma unroll
-    for (int pb = 0; pb < 2; pb++)
+      for (int e = 0; e < 8; e++) v_scale[e] = vs[(size_t)b * max_ctx + p0 + 8 * c + e];
 #pragma unroll
-      for (int j = 0; j < 4; j++)
-        kf[pb][j] = *reinterpret_cast<const half8_t *>(kbase + (size_t)(pb * 16 + r) * HD + 32 * c + 8 * j);
+      for (int pb = 0; pb < 2; pb++) {
+        k_scale[pb] = ks[(size_t)b * max_ctx + p0 + pb * 16 + r];
 #pragma unroll
-    for (int t = 0; t < 8; t++)
-      vf[t] = *reinterpret_cast<const half8_t *>(vbase + ((size_t)c * HD + t * 16 + r) * 8);
+        for (int j = 0; j < 4; j++) kf[pb][j] = i8x8_to_half8(kbase + (size_t)(pb * 16 + r) * HD + 32 * c + 8 * j, nullptr);
+      }
+#pragma unroll
+      for (int t = 0; t < 8; t++) vf[t] = i8x8_to_half8(vbase + ((size_t)c * HD + t * 16 + r) * 8, v_scale);
+    } else {
+      const _Float16 *kbase = static_cast<const _Float16 *>(kc_v) + k_off;
+      const _Float16 *vbase = static_cast<const _Float16 *>(vc_v) + v_off;
+#pragma unroll
+      for (int pb = 0; pb < 2; pb++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          kf[pb][j] = *reinterpret_cast<const half8_t *>(kbase + (size_t)(pb * 16 + r) * HD + 32 * c + 8 * j);
+#pragma unroll
+      for (int t = 0; t < 8; t++)
+        vf[t] = *reinterpret_cast<const half8_t *>(vbase + ((size_t)c * HD + t * 16 + r) * 8);
+    }
 
     float s[2];
 #pragma unroll
@@ -179,7 +212,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const _Float16 *__res
       for (int j = 0; j < 4; j++) d = __builtin_amdgcn_mfma_f32_16x16x32_f16(qa[j], kf[pb][j], d, 0, 0, 0);
       // lane (r, c): score of head c at position p0 + 16*pb + r
       const int p = p0 + pb * 16 + r;
-      s[pb] = (p < n_ctx) ? d[0] * scale : -INFINITY;
+      s[pb] = (p < n_ctx) ? d[0] * scale * k_scale[pb] : -INFINITY;
     }
     float mx = fmaxf(s[0], s[1]);
 #pragma unroll
@@ -369,6 +402,129 @@ __global__ void kv_random_fill_kernel(_Float16 *__restrict__ buf, size_t n, uint
   }
 }
 
+// ---- int8 cache: KvCache with KvDtype::I8 (crates/yscv-onnx/src/runner/kv_cache.rs:45-61) --------------------------------
+// A row = the kv_dim = Hkv * 128 values one position adds to K (or V): scale = absmax / 127 (1.0 when absmax <=
+// f32::EPSILON), q = clamp(round_half_away(v * (1 / scale)), -127, 127).
+__device__ __forceinline__ float block_max_256(float v, float *red) {
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  v = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  return v;
+}
+__device__ __forceinline__ int8_t kv_quant_one(float v, float inv) {
+#pragma clang fp contract(off)  // the product is rounded before the rounding rule looks at it, as in the reference
+  const float x = v * inv;
+  const float t = truncf(x);
+  const float rr = (fabsf(x - t) >= 0.5f) ? t + copysignf(1.0f, x) : t;
+  if (rr != rr) return 0;
+  return (int8_t)(int)fminf(fmaxf(rr, -127.0f), 127.0f);
+}
+__device__ __forceinline__ void kv_row_scale(float amax, float *scale, float *inv) {
+  *scale = (amax <= 1.1920929e-7f) ? 1.0f : __fdiv_rn(amax, 127.0f);
+  *inv = __fdiv_rn(1.0f, *scale);
+}
+
+// RoPE on q (in place) and k, then per-row int8 quantisation of the rotated k row and of the v row of this position.
+// One workgroup per batch row; dynamic LDS: 2 * Hkv * 128 floats.
+__global__ void __launch_bounds__(256) rope_append_i8_kernel(_Float16 *__restrict__ qkv, const int32_t *__restrict__ pos_ptr,
+                                                             int hq, int hkv, float theta, int max_ctx,
+                                                             int8_t *__restrict__ kc, float *__restrict__ ks,
+                                                             int8_t *__restrict__ vc, float *__restrict__ vs) {
+  constexpr int HD = 128, HALF = 64;
+  extern __shared__ float kv_lds[];
+  __shared__ float red[4];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const int pos = *pos_ptr;
+  const int kv_dim = hkv * HD;
+  float *kbuf = kv_lds, *vbuf = kv_lds + kv_dim;
+  _Float16 *row = qkv + (size_t)b * (hq + 2 * hkv) * HD;
+  float kmax = 0.0f, vmax = 0.0f;
+  for (int idx = tid; idx < (hq + hkv) * HALF; idx += 256) {
+    const int slot = idx / HALF, i = idx % HALF;
+    const float inv_freq = 1.0f / powf(theta, (float)(2 * i) / (float)HD);
+    float sn, cs;
+    sincosf(inv_freq * (float)pos, &sn, &cs);
+    _Float16 *src = row + (size_t)slot * HD;
+    const float x0 = (float)src[i], x1 = (float)src[i + HALF];
+    const float y0 = x0 * cs - x1 * sn, y1 = x0 * sn + x1 * cs;
+    if (slot < hq) {
+      src[i] = (_Float16)y0;
+      src[i + HALF] = (_Float16)y1;
+    } else {
+      kbuf[(slot - hq) * HD + i] = y0;
+      kbuf[(slot - hq) * HD + i + HALF] = y1;
+      kmax = fmaxf(kmax, fmaxf(fabsf(y0), fabsf(y1)));
+    }
+  }
+  for (int idx = tid; idx < kv_dim; idx += 256) {
+    const float v = (float)row[(size_t)(hq + hkv) * HD + idx];
+    vbuf[idx] = v;
+    vmax = fmaxf(vmax, fabsf(v));
+  }
+  __syncthreads();
+  kmax = block_max_256(kmax, red);
+  vmax = block_max_256(vmax, red);
+  float k_scale, k_inv, v_scale, v_inv;
+  kv_row_scale(kmax, &k_scale, &k_inv);
+  kv_row_scale(vmax, &v_scale, &v_inv);
+  if (tid == 0) {
+    ks[(size_t)b * max_ctx + pos] = k_scale;
+    vs[(size_t)b * max_ctx + pos] = v_scale;
+  }
+  for (int idx = tid; idx < kv_dim; idx += 256) {
+    const int kvh = idx / HD, i = idx % HD;
+    kc[(((size_t)b * hkv + kvh) * max_ctx + pos) * HD + i] = kv_quant_one(kbuf[idx], k_inv);
+    vc[((((size_t)b * hkv + kvh) * (max_ctx / 8) + pos / 8) * HD + i) * 8 + (pos & 7)] = kv_quant_one(vbuf[idx], v_inv);
+  }
+}
+
+// natural [batch][pos][kv_head][d] fp16 (host order) -> int8 cache rows; one workgroup per (position, batch row)
+__global__ void __launch_bounds__(256) kv_relayout_i8_kernel(const _Float16 *__restrict__ k_nat, const _Float16 *__restrict__ v_nat,
+                                                             int npos, int hkv, int max_ctx, int8_t *__restrict__ kc,
+                                                             float *__restrict__ ks, int8_t *__restrict__ vc,
+                                                             float *__restrict__ vs) {
+  constexpr int HD = 128;
+  __shared__ float red[4];
+  const int pos = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  const int kv_dim = hkv * HD;
+  const _Float16 *kr = k_nat + ((size_t)b * npos + pos) * kv_dim, *vr = v_nat + ((size_t)b * npos + pos) * kv_dim;
+  float kmax = 0.0f, vmax = 0.0f;
+  for (int idx = tid; idx < kv_dim; idx += 256) {
+    kmax = fmaxf(kmax, fabsf((float)kr[idx]));
+    vmax = fmaxf(vmax, fabsf((float)vr[idx]));
+  }
+  kmax = block_max_256(kmax, red);
+  vmax = block_max_256(vmax, red);
+  float k_scale, k_inv, v_scale, v_inv;
+  kv_row_scale(kmax, &k_scale, &k_inv);
+  kv_row_scale(vmax, &v_scale, &v_inv);
+  if (tid == 0) {
+    ks[(size_t)b * max_ctx + pos] = k_scale;
+    vs[(size_t)b * max_ctx + pos] = v_scale;
+  }
+  for (int idx = tid; idx < kv_dim; idx += 256) {
+    const int kvh = idx / HD, i = idx % HD;
+    kc[(((size_t)b * hkv + kvh) * max_ctx + pos) * HD + i] = kv_quant_one((float)kr[idx], k_inv);
+    vc[((((size_t)b * hkv + kvh) * (max_ctx / 8) + pos / 8) * HD + i) * 8 + (pos & 7)] = kv_quant_one((float)vr[idx], v_inv);
+  }
+}
+
+// benchmark fill of an int8 cache: uniform bytes in [-127, 127] and one constant scale, so values span about +-3.5
+__global__ void kv_random_fill_i8_kernel(int8_t *__restrict__ buf, size_t n, uint64_t seed) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    uint64_t z = (i + 1) * 0x9E3779B97F4A7C15ull + seed;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    buf[i] = (int8_t)((int)(z % 255u) - 127);
+  }
+}
+__global__ void fill_const_f32_kernel(float *p, size_t n, float v) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
 // ---- launchers -------------------------------------------------------------------------------------------
 int32_t launch_embed(const int32_t *tokens, const _Float16 *table, int batch, int d, int vocab, float *h,
                      hipStream_t s) {
@@ -412,10 +568,55 @@ int32_t launch_attention(const _Float16 *qkv, const _Float16 *kc, const _Float16
     return set_error(YSCV_HIP_ERR_UNSUPPORTED, "attention kernel handles 1..4 query heads per kv head");
   const int max_chunks = max_ctx / ATT_CHUNK;
   const float scale = 1.0f / sqrtf((float)hd);
-  hipLaunchKernelGGL(attn_partial_kernel, dim3(max_chunks, hkv, batch), dim3(256), 0, s, qkv, kc, vc, pos_ptr, hq,
+  hipLaunchKernelGGL(attn_partial_kernel<false>, dim3(max_chunks, hkv, batch), dim3(256), 0, s, qkv, kc, vc, nullptr, nullptr,
+                     pos_ptr, hq, hkv, max_ctx, max_chunks, scale, part);
+  YSCV_HIP_TRY(hipGetLastError());
+  hipLaunchKernelGGL(attn_combine_kernel, dim3(hq, batch), dim3(128), 0, s, part, pos_ptr, hq, max_chunks, out);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_attention_i8(const _Float16 *qkv, const int8_t *kc, const float *ks, const int8_t *vc, const float *vs,
+                            const int32_t *pos_ptr, int batch, int hq, int hkv, int hd, int max_ctx, float *part,
+                            _Float16 *out, hipStream_t s) {
+  if (hd != 128) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "attention kernel is built for head_dim 128, got %d", hd);
+  if (hq % hkv != 0 || hq / hkv > 4)
+    return set_error(YSCV_HIP_ERR_UNSUPPORTED, "attention kernel handles 1..4 query heads per kv head");
+  const int max_chunks = max_ctx / ATT_CHUNK;
+  const float scale = 1.0f / sqrtf((float)hd);
+  hipLaunchKernelGGL(attn_partial_kernel<true>, dim3(max_chunks, hkv, batch), dim3(256), 0, s, qkv, kc, vc, ks, vs, pos_ptr, hq,
                      hkv, max_ctx, max_chunks, scale, part);
   YSCV_HIP_TRY(hipGetLastError());
   hipLaunchKernelGGL(attn_combine_kernel, dim3(hq, batch), dim3(128), 0, s, part, pos_ptr, hq, max_chunks, out);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_rope_append_i8(_Float16 *qkv, const int32_t *pos_ptr, int batch, int hq, int hkv, int hd, float theta,
+                              int max_ctx, int8_t *kc, float *ks, int8_t *vc, float *vs, hipStream_t s) {
+  if (hd != 128) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "int8 cache append is built for head_dim 128, got %d", hd);
+  const size_t lds = (size_t)2 * hkv * hd * sizeof(float);
+  if (lds > 48 * 1024) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "int8 cache append: too many kv heads (%d)", hkv);
+  hipLaunchKernelGGL(rope_append_i8_kernel, dim3(batch), dim3(256), lds, s, qkv, pos_ptr, hq, hkv, theta, max_ctx, kc, ks, vc, vs);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_kv_relayout_i8(const _Float16 *k_nat, const _Float16 *v_nat, int batch, int npos, int hkv, int hd, int max_ctx,
+                              int8_t *kc, float *ks, int8_t *vc, float *vs, hipStream_t s) {
+  if (hd != 128) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "int8 cache is built for head_dim 128, got %d", hd);
+  hipLaunchKernelGGL(kv_relayout_i8_kernel, dim3(npos, batch), dim3(256), 0, s, k_nat, v_nat, npos, hkv, max_ctx, kc, ks, vc, vs);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_kv_random_fill_i8(int8_t *buf, size_t n, float *scales, size_t n_scales, float scale, uint64_t seed, hipStream_t s) {
+  size_t blocks = ceil_div(n, (size_t)256);
+  if (blocks > 65535) blocks = 65535;
+  hipLaunchKernelGGL(kv_random_fill_i8_kernel, dim3((unsigned)blocks), dim3(256), 0, s, buf, n, seed);
+  YSCV_HIP_TRY(hipGetLastError());
+  size_t sb = ceil_div(n_scales, (size_t)256);
+  hipLaunchKernelGGL(fill_const_f32_kernel, dim3((unsigned)(sb > 65535 ? 65535 : sb)), dim3(256), 0, s, scales, n_scales, scale);
   YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
 }

@@ -17,11 +17,13 @@ def _p(a):
 
 
 class Decoder:
-    def __init__(self, **cfg):
+    def __init__(self, kv_dtype="f16", **cfg):
+        """kv_dtype: 'f16' or 'i8' (per-row int8 cache, KvDtype::I8 of the reference's KvCache)."""
         self.cfg = dict(cfg)
+        self.kv_dtype = kv_dtype
         c = DecoderConfig(**cfg)
         h = C.c_void_p()
-        lib().decoder_create(C.byref(c), C.byref(h))
+        lib().decoder_create_kv(C.byref(c), {"f16": 0, "i8": 1}[kv_dtype], C.byref(h))
         self._h = h
         self.batch = 0
 
