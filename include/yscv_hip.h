@@ -338,6 +338,17 @@ int32_t yscv_hip_exec_qlinear_matmul(const float *a_dev, float a_scale, float a_
  * operators one after the other; counted as one qlinear_matmul_fast. */
 int32_t yscv_hip_exec_qdq_matmul(const float *x_dev, size_t m, float a_scale, const yscv_hip_i8_weight *b,
                                  float b_scale, float y_scale, float y_zp, float *out_dev, void *stream);
+/* DynamicQuantizeLinear feeding MatMulInteger, the pair ONNX Runtime's dynamic quantisation emits (exec_dynamic_quantize_linear,
+ * crates/yscv-onnx/src/runner/misc.rs:241-289, then exec_matmul_integer with a_zero_point = the y_zero_point just computed,
+ * runner/linear.rs:648-737), as one call: x_dev [m][k] f32 is reduced to its range, quantised to uint8 once into
+ * stream-ordered scratch, and multiplied against the prepacked int8 weight (b_zero_point 0); the zero point never leaves
+ * the device (the GEMM's epilogue reads it there and folds (128 - zp) * colsum(b)), the f32 carriers of the quantised
+ * activations are never written, no range scan and no host synchronisation.  out_dev [m][n] = f32 of the exact integer sum
+ * of (a_q - zp) * b; *y_scale_dev, *y_zp_dev as DynamicQuantizeLinear returns them.  Bit-identical to the two operators
+ * called one after the other.  Counted as matmul_integer_fallback (a non-zero a_zero_point sends the reference to its
+ * f32 matmul, linear.rs:701-736). */
+int32_t yscv_hip_exec_dql_matmul_integer(const float *x_dev, size_t m, const yscv_hip_i8_weight *b, float *out_dev,
+                                         float *y_scale_dev, float *y_zp_dev, void *stream);
 /* MatMulNBits (com.microsoft), the operator ONNX exporters emit for 4-bit weights: Y = A x dequant(B)^T + bias.  The
  * reference's dispatcher has no such operator (crates/yscv-onnx/src/runner/dispatch.rs:191-322), so its int4 branch
  * only ever sees weights it packed itself; here the initialisers of the node -- B [N][K/block][block/2] bytes, element

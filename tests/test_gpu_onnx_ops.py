@@ -375,3 +375,29 @@ def test_gemm_through_the_int4_branch(oracle, torch_cuda, ops, m, k, n, g, nk):
         assert np.array_equal(got, want.astype(np.float32)), (alpha, beta)
     with pytest.raises(ValueError):
         ops.exec_gemm_int4(a, w, c=_dev(torch, np.zeros(n + 1, np.float32)))
+
+
+@pytest.mark.parametrize("shape", [(1, 64, 16), (5, 200, 70), (33, 512, 128), (64, 4096, 256), (130, 1024, 48)])
+def test_dql_fused_into_matmul_integer(oracle, torch_cuda, ops, shape):
+    """DynamicQuantizeLinear -> MatMulInteger as one call: bit-identical to the two operators chained, and equal to the
+    checker's DynamicQuantizeLinear followed by the exact integer product."""
+    torch = torch_cuda
+    m, k, n = shape
+    rng = np.random.default_rng(m * 7 + k + n)
+    x = (rng.standard_normal((m, k)) * 3.0 + 0.7).astype(np.float32)
+    b = rng.integers(-127, 128, (k, n)).astype(np.float32)
+    pre = ops.PrepackedI8B(_dev(torch, b))
+    out, ys, yz = ops.exec_dql_matmul_integer(_dev(torch, x), pre)
+    y, s2, z2 = ops.exec_dynamic_quantize_linear(_dev(torch, x))
+    chained, _ = ops.exec_matmul_integer(y, None, a_zp=float(z2.item()), b_zp=0.0, prepacked=pre)
+    assert torch.equal(out, chained) and torch.equal(ys, s2) and torch.equal(yz, z2)
+    yq, sc, zp = oracle.dynamic_quantize_linear(x.ravel())
+    assert float(ys.item()) == np.float32(sc) and float(yz.item()) == float(zp)
+    want = (yq.reshape(m, k).astype(np.int64) - int(zp)) @ b.astype(np.int64)
+    assert np.array_equal(out.cpu().numpy(), want.astype(np.float32))
+    # constant input: range 0 .. c, every value quantises to 255 or to 0
+    xc = np.full((4, k), 2.5, np.float32)
+    out, ys, yz = ops.exec_dql_matmul_integer(_dev(torch, xc), pre)
+    yq, sc, zp = oracle.dynamic_quantize_linear(xc.ravel())
+    want = (yq.reshape(4, k).astype(np.int64) - int(zp)) @ b.astype(np.int64)
+    assert np.array_equal(out.cpu().numpy(), want.astype(np.float32))

@@ -114,6 +114,7 @@ _SIGNATURES = {
     "yscv_hip_exec_qlinear_matmul": [_vp, _f32, _f32, _vp, _vp, _f32, _f32, _f32, _f32, _sz, _sz, _sz, _vp,
                                      C.POINTER(_i32), _vp],
     "yscv_hip_exec_qdq_matmul": [_vp, _sz, _f32, _vp, _f32, _f32, _f32, _vp, _vp],
+    "yscv_hip_exec_dql_matmul_integer": [_vp, _sz, _vp, _vp, _vp, _vp, _vp],
     "yscv_hip_exec_matmul_nbits": [_vp, _i32, _sz, _vp, _vp, C.c_int64, C.c_int64, C.c_int64, C.c_int64, _vp, _i32, _vp],
     "yscv_hip_exec_gemm_int4": [_vp, _sz, _vp, _vp, _sz, _f32, _f32, _vp, _vp],
     "yscv_hip_exec_quantize_linear": [_vp, _sz, _f32, _f32, _vp, _vp],

@@ -108,6 +108,7 @@ struct I8Args {
   int ksteps;       // kp / 64
   int a_xor;        // 0x80808080 for uint8 activations, 0 for int8
   int zp_mul;       // multiplies col_sum in the epilogue
+  const float *a_zp_dev;  // null, or the uint8 zero point of A as an f32 in device memory (then zp_mul = 128 - that)
 };
 
 template <bool VEC>
@@ -215,7 +216,7 @@ __global__ void __launch_bounds__(I8_THREADS) i8_gemm_kernel(I8Args p) {
   for (int j = 0; j < 2; j++) {
     const int col = n0 + j * 16 + r;
     if (col >= p.n) continue;
-    const int32_t zc = p.zp_mul * p.col_sum[col];
+    const int32_t zc = (p.a_zp_dev ? 128 - (int)p.a_zp_dev[0] : p.zp_mul) * p.col_sum[col];
     const int32_t corr = p.corr ? p.corr[col] : 0;
     const float comp = p.composite_v ? p.composite_v[col] : p.composite;
 #pragma unroll
@@ -228,6 +229,8 @@ __global__ void __launch_bounds__(I8_THREADS) i8_gemm_kernel(I8Args p) {
         const size_t o = (size_t)row * p.n + col;
         if (p.mode == 0) {
           reinterpret_cast<int32_t *>(p.out)[o] = v;
+        } else if (p.mode == 3) {
+          reinterpret_cast<float *>(p.out)[o] = (float)v;
         } else if (p.mode == 2) {
           reinterpret_cast<int32_t *>(p.out)[o] = requant_dequant_bits(v, corr, comp, p.y_zp, p.round_mode, lo, hi, p.dq_scale);
         } else {
@@ -470,6 +473,7 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
   // then all waves store whole rows ---------------------------------------------------------------------
   __syncthreads();  // every wave is done with the ring
   const float lo = (float)p.lo, hi = (float)p.hi;
+  const int zp_mul = p.a_zp_dev ? 128 - (int)p.a_zp_dev[0] : p.zp_mul;
   if (wave < 4) {
 #pragma unroll
     for (int j = 0; j < NT; j++) {
@@ -478,7 +482,7 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
       float comp[4];
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        zc[e] = p.zp_mul * zc_all[j][e];
+        zc[e] = zp_mul * zc_all[j][e];
         corr[e] = p.corr ? corr_all[j][e] : 0;
         comp[e] = p.composite_v ? comp_all[j][e] : p.composite;
       }
@@ -490,6 +494,9 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
         for (int e = 0; e < 4; e++) v[e] = (int32_t)((uint32_t)acc[i][j][e] + (uint32_t)zc[e]);
         if (p.mode == 0) {
           *reinterpret_cast<int4_t *>(i8_ring + lrow * RS32 + lcol * 4) = int4_t{v[0], v[1], v[2], v[3]};
+        } else if (p.mode == 3) {
+          *reinterpret_cast<int4_t *>(i8_ring + lrow * RS32 + lcol * 4) =
+              int4_t{__float_as_int((float)v[0]), __float_as_int((float)v[1]), __float_as_int((float)v[2]), __float_as_int((float)v[3])};
         } else if (p.mode == 2) {
           int4_t f;
 #pragma unroll
@@ -586,6 +593,7 @@ int32_t launch_i8_gemm(const void *a, int a_is_u8, int a_zp, const yscv_hip_i8_w
   p.ksteps = (int)(b->kp / 64);
   p.a_xor = a_is_u8 ? (int)0x80808080u : 0;
   p.zp_mul = a_is_u8 ? (128 - a_zp) : -a_zp;
+  p.a_zp_dev = ep.a_zp_dev;
   const bool aligned = (reinterpret_cast<uintptr_t>(a) & 15) == 0;
   const bool out_ok = (reinterpret_cast<uintptr_t>(out) & 15) == 0;
   if (b->k % 64 == 0 && aligned && out_ok && m * b->k < ((size_t)1 << 31)) {

@@ -103,7 +103,7 @@ void note_int4_fallback();
 int32_t launch_i8_pack_b(const int8_t *b_kn, size_t k, size_t n, size_t kp, size_t np,
                          int8_t *frag, int32_t *col_sum, hipStream_t s);
 struct I8Epilogue {
-  int mode;  // 0: int32 out, 1: requantize to bytes, 2: requantize, then (q - y_zp) * dq_scale as f32
+  int mode;  // 0: int32 out, 1: requantize to bytes, 2: requantize, then (q - y_zp) * dq_scale as f32, 3: f32(int32) out
   const int32_t *corr;
   const float *composite_v;
   float composite;
@@ -111,6 +111,7 @@ struct I8Epilogue {
   int round_mode;
   int lo, hi;
   float dq_scale;
+  const float *a_zp_dev = nullptr;  // uint8 A only: its zero point as an f32 in device memory, used instead of a_zp
 };
 int32_t launch_i8_gemm(const void *a, int a_is_u8, int a_zp, const yscv_hip_i8_weight *b, size_t m,
                        void *out, const I8Epilogue &ep, hipStream_t s);

@@ -563,6 +563,41 @@ int32_t yscv_hip_exec_qdq_matmul(const float *x_dev, size_t m, float a_scale, co
   return YSCV_HIP_OK;
 }
 
+int32_t yscv_hip_exec_dql_matmul_integer(const float *x_dev, size_t m, const yscv_hip_i8_weight *b, float *out_dev,
+                                         float *y_scale_dev, float *y_zp_dev, void *stream) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(b != nullptr, "null int8 weight handle");
+  YSCV_REQUIRE(y_scale_dev && y_zp_dev, "null scale / zero-point pointer");
+  if (m == 0) return YSCV_HIP_OK;
+  YSCV_REQUIRE(x_dev && out_dev, "null x / out pointer");
+  hipStream_t s = as_stream(stream);
+  const size_t len = m * b->k;
+  // uint8 A and {scale, zero point} in one stream-ordered scratch block; nothing returns to the host
+  uint8_t *scratch = nullptr;
+  const size_t a_bytes = round_up(len, 256);
+  YSCV_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&scratch), a_bytes + 256, s));
+  float *scale_zp = reinterpret_cast<float *>(scratch + a_bytes);
+  int32_t st = launch_dynamic_quantize_linear(x_dev, len, scratch, scale_zp, s);
+  if (st == YSCV_HIP_OK) {
+    I8Epilogue ep{};
+    ep.mode = 3;                   // f32(acc): MatMulInteger's output carrier (linear.rs:693-697)
+    ep.a_zp_dev = scale_zp + 1;    // the zero point stays on the device: the GEMM folds (128 - zp) * colsum(b) itself
+    st = launch_i8_gemm(scratch, 1, 0, b, m, out_dev, ep, s);
+  }
+  hipError_t e1 = hipSuccess, e2 = hipSuccess;
+  if (st == YSCV_HIP_OK) {
+    e1 = hipMemcpyAsync(y_scale_dev, scale_zp, sizeof(float), hipMemcpyDeviceToDevice, s);
+    e2 = hipMemcpyAsync(y_zp_dev, scale_zp + 1, sizeof(float), hipMemcpyDeviceToDevice, s);
+  }
+  const hipError_t fe = hipFreeAsync(scratch, s);
+  YSCV_TRY(st);
+  YSCV_HIP_TRY(e1);
+  YSCV_HIP_TRY(e2);
+  YSCV_HIP_TRY(fe);
+  g_mmi_fallback.fetch_add(1, std::memory_order_relaxed);
+  return YSCV_HIP_OK;
+}
+
 int32_t yscv_hip_exec_matmul_nbits(const void *a_dev, int32_t a_dtype, size_t m, const yscv_hip_int4_weight *b,
                                    const float *bias_dev, int64_t attr_k, int64_t attr_n, int64_t attr_bits,
                                    int64_t attr_block_size, void *y_dev, int32_t y_dtype, void *stream) {

@@ -149,6 +149,19 @@ def exec_qdq_matmul(x, a_scale, prepacked: PrepackedI8B, b_scale, y_scale, y_zp:
     return out
 
 
+def exec_dql_matmul_integer(x, prepacked: PrepackedI8B):
+    """DynamicQuantizeLinear -> MatMulInteger (b_zero_point 0) in one call.  Returns (out [m][n] f32, y_scale [1], y_zp [1])."""
+    import torch
+
+    x = _dev_f32(x, "x")
+    if x.dim() != 2 or int(x.shape[1]) != prepacked.k:
+        raise ValueError("x must be [m][k] with k matching the prepacked weight")
+    out = torch.empty(int(x.shape[0]), prepacked.n, device=x.device, dtype=torch.float32)
+    sz = torch.empty(2, device=x.device, dtype=torch.float32)
+    lib().exec_dql_matmul_integer(_p(x), _sz(int(x.shape[0])), prepacked.handle, _p(out), _p(sz[0:1]), _p(sz[1:2]), _stream_ptr())
+    return out, sz[0:1], sz[1:2]
+
+
 class MatMulNBitsWeight:
     """The initialisers of one MatMulNBits node (com.microsoft) uploaded once: B [N][K/block][block/2] uint8 (element 2i
     in the low nibble), scales [N * K/block] float32 or float16, optional packed uint4 zero_points [N][ceil(K/block/2)]
