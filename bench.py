@@ -429,6 +429,8 @@ def main():
                          "(the run the rocprofv3 summaries of those kernels are taken from)")
     ap.add_argument("--graph-path", action="store_true",
                     help="time the multi-kernel path (one HIP-graph replay per step) instead of the single-launch kernel")
+    ap.add_argument("--no-check", action="store_true",
+                    help="skip the comparison of the single-launch kernel with the multi-kernel path (timing experiments)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (torch copy_ kernel, 3 launches): the known-size "
                          "kernel that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
@@ -471,7 +473,7 @@ def main():
     assert dec.weight_bytes() >= w_bytes
 
     persistent = args.batch == 1 and not args.graph_path
-    check = check_single_launch(dec, torch) if persistent else None
+    check = check_single_launch(dec, torch) if persistent and not args.no_check else None
     dt, dt_events = bench_decode(dec, torch, args.batch, args.steps, args.warmup, stream_ptr, persistent=persistent)
     tok_s = args.batch * args.steps / dt
     kv_row_bytes = 2 * cfg["n_layers"] * cfg["n_kv_heads"] * cfg["head_dim"] * 2  # K + V bytes one cached position adds

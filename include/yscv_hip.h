@@ -514,6 +514,10 @@ int32_t yscv_hip_decoder_read_logits(yscv_hip_decoder *d, float *out_host);
 #define YSCV_HIP_DEC_ACT_ATTN_OUT 3 /* [batch][n_heads * head_dim] */
 #define YSCV_HIP_DEC_ACT_FFN 4      /* [batch][d_ff] */
 int32_t yscv_hip_decoder_read_activation(yscv_hip_decoder *d, int32_t which, float *out_host, size_t capacity);
+/* Test aid: the single-launch path stamps what its workgroups hand to each other with a 24-bit tag that advances with
+ * every step; close to the end of the tag space yscv_hip_decoder_run clears the exchange buffers and starts the count
+ * again.  This sets the count (>= 1), so that a test reaches that point without half a million decode steps. */
+int32_t yscv_hip_decoder_debug_set_tag_epoch(yscv_hip_decoder *d, uint32_t epoch);
 /* Bytes of packed weights + scales one decode step streams through the projections. */
 int32_t yscv_hip_decoder_weight_bytes(const yscv_hip_decoder *d, size_t *bytes);
 int32_t yscv_hip_decoder_vocab(const yscv_hip_decoder *d, size_t *vocab);

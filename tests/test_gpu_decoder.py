@@ -211,6 +211,31 @@ def test_persistent_decode_matches_numpy_and_graph_path(prefill):
     assert np.abs(graph_logits - logits5).max() / np.abs(logits5).max() < 5e-3
 
 
+def test_single_launch_tags_wrap_around_cleanly():
+    """The 24-bit tags of the single-launch path: runs that straddle the end of the tag space (the host clears the
+    exchange buffers and restarts the count) give the same tokens and logits as a run far from it."""
+    import ctypes as C
+
+    from yscv_amd import lib
+
+    rng = np.random.default_rng(4400)
+    cfg = dict(PCFG)
+    dec, _ = _build(rng, cfg)
+    tokens = np.array([9], np.int32)
+    dec.reset(tokens, 0)
+    dec.run(12, persistent=True)
+    want_tok, want_logits = dec.tokens(0, 12)[:, 0].copy(), dec.logits().copy()
+    per_step = cfg["n_layers"] + 2
+    last_epoch = (1 << 24) // per_step
+    for back in (30, 13, 12, 5, 2, 1):      # the 12 steps start `back` epochs before the tag space ends
+        lib().decoder_debug_set_tag_epoch(dec._h, C.c_uint32(last_epoch - back))
+        dec.reset(tokens, 0)
+        dec.run(5, persistent=True)         # two launches, so that the wrap may fall between them or inside the window
+        dec.run(7, persistent=True)
+        assert np.array_equal(dec.tokens(0, 12)[:, 0], want_tok), back
+        assert np.array_equal(dec.logits(), want_logits), back
+
+
 def test_generate_matches_device_greedy_and_stops_at_eos():
     """generate() (generate.rs:58-118) with the decoder as the model: top_k = 1 reproduces the tokens the device picks
     greedily; an EOS token ends the loop without being stored; the sampling path runs with the default configuration."""

@@ -11,7 +11,8 @@ EPILOGUE_STORE, EPILOGUE_ADD_F32, EPILOGUE_SWIGLU = 0, 1, 2
 STATIC_SCRATCH_BYTES = 32 << 20
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "lib", "libyscv_hip.so")
+# YSCV_HIP_LIB points at another build of the same library (e.g. one with stage timestamps compiled in)
+_LIB_PATH = os.environ.get("YSCV_HIP_LIB") or os.path.join(_HERE, "lib", "libyscv_hip.so")
 
 STATUS_NAMES = {0: "OK", -1: "INVALID_ARG", -2: "DEVICE", -3: "OOM", -4: "UNSUPPORTED", -5: "NO_DEVICE"}
 
@@ -141,6 +142,7 @@ _SIGNATURES = {
     "yscv_hip_decoder_read_tokens": [_vp, _i32, _i32, _vp],
     "yscv_hip_decoder_read_logits": [_vp, _vp],
     "yscv_hip_decoder_read_activation": [_vp, _i32, _vp, _sz],
+    "yscv_hip_decoder_debug_set_tag_epoch": [_vp, C.c_uint32],
     "yscv_hip_decoder_weight_bytes": [_vp, C.POINTER(_sz)],
     "yscv_hip_decoder_vocab": [_vp, C.POINTER(_sz)],
     "yscv_hip_sample_token": [_vp, _sz, _sz, _f32, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32)],

@@ -37,7 +37,7 @@ namespace yscv {
 
 typedef unsigned long long u64;
 // Stage timestamps (wall clock, per workgroup and layer) for performance work: build with
-// -DYSCV_PERSIST_TRACE=1 and point PersistModel::dbg_t at a [G][n_layers][16] buffer.
+// -DYSCV_PERSIST_TRACE=1 (the decoder then allocates the [G][n_layers][PERSIST_TRACE_SLOTS] buffer).
 #ifndef YSCV_PERSIST_TRACE
 #define YSCV_PERSIST_TRACE 0
 #endif
@@ -224,12 +224,15 @@ __device__ __forceinline__ bool poll_backoff_ws(WaitState &ws, uint32_t *abort_f
   return true;
 }
 // barrier of the compute waves (the producer waves never join, so s_barrier cannot be used)
+// Every other wait of a compute wave is bounded, so every wave reaches its barriers; the bound here (minutes) only
+// keeps a wave from spinning for ever should one of its workgroup have died.
 __device__ __forceinline__ void compute_barrier(WaitState &ws, lds_u32 *ctr, int n_waves) {
   ws.bar_gen += n_waves;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
   if ((threadIdx.x & 63) == 0) {
     __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    while ((int)(__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) - ws.bar_gen) < 0)
+    unsigned n = 0;
+    while ((int)(__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) - ws.bar_gen) < 0 && ++n < 0x40000000u)
       __builtin_amdgcn_s_sleep(0);
   }
   __builtin_amdgcn_wave_barrier();
@@ -633,15 +636,18 @@ __device__ GEMV_INL GemvState gemv_stage(GemvArgs a, GemvState st) {
   // ---- one record: 8 rows x 512 k against fragment xa ------------------------------------------------------
   unsigned crec = st.crec;
   unsigned landed_seen = st.crec;  // the producer's count as last read: while it is ahead, no record waits for a poll
+  unsigned spins = 0;              // one budget for all records of the stage: a stalled stream costs it once, not per record
   auto consume = [&](bool single, const half8_t &xf, const float4_t &zf, float &acc) {
     if ((int)(landed_seen - (crec + 1)) < 0) {
-      unsigned spins = 0;
       while ((int)((landed_seen = __builtin_amdgcn_readfirstlane(
                         __hip_atomic_load(sync + wave, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP))) -
                    (crec + 1)) < 0) {
         __builtin_amdgcn_s_sleep(0);
-        if (++spins > 40000000u) {  // the stream stalled: never expected, but no wait here is unbounded
+        // the stream stalled (never expected) or another wave has given up: no wait here is unbounded
+        if (++spins > 40000000u ||
+            ((spins & 4095u) == 0 && __hip_atomic_load(a.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
           __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          spins = 40000000u;
           break;
         }
       }
@@ -738,7 +744,7 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
   auto nbw = [&](int kind) { return wg < m.ph[kind].nb ? (m.ph[kind].nb - wg + G - 1) / G : 0; };
   int dbg_layer = 0;
   auto mark = [&](int idx) {
-    if (YSCV_PERSIST_TRACE && m.dbg_t && tid == 0) m.dbg_t[((size_t)wg * L + dbg_layer) * 16 + idx] = wall_clock64();
+    if (YSCV_PERSIST_TRACE && m.dbg_t && tid == 0) m.dbg_t[((size_t)wg * L + dbg_layer) * PERSIST_TRACE_SLOTS + idx] = wall_clock64();
   };
   if (tid < 32) sync[tid] = 0;
   __syncthreads();
@@ -857,7 +863,7 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
     ga.in_buf = in_buf;
     ga.ss = with_ss ? in_buf + persist_vec_entries(m.ph[kind].k) : nullptr;
     ga.abort_flag = m.abort_flag;
-    ga.dbg_t = (YSCV_PERSIST_TRACE && m.dbg_t) ? m.dbg_t + ((size_t)wg * L + dbg_layer) * 16 + mk : nullptr;
+    ga.dbg_t = (YSCV_PERSIST_TRACE && m.dbg_t) ? m.dbg_t + ((size_t)wg * L + dbg_layer) * PERSIST_TRACE_SLOTS + mk : nullptr;
     ga.tag = tag;
     ga.ks = m.ph[kind].ks;
     ga.frags = m.ph[kind].frags;
@@ -973,10 +979,11 @@ decode_persistent_kernel(PersistModel m, int n_steps, int pos0, int step0, int m
         aa.tag = tag;
         aa.att_off = (uint32_t)(size_t)att_lds;
         aa.bar_off = (uint32_t)(size_t)(lds + RING_BYTES + PART_BYTES + ATT_BYTES) + 64;
-        aa.dbg_t = (YSCV_PERSIST_TRACE && m.dbg_t) ? m.dbg_t + ((size_t)wg * L + l) * 16 : nullptr;
+        aa.dbg_t = (YSCV_PERSIST_TRACE && m.dbg_t) ? m.dbg_t + ((size_t)wg * L + l) * PERSIST_TRACE_SLOTS : nullptr;
         ws = attn_items(aa, ws);
         mark(4);
         for (int head = G - 1 - wg; head < HQ; head += G) ws = attn_combine(aa, ws, head);
+        mark(16);
       }
       // ---- output projection + residual ------------------------------------------------------------------
       {

@@ -131,7 +131,9 @@ struct yscv_hip_decoder {
   unsigned long long *p_exch = nullptr;
   uint32_t *p_abort = nullptr;
   size_t p_stream_bytes = 0;
-  uint32_t epoch = 1;          // tag epoch of the next persistent step; never reused
+  size_t p_exch_entries = 0;
+  uint32_t epoch = 1;          // tag epoch of the next persistent step; tags are 24 bits wide: see yscv_hip_decoder_run
+  unsigned long long *p_trace = nullptr;  // stage timestamps (builds with YSCV_PERSIST_TRACE only)
 };
 
 // A captured step holds the addresses of the weights and of the workspace as they were at capture time: whatever
@@ -184,6 +186,7 @@ static void decoder_free(yscv_hip_decoder *d) {
   (void)hipFree(d->p_vc);
   (void)hipFree(d->p_exch);
   (void)hipFree(d->p_abort);
+  (void)hipFree(d->p_trace);
   delete d;
 }
 
@@ -249,6 +252,7 @@ static int32_t persist_setup(yscv_hip_decoder *d) {
   const size_t total_e = 2 * up(e_xn) + up(e_qkv) + up(e_ao) + up(e_act) + up(e_part) + up(e_arg);
   DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->p_exch), total_e * 8));
   DEC_HIP(hipMemset(d->p_exch, 0, total_e * 8));
+  d->p_exch_entries = total_e;
   unsigned long long *p = d->p_exch;
   m.xn = p;   p += up(e_xn);
   m.xn2 = p;  p += up(e_xn);
@@ -271,6 +275,12 @@ static int32_t persist_setup(yscv_hip_decoder *d) {
   m.history = d->history;
   m.abort_flag = d->p_abort;
   m.dbg_t = nullptr;
+#if defined(YSCV_PERSIST_TRACE) && YSCV_PERSIST_TRACE
+  // performance builds only: [G][n_layers][PERSIST_TRACE_SLOTS] stage timestamps, read back by yscv_hip_debug_persist_trace
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->p_trace), (size_t)G * c.n_layers * PERSIST_TRACE_SLOTS * 8));
+  DEC_HIP(hipMemset(d->p_trace, 0, (size_t)G * c.n_layers * PERSIST_TRACE_SLOTS * 8));
+  m.dbg_t = d->p_trace;
+#endif
   d->persist_ok = true;
   return YSCV_HIP_OK;
 }
@@ -769,6 +779,17 @@ int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_g
       return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the single-launch decode path does not support this model shape");
     if (d->batch != 1) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the single-launch decode path runs batch 1 only");
     if (n_steps == 0) return YSCV_HIP_OK;
+    // A tag is ((epoch + step) * (layers + 2) + 1 + layer) modulo 2^24.  Before the tag space wraps, the exchange
+    // buffers are cleared and the epoch starts again, so an entry left from half a million steps ago can never be taken
+    // for a fresh one.
+    const uint64_t per_step = (uint64_t)d->cfg.n_layers + 2;
+    YSCV_REQUIRE((uint64_t)n_steps * per_step < (1u << 23), "too many steps for one launch of the single-launch path");
+    if (((uint64_t)d->epoch + (uint64_t)n_steps + 1) * per_step + 2 >= (1u << 24)) {
+      hipLaunchKernelGGL(fill_i32_kernel, dim3(grid_for(d->p_exch_entries * 2)), dim3(256), 0, s,
+                         reinterpret_cast<int32_t *>(d->p_exch), d->p_exch_entries * 2, 0);
+      DEC_HIP(hipGetLastError());
+      d->epoch = 1;
+    }
     YSCV_TRY(launch_persist_decode(d->pm, n_steps, pos, step, d->cfg.max_steps, d->epoch, s));
     d->epoch += (uint32_t)n_steps;
     // position and step counters live on the device for the multi-kernel path: keep them in step
@@ -863,6 +884,28 @@ int32_t yscv_hip_decoder_read_activation(yscv_hip_decoder *d, int32_t which, flo
   std::vector<_Float16> tmp(elems);
   DEC_HIP(hipMemcpy(tmp.data(), src, elems * 2, hipMemcpyDeviceToHost));
   for (size_t i = 0; i < elems; i++) out_host[i] = (float)tmp[i];
+  return YSCV_HIP_OK;
+}
+
+#if defined(YSCV_PERSIST_TRACE) && YSCV_PERSIST_TRACE
+// Performance builds only (not declared in the public header): the stage timestamps of the last single-launch run,
+// [workgroups][layers][PERSIST_TRACE_SLOTS] ticks of the 100 MHz wall clock.
+__attribute__((visibility("default"))) int32_t yscv_hip_debug_persist_trace(yscv_hip_decoder *d, unsigned long long *out, size_t capacity,
+                                                                           int32_t *workgroups, int32_t *slots) {
+  YSCV_REQUIRE(d && out && d->p_trace, "no trace buffer");
+  const size_t n = (size_t)d->pm.G * d->cfg.n_layers * PERSIST_TRACE_SLOTS;
+  YSCV_REQUIRE(capacity >= n, "trace needs %zu entries", n);
+  DEC_HIP(hipDeviceSynchronize());
+  DEC_HIP(hipMemcpy(out, d->p_trace, n * 8, hipMemcpyDeviceToHost));
+  *workgroups = d->pm.G;
+  *slots = PERSIST_TRACE_SLOTS;
+  return YSCV_HIP_OK;
+}
+#endif
+
+int32_t yscv_hip_decoder_debug_set_tag_epoch(yscv_hip_decoder *d, uint32_t epoch) {
+  YSCV_REQUIRE(d != nullptr && epoch >= 1, "null decoder or epoch 0");
+  d->epoch = epoch;
   return YSCV_HIP_OK;
 }
 

@@ -27,6 +27,7 @@ namespace yscv {
 constexpr int PS_WAVES = 4;   // compute waves per workgroup = k slices of every projection
 constexpr int PS_REC_FULL = 2304;
 constexpr int PS_REC_SINGLE = 1280;
+constexpr int PERSIST_TRACE_SLOTS = 24;  // timestamps per (workgroup, layer) in builds with YSCV_PERSIST_TRACE
 enum : int { PK_QKV = 0, PK_O = 1, PK_GU = 2, PK_DOWN = 3, PK_LM = 4, PK_COUNT = 5 };
 
 struct PersistPhase {
@@ -66,7 +67,7 @@ struct PersistModel {
   int32_t *tokens;              // [1] current token (in: first token; out: last pick)
   int32_t *history;             // [max_steps]
   uint32_t *abort_flag;         // set when a bounded wait gave up
-  unsigned long long *dbg_t;    // null, or [G][n_layers][16] stage timestamps (builds with YSCV_PERSIST_TRACE)
+  unsigned long long *dbg_t;    // null, or [G][n_layers][PERSIST_TRACE_SLOTS] stage timestamps (builds with YSCV_PERSIST_TRACE)
 };
 
 // entries an exchange vector of k values occupies (padded to whole 512-k fragments per wave)
