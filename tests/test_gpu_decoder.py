@@ -74,6 +74,48 @@ def test_decode_steps_match_numpy(use_graph):
         cur = got_tok.copy()  # teacher-force the restatement with the GPU's picks
 
 
+@pytest.mark.parametrize("prefill", [5, 127, 128, 133, 250])
+def test_fused_attention_equals_the_separate_rope_append(prefill):
+    """Rotary embedding and cache append inside the attention kernel against the separate rope_append launch in front
+    of it: same arithmetic, so tokens, logits, the attention output, the rotated q and the appended cache rows must be
+    identical bit for bit.  The prefills put the current position at the start, the end and the middle of a
+    128-position chunk and leave chunks unused."""
+    import ctypes as C
+
+    from yscv_amd.capi import lib
+
+    rng = np.random.default_rng(4100 + prefill)
+    cfg = dict(CFG)
+    dec, _ = _build(rng, cfg)
+    B, steps = 3, 5
+    kv = []
+    for l in range(cfg["n_layers"]):
+        k = rng.standard_normal((B, prefill, cfg["n_kv_heads"], cfg["head_dim"])).astype(np.float16)
+        v = rng.standard_normal((B, prefill, cfg["n_kv_heads"], cfg["head_dim"])).astype(np.float16)
+        kv.append((k, v))
+    tokens = np.array([9, 130, 511], np.int32)
+    got = {}
+    for fused in (1, 0):
+        lib().decoder_debug_set_fused_attention(dec._h, C.c_int32(fused))
+        for l, (k, v) in enumerate(kv):
+            dec.set_kv(l, k, v)
+        dec.reset(tokens, prefill)
+        trace = []
+        for step in range(steps):
+            dec.run(1, use_graph=bool(step & 1))
+            trace.append((dec.logits().copy(), dec.activation("attn_out").copy(), dec.activation("qkv").copy()))
+        rows = [dec.get_kv(l, B, prefill, steps) for l in range(cfg["n_layers"])]
+        got[fused] = (dec.tokens(0, steps).copy(), trace, rows)
+    lib().decoder_debug_set_fused_attention(dec._h, C.c_int32(1))
+    assert np.array_equal(got[1][0], got[0][0])
+    for step in range(steps):
+        for a, b_, name in zip(got[1][1][step], got[0][1][step], ("logits", "attention output", "qkv")):
+            assert np.array_equal(a, b_), (step, name, np.abs(a - b_).max())
+    for l in range(cfg["n_layers"]):
+        for a, b_, name in zip(got[1][2][l], got[0][2][l], ("k", "v")):
+            assert np.array_equal(a, b_), ("appended rows", l, name, np.argwhere(a != b_)[:8].tolist())
+
+
 @pytest.mark.parametrize("use_graph", [False, True])
 def test_decode_with_int8_kv_cache_matches_numpy(use_graph):
     """--kv-dtype i8 (apps/llm-bench/src/main.rs:232-265; KvCache I8 storage, kv_cache.rs:45-79): rows quantised on

@@ -110,6 +110,8 @@ struct yscv_hip_decoder {
   // activations
   float *h = nullptr, *logits = nullptr, *attn_part = nullptr;
   _Float16 *xn = nullptr, *qkv = nullptr, *ao = nullptr, *act = nullptr;
+  _Float16 *qrot = nullptr;       // rotated query heads of the last fused attention launch (diagnostics)
+  bool fused_attn = true;         // fp16 cache: rope + append inside the attention kernel
   void *ws = nullptr;
   size_t ws_bytes = 0;
   int32_t *tokens = nullptr, *history = nullptr, *pos = nullptr, *step = nullptr;
@@ -169,6 +171,7 @@ static void decoder_free(yscv_hip_decoder *d) {
   (void)hipFree(d->h);
   (void)hipFree(d->logits);
   (void)hipFree(d->attn_part);
+  (void)hipFree(d->qrot);
   (void)hipFree(d->xn);
   (void)hipFree(d->qkv);
   (void)hipFree(d->ao);
@@ -342,6 +345,8 @@ static int32_t alloc_runtime(yscv_hip_decoder *d) {
   DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->act), B * (size_t)c.d_ff * 2));
   const size_t chunks = c.max_ctx / 128;
   DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->attn_part), B * c.n_heads * chunks * (c.head_dim + 2) * 4));
+  DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->qrot), B * (size_t)c.n_heads * c.head_dim * 2));
+  DEC_HIP(hipMemset(d->qrot, 0, B * (size_t)c.n_heads * c.head_dim * 2));
   DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->tokens), B * 4));
   DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->history), B * (size_t)c.max_steps * 4));
   DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->pos), 4));
@@ -405,6 +410,9 @@ static int32_t enqueue_step(yscv_hip_decoder *d, int batch, hipStream_t s) {
                                      L.kc8, L.ks, L.vc8, L.vs, s));
       YSCV_TRY(launch_attention_i8(d->qkv, L.kc8, L.ks, L.vc8, L.vs, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim,
                                    c.max_ctx, d->attn_part, d->ao, s));
+    } else if (d->fused_attn) {
+      YSCV_TRY(launch_attention_fused(d->qkv, L.kc, L.vc, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_theta,
+                                      c.max_ctx, d->attn_part, d->qrot, d->ao, s));
     } else {
       YSCV_TRY(launch_rope_append(d->qkv, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_theta, c.max_ctx,
                                   L.kc, L.vc, s));
@@ -883,6 +891,12 @@ int32_t yscv_hip_decoder_read_activation(yscv_hip_decoder *d, int32_t which, flo
   }
   std::vector<_Float16> tmp(elems);
   DEC_HIP(hipMemcpy(tmp.data(), src, elems * 2, hipMemcpyDeviceToHost));
+  if (which == YSCV_HIP_DEC_ACT_QKV && d->kv_dtype == YSCV_HIP_KV_F16 && d->fused_attn) {
+    // the fused attention kernel rotates q on the fly and leaves the buffer unrotated: report the rotated copy
+    const size_t qn = (size_t)c.n_heads * c.head_dim;
+    for (size_t b = 0; b < B; b++)
+      DEC_HIP(hipMemcpy(tmp.data() + b * qkv_n, d->qrot + b * qn, qn * 2, hipMemcpyDeviceToHost));
+  }
   for (size_t i = 0; i < elems; i++) out_host[i] = (float)tmp[i];
   return YSCV_HIP_OK;
 }
@@ -906,6 +920,13 @@ __attribute__((visibility("default"))) int32_t yscv_hip_debug_persist_trace(yscv
 int32_t yscv_hip_decoder_debug_set_tag_epoch(yscv_hip_decoder *d, uint32_t epoch) {
   YSCV_REQUIRE(d != nullptr && epoch >= 1, "null decoder or epoch 0");
   d->epoch = epoch;
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_debug_set_fused_attention(yscv_hip_decoder *d, int32_t on) {
+  YSCV_REQUIRE(d != nullptr, "null decoder");
+  drop_graph(d);  // a captured step holds the launches of the other variant
+  d->fused_attn = on != 0;
   return YSCV_HIP_OK;
 }
 

@@ -16,6 +16,11 @@ int32_t launch_kv_relayout(const _Float16 *k_nat, const _Float16 *v_nat, int bat
 int32_t launch_attention(const _Float16 *qkv, const _Float16 *kc, const _Float16 *vc, const int32_t *pos_ptr,
                          int batch, int hq, int hkv, int hd, int max_ctx, float *part, _Float16 *out,
                          hipStream_t s);
+// rope_append fused into the attention partials, then the merge (fp16 cache): `qrot` receives the rotated query heads
+// [batch][hq * 128] (diagnostics; qkv itself keeps the unrotated q)
+int32_t launch_attention_fused(const _Float16 *qkv, _Float16 *kc, _Float16 *vc, const int32_t *pos_ptr, int batch, int hq,
+                               int hkv, int hd, float theta, int max_ctx, float *part, _Float16 *qrot, _Float16 *out,
+                               hipStream_t s);
 // int8 cache (KvCache with KvDtype::I8): K int8 [batch][kv_head][max_ctx][128], V int8 [batch][kv_head][max_ctx/8][128][8],
 // one f32 scale per (batch row, position) for each of them
 int32_t launch_rope_append_i8(_Float16 *qkv, const int32_t *pos_ptr, int batch, int hq, int hkv, int hd, float theta,

@@ -56,6 +56,12 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const float *__restrict__ 
   }
 }
 
+// rotate-half of one pair, written with explicit fused multiply-adds so that every kernel that rotates rounds alike
+__device__ __forceinline__ void rope_pair(float x0, float x1, float cs, float sn, _Float16 &y0, _Float16 &y1) {
+  y0 = (_Float16)fmaf(x0, cs, -(x1 * sn));
+  y1 = (_Float16)fmaf(x0, sn, x1 * cs);
+}
+
 // ---- RoPE on q (in place) and k, then append k / v to the cache -------------------------------------
 // qkv: [batch][(Hq + 2*Hkv) * D] fp16, q heads first, then k heads, then v heads.
 // one workgroup per (batch row, head slot); head slots: Hq q heads, Hkv k heads, Hkv v heads.
@@ -76,7 +82,8 @@ __global__ void __launch_bounds__(64) rope_append_kernel(_Float16 *__restrict__ 
       float sn, cs;
       sincosf(ang, &sn, &cs);
       const float x0 = (float)src[i], x1 = (float)src[i + half_d];
-      const _Float16 y0 = (_Float16)(x0 * cs - x1 * sn), y1 = (_Float16)(x0 * sn + x1 * cs);
+      _Float16 y0, y1;
+      rope_pair(x0, x1, cs, sn, y0, y1);
       if (slot < hq) {
         src[i] = y0;
         src[i + half_d] = y1;
@@ -328,6 +335,207 @@ __global__ void __launch_bounds__(128) attn_combine_kernel(const float *__restri
   out[((size_t)b * hq + head) * HD + tid] = (_Float16)(o * inv);
 }
 
+// ---- rotary embedding + cache append + attention partials in ONE launch (fp16 cache) ------------------------------
+// Same arithmetic as rope_append_kernel -> attn_partial_kernel<false>, without the kernel boundary between them:
+//   * every workgroup rotates the query heads of its kv head itself (one (i, i + 64) pair per thread, through LDS)
+//     while its K / V loads are in flight; the rotated q is never written back (the workgroups of the other chunks
+//     read the unrotated one at the same time), only the workgroup of chunk 0 leaves a copy in `qrot` for diagnostics;
+//   * the workgroup whose chunk holds the current position rotates k, appends k and v to the cache and patches the
+//     new row into the registers of the wave that owns the position (the loads issued up front saw the old bytes).
+// attn_combine_kernel follows as a launch of its own.  (Merging the chunks in the same launch as well -- partials
+// through agent-scope stores, an arrival counter per (batch row, kv head), the last workgroup merges -- computed the
+// same values but was slower than the separate launch: 36.9 against 29.2 + 4.7 us at batch 16, context 2048; with an
+// acquire-release counter, whose cache write-back every workgroup pays, 113 us.)
+__global__ void __launch_bounds__(256) attn_fused_kernel(const _Float16 *__restrict__ qkv, _Float16 *kc, _Float16 *vc,
+                                                         const int32_t *__restrict__ pos_ptr, int hq, int hkv, int max_ctx,
+                                                         int max_chunks, float scale, float theta,
+                                                         float *__restrict__ part, _Float16 *__restrict__ qrot) {
+  constexpr int HD = 128;
+  __shared__ __attribute__((aligned(16))) _Float16 q_lds[4][HD];
+  __shared__ __attribute__((aligned(16))) _Float16 knew[HD], vnew[HD];
+  __shared__ __attribute__((aligned(16))) _Float16 p_lds[ATT_WAVES][4][32];
+  __shared__ float w_m[ATT_WAVES][4], w_l[ATT_WAVES][4];
+  __shared__ float w_o[ATT_WAVES][4][HD];
+  const int chunk = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, c = lane >> 4;
+  const int group = hq / hkv;
+  const int pos = *pos_ptr;
+  const int n_ctx = pos + 1;
+  const int live_chunks = (n_ctx + ATT_CHUNK - 1) / ATT_CHUNK;
+  if (chunk >= live_chunks) return;  // uniform in the workgroup, before any barrier
+  const int p0 = chunk * ATT_CHUNK + wave * ATT_POS_PER_WAVE;
+  const int row_elems = (hq + 2 * hkv) * HD;
+  const bool wave_live = p0 < n_ctx;
+  const bool owner = (pos / ATT_CHUNK) == chunk;  // this workgroup's positions include the current token
+
+  // ---- K / V of this wave's 32 positions: requested before anything else ----
+  const size_t k_off = (((size_t)b * hkv + kvh) * max_ctx + p0) * HD;
+  const size_t v_off = ((((size_t)b * hkv + kvh) * (max_ctx / 8) + p0 / 8) * HD) * 8;
+  half8_t kf[2][4], vf[8];
+  if (wave_live) {
+    const _Float16 *kbase = kc + k_off;
+    const _Float16 *vbase = vc + v_off;
+#pragma unroll
+    for (int pb = 0; pb < 2; pb++)
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        kf[pb][j] = *reinterpret_cast<const half8_t *>(kbase + (size_t)(pb * 16 + r) * HD + 32 * c + 8 * j);
+#pragma unroll
+    for (int t = 0; t < 8; t++) vf[t] = *reinterpret_cast<const half8_t *>(vbase + ((size_t)c * HD + t * 16 + r) * 8);
+  }
+
+  // ---- rotary embedding: thread (h = tid / 64, i = tid % 64) turns the pair (i, i + 64) of query head h ----
+  {
+    const int h = tid >> 6, i = tid & 63;
+    const float inv_freq = 1.0f / powf(theta, (float)(2 * i) / (float)HD);
+    const float ang = inv_freq * (float)pos;
+    float sn, cs;
+    sincosf(ang, &sn, &cs);
+    if (h < group) {
+      const int head = kvh * group + h;
+      const _Float16 *src = qkv + (size_t)b * row_elems + (size_t)head * HD;
+      const float x0 = (float)src[i], x1 = (float)src[i + HD / 2];
+      _Float16 y0, y1;
+      rope_pair(x0, x1, cs, sn, y0, y1);
+      q_lds[h][i] = y0;
+      q_lds[h][i + HD / 2] = y1;
+      if (chunk == 0) {
+        qrot[((size_t)b * hq + head) * HD + i] = y0;
+        qrot[((size_t)b * hq + head) * HD + i + HD / 2] = y1;
+      }
+    }
+    if (owner) {
+      if (h == 0) {
+        const _Float16 *src = qkv + (size_t)b * row_elems + (size_t)(hq + kvh) * HD;
+        const float x0 = (float)src[i], x1 = (float)src[i + HD / 2];
+        _Float16 y0, y1;
+      rope_pair(x0, x1, cs, sn, y0, y1);
+        knew[i] = y0;
+        knew[i + HD / 2] = y1;
+        _Float16 *dst = kc + (((size_t)b * hkv + kvh) * max_ctx + pos) * HD;
+        dst[i] = y0;
+        dst[i + HD / 2] = y1;
+      } else if (h == 1 || h == 2) {
+        const int dd = (h - 1) * 64 + i;
+        const _Float16 v = qkv[(size_t)b * row_elems + (size_t)(hq + hkv + kvh) * HD + dd];
+        vnew[dd] = v;
+        vc[((((size_t)b * hkv + kvh) * (max_ctx / 8) + pos / 8) * HD + dd) * 8 + (pos & 7)] = v;
+      }
+    }
+  }
+  __syncthreads();
+
+  float m_h = -INFINITY, l_h = 0.0f;
+  float o_acc[8];
+#pragma unroll
+  for (int t = 0; t < 8; t++) o_acc[t] = 0.0f;
+
+  if (wave_live) {
+    half8_t qa[4];
+    {
+      const int h = r >> 2;
+      const bool valid = ((r & 3) == 0) && h < group;
+      const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        qa[j] = valid ? *reinterpret_cast<const half8_t *>(&q_lds[h & 3][32 * c + 8 * j]) : z;
+    }
+    // the row appended in this launch: the loads above read whatever the cache held before
+    const int rel = pos - p0;
+    if (owner && rel >= 0 && rel < ATT_POS_PER_WAVE) {
+#pragma unroll
+      for (int pb = 0; pb < 2; pb++)
+        if (rel == pb * 16 + r) {
+#pragma unroll
+          for (int j = 0; j < 4; j++) kf[pb][j] = *reinterpret_cast<const half8_t *>(&knew[32 * c + 8 * j]);
+        }
+      const int e_new = rel - 8 * c;
+      if (e_new >= 0 && e_new < 8) {
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+          const _Float16 nv = vnew[t * 16 + r];
+#pragma unroll
+          for (int e = 0; e < 8; e++)
+            if (e == e_new) vf[t][e] = nv;
+        }
+      }
+    }
+
+    float s[2];
+#pragma unroll
+    for (int pb = 0; pb < 2; pb++) {
+      float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int j = 0; j < 4; j++) d = __builtin_amdgcn_mfma_f32_16x16x32_f16(qa[j], kf[pb][j], d, 0, 0, 0);
+      const int p = p0 + pb * 16 + r;
+      s[pb] = (p < n_ctx) ? d[0] * scale : -INFINITY;
+    }
+    float mx = fmaxf(s[0], s[1]);
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    const float e0 = (s[0] == -INFINITY) ? 0.0f : __expf(s[0] - mx);
+    const float e1 = (s[1] == -INFINITY) ? 0.0f : __expf(s[1] - mx);
+    float sum = e0 + e1;
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    m_h = mx;
+    l_h = sum;
+    if (c < 4) {
+      p_lds[wave][c][r] = (_Float16)e0;
+      p_lds[wave][c][16 + r] = (_Float16)e1;
+    }
+    __builtin_amdgcn_wave_barrier();
+    half8_t pa = {0, 0, 0, 0, 0, 0, 0, 0};
+    if ((r & 3) == 0 && (r >> 2) < group) pa = *reinterpret_cast<const half8_t *>(&p_lds[wave][r >> 2][8 * c]);
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      half8_t vv = vf[t];
+      if (p0 + 8 * c >= n_ctx) vv = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      else if (p0 + 8 * c + 8 > n_ctx) {
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+          if (p0 + 8 * c + e >= n_ctx) vv[e] = (_Float16)0.0f;
+      }
+      float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
+      d = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vv, d, 0, 0, 0);
+      o_acc[t] = d[0];
+    }
+  }
+
+  // ---- merge the 4 waves, write this chunk's partial ----
+  if (c < 4) {
+    if (r == 0) {
+      w_m[wave][c] = m_h;
+      w_l[wave][c] = l_h;
+    }
+#pragma unroll
+    for (int t = 0; t < 8; t++) w_o[wave][c][t * 16 + r] = o_acc[t];
+  }
+  __syncthreads();
+  for (int idx = tid; idx < group * HD; idx += blockDim.x) {
+    const int h = idx / HD, dd = idx % HD;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < ATT_WAVES; w++) mx = fmaxf(mx, w_m[w][h]);
+    float l = 0.0f, o = 0.0f;
+#pragma unroll
+    for (int w = 0; w < ATT_WAVES; w++) {
+      const float f = (w_m[w][h] == -INFINITY) ? 0.0f : __expf(w_m[w][h] - mx);
+      l += w_l[w][h] * f;
+      o += w_o[w][h][dd] * f;
+    }
+    const int head = kvh * group + h;
+    float *dst = part + (((size_t)b * hq + head) * max_chunks + chunk) * (HD + 2);
+    dst[2 + dd] = o;
+    if (dd == 0) {
+      dst[0] = mx;
+      dst[1] = l;
+    }
+  }
+
+}
+
 // ---- greedy pick: last index among equal maxima; also records the token and advances the position ------
 __global__ void __launch_bounds__(1024) argmax_kernel(const float *__restrict__ logits, int vocab,
                                                       int32_t *__restrict__ tokens, int32_t *__restrict__ history,
@@ -570,6 +778,22 @@ int32_t launch_attention(const _Float16 *qkv, const _Float16 *kc, const _Float16
   const float scale = 1.0f / sqrtf((float)hd);
   hipLaunchKernelGGL(attn_partial_kernel<false>, dim3(max_chunks, hkv, batch), dim3(256), 0, s, qkv, kc, vc, nullptr, nullptr,
                      pos_ptr, hq, hkv, max_ctx, max_chunks, scale, part);
+  YSCV_HIP_TRY(hipGetLastError());
+  hipLaunchKernelGGL(attn_combine_kernel, dim3(hq, batch), dim3(128), 0, s, part, pos_ptr, hq, max_chunks, out);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_attention_fused(const _Float16 *qkv, _Float16 *kc, _Float16 *vc, const int32_t *pos_ptr, int batch, int hq,
+                               int hkv, int hd, float theta, int max_ctx, float *part, _Float16 *qrot, _Float16 *out,
+                               hipStream_t s) {
+  if (hd != 128) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "attention kernel is built for head_dim 128, got %d", hd);
+  if (hq % hkv != 0 || hq / hkv > 4)
+    return set_error(YSCV_HIP_ERR_UNSUPPORTED, "attention kernel handles 1..4 query heads per kv head");
+  const int max_chunks = max_ctx / ATT_CHUNK;
+  const float scale = 1.0f / sqrtf((float)hd);
+  hipLaunchKernelGGL(attn_fused_kernel, dim3(max_chunks, hkv, batch), dim3(256), 0, s, qkv, kc, vc, pos_ptr, hq, hkv, max_ctx,
+                     max_chunks, scale, theta, part, qrot);
   YSCV_HIP_TRY(hipGetLastError());
   hipLaunchKernelGGL(attn_combine_kernel, dim3(hq, batch), dim3(128), 0, s, part, pos_ptr, hq, max_chunks, out);
   YSCV_HIP_TRY(hipGetLastError());
