@@ -77,6 +77,31 @@ struct DevBuf {
   }
 };
 
+// Scratch from the stream-ordered allocator: allocation and release are queued on the stream like the kernels that
+// use the memory, so the call that owns the buffer can return without waiting for the device.
+struct StreamBuf {
+  void *p = nullptr;
+  hipStream_t s = nullptr;
+  ~StreamBuf() {
+    if (p) (void)hipFreeAsync(p, s);
+  }
+  int32_t alloc(size_t bytes, hipStream_t stream) {
+    if (bytes == 0) bytes = 4;
+    s = stream;
+    hipError_t e = hipMallocAsync(&p, bytes, s);
+    if (e != hipSuccess) {
+      p = nullptr;
+      return set_error(e == hipErrorOutOfMemory ? YSCV_HIP_ERR_OOM : YSCV_HIP_ERR_DEVICE,
+                       "hipMallocAsync(%zu) failed: %s", bytes, hipGetErrorString(e));
+    }
+    return YSCV_HIP_OK;
+  }
+  template <typename T>
+  T *as() const {
+    return static_cast<T *>(p);
+  }
+};
+
 inline size_t ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }
 inline size_t round_up(size_t a, size_t b) { return ceil_div(a, b) * b; }
 

@@ -95,6 +95,17 @@ __device__ __forceinline__ int32_t requant_dequant_bits(int32_t acc, int32_t cor
   return __float_as_int(__fmul_rn(__fsub_rn((float)q, y_zp), dq_scale));
 }
 
+// requantise and keep the value as an f32 carrier, the form exec_qlinear_matmul returns (crates/yscv-onnx/src/runner/
+// linear.rs:481-485): clamp keeps a NaN
+__device__ __forceinline__ int32_t requant_f32_bits(int32_t acc, int32_t corr, float comp, float y_zp, int round_mode,
+                                                    float lo, float hi) {
+  int32_t a = (int32_t)((uint32_t)acc + (uint32_t)corr);
+  float v = __fadd_rn(__fmul_rn((float)a, comp), y_zp);
+  float r = round_mode == YSCV_HIP_ROUND_HALF_AWAY ? round_half_away(v) : rintf(v);
+  if (r == r) r = fminf(fmaxf(r, lo), hi);
+  return __float_as_int(r);
+}
+
 struct I8Args {
   const uint8_t *a;   // [m][k]
   const int8_t *frag; // packed B
@@ -103,7 +114,7 @@ struct I8Args {
   const int32_t *corr;
   const float *composite_v;
   float composite, y_zp, dq_scale;
-  int round_mode, lo, hi, mode;  // mode 0: int32 out, 1: requantised bytes, 2: requantise + dequantise to f32
+  int round_mode, lo, hi, mode;  // as I8Epilogue::mode
   int m, n, k;
   int ksteps;       // kp / 64
   int a_xor;        // 0x80808080 for uint8 activations, 0 for int8
@@ -233,6 +244,8 @@ __global__ void __launch_bounds__(I8_THREADS) i8_gemm_kernel(I8Args p) {
           reinterpret_cast<float *>(p.out)[o] = (float)v;
         } else if (p.mode == 2) {
           reinterpret_cast<int32_t *>(p.out)[o] = requant_dequant_bits(v, corr, comp, p.y_zp, p.round_mode, lo, hi, p.dq_scale);
+        } else if (p.mode == 4) {
+          reinterpret_cast<int32_t *>(p.out)[o] = requant_f32_bits(v, corr, comp, p.y_zp, p.round_mode, lo, hi);
         } else {
           int q = requant_one(v, corr, comp, p.y_zp, p.round_mode, lo, hi);
           reinterpret_cast<uint8_t *>(p.out)[o] = (uint8_t)q;
@@ -502,6 +515,11 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
 #pragma unroll
           for (int e = 0; e < 4; e++)
             f[e] = requant_dequant_bits(v[e], corr[e], comp[e], p.y_zp, p.round_mode, lo, hi, p.dq_scale);
+          *reinterpret_cast<int4_t *>(i8_ring + lrow * RS32 + lcol * 4) = f;
+        } else if (p.mode == 4) {
+          int4_t f;
+#pragma unroll
+          for (int e = 0; e < 4; e++) f[e] = requant_f32_bits(v[e], corr[e], comp[e], p.y_zp, p.round_mode, lo, hi);
           *reinterpret_cast<int4_t *>(i8_ring + lrow * RS32 + lcol * 4) = f;
         } else {
           uint32_t packed = 0;

@@ -103,7 +103,8 @@ void note_int4_fallback();
 int32_t launch_i8_pack_b(const int8_t *b_kn, size_t k, size_t n, size_t kp, size_t np,
                          int8_t *frag, int32_t *col_sum, hipStream_t s);
 struct I8Epilogue {
-  int mode;  // 0: int32 out, 1: requantize to bytes, 2: requantize, then (q - y_zp) * dq_scale as f32, 3: f32(int32) out
+  int mode;  // 0: int32 out, 1: requantize to bytes, 2: requantize, then (q - y_zp) * dq_scale as f32, 3: f32(int32) out,
+             // 4: requantize, the quantised value kept as f32 (a NaN stays a NaN)
   const int32_t *corr;
   const float *composite_v;
   float composite;

@@ -279,19 +279,36 @@ struct MatmulArgs {
 };
 
 int32_t run_fast(const MatmulArgs &g) {
+  if (g.b_packed) {
+    // the usual case, a weight packed at load time: cast kernel + GEMM whose epilogue writes the f32 carriers, the
+    // int8 copy of A in stream-ordered scratch -- nothing here waits for the device
+    StreamBuf a8;
+    YSCV_TRY(a8.alloc(g.m * g.k, g.s));
+    hipLaunchKernelGGL(cast_as_i8_kernel, dim3(grid_for(g.m * g.k)), dim3(256), 0, g.s, g.a, g.m * g.k, 0, a8.as<int8_t>());
+    YSCV_HIP_TRY(hipGetLastError());
+    I8Epilogue ep{};
+    if (g.op == OP_QLINEAR) {
+      ep.mode = 4;
+      ep.composite = (g.a_scale * g.b_scale) / g.y_scale;
+      ep.y_zp = g.y_zp;
+      ep.round_mode = YSCV_HIP_ROUND_HALF_AWAY;
+      ep.lo = -128;
+      ep.hi = 127;
+    } else {
+      ep.mode = 3;
+    }
+    return launch_i8_gemm(a8.p, 0, 0, g.b_packed, g.m, g.out, ep, g.s);
+  }
   DevBuf a8, b8, acc;
   YSCV_TRY(a8.alloc(g.m * g.k));
   YSCV_TRY(acc.alloc(g.m * g.n * sizeof(int32_t)));
   hipLaunchKernelGGL(cast_as_i8_kernel, dim3(grid_for(g.m * g.k)), dim3(256), 0, g.s, g.a, g.m * g.k, 0, a8.as<int8_t>());
   TempWeight tmp;
-  const yscv_hip_i8_weight *w = g.b_packed;
-  if (!w) {
-    YSCV_TRY(b8.alloc(g.k * g.n));
-    hipLaunchKernelGGL(cast_as_i8_kernel, dim3(grid_for(g.k * g.n)), dim3(256), 0, g.s, g.b, g.k * g.n, 0,
-                       b8.as<int8_t>());
-    YSCV_TRY(pack_device_i8(b8.as<int8_t>(), g.k, g.n, g.s, &tmp.w));
-    w = tmp.w;
-  }
+  YSCV_TRY(b8.alloc(g.k * g.n));
+  hipLaunchKernelGGL(cast_as_i8_kernel, dim3(grid_for(g.k * g.n)), dim3(256), 0, g.s, g.b, g.k * g.n, 0,
+                     b8.as<int8_t>());
+  YSCV_TRY(pack_device_i8(b8.as<int8_t>(), g.k, g.n, g.s, &tmp.w));
+  const yscv_hip_i8_weight *w = tmp.w;
   I8Epilogue ep{};
   ep.mode = 0;
   YSCV_TRY(launch_i8_gemm(a8.p, 0, 0, w, g.m, acc.p, ep, g.s));
@@ -300,7 +317,7 @@ int32_t run_fast(const MatmulArgs &g) {
                      (const int32_t *)nullptr, 0, 0, g.m, g.n, g.op == OP_QLINEAR ? 1 : 0, composite, 0.0, g.y_scale,
                      g.y_zp, g.out);
   YSCV_HIP_TRY(hipGetLastError());
-  YSCV_HIP_TRY(hipStreamSynchronize(g.s));  // the scratch buffers are released on return
+  YSCV_HIP_TRY(hipStreamSynchronize(g.s));  // the scratch buffers and the temporary weight are released on return
   return YSCV_HIP_OK;
 }
 
@@ -685,14 +702,13 @@ int32_t yscv_hip_exec_dynamic_quantize_linear(const float *x_dev, size_t len, fl
   YSCV_REQUIRE(y_scale_dev && y_zp_dev, "null scale / zero-point pointer");
   YSCV_REQUIRE(len == 0 || (x_dev && y_dev), "null pointer");
   hipStream_t s = as_stream(stream);
-  DevBuf q, sz;
-  YSCV_TRY(q.alloc(len));
-  YSCV_TRY(sz.alloc(2 * sizeof(float)));
+  StreamBuf q, sz;  // released in stream order: the call does not wait for the device
+  YSCV_TRY(q.alloc(len, s));
+  YSCV_TRY(sz.alloc(2 * sizeof(float), s));
   YSCV_TRY(launch_dynamic_quantize_linear(x_dev, len, q.as<uint8_t>(), sz.as<float>(), s));
   hipLaunchKernelGGL(u8_to_f32_kernel, dim3(grid_for(len)), dim3(256), 0, s, q.as<uint8_t>(), len, sz.as<float>(),
                      y_dev, y_scale_dev, y_zp_dev);
   YSCV_HIP_TRY(hipGetLastError());
-  YSCV_HIP_TRY(hipStreamSynchronize(s));
   return YSCV_HIP_OK;
 }
 
