@@ -360,7 +360,14 @@ def extra_kernels(torch, stream_ptr):
         th = tavg(gemv_hot, 56)
         c1[name] = {"us_per_call_whole_op": round(t * 1e6, 2), "GB/s_whole_op": round(byt / t / 1e9, 1),
                     "hot_us_per_call": round(th * 1e6, 2), "hot_GB/s": round(byt / th / 1e9, 1)}
-    c1["note"] = ("cold = 56 rotating weight copies (587 MB, > 2x the 256 MB Infinity Cache), hot = one copy; one kernel per "
+    from yscv_amd.capi import lib as _lib
+    import ctypes as _C
+
+    def empty():
+        _lib().launch_empty(_C.c_void_p(torch.cuda.current_stream().cuda_stream))
+
+    c1["launch_floor_us"] = round(tavg(empty, 200) * 1e6, 2)
+    c1["note"] = ("launch_floor_us = an empty kernel of the same grid timed the same way (nodes of one graph); cold = 56 rotating weight copies (587 MB, > 2x the 256 MB Infinity Cache), hot = one copy; one kernel per "
                   "call, the f32 input is normalised and split inside it")
     out["config1_gemv_m1_k4096_n4096"] = c1
     del ring
@@ -412,6 +419,38 @@ def extra_kernels(torch, stream_ptr):
                             "TFLOP/s": round(fl / t / 1e12, 1), "frac_of_mfma_peak": round(fl / t / 1e12 / MFMA_BF16_PEAK, 4),
                             "kernel": "int4_skinny_kernel" if m <= 16 else "int4_gemm_ring_kernel"}
     out["config5_lm_head_sweep_k4096_n128256"] = sweep
+
+    # where the skinny kernel hands over to the MFMA GEMM: both kernels on either side of m = 16 (event-timed eager
+    # calls: the forced modes take their scratch from the stream-ordered allocator)
+    def teager(fn, reps=20):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        s_, e_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s_.record()
+        for _ in range(reps):
+            fn()
+        e_.record()
+        torch.cuda.synchronize()
+        return s_.elapsed_time(e_) * 1e-3 / reps
+
+    x16, x32 = torch.randn(16, k, device="cuda").bfloat16(), torch.randn(32, k, device="cuda").bfloat16()
+    x17 = torch.randn(17, k, device="cuda").bfloat16()
+    y16 = torch.empty(16, n, device="cuda", dtype=torch.bfloat16)
+    y17 = torch.empty(17, n, device="cuda", dtype=torch.bfloat16)
+    y32 = torch.empty(32, n, device="cuda", dtype=torch.bfloat16)
+
+    def two_passes():
+        w.matmul(x32[:16], out=y32[:16], mode="gemv")
+        w.matmul(x32[16:], out=y32[16:], mode="gemv")
+
+    out["switch_skinny_to_gemm_lm_head"] = {
+        "m16_skinny_us": round(teager(lambda: w.matmul(x16, out=y16, mode="gemv")) * 1e6, 1),
+        "m17_gemm_us": round(teager(lambda: w.matmul(x17, out=y17, mode="gemm")) * 1e6, 1),
+        "m32_two_skinny_passes_us": round(teager(two_passes) * 1e6, 1),
+        "m32_gemm_us": round(teager(lambda: w.matmul(x32, out=y32, mode="gemm")) * 1e6, 1),
+        "note": "yscv_hip_int4_matmul switches at m = 16: one skinny pass up to 16 rows, above that the LDS-ring MFMA GEMM, "
+                "whose smallest tile has 32 rows (m = 17 costs what m = 32 costs)"}
     w.close()
     return out
 

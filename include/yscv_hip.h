@@ -79,6 +79,10 @@ int32_t yscv_hip_device_info(char *buf, size_t buf_len);
  * its microbenchmark relates the dispatch kernels to its own scalar loops ("SIMD speedup vs scalar",
  * apps/llm-bench/src/bin/kernel_bench.rs:187), not to a machine peak. */
 int32_t yscv_hip_measure_peaks(double *hbm_read_gbs, double *mfma_f16_tflops, double *mfma_i8_tops);
+/* Calibration: one launch of a kernel that does nothing (one 512-thread workgroup per CU) on `stream`.  A benchmark
+ * that times many of them, back to back or as the nodes of a graph, gets the floor under the duration of any kernel
+ * (what a single short GEMV cannot go below).  No counterpart in the reference. */
+int32_t yscv_hip_launch_empty(void *stream);
 
 /* Device memory helpers for hosts without their own HIP binding. */
 int32_t yscv_hip_malloc(void **dev_ptr, size_t bytes);

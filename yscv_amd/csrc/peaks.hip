@@ -63,10 +63,27 @@ struct Events {
   }
 };
 
+__global__ void __launch_bounds__(512) empty_kernel(uint32_t *flag) {
+  if (flag == nullptr) __builtin_amdgcn_s_sleep(1);  // never true for the launcher below; keeps the body from being dropped
+}
+
 }  // namespace
 }  // namespace yscv
 
 using namespace yscv;
+
+// One launch of a kernel that does nothing, with the grid every decode-sized kernel here uses (one 512-thread workgroup
+// per CU): timed back to back or as the nodes of a graph it gives the floor under any kernel's duration.
+extern "C" int32_t yscv_hip_launch_empty(void *stream) {
+  const Context *ctx = nullptr;
+  YSCV_TRY(ensure_context(&ctx));
+  static uint32_t *flag = nullptr;  // any non-null device address; never dereferenced
+  if (!flag) YSCV_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&flag), 64));
+  const int wgs = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  hipLaunchKernelGGL(empty_kernel, dim3(wgs), dim3(512), 0, static_cast<hipStream_t>(stream), flag);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
 
 extern "C" int32_t yscv_hip_measure_peaks(double *hbm_read_gbs, double *mfma_f16_tflops, double *mfma_i8_tops) {
   const Context *ctx = nullptr;
