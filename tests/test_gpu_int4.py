@@ -376,6 +376,39 @@ def test_lm_head_sweep_sampled_at_full_size(oracle, K, torch_cuda):
     w.close()
 
 
+def test_ring_gemm_every_output_at_lm_head_shape(K, torch_cuda):
+    """Every element of the MFMA GEMM's output at the LM-head shape (K=4096, N=128256), for row counts that select
+    each tile shape (32-, 64-row, 128 x 256, 256 x 128), three calls each: against an fp32 product with the dequantised
+    weight on the GPU (tolerance of the bf16 output), and bit-identical from call to call.  A sampled check misses a
+    weight tile that goes wrong now and then (a few 16-column blocks of a hundred thousand columns)."""
+    torch = torch_cuda
+    rng = np.random.default_rng(56)
+    k, n, g = 4096, 128256, 32
+    b = rng.integers(0, 256, n * k // 2, dtype=np.uint8)
+    scales16 = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float16)
+    w = K.PackedInt4Weight(b, scales16, g, n, k, nibble_format=K.NIBBLE_UNSIGNED)
+    bt = torch.from_numpy(b.reshape(n, k // 2)).cuda()
+    wd = torch.stack(((bt & 15).float() - 8.0, (bt >> 4).float() - 8.0), dim=2).reshape(n, k // g, g)
+    del bt
+    wd = (wd * torch.from_numpy(scales16.reshape(n, k // g).astype(np.float32)).cuda()[:, :, None]).reshape(n, k)
+    x_all = torch.from_numpy(rng.standard_normal((256, k)).astype(np.float32)).bfloat16().cuda()
+    for m in (24, 64, 96, 128, 200, 256):
+        x = x_all[:m].contiguous()
+        ref = x.float() @ wd.T
+        bound = float(ref.abs().max()) * 2.0 ** -7
+        first = None
+        for rep in range(3):
+            y = w.matmul(x)
+            err = float((y.float() - ref).abs().nan_to_num(1e9).max())
+            assert err <= bound, (m, rep, err, bound)
+            if first is None:
+                first = y
+            else:
+                assert torch.equal(y, first), (m, rep)
+        del ref
+    w.close()
+
+
 def test_weight_loaded_from_a_file_equals_the_uploaded_one(K, torch_cuda, tmp_path):
     """yscv_hip_int4_weight_load: the on-disk form carries exactly the arguments of the upload call."""
     torch = torch_cuda

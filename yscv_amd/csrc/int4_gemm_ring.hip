@@ -361,13 +361,12 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
     });
     publish(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, std::integral_constant<int, SA / 2 - 1>{},
             std::integral_constant<int, SA / 2>{});
-    int s0 = 0;
-    for (; s0 + SA <= last; s0 += SA) g4_static_for<0, SA>([&](auto uc) { step(s0 + decltype(uc)::value, uc); });
-    // the remaining 0 .. SA-1 steps as straight-line code
-    g4_static_for<1, SA>([&](auto rc) {
-      constexpr int R = decltype(rc)::value;
-      if (last - s0 == R) g4_static_for<0, R>([&](auto uc) { step(s0 + decltype(uc)::value, uc); });
-    });
+    // The steps run in whole groups of SA, one loop and nothing after it: `last` steps are needed, the group is
+    // completed with steps past the end (they publish the last stage again into a slot nobody reads; the MMA waves
+    // answer their barriers, see below).  Straight-line code for the 1 .. SA-1 left-over steps behind the loop gave the
+    // compiler a place to move the tile registers of loads still in flight (copies at the entry of each left-over
+    // path, executed before the data had landed): wrong weights in the last stages, now and then.
+    for (int s0 = 0; s0 < last; s0 += SA) g4_static_for<0, SA>([&](auto uc) { step(s0 + decltype(uc)::value, uc); });
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     // the registers of the loads issued past the end stay reserved until those loads have landed
 #pragma unroll
@@ -417,6 +416,9 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
       aslot = naslot;
       bslot = nbslot;
     }
+    // the producers run their steps in whole groups of SA: answer the barriers of the steps past the last stage
+    const int steps = nstages - 1;
+    for (int e = steps; e < (steps + SA - 1) / SA * SA; e++) __builtin_amdgcn_s_barrier();
   }
 
   // ---- epilogue: lane (c, r) of an MMA wave holds y[16 i + r][16 j + 4 c + 0..3] of its part; through LDS so that

@@ -504,26 +504,25 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
   // Meet the other k slices in LDS, once per UB blocks: every wave leaves its UB x NI x 64 partial sums, and after
   // one barrier the sums are shared out over the waves in 64-lane pieces (piece q = block q / NI of the group,
   // accumulator q % NI), rotating so that no wave is always the late one.
+  // the wave index as the scalar it is (the compiler takes anything derived from threadIdx for a per-lane value, and
+  // the piece loop below would then run under exec masks with its indices in vector registers)
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  int exm = 0;  // reductions done so far, modulo the number of waves: rotates the piece-to-wave assignment
+
   auto reduce_store = [&](const float (&accs)[UB][NI], int nt0, int ex) {
     float *buf = red + (size_t)(ex & 1) * waves * (UB * NI) * 64;
+    {
+      float *wb = buf + wave * (UB * NI) * 64 + lane;
 #pragma unroll
-    for (int u = 0; u < UB; u++)
+      for (int u = 0; u < UB; u++)
 #pragma unroll
-      for (int i = 0; i < NI; i++) buf[((wave * UB + u) * NI + i) * 64 + lane] = accs[u][i];
+        for (int i = 0; i < NI; i++) wb[(u * NI + i) * 64] = accs[u][i];
+    }
     lds_barrier();
-    for (int q = (wave + ex) % waves; q < UB * NI; q += waves) {
+    // epilogue of one finished 64-lane piece q = u * NI + i: block u of the group, accumulator i
+    auto finish = [&](float v, int q) {
       const int u = q / NI, i = q % NI;
       const int col = (nt0 + u * stride) * 16 + r;
-      // the slices are fetched four at a time (two LDS round trips, few registers), then added in slice order
-      float v = 0.0f;
-#pragma unroll
-      for (int w0 = 0; w0 < 8; w0 += 4) {
-        float part[4];
-#pragma unroll
-        for (int w = 0; w < 4; w++) part[w] = w0 + w < waves ? buf[(((w0 + w) * UB + u) * NI + i) * 64 + lane] : 0.0f;
-#pragma unroll
-        for (int w = 0; w < 4; w++) v += part[w];
-      }
       const int mrow = c * NI + i;
       const bool live = mrow < a.m && col < a.n;
       if (a.ksg > 1) {
@@ -545,6 +544,43 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
           store_out(a.y, (size_t)mrow * a.n + col, v, a.y_dtype);
         }
       }
+    };
+    int q = wave_s + exm;
+    if (q >= waves) q -= waves;
+    exm = exm + 1 == waves ? 0 : exm + 1;
+    // slice w of piece q sits at buf[(w * UB * NI + q) * 64 + lane]: one base per piece, constant offsets per slice
+    if (waves == 8 && UB * NI == 16) {
+      // the usual shape, two pieces per wave (q and q + 8): all sixteen slices are requested in one go (one LDS round
+      // trip per reduction instead of four), then added in slice order
+      const float *rb = buf + q * 64 + lane;
+      float p0[8], p1[8];
+#pragma unroll
+      for (int w = 0; w < 8; w++) {
+        p0[w] = rb[w * (UB * NI) * 64];
+        p1[w] = rb[w * (UB * NI) * 64 + 8 * 64];
+      }
+      float v0 = 0.0f, v1 = 0.0f;
+#pragma unroll
+      for (int w = 0; w < 8; w++) {
+        v0 += p0[w];
+        v1 += p1[w];
+      }
+      finish(v0, q);
+      finish(v1, q + 8);
+      return;
+    }
+    for (; q < UB * NI; q += waves) {
+      const float *rb = buf + q * 64 + lane;
+      float v = 0.0f;
+#pragma unroll
+      for (int w0 = 0; w0 < 8; w0 += 4) {  // four slices at a time: two LDS round trips, few registers
+        float part[4];
+#pragma unroll
+        for (int w = 0; w < 4; w++) part[w] = w0 + w < waves ? rb[(w0 + w) * (UB * NI) * 64] : 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) v += part[w];
+      }
+      finish(v, q);
     }
   };
 
