@@ -287,6 +287,18 @@ def test_full_depth_single_launch_agrees_with_multi_kernel_path(nibbles):
     for b in range(B):
         assert picks[b] == greedy_pick(many[b])
     assert len({int(p) for p in picks}) > 1  # different rows, different inputs
+    # no path has a result that depends on timing (no atomics on shared sums, fixed merge orders): the same state gives
+    # the same bits, three times over 24 steps
+    for persistent, b in ((True, 1), (False, 1), (False, B)):
+        want = None
+        for rep in range(3):
+            dec.reset(tokens[:b], start)
+            dec.run(24, use_graph=True, persistent=persistent)
+            got = (dec.tokens(0, 24).copy(), dec.logits().copy())
+            if want is None:
+                want = got
+            else:
+                assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]), (persistent, b, rep)
     dec.close()
 
 

@@ -376,11 +376,12 @@ def test_lm_head_sweep_sampled_at_full_size(oracle, K, torch_cuda):
     w.close()
 
 
-def test_ring_gemm_every_output_at_lm_head_shape(K, torch_cuda):
-    """Every element of the MFMA GEMM's output at the LM-head shape (K=4096, N=128256), for row counts that select
-    each tile shape (32-, 64-row, 128 x 256, 256 x 128), three calls each: against an fp32 product with the dequantised
-    weight on the GPU (tolerance of the bf16 output), and bit-identical from call to call.  A sampled check misses a
-    weight tile that goes wrong now and then (a few 16-column blocks of a hundred thousand columns)."""
+def test_every_output_at_lm_head_shape(K, torch_cuda):
+    """Every element of the output at the LM-head shape (K=4096, N=128256), for row counts that select the skinny kernel
+    with one, two and four accumulators and each tile shape of the MFMA GEMM (32-, 64-row, 128 x 256, 256 x 128), three
+    calls each: against an fp32 product with the dequantised weight on the GPU (tolerance of the bf16 output), and
+    bit-identical from call to call.  A sampled check misses a weight tile that goes wrong now and then (a few
+    16-column blocks of a hundred thousand columns)."""
     torch = torch_cuda
     rng = np.random.default_rng(56)
     k, n, g = 4096, 128256, 32
@@ -392,7 +393,7 @@ def test_ring_gemm_every_output_at_lm_head_shape(K, torch_cuda):
     del bt
     wd = (wd * torch.from_numpy(scales16.reshape(n, k // g).astype(np.float32)).cuda()[:, :, None]).reshape(n, k)
     x_all = torch.from_numpy(rng.standard_normal((256, k)).astype(np.float32)).bfloat16().cuda()
-    for m in (24, 64, 96, 128, 200, 256):
+    for m in (1, 4, 8, 16, 24, 64, 96, 128, 200, 256):
         x = x_all[:m].contiguous()
         ref = x.float() @ wd.T
         bound = float(ref.abs().max()) * 2.0 ** -7
