@@ -517,3 +517,53 @@ def test_fused_epilogues_at_decoder_shapes(oracle, K, torch_cuda, n, k, m):
     with pytest.raises(Exception, match="m <= 16"):
         w.matmul_fused(torch.zeros(17, k, device="cuda", dtype=torch.float16), torch.zeros(17, n, device="cuda"), K.EPILOGUE_STORE)
     w.close()
+
+
+def _dequant_on_gpu(torch, b, scales, n, k, g, zq=None):
+    """[n][k] f32 weight from packed nibbles (element 2i in the low nibble), per-group scales and zero points."""
+    bt = torch.from_numpy(b.reshape(n, k // 2)).cuda()
+    q = torch.stack(((bt & 15).float(), (bt >> 4).float()), dim=2).reshape(n, k // g, g)
+    z = 8.0 if zq is None else torch.from_numpy(zq.astype(np.float32)).cuda()[:, :, None]
+    sc = torch.from_numpy(scales.reshape(n, k // g).astype(np.float32)).cuda()[:, :, None]
+    return ((q - z) * sc).reshape(n, k)
+
+
+def test_random_shapes_every_output(K, torch_cuda):
+    """Forty shapes drawn from a fixed seed -- row counts on both sides of every kernel and tile switch, ragged N, K from
+    one tile to the down projection's 14336, all group sizes, zero points, f32 / fp16 scales, every activation type --
+    with EVERY output element held against an fp32 product on the GPU (bar: the int4 tolerance of the kernels, plus the
+    rounding of a 16-bit output), twice, the second call bit-identical to the first."""
+    torch = torch_cuda
+    rng = np.random.default_rng(20260)
+    ms = [1, 2, 4, 5, 8, 9, 16, 17, 31, 32, 33, 64, 65, 100, 128, 129, 255, 256, 257, 384, 513]
+    for case in range(40):
+        m = int(rng.choice(ms))
+        g = int(rng.choice([32, 32, 64, 128]))
+        k = int(rng.choice([128, 256, 384, 1024, 2048, 4096, 14336]))
+        if k % g:
+            k = (k // g) * g
+        n = int(rng.choice([16, 48, 100, 257, 1000, 4096, 6144, 11008, 24011]))
+        if m * n * k > 2.2e11:  # keep the case under a second
+            n = 1000
+        sf16 = bool(rng.integers(0, 2))
+        has_zp = bool(rng.integers(0, 2))
+        xdt = [torch.float32, torch.float16, torch.bfloat16][int(rng.integers(0, 3))]
+        b = rng.integers(0, 256, n * k // 2, dtype=np.uint8)
+        scales = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float16 if sf16 else np.float32)
+        zq = rng.integers(5, 12, (n, k // g)) if has_zp else None
+        w = K.PackedInt4Weight(b, scales, g, n, k, zero_points=pack_zero_points(zq) if has_zp else None,
+                               nibble_format=K.NIBBLE_UNSIGNED)
+        wd = _dequant_on_gpu(torch, b, scales, n, k, g, zq)
+        x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).to(xdt).cuda()
+        ref = x.float() @ wd.T
+        y = w.matmul(x)
+        tag = (case, m, n, k, g, sf16, has_zp, str(xdt))
+        assert tuple(y.shape) == (m, n) and y.dtype == xdt, tag
+        err = float((y.float() - ref).abs().nan_to_num(1e9).max())
+        top = float(ref.abs().max())
+        out_round = {torch.float32: 0.0, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[xdt]
+        assert err <= top * (1e-3 + out_round) + 1e-6, tag + (err, top)
+        assert err <= 1e-3 * np.sqrt(k) * float(x.float().abs().max()), tag + (err,)
+        assert torch.equal(w.matmul(x), y), tag
+        w.close()
+        del wd, ref
