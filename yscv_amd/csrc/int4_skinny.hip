@@ -572,13 +572,21 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
     for (; q < UB * NI; q += waves) {
       const float *rb = buf + q * 64 + lane;
       float v = 0.0f;
+      if (waves == 8) {  // all eight slices in one LDS round trip
+        float part[8];
 #pragma unroll
-      for (int w0 = 0; w0 < 8; w0 += 4) {  // four slices at a time: two LDS round trips, few registers
-        float part[4];
+        for (int w = 0; w < 8; w++) part[w] = rb[w * (UB * NI) * 64];
 #pragma unroll
-        for (int w = 0; w < 4; w++) part[w] = w0 + w < waves ? rb[(w0 + w) * (UB * NI) * 64] : 0.0f;
+        for (int w = 0; w < 8; w++) v += part[w];
+      } else {
 #pragma unroll
-        for (int w = 0; w < 4; w++) v += part[w];
+        for (int w0 = 0; w0 < 8; w0 += 4) {  // four slices at a time: two LDS round trips, few registers
+          float part[4];
+#pragma unroll
+          for (int w = 0; w < 4; w++) part[w] = w0 + w < waves ? rb[(w0 + w) * (UB * NI) * 64] : 0.0f;
+#pragma unroll
+          for (int w = 0; w < 4; w++) v += part[w];
+        }
       }
       finish(v, q);
     }
