@@ -36,16 +36,49 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const float *__restrict__ 
   __shared__ float red[4];
   const int b = blockIdx.x;
   const float *row = h + (size_t)b * d;
+  // a row of up to 8192 values stays in registers between the two passes (one memory round trip instead of two);
+  // longer rows are read again
+  constexpr int KEEP = 8;
+  float4_t keep[KEEP];
+  const bool fits = d <= KEEP * 256 * 4;
   float ss = 0.0f;
-  for (int i = threadIdx.x * 4; i < d; i += blockDim.x * 4) {
-    float4_t v = *reinterpret_cast<const float4_t *>(row + i);
-    ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+  if (fits) {
+#pragma unroll
+    for (int u = 0; u < KEEP; u++) {
+      const int i = (u * 256 + (int)threadIdx.x) * 4;
+      keep[u] = i < d ? *reinterpret_cast<const float4_t *>(row + i) : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+#pragma unroll
+    for (int u = 0; u < KEEP; u++) {
+      const float4_t v = keep[u];
+      if ((u * 256 + (int)threadIdx.x) * 4 < d) ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+    }
+  } else {
+    for (int i = threadIdx.x * 4; i < d; i += blockDim.x * 4) {
+      float4_t v = *reinterpret_cast<const float4_t *>(row + i);
+      ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+    }
   }
   for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
   __syncthreads();
   ss = red[0] + red[1] + red[2] + red[3];
   const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+  if (fits) {
+#pragma unroll
+    for (int u = 0; u < KEEP; u++) {
+      const int i = (u * 256 + (int)threadIdx.x) * 4;
+      if (i < d) {
+        const float4_t v = keep[u];
+        const float4_t g = *reinterpret_cast<const float4_t *>(gamma + i);
+        half4_t o;
+#pragma unroll
+        for (int e = 0; e < 4; e++) o[e] = (_Float16)(v[e] * inv * g[e]);
+        *reinterpret_cast<half4_t *>(out + (size_t)b * d + i) = o;
+      }
+    }
+    return;
+  }
   for (int i = threadIdx.x * 4; i < d; i += blockDim.x * 4) {
     float4_t v = *reinterpret_cast<const float4_t *>(row + i);
     float4_t g = *reinterpret_cast<const float4_t *>(gamma + i);
@@ -303,6 +336,36 @@ __global__ void __launch_bounds__(128) attn_combine_kernel(const float *__restri
   const int n_ctx = *pos_ptr + 1;
   const int chunks = (n_ctx + ATT_CHUNK - 1) / ATT_CHUNK;
   const float *src = part + (((size_t)b * hq + head) * max_chunks) * (HD + 2);
+  constexpr int FAST = 32;  // contexts up to 32 chunks: every load of the kernel is requested at once
+  if (chunks <= FAST) {
+    float po[FAST];
+#pragma unroll
+    for (int ch = 0; ch < FAST; ch++) po[ch] = src[(size_t)(ch < chunks ? ch : chunks - 1) * (HD + 2) + 2 + tid];
+    float pm = -INFINITY, pl = 0.0f;
+    if (tid < chunks) {
+      pm = src[(size_t)tid * (HD + 2)];
+      pl = src[(size_t)tid * (HD + 2) + 1];
+    }
+    float mx = pm;
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    if ((tid & 63) == 0) red_m[tid >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(red_m[0], red_m[1]);
+    const float f = (pm == -INFINITY) ? 0.0f : __expf(pm - mx);
+    if (tid < chunks) wgt[tid] = f;
+    float l = pl * f;
+    for (int off = 32; off > 0; off >>= 1) l += __shfl_xor(l, off, 64);
+    if ((tid & 63) == 0) red_l[tid >> 6] = l;
+    __syncthreads();
+    l = red_l[0] + red_l[1];
+    float o = 0.0f;
+#pragma unroll
+    for (int ch = 0; ch < FAST; ch++)
+      if (ch < chunks) o += po[ch] * wgt[ch];
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    out[((size_t)b * hq + head) * HD + tid] = (_Float16)(o * inv);
+    return;
+  }
   // maximum over all chunks
   float mx = -INFINITY;
   for (int ch = tid; ch < chunks; ch += 128) mx = fmaxf(mx, src[(size_t)ch * (HD + 2)]);

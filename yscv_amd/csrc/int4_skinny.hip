@@ -664,18 +664,19 @@ __global__ void int4_skinny_finalize_kernel(const float *__restrict__ partial, i
   }
   for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total;
        idx += (size_t)gridDim.x * blockDim.x) {
-    // issue the loads of this element together (one memory round trip), then add in slice order
+    // issue the loads of this element together (one memory round trip), the residual it is added to included, then
+    // add in slice order
     float p[8];
 #pragma unroll
     for (int s = 0; s < 8; s++) p[s] = s < ksg ? partial[(size_t)s * total + idx] : 0.0f;
+    const float before = epi == EPI_ADD_F32 ? reinterpret_cast<const float *>(y)[idx] : 0.0f;
     float v = 0.0f;
 #pragma unroll
     for (int s = 0; s < 8; s++) v += p[s];
     for (int s = 8; s < ksg; s++) v += partial[(size_t)s * total + idx];
     if (row_scale) v *= row_scale[idx / n];
     if (epi == EPI_ADD_F32) {
-      float *dst = reinterpret_cast<float *>(y) + idx;
-      *dst = *dst + v;
+      reinterpret_cast<float *>(y)[idx] = before + v;
     } else {
       store_out(y, idx, v, y_dtype);
     }
@@ -750,6 +751,15 @@ static int32_t launch_one(const SkinnyArgs &a, const SkinnyPlan &plan, hipStream
     return launch_p<SPLIT, NI, GM, SF16, HAS_ZP, 2>(a, plan, s);
   } else {
     constexpr int P = SPLIT == 2 ? 1 : (SF16 && !HAS_ZP ? 4 : 3);
+    if constexpr (P == 4) {
+      // A workgroup with one or two blocks (the short projections of a decode step) gets a ring of that depth: the
+      // requests past the last block that keep a deeper ring's load count fixed are real instructions, each holds the
+      // CU's memory pipeline for sixteen cycles whatever it asks for, and with one block three quarters of the ring
+      // fill would be such fillers (2 of the 8 us of an output projection at m = 16).
+      const int blocks_per_wg = (a.nt + plan.grid_x - 1) / plan.grid_x;
+      if (blocks_per_wg == 1) return launch_p<SPLIT, NI, GM, SF16, HAS_ZP, 1>(a, plan, s);
+      if (blocks_per_wg == 2) return launch_p<SPLIT, NI, GM, SF16, HAS_ZP, 2>(a, plan, s);
+    }
     return launch_p<SPLIT, NI, GM, SF16, HAS_ZP, P>(a, plan, s);
   }
 }
