@@ -33,7 +33,7 @@ MFMA_I8_PEAK = 5000.0       # TOP/s dense
 # plain 256 MiB copy gives for FETCH_SIZE on this GPU, + write 38 KiB x 1.0): profiles/int4_skinny_decode7b_graph_path.md
 SKINNY_TRAFFIC_BYTES = 31_385_000
 # HBM bytes per decode step of the single-launch kernel from the same kind of counter runs (None until measured)
-PERSIST_TRAFFIC_BYTES_PER_STEP = 4_427_000_000  # fetch 4.336 GB (x2.0 scale) + write 0.090 GB: profiles/decode_persistent_7b.md
+PERSIST_TRAFFIC_BYTES_PER_STEP = 4_429_000_000  # fetch 4.337 GB (x2.0 scale) + write 0.092 GB: profiles/decode_persistent_7b.md
 
 CFG7B = dict(n_layers=32, d_model=4096, n_heads=32, n_kv_heads=8, head_dim=128, d_ff=14336, vocab=32000,
              group_size=32, max_batch=16, max_ctx=2048 + 512, max_steps=1024, rope_theta=10000.0, rms_eps=1e-5)
