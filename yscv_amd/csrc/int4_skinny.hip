@@ -751,7 +751,7 @@ static int32_t launch_one(const SkinnyArgs &a, const SkinnyPlan &plan, hipStream
     return launch_p<SPLIT, NI, GM, SF16, HAS_ZP, 2>(a, plan, s);
   } else {
     constexpr int P = SPLIT == 2 ? 1 : (SF16 && !HAS_ZP ? 4 : 3);
-    if constexpr (P == 4) {
+    if constexpr (SPLIT == 1) {
       // A workgroup with one or two blocks (the short projections of a decode step) gets a ring of that depth: the
       // requests past the last block that keep a deeper ring's load count fixed are real instructions, each holds the
       // CU's memory pipeline for sixteen cycles whatever it asks for, and with one block three quarters of the ring
