@@ -494,9 +494,11 @@ int32_t yscv_hip_decoder_reset(yscv_hip_decoder *d, int32_t batch, int32_t start
 /* Run n_steps decode steps (asynchronously on `stream`).  use_graph = 0 launches the kernels of a step one
  * by one, 1 replays one captured HIP graph per step, 2 runs all n_steps in ONE cooperative launch of the
  * persistent decode kernel (batch 1 only; YSCV_HIP_ERR_UNSUPPORTED with the reason in the error text when
- * the model shape or the device cannot run it).  All three produce the same tokens.  Fails if the KV cache
+ * the model shape or the device cannot run it), YSCV_HIP_DECODE_AUTO picks 2 where it applies (batch 1, fp16
+ * cache, supported shape) and 1 otherwise.  All produce the same tokens.  Fails if the KV cache
  * or the token history would overflow (KvCache::append returns an error in the same situation,
  * kv_cache.rs:160-185). */
+#define YSCV_HIP_DECODE_AUTO 3
 int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_graph, void *stream);
 /* Measurement aid: enqueue only the int4 projections of n_steps decode steps (same weights, same
  * order, same buffers as a real step, no attention / norm / sampling), so that the projections'

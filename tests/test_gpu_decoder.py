@@ -293,13 +293,13 @@ def test_generate_matches_device_greedy_and_stops_at_eos():
     got = dec.generate(prompt, max_tokens=12, top_k=1, top_p=1.0)
     # the same through the device-side greedy loop: feed the prompt, then let the decoder run on its own picks
     dec.reset(np.array([prompt[0]], np.int32), 0)
-    dec.run(1, use_graph=False)
+    dec.run(1, auto=True)  # the path generate() takes: the fastest one the decoder has
     for p, t in enumerate(prompt[1:], start=1):
         dec.reset(np.array([t], np.int32), p)
-        dec.run(1, use_graph=False)
+        dec.run(1, auto=True)
     first = int(dec.tokens(0, 1)[0, 0])
     dec.reset(np.array([first], np.int32), len(prompt))
-    dec.run(11, use_graph=False)
+    dec.run(11, auto=True)
     want = [first] + dec.tokens(0, 11)[:, 0].tolist()
     assert got.tolist() == want
     # EOS: the third generated token as EOS stops after two

@@ -780,6 +780,8 @@ int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_g
                d->cfg.max_ctx);
   YSCV_REQUIRE(step + n_steps <= d->cfg.max_steps, "token history overflow: %d + %d > max_steps %d", step, n_steps,
                d->cfg.max_steps);
+  if (use_graph == YSCV_HIP_DECODE_AUTO)  // the fastest path this decoder has for its batch
+    use_graph = (d->batch == 1 && d->persist_ok && d->kv_dtype == YSCV_HIP_KV_F16) ? 2 : 1;
   if (use_graph == 2) {
     if (d->kv_dtype != YSCV_HIP_KV_F16)
       return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the single-launch decode path reads an fp16 KV cache only");

@@ -111,7 +111,7 @@ int32_t yscv_hip_decoder_generate(yscv_hip_decoder *d, const uint32_t *input_ids
     YSCV_REQUIRE(input_ids[p] < vocab, "prompt token %u outside the vocabulary (%zu)", input_ids[p], vocab);
     const int32_t tok = (int32_t)input_ids[p];
     YSCV_TRY(yscv_hip_decoder_reset(d, 1, (int32_t)p, &tok));
-    YSCV_TRY(yscv_hip_decoder_run(d, 1, 0, nullptr));
+    YSCV_TRY(yscv_hip_decoder_run(d, 1, YSCV_HIP_DECODE_AUTO, nullptr));
   }
   for (size_t g = 0; g < cfg->max_tokens; g++) {
     YSCV_TRY(yscv_hip_decoder_read_logits(d, logits.data()));
@@ -135,7 +135,7 @@ int32_t yscv_hip_decoder_generate(yscv_hip_decoder *d, const uint32_t *input_ids
     if (g + 1 == cfg->max_tokens) break;
     const int32_t tok = (int32_t)next;
     YSCV_TRY(yscv_hip_decoder_reset(d, 1, (int32_t)(tokens.size() - 1), &tok));
-    YSCV_TRY(yscv_hip_decoder_run(d, 1, 0, nullptr));
+    YSCV_TRY(yscv_hip_decoder_run(d, 1, YSCV_HIP_DECODE_AUTO, nullptr));
   }
   return YSCV_HIP_OK;
 }

@@ -69,10 +69,11 @@ class Decoder:
         self.batch = t.size
         lib().decoder_reset(self._h, int(t.size), int(start_pos), _p(t))
 
-    def run(self, n_steps, use_graph=True, stream=None, persistent=False):
+    def run(self, n_steps, use_graph=True, stream=None, persistent=False, auto=False):
         """use_graph: replay one captured HIP graph per step; persistent: run all steps inside one
-        cooperative launch (batch 1, shapes the single-launch kernel supports)."""
-        mode = 2 if persistent else int(bool(use_graph))
+        cooperative launch (batch 1, shapes the single-launch kernel supports); auto: the fastest of the two
+        that applies (YSCV_HIP_DECODE_AUTO, what generate() uses)."""
+        mode = 3 if auto else (2 if persistent else int(bool(use_graph)))
         lib().decoder_run(self._h, int(n_steps), mode, C.c_void_p(stream) if stream else None)
 
     def run_projections(self, n_steps, stream=None):
