@@ -91,12 +91,16 @@ def kv_i8_roundtrip(rows):
 
 
 class RefDecoder:
-    def __init__(self, cfg: dict, linears: dict, norms: dict, emb16, kv_i8: bool = False):
+    def __init__(self, cfg: dict, linears: dict, norms: dict, emb16, kv_i8: bool = False, round_f16: bool = True):
         """linears[(layer, kind)] = (packed, scales16) with kind in q k v o gate up down, and
         linears[('lm_head',)]; norms[(layer, 'attn'|'ffn')], norms[('final',)] f32 gamma.
         kv_i8: the cache stores per-row int8 (KvDtype::I8); the rotated key of a new token is then quantised from its f32
-        value, not from an fp16 rounding of it."""
+        value, not from an fp16 rounding of it.
+        round_f16=False drops every fp16 rounding of an activation: f32 from the embedding row to the logits, which
+        is what the reference's CPU path computes (its activations are f32 tensors); the default rounds where the
+        GPU decoder's multi-launch path without folded norms stores fp16."""
         self.c = cfg
+        self._r = f16 if round_f16 else (lambda x: np.asarray(x, np.float32))
         self.kv_i8 = kv_i8
         g = cfg["group_size"]
         D, hd = cfg["d_model"], cfg["head_dim"]
@@ -122,11 +126,11 @@ class RefDecoder:
             self.kc[layer][b], self.vc[layer][b] = kb, vb
 
     def _rmsnorm(self, h, gamma):
-        return f16(rmsnorm(h, gamma, self.c["rms_eps"]))
+        return self._r(rmsnorm(h, gamma, self.c["rms_eps"]))
 
     def _rope(self, x, pos):
         """x: [heads][d]."""
-        return f16(rope(x, pos, self.c["rope_theta"]))
+        return self._r(rope(x, pos, self.c["rope_theta"]))
 
     def step(self, tokens, pos):
         """tokens: int [batch]; pos: position the new token is written at.  Returns logits f32 [batch][vocab].
@@ -139,9 +143,9 @@ class RefDecoder:
         h = self.emb[np.asarray(tokens)].astype(np.float32)
         for l in range(c["n_layers"]):
             xn = self._rmsnorm(h, self.norms[(l, "attn")])
-            q = f16(xn @ self.w[(l, "q")].T).reshape(B, nh, hd)
-            k = f16(xn @ self.w[(l, "k")].T).reshape(B, nkv, hd)
-            v = f16(xn @ self.w[(l, "v")].T).reshape(B, nkv, hd)
+            q = self._r(xn @ self.w[(l, "q")].T).reshape(B, nh, hd)
+            k = self._r(xn @ self.w[(l, "k")].T).reshape(B, nkv, hd)
+            v = self._r(xn @ self.w[(l, "v")].T).reshape(B, nkv, hd)
             ao = np.zeros((B, nh, hd), np.float32)
             qkv = np.zeros((B, (nh + 2 * nkv) * hd), np.float32)
             for b in range(B):
@@ -154,12 +158,12 @@ class RefDecoder:
                 self.kc[l][b] = np.concatenate([self.kc[l][b][:pos], k_row[None]], 0)
                 self.vc[l][b] = np.concatenate([self.vc[l][b][:pos], v_row[None]], 0)
                 ao[b] = gqa_attend(qr, self.kc[l][b], self.vc[l][b], groups)
-            ao = f16(ao.reshape(B, nh * hd))
+            ao = self._r(ao.reshape(B, nh * hd))
             h = h + ao @ self.w[(l, "o")].T
             xn = self._rmsnorm(h, self.norms[(l, "ffn")])
             gt = xn @ self.w[(l, "gate")].T
             up = xn @ self.w[(l, "up")].T
-            act = f16(swiglu(gt, up))
+            act = self._r(swiglu(gt, up))
             h = h + act @ self.w[(l, "down")].T
         xn = self._rmsnorm(h, self.norms[("final",)])
         self.trace = {"qkv": qkv, "attn_out": ao, "ffn": act, "residual": h.astype(np.float32), "normed": xn}

@@ -7,8 +7,15 @@ SwiGLU 14336, vocab 32000, int4 group 32 with fp16 scales, fp16 KV cache at cont
   125-block LM head per workgroup are all exercised against an independent result.
 * All 32 layers: the single-launch kernel against the multi-kernel path (tokens and logits), step by step and as one
   launch, and row 0 of a batch-16 step against the batch-1 step.
-Tolerances: the activations between stages are fp16 on the GPU and in the checker (same rounding points), the
-projections sum in another order than numpy: 1e-2 of max|logit| is the float bar of the int4 path.
+Tolerances: the logits are held to 1e-2 of max|logit| (the float bar of the int4 path) against TWO results of the
+checker: f32 from the embedding row to the logits, which is what the reference's CPU path computes, and the same with
+every activation rounded to fp16 where the GPU's multi-launch path stores fp16.  The GPU paths round at slightly
+different points (the single-launch kernel and the folded norms keep some values in f32 longer, or round before the
+norm's row factor is applied instead of after), so they sit as far from the f32 result as the rounded checker does
+(1e-3 .. 4e-3 here), not closer to one than to the other.  With the int8 cache a key or value whose scaled magnitude
+lies next to a rounding boundary takes the neighbouring int8 code as soon as its input differs in the last fp16 bit,
+a step of 1/127 of the row's maximum: there the rounded checker itself is up to 1.6e-2 from the f32 one, and the bar
+for the logits is 3e-2 (every stage-level check keeps its own, tighter bound).
 
 Weights of the two-layer model are uniform over the nibbles 1..15, i.e. symmetric about the zero point 8.  Uniform
 0..15 (what the benchmark's random init draws) has mean -0.5 after the zero point: with positive RMSNorm gains every
@@ -59,12 +66,14 @@ def _build_two_layers():
     dec.set_embedding(emb)
     dec.finalize()
     ref = RefDecoder(cfg, linears, norms, emb)
+    ref.f32 = RefDecoder(cfg, linears, norms, emb, round_f16=False)
     B = cfg["max_batch"]
     for l in range(cfg["n_layers"]):
         k = rng.standard_normal((B, PREFILL, cfg["n_kv_heads"], hd), dtype=np.float32).astype(np.float16)
         v = rng.standard_normal((B, PREFILL, cfg["n_kv_heads"], hd), dtype=np.float32).astype(np.float16)
         dec.set_kv(l, k, v)
         ref.set_kv(l, k.astype(np.float32), v.astype(np.float32))
+        ref.f32.set_kv(l, k.astype(np.float32), v.astype(np.float32))
     return cfg, dec, ref, linears
 
 
@@ -78,14 +87,18 @@ def two_layers():
     dec.close()
 
 
-def _check_rows(got_logits, got_tok, exp_logits, what):
+def _check_rows(got_logits, got_tok, exp_logits, exp_f32, what, tol=1e-2):
+    """Logits against the rounded and the f32 result of the checker; returns the worst row of each."""
     from oracle.decoder_ref import greedy_pick
 
+    worst = [0.0, 0.0]
     for b in range(exp_logits.shape[0]):
-        err = np.abs(got_logits[b] - exp_logits[b]).max() / np.abs(exp_logits[b]).max()
-        assert err < 1e-2, (what, b, err)
+        for i, exp in enumerate((exp_logits, exp_f32)):
+            err = np.abs(got_logits[b] - exp[b]).max() / np.abs(exp[b]).max()
+            assert err < tol, (what, "rounded" if i == 0 else "f32", b, err)
+            worst[i] = max(worst[i], float(err))
         assert got_tok[b] == greedy_pick(got_logits[b]), (what, b)  # the exact rule, on the GPU's own logits
-    return max(np.abs(got_logits[b] - exp_logits[b]).max() / np.abs(exp_logits[b]).max() for b in range(exp_logits.shape[0]))
+    return worst
 
 
 def test_single_launch_batch1_at_7b_widths_matches_numpy(two_layers):
@@ -97,9 +110,9 @@ def test_single_launch_batch1_at_7b_widths_matches_numpy(two_layers):
     for step in range(3):
         dec.run(1, persistent=True)
         got_logits, got_tok = dec.logits(), dec.tokens(step, 1)[0]
-        exp = ref.step(cur, PREFILL + step)
-        worst = _check_rows(got_logits, got_tok, exp, f"persistent step {step}")
-        print(f"[7b widths, single launch] step {step}: rel err {worst:.2e}", flush=True)
+        exp, exp32 = ref.step(cur, PREFILL + step), ref.f32.step(cur, PREFILL + step)
+        worst = _check_rows(got_logits, got_tok, exp, exp32, f"persistent step {step}")
+        print(f"[7b widths, single launch] step {step}: rel err {worst[0]:.2e} (f32 checker {worst[1]:.2e})", flush=True)
         seen.append(int(got_tok[0]))
         cur = got_tok.copy()
     last = dec.logits().copy()
@@ -168,10 +181,10 @@ def test_multi_kernel_batch16_at_7b_widths_matches_numpy(two_layers, oracle):
     for step in range(2):
         dec.run(1, use_graph=True)
         got_logits, got_tok = dec.logits(), dec.tokens(step, 1)[0]
-        exp = ref.step(cur, PREFILL + step)
-        worst = _check_rows(got_logits, got_tok, exp, f"batch 16 step {step}")
+        exp, exp32 = ref.step(cur, PREFILL + step), ref.f32.step(cur, PREFILL + step)
+        worst = _check_rows(got_logits, got_tok, exp, exp32, f"batch 16 step {step}")
         att, lm = _stage_checks(oracle, cfg, dec, ref, linears, PREFILL + step, B)
-        print(f"[7b widths, batch 16] step {step}: worst row rel err {worst:.2e}; stage level: attention {att:.1e}, "
+        print(f"[7b widths, batch 16] step {step}: worst row rel err {worst[0]:.2e} (f32 checker {worst[1]:.2e}); stage level: attention {att:.1e}, "
               f"lm_head {lm:.1e}", flush=True)
         cur = got_tok.copy()
     # eager launches give the same stream as the graph replays
@@ -205,6 +218,7 @@ def test_multi_kernel_int8_cache_at_7b_widths_matches_numpy(two_layers):
     dec.set_embedding(emb16)
     dec.finalize()
     ref = RefDecoder(cfg, linears, ref16.norms, emb16, kv_i8=True)
+    ref32 = RefDecoder(cfg, linears, ref16.norms, emb16, kv_i8=True, round_f16=False)
     rng = np.random.default_rng(7100)
     B = cfg["max_batch"]
     for l in range(cfg["n_layers"]):
@@ -212,15 +226,16 @@ def test_multi_kernel_int8_cache_at_7b_widths_matches_numpy(two_layers):
         v = rng.standard_normal((B, PREFILL, cfg["n_kv_heads"], hd), dtype=np.float32).astype(np.float16)
         dec.set_kv(l, k, v)
         ref.set_kv(l, k.astype(np.float32), v.astype(np.float32))
+        ref32.set_kv(l, k.astype(np.float32), v.astype(np.float32))
     tokens = np.array([11, 2222, 13333, 31999], np.int32)
     dec.reset(tokens, PREFILL)
     cur = tokens.copy()
     for step in range(3):
         dec.run(1, use_graph=True)
         got_logits, got_tok = dec.logits(), dec.tokens(step, 1)[0]
-        exp = ref.step(cur, PREFILL + step)
-        worst = _check_rows(got_logits, got_tok, exp, f"int8 cache step {step}")
-        print(f"[7b widths, int8 cache] step {step}: worst row rel err {worst:.2e}", flush=True)
+        exp, exp32 = ref.step(cur, PREFILL + step), ref32.step(cur, PREFILL + step)
+        worst = _check_rows(got_logits, got_tok, exp, exp32, f"int8 cache step {step}", tol=3e-2)
+        print(f"[7b widths, int8 cache] step {step}: worst row rel err {worst[0]:.2e} (f32 checker {worst[1]:.2e})", flush=True)
         cur = got_tok.copy()
     dec.close()
 

@@ -261,15 +261,20 @@ def test_ref_decoder_steps_match_float64_transcription():
     cfg = dict(CFG)
     lin, norms, emb, shapes = _tiny_model(rng, cfg)
     ref = R.RefDecoder(cfg, lin, norms, emb)
+    ref32 = R.RefDecoder(cfg, lin, norms, emb, round_f16=False)
     kc = [[] for _ in range(cfg["n_layers"])]
     vc = [[] for _ in range(cfg["n_layers"])]
     tok = 3
     for pos in range(3):
         got = ref.step(np.array([tok, tok]), pos)
+        got32 = ref32.step(np.array([tok, tok]), pos)
         want = _step_f64(cfg, lin, norms, emb, shapes, kc, vc, tok, pos)
-        # fp16 roundings of the checker's activations are the only difference: ~1e-3 relative
+        # fp16 roundings of the checker's activations are the only difference: ~1e-3 relative; without them
+        # (round_f16=False) what is left is f32 against float64 arithmetic
         scale = np.abs(want).max()
         assert np.abs(got[0] - want).max() / scale < 5e-3, pos
+        assert np.abs(got32[0] - want).max() / scale < 2e-5, pos
+        assert not np.array_equal(got[0], got32[0])
         np.testing.assert_array_equal(got[0], got[1])  # batch rows are independent
         tok = R.greedy_pick(got[0])
 

@@ -145,6 +145,7 @@ _SIGNATURES = {
     "yscv_hip_decoder_read_activation": [_vp, _i32, _vp, _sz],
     "yscv_hip_decoder_debug_set_tag_epoch": [_vp, C.c_uint32],
     "yscv_hip_decoder_debug_set_fused_attention": [_vp, C.c_int32],
+    "yscv_hip_decoder_debug_set_folded_norm": [_vp, C.c_int32],
     "yscv_hip_decoder_weight_bytes": [_vp, C.POINTER(_sz)],
     "yscv_hip_decoder_vocab": [_vp, C.POINTER(_sz)],
     "yscv_hip_sample_token": [_vp, _sz, _sz, _f32, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32)],

@@ -139,7 +139,8 @@ int32_t int4_workspace_bytes(const yscv_hip_int4_weight *w, size_t m, int x_dtyp
 // `ws` may be null: scratch then comes from the stream-ordered allocator, so concurrent callers
 // on different streams never share it.
 int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, void *y, int y_dtype, size_t m,
-                    int force /*0 auto, 1 skinny, 2 gemm*/, int epi, void *ws, size_t ws_bytes, hipStream_t s) {
+                    int force /*0 auto, 1 skinny, 2 gemm*/, int epi, void *ws, size_t ws_bytes, hipStream_t s,
+                    const NormFold *nf) {
   const Context *ctx = nullptr;
   YSCV_TRY(ensure_context(&ctx));
   YSCV_REQUIRE(w != nullptr, "null int4 weight handle");
@@ -147,6 +148,8 @@ int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, v
   YSCV_REQUIRE(valid_act_dtype(x_dtype) && valid_act_dtype(y_dtype), "unknown dtype code");
   if (m == 0) return YSCV_HIP_OK;
   if (force == 1 && m > 16) return set_error(YSCV_HIP_ERR_INVALID_ARG, "gemv entry point handles m <= 16, got %zu", m);
+  if (nf && (!w->tiled || m > 16 || x_dtype != YSCV_HIP_F16))
+    return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the folded norm exists for the skinny kernel on fp16 activations only");
   if (!w->tiled) {
     if (epi != EPI_STORE) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "fused epilogues need the tiled layout");
     note_int4_fallback();
@@ -205,7 +208,7 @@ int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, v
     st = launch_x_prep(x, x_dtype, m, w->k, L.k_pad, run_split, const_cast<_Float16 *>(xh), xl, row_scale, s);
   if (st == YSCV_HIP_OK) {
     if (L.skinny)
-      st = launch_int4_skinny(w, L.plan, xh, xl, xraw, row_scale, L.k_pad, L.split, y, y_dtype, m, partial, epi, s);
+      st = launch_int4_skinny(w, L.plan, xh, xl, xraw, row_scale, L.k_pad, L.split, y, y_dtype, m, partial, epi, s, nf);
     else
       st = launch_int4_gemm(w, xh, xl, row_scale, L.k_pad, run_split, y, y_dtype, m, s);
   }

@@ -149,50 +149,6 @@ __device__ __forceinline__ int xidx(int i, int ks, int frags) {
   const int r = k2 >> 5, c = (k2 >> 3) & 3, q = (k2 & 7) >> 1;
   return ((v * frags + f) << 8) + ((q >> 1) << 7) + 2 * (16 * c + r) + (q & 1);
 }
-// Cross-lane moves without LDS: __shfl_* compiles to ds_bpermute_b32, about a hundred cycles each when one depends
-// on the other, and a layer has some ninety of them on its critical path.  Within a row of 16 lanes DPP does the
-// same in one vector instruction; v_permlane16_swap / v_permlane32_swap exchange rows and halves of the wave.
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
-}
-constexpr int DPP_XOR1 = 0xB1, DPP_XOR2 = 0x4E;         // quad_perm [1,0,3,2], [2,3,0,1]
-constexpr int DPP_NEXT1 = 0xF5, DPP_NEXT2 = 0xEE;       // quad_perm [1,1,3,3], [2,3,2,3]: lane + 1 / lane + 2 inside a quad
-constexpr int DPP_ROR4 = 0x124, DPP_ROR8 = 0x128;       // row_ror:4, row_ror:8 (= lane ^ 8 inside a row)
-constexpr int DPP_HALF_MIRROR = 0x141;                  // lane -> 7 - lane inside each group of 8
-typedef uint32_t swap_pair_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ void xor16_pair(float v, float &x, float &y) {  // {x, y} = {v[lane & ~16], v[lane | 16]}
-  const swap_pair_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  x = __uint_as_float(r[0]);
-  y = __uint_as_float(r[1]);
-}
-__device__ __forceinline__ void xor32_pair(float v, float &x, float &y) {  // {x, y} = {v[lane & ~32], v[lane | 32]}
-  const swap_pair_t r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  x = __uint_as_float(r[0]);
-  y = __uint_as_float(r[1]);
-}
-__device__ __forceinline__ float sum_xor16_xor32(float v) {  // v + v[lane ^ 16], then the same over lane ^ 32
-  float x, y;
-  xor16_pair(v, x, y);
-  v = x + y;
-  xor32_pair(v, x, y);
-  return x + y;
-}
-__device__ __forceinline__ float row_sum16(float v) {  // sum over the 16 lanes of a row, in every lane
-  v += dpp_move<DPP_XOR1>(v);
-  v += dpp_move<DPP_XOR2>(v);
-  v += dpp_move<DPP_ROR4>(v);
-  v += dpp_move<DPP_ROR8>(v);
-  return v;
-}
-__device__ __forceinline__ float row_max16(float v) {
-  v = fmaxf(v, dpp_move<DPP_XOR1>(v));
-  v = fmaxf(v, dpp_move<DPP_XOR2>(v));
-  v = fmaxf(v, dpp_move<DPP_HALF_MIRROR>(v));
-  v = fmaxf(v, dpp_move<DPP_ROR8>(v));
-  return v;
-}
-__device__ __forceinline__ float wave_sum(float v) { return sum_xor16_xor32(row_sum16(v)); }
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + __expf(-g)); }
 // order of the greedy pick: higher value wins, equal (or unordered) values -> larger index
 __device__ __forceinline__ bool better(float va, int ia, float vb, int ib) {

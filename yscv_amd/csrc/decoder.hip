@@ -4,6 +4,7 @@
 // One decode step is a fixed sequence of kernel launches that reads the position from device
 // memory, so the step is captured once into a HIP graph and replayed for every token.
 #include <algorithm>
+#include <cmath>
 #include <vector>
 
 #include "decoder.hpp"
@@ -112,6 +113,14 @@ struct yscv_hip_decoder {
   _Float16 *xn = nullptr, *qkv = nullptr, *ao = nullptr, *act = nullptr;
   _Float16 *qrot = nullptr;       // rotated query heads of the last fused attention launch (diagnostics)
   bool fused_attn = true;         // fp16 cache: rope + append inside the attention kernel
+  // RMSNorm folded into the projections around it (NormFold, kernels.hpp): two buffers of partial sums of squares,
+  // written and read in turn, each with the power of two per row that xn's rows were multiplied by
+  bool fold_norm = false;         // decided in finish_setup from the shapes
+  bool fold_norm_wanted = true;   // test aid: yscv_hip_decoder_debug_set_folded_norm
+  float *ss[2] = {nullptr, nullptr};
+  float *pre[2] = {nullptr, nullptr};
+  int ss_stride = 0;
+  int last_ss = 0, last_ss_count = 0;  // what the final norm's consumer read in the last enqueued step
   void *ws = nullptr;
   size_t ws_bytes = 0;
   int32_t *tokens = nullptr, *history = nullptr, *pos = nullptr, *step = nullptr;
@@ -172,6 +181,10 @@ static void decoder_free(yscv_hip_decoder *d) {
   (void)hipFree(d->logits);
   (void)hipFree(d->attn_part);
   (void)hipFree(d->qrot);
+  (void)hipFree(d->ss[0]);
+  (void)hipFree(d->ss[1]);
+  (void)hipFree(d->pre[0]);
+  (void)hipFree(d->pre[1]);
   (void)hipFree(d->xn);
   (void)hipFree(d->qkv);
   (void)hipFree(d->ao);
@@ -347,6 +360,14 @@ static int32_t alloc_runtime(yscv_hip_decoder *d) {
   DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->attn_part), B * c.n_heads * chunks * (c.head_dim + 2) * 4));
   DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->qrot), B * (size_t)c.n_heads * c.head_dim * 2));
   DEC_HIP(hipMemset(d->qrot, 0, B * (size_t)c.n_heads * c.head_dim * 2));
+  d->ss_stride = c.d_model / 16;
+  for (int i = 0; i < 2; i++) {
+    DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->ss[i]), B * (size_t)d->ss_stride * 4));
+    DEC_HIP(hipMemset(d->ss[i], 0, B * (size_t)d->ss_stride * 4));
+    const std::vector<float> ones(B, 1.0f);
+    DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->pre[i]), B * 4));
+    DEC_HIP(hipMemcpy(d->pre[i], ones.data(), B * 4, hipMemcpyHostToDevice));
+  }
   DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->tokens), B * 4));
   DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->history), B * (size_t)c.max_steps * 4));
   DEC_HIP(hipMalloc(reinterpret_cast<void **>(&d->pos), 4));
@@ -393,6 +414,25 @@ static int32_t finish_setup(yscv_hip_decoder *d) {
     }
     DEC_HIP(hipMemcpy(d->p_gammas + 2 * d->layers.size() * D, d->final_norm, D * 4, hipMemcpyDeviceToDevice));
   }
+  // the norms fold into the projections when the second pass of a K-split update can take whole 256-column pieces
+  // and the projections that consume a norm are not K-split themselves
+  {
+    const Context *ctx = nullptr;
+    YSCV_TRY(ensure_context(&ctx));
+    // (a consuming projection adds up at most 256 partial sums per row, four rows per wave of 512 k)
+    bool ok = d->cfg.d_model % 256 == 0 && d->cfg.d_model <= 4096 && d->fold_norm_wanted &&
+              d->cfg.max_batch <= 4 * ((d->cfg.d_model + 511) / 512);
+    for (auto &L : d->layers)
+      for (auto *w : {L.wqkv, L.wgu}) ok = ok && w->tiled && plan_int4_skinny(w, d->cfg.max_batch, 1, ctx->num_cus).ksg == 1;
+    ok = ok && d->lm_head->tiled && plan_int4_skinny(d->lm_head, d->cfg.max_batch, 1, ctx->num_cus).ksg == 1;
+    for (auto &L : d->layers) ok = ok && L.wo->tiled && L.wdown->tiled;
+    // every projection takes its fp16 activations as they are (no padded copy with a row scale of its own)
+    auto direct = [](const yscv_hip_int4_weight *w) { return w->ktp * 128 == w->k; };
+    for (auto &L : d->layers)
+      for (auto *w : {L.wqkv, L.wo, L.wgu, L.wdown}) ok = ok && direct(w);
+    ok = ok && direct(d->lm_head);
+    d->fold_norm = ok;
+  }
   d->finalized = true;
   return YSCV_HIP_OK;
 }
@@ -401,10 +441,45 @@ static int32_t finish_setup(yscv_hip_decoder *d) {
 static int32_t enqueue_step(yscv_hip_decoder *d, int batch, hipStream_t s) {
   const auto &c = d->cfg;
   const int D = c.d_model;
-  YSCV_TRY(launch_embed(d->tokens, d->emb, batch, D, c.vocab, d->h, s));
-  for (auto &L : d->layers) {
-    YSCV_TRY(launch_rmsnorm(d->h, L.attn_norm, batch, D, c.rms_eps, d->xn, s));
-    YSCV_TRY(int4_run_ws(L.wqkv, d->xn, YSCV_HIP_F16, d->qkv, YSCV_HIP_F16, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s));
+  const bool fold = d->fold_norm;
+  // folded norms: `cur` is the buffer of partial sums the next consumer reads, `cnt` how many partials a row has there
+  int cur = 0, cnt = 0;
+  // `feeds_update`: a residual update follows this norm's projection and takes its row scales from it
+  auto consumer = [&](NormFold &nf, bool feeds_update) {
+    nf.ss_in = d->ss[cur];
+    nf.pre_in = d->pre[cur];
+    nf.pre_next = feeds_update ? d->pre[cur ^ 1] : nullptr;
+    nf.ss_in_count = cnt;
+    nf.ss_in_stride = d->ss_stride;
+    nf.inv_d = 1.0f / (float)D;
+    nf.eps = c.rms_eps;
+  };
+  auto producer = [&](NormFold &nf, const float *gamma, int *count_out) {
+    nf.gamma_next = gamma;
+    nf.pre = d->pre[cur ^ 1];
+    nf.xg = d->xn;
+    nf.ss_out = d->ss[cur ^ 1];
+    nf.ss_out_stride = d->ss_stride;
+    nf.ss_out_count = count_out;
+  };
+  if (fold) {
+    YSCV_TRY(launch_embed_norm(d->tokens, d->emb, batch, D, c.vocab, c.rms_eps, d->h, d->layers[0].attn_norm, d->xn, d->ss[0],
+                               d->ss_stride, d->pre[0], s));
+    cur = 0;
+    cnt = 1;
+  } else {
+    YSCV_TRY(launch_embed(d->tokens, d->emb, batch, D, c.vocab, d->h, s));
+  }
+  for (size_t li = 0; li < d->layers.size(); li++) {
+    auto &L = d->layers[li];
+    if (fold) {
+      NormFold nf;
+      consumer(nf, true);
+      YSCV_TRY(int4_run_ws(L.wqkv, d->xn, YSCV_HIP_F16, d->qkv, YSCV_HIP_F16, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s, &nf));
+    } else {
+      YSCV_TRY(launch_rmsnorm(d->h, L.attn_norm, batch, D, c.rms_eps, d->xn, s));
+      YSCV_TRY(int4_run_ws(L.wqkv, d->xn, YSCV_HIP_F16, d->qkv, YSCV_HIP_F16, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s));
+    }
     if (d->kv_dtype == YSCV_HIP_KV_I8) {
       YSCV_TRY(launch_rope_append_i8(d->qkv, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_theta, c.max_ctx,
                                      L.kc8, L.ks, L.vc8, L.vs, s));
@@ -419,13 +494,37 @@ static int32_t enqueue_step(yscv_hip_decoder *d, int batch, hipStream_t s) {
       YSCV_TRY(launch_attention(d->qkv, L.kc, L.vc, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim, c.max_ctx,
                                 d->attn_part, d->ao, s));
     }
-    YSCV_TRY(int4_run_ws(L.wo, d->ao, YSCV_HIP_F16, d->h, YSCV_HIP_F32, batch, 1, EPI_ADD_F32, d->ws, d->ws_bytes, s));
-    YSCV_TRY(launch_rmsnorm(d->h, L.ffn_norm, batch, D, c.rms_eps, d->xn, s));
-    YSCV_TRY(int4_run_ws(L.wgu, d->xn, YSCV_HIP_F16, d->act, YSCV_HIP_F16, batch, 1, EPI_SWIGLU, d->ws, d->ws_bytes, s));
-    YSCV_TRY(int4_run_ws(L.wdown, d->act, YSCV_HIP_F16, d->h, YSCV_HIP_F32, batch, 1, EPI_ADD_F32, d->ws, d->ws_bytes, s));
+    if (fold) {
+      // o: h += W ao, and the ffn norm's inputs; gate/up reads them; down: h += W act, and the next norm's inputs
+      NormFold po, cg, pd;
+      int n_o = 0, n_d = 0;
+      producer(po, L.ffn_norm, &n_o);
+      YSCV_TRY(int4_run_ws(L.wo, d->ao, YSCV_HIP_F16, d->h, YSCV_HIP_F32, batch, 1, EPI_ADD_F32, d->ws, d->ws_bytes, s, &po));
+      cur ^= 1;
+      cnt = n_o;
+      consumer(cg, true);
+      YSCV_TRY(int4_run_ws(L.wgu, d->xn, YSCV_HIP_F16, d->act, YSCV_HIP_F16, batch, 1, EPI_SWIGLU, d->ws, d->ws_bytes, s, &cg));
+      producer(pd, li + 1 < d->layers.size() ? d->layers[li + 1].attn_norm : d->final_norm, &n_d);
+      YSCV_TRY(int4_run_ws(L.wdown, d->act, YSCV_HIP_F16, d->h, YSCV_HIP_F32, batch, 1, EPI_ADD_F32, d->ws, d->ws_bytes, s, &pd));
+      cur ^= 1;
+      cnt = n_d;
+    } else {
+      YSCV_TRY(int4_run_ws(L.wo, d->ao, YSCV_HIP_F16, d->h, YSCV_HIP_F32, batch, 1, EPI_ADD_F32, d->ws, d->ws_bytes, s));
+      YSCV_TRY(launch_rmsnorm(d->h, L.ffn_norm, batch, D, c.rms_eps, d->xn, s));
+      YSCV_TRY(int4_run_ws(L.wgu, d->xn, YSCV_HIP_F16, d->act, YSCV_HIP_F16, batch, 1, EPI_SWIGLU, d->ws, d->ws_bytes, s));
+      YSCV_TRY(int4_run_ws(L.wdown, d->act, YSCV_HIP_F16, d->h, YSCV_HIP_F32, batch, 1, EPI_ADD_F32, d->ws, d->ws_bytes, s));
+    }
   }
-  YSCV_TRY(launch_rmsnorm(d->h, d->final_norm, batch, D, c.rms_eps, d->xn, s));
-  YSCV_TRY(int4_run_ws(d->lm_head, d->xn, YSCV_HIP_F16, d->logits, YSCV_HIP_F32, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s));
+  if (fold) {
+    NormFold nf;
+    consumer(nf, false);
+    d->last_ss = cur;
+    d->last_ss_count = cnt;
+    YSCV_TRY(int4_run_ws(d->lm_head, d->xn, YSCV_HIP_F16, d->logits, YSCV_HIP_F32, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s, &nf));
+  } else {
+    YSCV_TRY(launch_rmsnorm(d->h, d->final_norm, batch, D, c.rms_eps, d->xn, s));
+    YSCV_TRY(int4_run_ws(d->lm_head, d->xn, YSCV_HIP_F16, d->logits, YSCV_HIP_F32, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s));
+  }
   YSCV_TRY(launch_argmax(d->logits, batch, c.vocab, d->tokens, d->history, d->step, c.max_steps, s));
   YSCV_TRY(launch_advance(d->pos, d->step, s));
   return YSCV_HIP_OK;
@@ -838,14 +937,56 @@ int32_t yscv_hip_decoder_run_projections(yscv_hip_decoder *d, int32_t n_steps, v
   YSCV_REQUIRE(d->batch >= 1, "call yscv_hip_decoder_reset first");
   hipStream_t s = as_stream(stream);
   const int batch = d->batch;
+  const auto &c = d->cfg;
   for (int i = 0; i < n_steps; i++) {
-    for (auto &L : d->layers) {
-      YSCV_TRY(int4_run_ws(L.wqkv, d->xn, YSCV_HIP_F16, d->qkv, YSCV_HIP_F16, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s));
-      YSCV_TRY(int4_run_ws(L.wo, d->ao, YSCV_HIP_F16, d->h, YSCV_HIP_F32, batch, 1, EPI_ADD_F32, d->ws, d->ws_bytes, s));
-      YSCV_TRY(int4_run_ws(L.wgu, d->xn, YSCV_HIP_F16, d->act, YSCV_HIP_F16, batch, 1, EPI_SWIGLU, d->ws, d->ws_bytes, s));
-      YSCV_TRY(int4_run_ws(L.wdown, d->act, YSCV_HIP_F16, d->h, YSCV_HIP_F32, batch, 1, EPI_ADD_F32, d->ws, d->ws_bytes, s));
+    // the same calls as in a real step, folded norms included (their partial sums are whatever the buffers hold)
+    int cur = 0, cnt = 1;
+    auto consumer = [&](NormFold &nf, bool feeds_update) {
+      nf.ss_in = d->ss[cur];
+      nf.pre_in = d->pre[cur];
+      nf.pre_next = feeds_update ? d->pre[cur ^ 1] : nullptr;
+      nf.ss_in_count = cnt;
+      nf.ss_in_stride = d->ss_stride;
+      nf.inv_d = 1.0f / (float)c.d_model;
+      nf.eps = c.rms_eps;
+    };
+    auto producer = [&](NormFold &nf, const float *gamma, int *count_out) {
+      nf.gamma_next = gamma;
+      nf.pre = d->pre[cur ^ 1];
+      nf.xg = d->xn;
+      nf.ss_out = d->ss[cur ^ 1];
+      nf.ss_out_stride = d->ss_stride;
+      nf.ss_out_count = count_out;
+    };
+    for (size_t li = 0; li < d->layers.size(); li++) {
+      auto &L = d->layers[li];
+      NormFold cq, po, cg, pd;
+      int n_o = 0, n_d = 0;
+      if (d->fold_norm) consumer(cq, true);
+      YSCV_TRY(int4_run_ws(L.wqkv, d->xn, YSCV_HIP_F16, d->qkv, YSCV_HIP_F16, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s,
+                           d->fold_norm ? &cq : nullptr));
+      if (d->fold_norm) producer(po, L.ffn_norm, &n_o);
+      YSCV_TRY(int4_run_ws(L.wo, d->ao, YSCV_HIP_F16, d->h, YSCV_HIP_F32, batch, 1, EPI_ADD_F32, d->ws, d->ws_bytes, s,
+                           d->fold_norm ? &po : nullptr));
+      if (d->fold_norm) {
+        cur ^= 1;
+        cnt = n_o;
+        consumer(cg, true);
+      }
+      YSCV_TRY(int4_run_ws(L.wgu, d->xn, YSCV_HIP_F16, d->act, YSCV_HIP_F16, batch, 1, EPI_SWIGLU, d->ws, d->ws_bytes, s,
+                           d->fold_norm ? &cg : nullptr));
+      if (d->fold_norm) producer(pd, li + 1 < d->layers.size() ? d->layers[li + 1].attn_norm : d->final_norm, &n_d);
+      YSCV_TRY(int4_run_ws(L.wdown, d->act, YSCV_HIP_F16, d->h, YSCV_HIP_F32, batch, 1, EPI_ADD_F32, d->ws, d->ws_bytes, s,
+                           d->fold_norm ? &pd : nullptr));
+      if (d->fold_norm) {
+        cur ^= 1;
+        cnt = n_d;
+      }
     }
-    YSCV_TRY(int4_run_ws(d->lm_head, d->xn, YSCV_HIP_F16, d->logits, YSCV_HIP_F32, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s));
+    NormFold cl;
+    if (d->fold_norm) consumer(cl, false);
+    YSCV_TRY(int4_run_ws(d->lm_head, d->xn, YSCV_HIP_F16, d->logits, YSCV_HIP_F32, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s,
+                         d->fold_norm ? &cl : nullptr));
   }
   return YSCV_HIP_OK;
 }
@@ -900,6 +1041,19 @@ int32_t yscv_hip_decoder_read_activation(yscv_hip_decoder *d, int32_t which, flo
       DEC_HIP(hipMemcpy(tmp.data() + b * qkv_n, d->qrot + b * qn, qn * 2, hipMemcpyDeviceToHost));
   }
   for (size_t i = 0; i < elems; i++) out_host[i] = (float)tmp[i];
+  if (which == YSCV_HIP_DEC_ACT_NORMED && d->fold_norm && d->last_ss_count > 0) {
+    // folded norm: the buffer holds fp16(h * gamma * pre[row]); what the consumer multiplied by its weights is that
+    // times the row factor it worked out from the partial sums of squares and pre[row]
+    std::vector<float> ss((size_t)B * d->ss_stride), pre(B);
+    DEC_HIP(hipMemcpy(ss.data(), d->ss[d->last_ss], ss.size() * 4, hipMemcpyDeviceToHost));
+    DEC_HIP(hipMemcpy(pre.data(), d->pre[d->last_ss], B * 4, hipMemcpyDeviceToHost));
+    for (size_t b = 0; b < B; b++) {
+      float t = 0.0f;
+      for (int j = 0; j < d->last_ss_count; j++) t += ss[b * d->ss_stride + j];
+      const float f = 1.0f / (pre[b] * std::sqrt(t / (float)c.d_model + c.rms_eps));
+      for (size_t i = 0; i < (size_t)c.d_model; i++) out_host[b * c.d_model + i] *= f;
+    }
+  }
   return YSCV_HIP_OK;
 }
 
@@ -929,6 +1083,14 @@ int32_t yscv_hip_decoder_debug_set_fused_attention(yscv_hip_decoder *d, int32_t 
   YSCV_REQUIRE(d != nullptr, "null decoder");
   drop_graph(d);  // a captured step holds the launches of the other variant
   d->fused_attn = on != 0;
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_debug_set_folded_norm(yscv_hip_decoder *d, int32_t on) {
+  YSCV_REQUIRE(d != nullptr, "null decoder");
+  drop_graph(d);
+  d->fold_norm_wanted = on != 0;
+  if (d->finalized) YSCV_TRY(finish_setup(d));
   return YSCV_HIP_OK;
 }
 

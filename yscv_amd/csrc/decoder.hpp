@@ -7,6 +7,10 @@ namespace yscv {
 
 int32_t launch_embed(const int32_t *tokens, const _Float16 *table, int batch, int d, int vocab, float *h,
                      hipStream_t s);
+// embedding lookup + the first norm in its folded form (NormFold in kernels.hpp): one partial sum of squares and the
+// power-of-two scale of xg per row
+int32_t launch_embed_norm(const int32_t *tokens, const _Float16 *table, int batch, int d, int vocab, float eps, float *h,
+                          const float *gamma, _Float16 *xg, float *ss_out, int ss_stride, float *pre, hipStream_t s);
 int32_t launch_rmsnorm(const float *h, const float *gamma, int batch, int d, float eps, _Float16 *out,
                        hipStream_t s);
 int32_t launch_rope_append(_Float16 *qkv, const int32_t *pos_ptr, int batch, int hq, int hkv, int hd, float theta,

@@ -18,6 +18,7 @@
 // Q K^T) or 8 consecutive positions of one d (V, B operand of P V) as one 128-bit load.
 #include "decoder.hpp"
 #include "int4_common.hpp"
+#include "kernels.hpp"
 
 namespace yscv {
 
@@ -28,6 +29,43 @@ __global__ void embed_kernel(const int32_t *__restrict__ tokens, const _Float16 
   int tok = tokens[b];
   tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
   for (int i = threadIdx.x; i < d; i += blockDim.x) h[(size_t)b * d + i] = (float)table[(size_t)tok * d + i];
+}
+
+// embedding lookup that also feeds the first norm in its folded form (NormFold, kernels.hpp): the row stays in
+// registers (d <= 4096) until its sum of squares is known, which gives the power of two pre[b] near 1 / (4 rms);
+// xg = fp16(h * gamma * pre[b]), and the sum as the row's single partial
+__global__ void __launch_bounds__(256) embed_norm_kernel(const int32_t *__restrict__ tokens, const _Float16 *__restrict__ table,
+                                                         int d, int vocab, float eps, float *__restrict__ h,
+                                                         const float *__restrict__ gamma, _Float16 *__restrict__ xg,
+                                                         float *__restrict__ ss_out, int ss_stride, float *__restrict__ pre) {
+  __shared__ float red4[4];
+  const int b = blockIdx.x;
+  int tok = tokens[b];
+  tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+  constexpr int KEEP = 16;
+  float keep[KEEP];
+  float sq = 0.0f;
+#pragma unroll
+  for (int u = 0; u < KEEP; u++) {
+    const int i = u * 256 + (int)threadIdx.x;
+    keep[u] = i < d ? (float)table[(size_t)tok * d + i] : 0.0f;
+    if (i < d) h[(size_t)b * d + i] = keep[u];
+    sq += keep[u] * keep[u];
+  }
+  sq = wave_sum(sq);
+  if ((threadIdx.x & 63) == 0) red4[threadIdx.x >> 6] = sq;
+  __syncthreads();
+  const float total = ((red4[0] + red4[1]) + red4[2]) + red4[3];
+  const float scale = norm_fold_prescale(1.0f / sqrtf(total / (float)d + eps));
+#pragma unroll
+  for (int u = 0; u < KEEP; u++) {
+    const int i = u * 256 + (int)threadIdx.x;
+    if (i < d) xg[(size_t)b * d + i] = (_Float16)fminf(fmaxf(keep[u] * gamma[i] * scale, -65504.0f), 65504.0f);
+  }
+  if (threadIdx.x == 0) {
+    ss_out[(size_t)b * ss_stride] = total;
+    pre[b] = scale;
+  }
 }
 
 // ---- RMSNorm: f32 residual -> fp16 normalised activations -----------------------------------------
@@ -800,6 +838,15 @@ __global__ void fill_const_f32_kernel(float *p, size_t n, float v) {
 int32_t launch_embed(const int32_t *tokens, const _Float16 *table, int batch, int d, int vocab, float *h,
                      hipStream_t s) {
   hipLaunchKernelGGL(embed_kernel, dim3(batch), dim3(256), 0, s, tokens, table, d, vocab, h);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_embed_norm(const int32_t *tokens, const _Float16 *table, int batch, int d, int vocab, float eps, float *h,
+                          const float *gamma, _Float16 *xg, float *ss_out, int ss_stride, float *pre, hipStream_t s) {
+  if (d > 4096) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "embedding with a folded norm: rows of at most 4096 values");
+  hipLaunchKernelGGL(embed_norm_kernel, dim3(batch), dim3(256), 0, s, tokens, table, d, vocab, eps, h, gamma, xg, ss_out, ss_stride,
+                     pre);
   YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
 }

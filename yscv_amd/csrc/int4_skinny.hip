@@ -63,6 +63,17 @@ struct SkinnyArgs {
   int ksg;
   int epi;         // EPI_STORE / EPI_ADD_F32 / EPI_SWIGLU
   int slices;      // ktp / TPW: number of wave-sized k slices that exist
+  // RMSNorm folded into the projections around it (NormFold in kernels.hpp); all null / 0 when unused
+  const float *gamma_next;  // producer: scale vector of the norm that follows the residual update
+  const float *pre;         // producer: power of two per row, [m]
+  _Float16 *xg;             // producer: fp16(h_new * gamma_next * pre[row]), [m][n]
+  float *ss_out;            // producer: sums of h_new^2 per row and 16-column block, [m][ss_out_stride]
+  int ss_out_stride;
+  const float *ss_in;       // consumer: partial sums of squares of the rows it multiplies, [m][ss_in_stride]
+  const float *pre_in;      // consumer: what the rows of its activations were multiplied by, [m]
+  float *pre_next;          // consumer, may be null: power of two per row for the residual update behind this norm
+  int ss_in_count, ss_in_stride;
+  float ss_inv_d, ss_eps;
 };
 
 // Scales of one (tile, row) kept in their storage type until used: 1, 2 or 4 values.
@@ -179,6 +190,46 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
     }
   };
   if constexpr (EARLY) fill_ring();
+  // folded norm, consumer side: this wave's share of the partial sums of squares (see further down), requested
+  // here so that their round trip overlaps the activations'
+  constexpr int kSsRowsPerWave = 4;  // rows wave, wave + waves, ...: the launcher checks that four per wave cover m
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  float ss_pre[kSsRowsPerWave][4], ss_scale[kSsRowsPerWave];
+  if (a.ss_in) {
+#pragma unroll
+    for (int u = 0; u < kSsRowsPerWave; u++) {
+      const int row = wave_u + u * waves;
+      ss_scale[u] = a.pre_in[min(row, a.m - 1)];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const int j = 4 * lane + e;
+        ss_pre[u][e] = (row < a.m && j < a.ss_in_count) ? a.ss_in[(size_t)row * a.ss_in_stride + j] : 0.0f;
+      }
+    }
+  }
+
+  // folded norm, producer side: the residual values and the gammas this wave's first two pieces of the first
+  // reduction will need, requested now (their round trip would otherwise sit at the end of a one-block kernel)
+  // (only in the instantiations with a ring of one or two blocks, where a residual update of a decode step lands and
+  // registers are to spare)
+  constexpr bool PREFETCH_H = P <= 2;
+  float h_pre[2] = {0.0f, 0.0f}, g_pre[2] = {0.0f, 0.0f}, p_pre[2] = {0.0f, 0.0f};
+  if (PREFETCH_H && a.xg) {
+#pragma unroll
+    for (int sl = 0; sl < 2; sl++) {
+      const int q = wave_u + sl * waves;
+      if (q < UB * NI) {  // uniform in the wave
+        const int u = q / NI, i = q % NI;
+        const int col = ((int)blockIdx.x + u * stride) * 16 + r;
+        const int mrow = c * NI + i;
+        if (col < a.n) g_pre[sl] = a.gamma_next[col];
+        if (mrow < a.m && col < a.n) {
+          h_pre[sl] = reinterpret_cast<const float *>(a.y)[(size_t)mrow * a.n + col];
+          p_pre[sl] = a.pre[mrow];
+        }
+      }
+    }
+  }
 
   // ---- activations -> registers, in A-operand order ------------------------------------------
   // MFMA row `r` carries batch row m when r == 4*(m / NI) + (m % NI): the useful results then sit
@@ -370,6 +421,28 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
       }
     }
   }
+  // Folded RMSNorm, consumer side: the row factors 1 / (pre * sqrt(sum(h^2) / d + eps)) come from the partial sums the
+  // kernel that wrote the residual left behind and from the power of two it scaled the row with.  Row q is added up by wave q % waves (four consecutive partials per
+  // lane, requested further up together with the activations, then a fixed tree of DPP moves and lane swaps: the
+  // same order in every run); the sixteen factors meet in LDS behind the barrier of the first reduction, which every
+  // use of them follows.
+  float *rs_lds = red + (size_t)2 * waves * (UB * NI) * 64;
+  if (a.ss_in) {
+#pragma unroll
+    for (int u = 0; u < kSsRowsPerWave; u++) {
+      const int row = wave_u + u * waves;
+      if (row < a.m) {  // uniform in the wave
+        const float t = wave_sum((ss_pre[u][0] + ss_pre[u][1]) + (ss_pre[u][2] + ss_pre[u][3]));
+        const float inv_rms = 1.0f / sqrtf(t * a.ss_inv_d + a.ss_eps);
+        if (lane == 0) {
+          rs_lds[row] = inv_rms / ss_scale[u];
+          // one workgroup leaves the scale of the next residual update behind (every workgroup holds the same bits)
+          if (a.pre_next && blockIdx.x == 0 && blockIdx.y == 0) a.pre_next[row] = norm_fold_prescale(inv_rms);
+        }
+      }
+    }
+  }
+
   // RAWX: accumulator i of lane (c, .) belongs to row c * NI + i, which lanes 4 c + i (+16, +32, +48) loaded
   float acc_scale[NI];
 #pragma unroll
@@ -493,9 +566,7 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
 
   // row scales of the activation pass, one per accumulator of this lane (loaded once: a load inside the loop
   // would make the compiler wait for every weight block in flight)
-  float rs[NI];
-#pragma unroll
-  for (int i = 0; i < NI; i++) rs[i] = 1.0f;
+  float4_t rs = {1.0f, 1.0f, 1.0f, 1.0f};  // (a vector: an array here ended up in scratch memory once the epilogues grew)
   if (a.row_scale) {  // one branch around all of them: rows past m read the last row's scale and are never stored
 #pragma unroll
     for (int i = 0; i < NI; i++) rs[i] = a.row_scale[min(c * NI + i, a.m - 1)];
@@ -520,7 +591,7 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
     }
     lds_barrier();
     // epilogue of one finished 64-lane piece q = u * NI + i: block u of the group, accumulator i
-    auto finish = [&](float v, int q) {
+    auto finish = [&](float v, int q, int slot) {
       const int u = q / NI, i = q % NI;
       const int col = (nt0 + u * stride) * 16 + r;
       const int mrow = c * NI + i;
@@ -531,7 +602,27 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
         float rsv = rs[0];
 #pragma unroll
         for (int ii = 1; ii < NI; ii++) rsv = (i == ii) ? rs[ii] : rsv;
+        if (a.ss_in) rsv = rs_lds[min(mrow, a.m - 1)];
         v *= rsv;
+        if (a.epi == EPI_ADD_F32 && a.xg) {
+          // residual update that also feeds the next norm: h_new, its fp16 image times gamma and the row's power of two, and the sum of
+          // h_new^2 over the sixteen columns of this block (the lanes r = 0..15 of a lane group), one per row
+          float hn = 0.0f;
+          if (live) {
+            float *hp = reinterpret_cast<float *>(a.y) + (size_t)mrow * a.n + col;
+            const bool pre = PREFETCH_H && ex == 0 && slot >= 0 && slot < 2;  // requested at the start of the kernel
+            const float hold = pre ? (slot == 0 ? h_pre[0] : h_pre[1]) : *hp;
+            const float gam = pre ? (slot == 0 ? g_pre[0] : g_pre[1]) : a.gamma_next[col];
+            const float pw = pre ? (slot == 0 ? p_pre[0] : p_pre[1]) : a.pre[mrow];
+            hn = hold + v;
+            *hp = hn;
+            const float gx = fminf(fmaxf(hn * gam * pw, -65504.0f), 65504.0f);
+            a.xg[(size_t)mrow * a.n + col] = (_Float16)gx;
+          }
+          const float sq = row_sum16(hn * hn);
+          if (r == 0 && mrow < a.m && (nt0 + u * stride) < a.nt) a.ss_out[(size_t)mrow * a.ss_out_stride + (nt0 + u * stride)] = sq;
+          return;
+        }
         if (a.epi == EPI_SWIGLU) {
           // rows 2i / 2i+1 of the weight are gate_i / up_i: neighbours in the wave
           const float up = __shfl_xor(v, 1, 64);
@@ -565,11 +656,11 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
         v0 += p0[w];
         v1 += p1[w];
       }
-      finish(v0, q);
-      finish(v1, q + 8);
+      finish(v0, q, 0);
+      finish(v1, q + 8, 1);
       return;
     }
-    for (; q < UB * NI; q += waves) {
+    for (int slot = 0; q < UB * NI; q += waves, slot++) {
       const float *rb = buf + q * 64 + lane;
       float v = 0.0f;
       if (waves == 8) {  // all eight slices in one LDS round trip
@@ -588,7 +679,7 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
           for (int w = 0; w < 4; w++) v += part[w];
         }
       }
-      finish(v, q);
+      finish(v, q, slot);
     }
   };
 
@@ -683,6 +774,36 @@ __global__ void int4_skinny_finalize_kernel(const float *__restrict__ partial, i
   }
 }
 
+// The second pass of a K-split residual update that also feeds the next norm (NormFold): one workgroup per (row, 256
+// columns); h += sum of the partials in slice order, xg = fp16(h * gamma * pre[row]), and the sum of h^2 over the 256 columns
+// (fixed order: shuffle tree per wave, then the four waves in turn) as one partial of the row.  n % 256 == 0.
+__global__ void __launch_bounds__(256) int4_skinny_finalize_norm_kernel(const float *__restrict__ partial, int ksg, int m, int n,
+                                                                        float *__restrict__ h, const float *__restrict__ gamma,
+                                                                        const float *__restrict__ pre, _Float16 *__restrict__ xg, float *__restrict__ ss_out,
+                                                                        int ss_stride) {
+  __shared__ float red4[4];
+  const int chunks = n >> 8;
+  const int row = blockIdx.x / chunks, chunk = blockIdx.x % chunks;
+  const size_t total = (size_t)m * n;
+  const size_t idx = (size_t)row * n + (size_t)chunk * 256 + threadIdx.x;
+  float p[8];
+#pragma unroll
+  for (int s = 0; s < 8; s++) p[s] = s < ksg ? partial[(size_t)s * total + idx] : 0.0f;
+  const float before = h[idx];
+  const float g = gamma[chunk * 256 + threadIdx.x] * pre[row];
+  float v = 0.0f;
+#pragma unroll
+  for (int s = 0; s < 8; s++) v += p[s];
+  for (int s = 8; s < ksg; s++) v += partial[(size_t)s * total + idx];
+  const float hn = before + v;
+  h[idx] = hn;
+  xg[idx] = (_Float16)fminf(fmaxf(hn * g, -65504.0f), 65504.0f);
+  const float sq = wave_sum(hn * hn);
+  if ((threadIdx.x & 63) == 0) red4[threadIdx.x >> 6] = sq;
+  __syncthreads();
+  if (threadIdx.x == 0) ss_out[(size_t)row * ss_stride + chunk] = ((red4[0] + red4[1]) + red4[2]) + red4[3];
+}
+
 SkinnyPlan plan_int4_skinny(const yscv_hip_int4_weight *w, size_t m, int split, int num_cus) {
   (void)split;
   SkinnyPlan p;
@@ -708,7 +829,7 @@ SkinnyPlan plan_int4_skinny(const yscv_hip_int4_weight *w, size_t m, int split, 
 template <int SPLIT, int NI, int GM, bool SF16, bool HAS_ZP, int P>
 static int32_t launch_p(const SkinnyArgs &a, const SkinnyPlan &plan, hipStream_t s) {
   constexpr int UB = skinny_ub(NI, P);
-  const size_t lds = (size_t)2 * plan.waves * UB * NI * 64 * sizeof(float);
+  const size_t lds = (size_t)2 * plan.waves * UB * NI * 64 * sizeof(float) + 64;  // + the sixteen row factors of a folded norm
   if constexpr (SPLIT == 2) {
     if (a.xf != nullptr) {
       const size_t stage = NI == 1 ? (size_t)plan.waves * kStageWave : 0;
@@ -717,7 +838,7 @@ static int32_t launch_p(const SkinnyArgs &a, const SkinnyPlan &plan, hipStream_t
         static hipError_t attr_err = hipSuccess;
         std::call_once(once, [] {
           attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(int4_skinny_kernel<SPLIT, NI, GM, SF16, HAS_ZP, P, 1>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, 8 * (2 * UB * NI * 64 * 4 + kStageWave));
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 8 * (2 * UB * NI * 64 * 4 + kStageWave) + 64);
         });
         if (attr_err != hipSuccess)
           return set_error(YSCV_HIP_ERR_DEVICE, "cannot reserve LDS for the activation staging: %s", hipGetErrorString(attr_err));
@@ -780,7 +901,7 @@ static int32_t launch_gm(const SkinnyArgs &a, const SkinnyPlan &plan, int gm, bo
 
 int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan, const _Float16 *xh,
                            const _Float16 *xl, const void *xraw, const float *row_scale, size_t k_pad, int split,
-                           void *y, int y_dtype, size_t m, float *partial, int epi, hipStream_t s) {
+                           void *y, int y_dtype, size_t m, float *partial, int epi, hipStream_t s, const NormFold *nf) {
   if (!w->tiled) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "skinny int4 kernel needs the tiled layout");
   if (m == 0 || m > 16) return set_error(YSCV_HIP_ERR_INVALID_ARG, "skinny int4 kernel handles 1 <= m <= 16, got %zu", m);
   if (plan.ksg > 1 && !partial) return set_error(YSCV_HIP_ERR_INVALID_ARG, "k-split needs a partial buffer");
@@ -808,6 +929,50 @@ int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan
   a.ksg = plan.ksg;
   a.epi = epi;
   a.slices = (int)(w->ktp / TPW);
+  a.gamma_next = nullptr;
+  a.xg = nullptr;
+  a.pre = a.pre_in = nullptr;
+  a.pre_next = nullptr;
+  a.ss_out = nullptr;
+  a.ss_out_stride = 0;
+  a.ss_in = nullptr;
+  a.ss_in_count = a.ss_in_stride = 0;
+  a.ss_inv_d = a.ss_eps = 0.0f;
+  const bool produce = nf && nf->xg != nullptr;
+  if (produce && row_scale) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "folded norm: the producing call takes activations as they are");
+  if (nf) {
+    if (nf->ss_in) {
+      if (plan.ksg > 1) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "folded norm: the consuming projection must not be K-split");
+      if (m > (size_t)4 * plan.waves || nf->ss_in_count > 256)
+        return set_error(YSCV_HIP_ERR_UNSUPPORTED, "folded norm: %zu rows on %d waves, %d partial sums per row", m, plan.waves, nf->ss_in_count);
+      if (split != 1 || xraw) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "folded norm: fp16 activations only");
+      if (!nf->pre_in) return set_error(YSCV_HIP_ERR_INVALID_ARG, "folded norm: the row scales of the activations are missing");
+      a.ss_in = nf->ss_in;
+      a.pre_in = nf->pre_in;
+      a.pre_next = nf->pre_next;
+      a.ss_in_count = nf->ss_in_count;
+      a.ss_in_stride = nf->ss_in_stride;
+      a.ss_inv_d = nf->inv_d;
+      a.ss_eps = nf->eps;
+    }
+    if (produce) {
+      if (epi != EPI_ADD_F32 || !nf->gamma_next || !nf->ss_out || !nf->ss_out_count || !nf->pre)
+        return set_error(YSCV_HIP_ERR_INVALID_ARG, "folded norm: the producing call is a residual update with gamma and a place for the sums");
+      if (plan.ksg > 1) {
+        if (w->n % 256 != 0 || plan.ksg > 64 || nf->ss_out_stride < (int)(w->n / 256))
+          return set_error(YSCV_HIP_ERR_UNSUPPORTED, "folded norm: K-split update needs n a multiple of 256");
+        *nf->ss_out_count = (int)(w->n / 256);
+      } else {
+        if (nf->ss_out_stride < (int)w->nt) return set_error(YSCV_HIP_ERR_INVALID_ARG, "folded norm: room for %zu partial sums per row", w->nt);
+        a.gamma_next = nf->gamma_next;
+        a.pre = nf->pre;
+        a.xg = nf->xg;
+        a.ss_out = nf->ss_out;
+        a.ss_out_stride = nf->ss_out_stride;
+        *nf->ss_out_count = (int)w->nt;
+      }
+    }
+  }
   if (epi == EPI_ADD_F32 && y_dtype != YSCV_HIP_F32)
     return set_error(YSCV_HIP_ERR_INVALID_ARG, "residual accumulation needs an f32 output");
   if (epi == EPI_SWIGLU && (w->n & 1)) return set_error(YSCV_HIP_ERR_INVALID_ARG, "SwiGLU epilogue needs an even row count");
@@ -821,6 +986,12 @@ int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan
   else
     st = small ? launch_gm<1, 1>(a, plan, w->gm, sf16, w->has_zp, s) : launch_gm<1, 4>(a, plan, w->gm, sf16, w->has_zp, s);
   YSCV_TRY(st);
+  if (plan.ksg > 1 && produce) {
+    hipLaunchKernelGGL(int4_skinny_finalize_norm_kernel, dim3((unsigned)(m * (w->n / 256))), dim3(256), 0, s, partial, plan.ksg,
+                       (int)m, (int)w->n, static_cast<float *>(y), nf->gamma_next, nf->pre, nf->xg, nf->ss_out, nf->ss_out_stride);
+    YSCV_HIP_TRY(hipGetLastError());
+    return YSCV_HIP_OK;
+  }
   if (plan.ksg > 1) {
     const size_t total = epi == EPI_SWIGLU ? m * (w->n / 2) : m * w->n;
     int blocks = (int)ceil_div(total, (size_t)256);

@@ -57,6 +57,32 @@ int32_t launch_x_prep(const void *x, int x_dtype, size_t m, size_t k, size_t k_p
 // epilogues of the skinny kernel
 enum : int { EPI_STORE = 0, EPI_ADD_F32 = 1, EPI_SWIGLU = 2 };
 
+// RMSNorm folded into the projections on either side of it (decode loop).  The kernel that updates the residual
+// stream h (EPI_ADD_F32) also writes what the norm's consumer needs: xg = fp16(h_new * gamma * pre[row]) and, per row,
+// partial sums of h_new^2 over fixed column blocks.  pre[row] is a power of two near 1 / (4 rms) of the row as the
+// norm BEFORE this update saw it (the kernel that consumed that norm leaves it behind; the embedding lookup works
+// it out from its own row): an unnormalised row would otherwise leave fp16's range at either end, and a power of two
+// leaves the rounding what it is.  A row may grow 2^18 / (its largest |value| / rms * gamma) fold within one update
+// before an element saturates at fp16's maximum, and shrink 2^12 fold before its typical element loses precision.
+// The projection that consumes xg works out inv = 1 / (pre * sqrt(sum / d + eps)) per row from the partials and
+// applies it to its f32 sums: the same product as RMSNorm followed by the projection, with the fp16 rounding taken
+// before the row factor instead of after it.
+struct NormFold {
+  // producer side (with EPI_ADD_F32): all null when the call does not feed a norm
+  const float *gamma_next = nullptr;  // [n]
+  const float *pre = nullptr;         // [m] power of two per row
+  _Float16 *xg = nullptr;             // [m][n]
+  float *ss_out = nullptr;            // [m][ss_out_stride]; the call reports how many partials per row it wrote
+  int ss_out_stride = 0;
+  int *ss_out_count = nullptr;        // host
+  // consumer side: null when the activations are already normalised
+  const float *ss_in = nullptr;       // [m][ss_in_stride]
+  const float *pre_in = nullptr;      // [m] what the rows of xg were multiplied by
+  float *pre_next = nullptr;          // [m] or null: receives the power of two for the update that follows this norm
+  int ss_in_count = 0, ss_in_stride = 0;
+  float inv_d = 0.0f, eps = 0.0f;
+};
+
 struct SkinnyPlan {
   int tpw;     // 128-k tiles per wave
   int waves;   // wavefronts per workgroup (= k-slices per workgroup)
@@ -69,7 +95,8 @@ SkinnyPlan plan_int4_skinny(const yscv_hip_int4_weight *w, size_t m, int split, 
 // normalises (and for f32 splits) them itself and xh, xl, row_scale are not used
 int32_t launch_int4_skinny(const yscv_hip_int4_weight *w, const SkinnyPlan &plan, const _Float16 *xh,
                            const _Float16 *xl, const void *xraw, const float *row_scale, size_t k_pad, int split,
-                           void *y, int y_dtype, size_t m, float *partial, int epi, hipStream_t s);
+                           void *y, int y_dtype, size_t m, float *partial, int epi, hipStream_t s,
+                           const NormFold *nf = nullptr);
 int32_t launch_int4_generic(const yscv_hip_int4_weight *w, const void *x, int x_dtype, void *y,
                             int y_dtype, size_t m, hipStream_t s);
 int32_t launch_int4_gemm(const yscv_hip_int4_weight *w, const _Float16 *xh, const _Float16 *xl,
@@ -85,7 +112,7 @@ int32_t launch_int4_gemm_ring(const yscv_hip_int4_weight *w, const _Float16 *xh,
 // Whole int4 call (activation preparation + kernel) with caller-provided scratch; ws may be null.
 int32_t int4_workspace_bytes(const yscv_hip_int4_weight *w, size_t m, int x_dtype, int force, size_t *bytes);
 int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, void *y, int y_dtype, size_t m,
-                    int force, int epi, void *ws, size_t ws_bytes, hipStream_t s);
+                    int force, int epi, void *ws, size_t ws_bytes, hipStream_t s, const NormFold *nf = nullptr);
 
 int32_t int4_create_from_device(const uint8_t *d_packed, const void *d_scales, int scale_dtype, int nibble_format,
                                 size_t n, size_t k, size_t g, yscv_hip_int4_weight **out);
