@@ -529,8 +529,9 @@ int32_t yscv_hip_decoder_debug_set_tag_epoch(yscv_hip_decoder *d, uint32_t epoch
  * one against the other.  Drops a captured graph.  No counterpart in the reference. */
 int32_t yscv_hip_decoder_debug_set_fused_attention(yscv_hip_decoder *d, int32_t on);
 /* Test aid: the multi-kernel path folds every RMSNorm into the projections around it when the shapes allow (the
- * kernel that updates the residual stream also writes fp16(h * gamma / 16) and per-row partial sums of h^2; the
- * projection that follows applies 16 / sqrt(mean(h^2) + eps) to its sums); 0 switches back to RMSNorm as a launch of
+ * kernel that updates the residual stream also writes fp16(h * gamma * p), p a power of two per row near
+ * 1 / (4 rms) of the row before the update, and per-row partial sums of h^2; the projection that follows applies
+ * 1 / (p * sqrt(mean(h^2) + eps)) to its sums); 0 switches back to RMSNorm as a launch of
  * its own, so that a test can hold one against the other (same product, the fp16 rounding taken before the row factor
  * instead of after it).  Drops a captured graph.  No counterpart in the reference. */
 int32_t yscv_hip_decoder_debug_set_folded_norm(yscv_hip_decoder *d, int32_t on);
