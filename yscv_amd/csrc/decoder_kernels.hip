@@ -42,15 +42,35 @@ __global__ void __launch_bounds__(256) embed_norm_kernel(const int32_t *__restri
   const int b = blockIdx.x;
   int tok = tokens[b];
   tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
-  constexpr int KEEP = 16;
-  float keep[KEEP];
+  // eight consecutive values per thread and piece, two pieces: 4096 values at most (d is a multiple of 8)
+  constexpr int PIECES = 2;
+  half8_t raw[PIECES];
+  float4_t gam[PIECES][2];
+#pragma unroll
+  for (int u = 0; u < PIECES; u++) {
+    const int i = (u * 256 + (int)threadIdx.x) * 8;
+    const bool in = i < d;
+    raw[u] = in ? *reinterpret_cast<const half8_t *>(table + (size_t)tok * d + i) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    // gamma is requested with the row, not after the sum
+    gam[u][0] = in ? *reinterpret_cast<const float4_t *>(gamma + i) : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    gam[u][1] = in ? *reinterpret_cast<const float4_t *>(gamma + i + 4) : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  }
   float sq = 0.0f;
 #pragma unroll
-  for (int u = 0; u < KEEP; u++) {
-    const int i = u * 256 + (int)threadIdx.x;
-    keep[u] = i < d ? (float)table[(size_t)tok * d + i] : 0.0f;
-    if (i < d) h[(size_t)b * d + i] = keep[u];
-    sq += keep[u] * keep[u];
+  for (int u = 0; u < PIECES; u++) {
+    const int i = (u * 256 + (int)threadIdx.x) * 8;
+    if (i < d) {
+      float4_t lo, hi;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        lo[e] = (float)raw[u][e];
+        hi[e] = (float)raw[u][4 + e];
+      }
+      *reinterpret_cast<float4_t *>(h + (size_t)b * d + i) = lo;
+      *reinterpret_cast<float4_t *>(h + (size_t)b * d + i + 4) = hi;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) sq += (float)raw[u][e] * (float)raw[u][e];
   }
   sq = wave_sum(sq);
   if ((threadIdx.x & 63) == 0) red4[threadIdx.x >> 6] = sq;
@@ -58,9 +78,15 @@ __global__ void __launch_bounds__(256) embed_norm_kernel(const int32_t *__restri
   const float total = ((red4[0] + red4[1]) + red4[2]) + red4[3];
   const float scale = norm_fold_prescale(1.0f / sqrtf(total / (float)d + eps));
 #pragma unroll
-  for (int u = 0; u < KEEP; u++) {
-    const int i = u * 256 + (int)threadIdx.x;
-    if (i < d) xg[(size_t)b * d + i] = (_Float16)fminf(fmaxf(keep[u] * gamma[i] * scale, -65504.0f), 65504.0f);
+  for (int u = 0; u < PIECES; u++) {
+    const int i = (u * 256 + (int)threadIdx.x) * 8;
+    if (i < d) {
+      half8_t o;
+#pragma unroll
+      for (int e = 0; e < 8; e++)
+        o[e] = (_Float16)fminf(fmaxf((float)raw[u][e] * gam[u][e >> 2][e & 3] * scale, -65504.0f), 65504.0f);
+      *reinterpret_cast<half8_t *>(xg + (size_t)b * d + i) = o;
+    }
   }
   if (threadIdx.x == 0) {
     ss_out[(size_t)b * ss_stride] = total;
@@ -647,13 +673,35 @@ __global__ void __launch_bounds__(1024) argmax_kernel(const float *__restrict__ 
   const float *row = logits + (size_t)b * vocab;
   float best = -INFINITY;
   int bi = -1;
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-    const float v = row[i];
-    // max_by keeps the later element unless the earlier one compares Greater; NaN compares Equal
+  // max_by keeps the later element unless the earlier one compares Greater; NaN compares Equal
+  auto take = [&](float v, int i) {
     if (bi < 0 || !(best > v)) {
       best = v;
       bi = i;
     }
+  };
+  if ((vocab & 3) == 0) {
+    // four consecutive values per thread and request, eight requests in flight, visited in index order
+    const float4_t *row4 = reinterpret_cast<const float4_t *>(row);
+    const int n4 = vocab >> 2;
+    for (int i0 = 0; i0 < n4; i0 += 8 * (int)blockDim.x) {
+      float4_t v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int i = i0 + u * (int)blockDim.x + (int)threadIdx.x;
+        v[u] = i < n4 ? row4[i] : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int i = i0 + u * (int)blockDim.x + (int)threadIdx.x;
+        if (i < n4) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) take(v[u][e], 4 * i + e);
+        }
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) take(row[i], i);
   }
   // combine: higher value wins, equal values -> larger index; an unordered pair keeps the larger index too
   auto better = [](float va, int ia, float vb, int ib) {
@@ -844,7 +892,7 @@ int32_t launch_embed(const int32_t *tokens, const _Float16 *table, int batch, in
 
 int32_t launch_embed_norm(const int32_t *tokens, const _Float16 *table, int batch, int d, int vocab, float eps, float *h,
                           const float *gamma, _Float16 *xg, float *ss_out, int ss_stride, float *pre, hipStream_t s) {
-  if (d > 4096) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "embedding with a folded norm: rows of at most 4096 values");
+  if (d > 4096 || d % 8 != 0) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "embedding with a folded norm: rows of at most 4096 values, a multiple of 8");
   hipLaunchKernelGGL(embed_norm_kernel, dim3(batch), dim3(256), 0, s, tokens, table, d, vocab, eps, h, gamma, xg, ss_out, ss_stride,
                      pre);
   YSCV_HIP_TRY(hipGetLastError());
