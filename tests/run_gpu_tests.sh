@@ -2,5 +2,4 @@
 # One-process GPU test run with a per-test time limit (a hang names its test).
 set -o pipefail
 cd "$(dirname "$0")/.."
-mkdir -p gpurun_out
 exec timeout -k 10 900 python -u -m pytest tests -m gpu -x -v --timeout 120 --timeout-method thread "$@"
