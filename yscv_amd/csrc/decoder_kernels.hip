@@ -509,7 +509,11 @@ __global__ void __launch_bounds__(256) attn_fused_kernel(const _Float16 *__restr
       for (int j = 0; j < 4; j++)
         kf[pb][j] = *reinterpret_cast<const half8_t *>(kbase + (size_t)(pb * 16 + r) * HD + 32 * c + 8 * j);
 #pragma unroll
-    for (int t = 0; t < 8; t++) vf[t] = *reinterpret_cast<const half8_t *>(vbase + ((size_t)c * HD + t * 16 + r) * 8);
+    // V arrives in whole lines that nothing reads again in this launch: streaming loads keep them from displacing the
+    // K lines, which four requests share (K through streaming loads costs more than it saves: a line evicted between
+    // two of its requests is fetched again)
+    for (int t = 0; t < 8; t++)
+      vf[t] = __builtin_nontemporal_load(reinterpret_cast<const half8_t *>(vbase + ((size_t)c * HD + t * 16 + r) * 8));
   }
 
   // ---- rotary embedding: thread (h = tid / 64, i = tid % 64) turns the pair (i, i + 64) of query head h ----
