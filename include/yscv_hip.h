@@ -524,7 +524,7 @@ int32_t yscv_hip_decoder_read_activation(yscv_hip_decoder *d, int32_t which, flo
  * every step; close to the end of the tag space yscv_hip_decoder_run clears the exchange buffers and starts the count
  * again.  This sets the count (>= 1), so that a test reaches that point without half a million decode steps. */
 int32_t yscv_hip_decoder_debug_set_tag_epoch(yscv_hip_decoder *d, uint32_t epoch);
-/* Test aid: the multi-kernel path with an fp16 cache runs rotary embedding and cache append inside the attention kernel;
+/* Test aid: the multi-kernel path runs rotary embedding and cache append (fp16 or int8) inside the attention kernel;
  * 0 switches to the separate rope_append launch in front of it, which computes the same values, so that a test can hold
  * one against the other.  Drops a captured graph.  No counterpart in the reference. */
 int32_t yscv_hip_decoder_debug_set_fused_attention(yscv_hip_decoder *d, int32_t on);

@@ -86,19 +86,21 @@ def test_decode_steps_match_numpy(use_graph):
         cur = got_tok.copy()  # teacher-force the restatement with the GPU's picks
 
 
+@pytest.mark.parametrize("kv_dtype", ["f16", "i8"])
 @pytest.mark.parametrize("prefill", [5, 127, 128, 133, 250])
-def test_fused_attention_equals_the_separate_rope_append(prefill):
+def test_fused_attention_equals_the_separate_rope_append(prefill, kv_dtype):
     """Rotary embedding and cache append inside the attention kernel against the separate rope_append launch in front
     of it: same arithmetic, so tokens, logits, the attention output, the rotated q and the appended cache rows must be
     identical bit for bit.  The prefills put the current position at the start, the end and the middle of a
-    128-position chunk and leave chunks unused."""
+    128-position chunk and leave chunks unused.  With the int8 cache the appended row's scales span all kv heads, which
+    every workgroup that appends works out for itself."""
     import ctypes as C
 
     from yscv_amd.capi import lib
 
     rng = np.random.default_rng(4100 + prefill)
     cfg = dict(CFG)
-    dec, _ = _build(rng, cfg)
+    dec, _ = _build(rng, cfg, kv_dtype=kv_dtype)
     B, steps = 3, 5
     kv = []
     for l in range(cfg["n_layers"]):

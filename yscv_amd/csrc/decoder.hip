@@ -112,7 +112,7 @@ struct yscv_hip_decoder {
   float *h = nullptr, *logits = nullptr, *attn_part = nullptr;
   _Float16 *xn = nullptr, *qkv = nullptr, *ao = nullptr, *act = nullptr;
   _Float16 *qrot = nullptr;       // rotated query heads of the last fused attention launch (diagnostics)
-  bool fused_attn = true;         // fp16 cache: rope + append inside the attention kernel
+  bool fused_attn = true;         // rope + append inside the attention kernel
   // RMSNorm folded into the projections around it (NormFold, kernels.hpp): two buffers of partial sums of squares,
   // written and read in turn, each with the power of two per row that xn's rows were multiplied by
   bool fold_norm = false;         // decided in finish_setup from the shapes
@@ -480,7 +480,10 @@ static int32_t enqueue_step(yscv_hip_decoder *d, int batch, hipStream_t s) {
       YSCV_TRY(launch_rmsnorm(d->h, L.attn_norm, batch, D, c.rms_eps, d->xn, s));
       YSCV_TRY(int4_run_ws(L.wqkv, d->xn, YSCV_HIP_F16, d->qkv, YSCV_HIP_F16, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s));
     }
-    if (d->kv_dtype == YSCV_HIP_KV_I8) {
+    if (d->kv_dtype == YSCV_HIP_KV_I8 && d->fused_attn) {
+      YSCV_TRY(launch_attention_fused_i8(d->qkv, L.kc8, L.ks, L.vc8, L.vs, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim,
+                                         c.rope_theta, c.max_ctx, d->attn_part, d->qrot, d->ao, s));
+    } else if (d->kv_dtype == YSCV_HIP_KV_I8) {
       YSCV_TRY(launch_rope_append_i8(d->qkv, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_theta, c.max_ctx,
                                      L.kc8, L.ks, L.vc8, L.vs, s));
       YSCV_TRY(launch_attention_i8(d->qkv, L.kc8, L.ks, L.vc8, L.vs, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim,
@@ -1034,7 +1037,7 @@ int32_t yscv_hip_decoder_read_activation(yscv_hip_decoder *d, int32_t which, flo
   }
   std::vector<_Float16> tmp(elems);
   DEC_HIP(hipMemcpy(tmp.data(), src, elems * 2, hipMemcpyDeviceToHost));
-  if (which == YSCV_HIP_DEC_ACT_QKV && d->kv_dtype == YSCV_HIP_KV_F16 && d->fused_attn) {
+  if (which == YSCV_HIP_DEC_ACT_QKV && d->fused_attn) {
     // the fused attention kernel rotates q on the fly and leaves the buffer unrotated: report the rotated copy
     const size_t qn = (size_t)c.n_heads * c.head_dim;
     for (size_t b = 0; b < B; b++)

@@ -34,6 +34,10 @@ int32_t launch_kv_relayout_i8(const _Float16 *k_nat, const _Float16 *v_nat, int 
 int32_t launch_attention_i8(const _Float16 *qkv, const int8_t *kc, const float *ks, const int8_t *vc, const float *vs,
                             const int32_t *pos_ptr, int batch, int hq, int hkv, int hd, int max_ctx, float *part,
                             _Float16 *out, hipStream_t s);
+// rope_append_i8 fused into the attention partials, then the merge (int8 cache); `qrot` as in launch_attention_fused
+int32_t launch_attention_fused_i8(const _Float16 *qkv, int8_t *kc, float *ks, int8_t *vc, float *vs, const int32_t *pos_ptr,
+                                  int batch, int hq, int hkv, int hd, float theta, int max_ctx, float *part, _Float16 *qrot,
+                                  _Float16 *out, hipStream_t s);
 int32_t launch_kv_random_fill_i8(int8_t *buf, size_t n, float *scales, size_t n_scales, float scale, uint64_t seed, hipStream_t s);
 int32_t launch_argmax(const float *logits, int batch, int vocab, int32_t *tokens, int32_t *history,
                       int32_t *step_ptr, int max_steps, hipStream_t s);

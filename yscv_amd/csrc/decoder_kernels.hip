@@ -153,10 +153,34 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const float *__restrict__ 
   }
 }
 
+// sin and cos of the angle of pair i at position pos: inv_freq[i] = 1 / theta^(2i / d)
+struct SinCos {
+  float sn, cs;
+};
+__device__ __forceinline__ SinCos rope_sincos(float theta, int i, int d, int pos) {
+  const float inv_freq = 1.0f / powf(theta, (float)(2 * i) / (float)d);
+  SinCos r;
+  sincosf(inv_freq * (float)pos, &r.sn, &r.cs);
+  return r;
+}
+
 // rotate-half of one pair, written with explicit fused multiply-adds so that every kernel that rotates rounds alike
+__device__ __forceinline__ void rope_pair_f32(float x0, float x1, float cs, float sn, float &y0, float &y1) {
+  y0 = fmaf(x0, cs, -(x1 * sn));
+  y1 = fmaf(x0, sn, x1 * cs);
+}
+// f32 -> fp16 of a value that exists as an f32 first.  Without the empty asm the compiler may merge the conversion
+// into the multiply-add that produced the value (a mixed-precision fma that rounds once, straight to fp16), in one
+// kernel and not in another: one rotated q element in a few thousand then differs by an fp16 ulp between them.
+__device__ __forceinline__ _Float16 f16_of_f32(float v) {
+  asm volatile("" : "+v"(v));
+  return (_Float16)v;
+}
 __device__ __forceinline__ void rope_pair(float x0, float x1, float cs, float sn, _Float16 &y0, _Float16 &y1) {
-  y0 = (_Float16)fmaf(x0, cs, -(x1 * sn));
-  y1 = (_Float16)fmaf(x0, sn, x1 * cs);
+  float f0, f1;
+  rope_pair_f32(x0, x1, cs, sn, f0, f1);
+  y0 = f16_of_f32(f0);
+  y1 = f16_of_f32(f1);
 }
 
 // ---- RoPE on q (in place) and k, then append k / v to the cache -------------------------------------
@@ -174,10 +198,8 @@ __global__ void __launch_bounds__(64) rope_append_kernel(_Float16 *__restrict__ 
   if (slot < hq + hkv) {
     // rotate-half: (x[i], x[i + d/2]) -> (x0 cos - x1 sin, x0 sin + x1 cos)
     for (int i = threadIdx.x; i < half_d; i += blockDim.x) {
-      const float inv_freq = 1.0f / powf(theta, (float)(2 * i) / (float)hd);
-      const float ang = inv_freq * (float)pos;
-      float sn, cs;
-      sincosf(ang, &sn, &cs);
+      const SinCos sc = rope_sincos(theta, i, hd, pos);
+      const float sn = sc.sn, cs = sc.cs;
       const float x0 = (float)src[i], x1 = (float)src[i + half_d];
       _Float16 y0, y1;
       rope_pair(x0, x1, cs, sn, y0, y1);
@@ -519,10 +541,8 @@ __global__ void __launch_bounds__(256) attn_fused_kernel(const _Float16 *__restr
   // ---- rotary embedding: thread (h = tid / 64, i = tid % 64) turns the pair (i, i + 64) of query head h ----
   {
     const int h = tid >> 6, i = tid & 63;
-    const float inv_freq = 1.0f / powf(theta, (float)(2 * i) / (float)HD);
-    const float ang = inv_freq * (float)pos;
-    float sn, cs;
-    sincosf(ang, &sn, &cs);
+    const SinCos sc = rope_sincos(theta, i, HD, pos);
+    const float sn = sc.sn, cs = sc.cs;
     if (h < group) {
       const int head = kvh * group + h;
       const _Float16 *src = qkv + (size_t)b * row_elems + (size_t)head * HD;
@@ -804,15 +824,15 @@ __global__ void __launch_bounds__(256) rope_append_i8_kernel(_Float16 *__restric
   float kmax = 0.0f, vmax = 0.0f;
   for (int idx = tid; idx < (hq + hkv) * HALF; idx += 256) {
     const int slot = idx / HALF, i = idx % HALF;
-    const float inv_freq = 1.0f / powf(theta, (float)(2 * i) / (float)HD);
-    float sn, cs;
-    sincosf(inv_freq * (float)pos, &sn, &cs);
+    const SinCos sc = rope_sincos(theta, i, HD, pos);
+    const float sn = sc.sn, cs = sc.cs;
     _Float16 *src = row + (size_t)slot * HD;
     const float x0 = (float)src[i], x1 = (float)src[i + HALF];
-    const float y0 = x0 * cs - x1 * sn, y1 = x0 * sn + x1 * cs;
+    float y0, y1;
+    rope_pair_f32(x0, x1, cs, sn, y0, y1);
     if (slot < hq) {
-      src[i] = (_Float16)y0;
-      src[i + HALF] = (_Float16)y1;
+      src[i] = f16_of_f32(y0);
+      src[i + HALF] = f16_of_f32(y1);
     } else {
       kbuf[(slot - hq) * HD + i] = y0;
       kbuf[(slot - hq) * HD + i + HALF] = y1;
@@ -838,6 +858,238 @@ __global__ void __launch_bounds__(256) rope_append_i8_kernel(_Float16 *__restric
     const int kvh = idx / HD, i = idx % HD;
     kc[(((size_t)b * hkv + kvh) * max_ctx + pos) * HD + i] = kv_quant_one(kbuf[idx], k_inv);
     vc[((((size_t)b * hkv + kvh) * (max_ctx / 8) + pos / 8) * HD + i) * 8 + (pos & 7)] = kv_quant_one(vbuf[idx], v_inv);
+  }
+}
+
+// ---- rotary embedding + int8 cache append + attention partials in ONE launch (int8 cache) ---------------------------
+// rope_append_i8_kernel -> attn_partial_kernel<true> without the kernel boundary, as attn_fused_kernel does it for the
+// fp16 cache.  The scale of an int8 row spans all kv heads of the position, so each of the Hkv workgroups whose chunk
+// holds the current position rotates the whole k row (Hkv * 64 pairs) and scans the whole v row to get the two scales
+// (all of them write the same two values), then quantises and appends its own head's 128 + 128 values and patches
+// them, with the new scales, into the registers of the wave that owns the position.  Dynamic LDS: Hkv * 128 floats.
+__global__ void __launch_bounds__(256) attn_fused_i8_kernel(const _Float16 *__restrict__ qkv, int8_t *kc, float *ks, int8_t *vc,
+                                                            float *vs, const int32_t *__restrict__ pos_ptr, int hq, int hkv,
+                                                            int max_ctx, int max_chunks, float scale, float theta,
+                                                            float *__restrict__ part, _Float16 *__restrict__ qrot) {
+  constexpr int HD = 128;
+  typedef int8_t char8_t __attribute__((ext_vector_type(8)));
+  extern __shared__ float krow_lds[];  // owner only: the rotated k row of every kv head, f32
+  __shared__ __attribute__((aligned(16))) _Float16 q_lds[4][HD];
+  __shared__ __attribute__((aligned(16))) _Float16 knew[HD], vnew[HD];  // k as its int8 value, v as q * scale
+  __shared__ float red[4], new_k_scale;
+  __shared__ __attribute__((aligned(16))) _Float16 p_lds[ATT_WAVES][4][32];
+  __shared__ float w_m[ATT_WAVES][4], w_l[ATT_WAVES][4];
+  __shared__ float w_o[ATT_WAVES][4][HD];
+  const int chunk = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, c = lane >> 4;
+  const int group = hq / hkv;
+  const int pos = *pos_ptr;
+  const int n_ctx = pos + 1;
+  const int live_chunks = (n_ctx + ATT_CHUNK - 1) / ATT_CHUNK;
+  if (chunk >= live_chunks) return;  // uniform in the workgroup, before any barrier
+  const int p0 = chunk * ATT_CHUNK + wave * ATT_POS_PER_WAVE;
+  const int row_elems = (hq + 2 * hkv) * HD;
+  const bool wave_live = p0 < n_ctx;
+  const bool owner = (pos / ATT_CHUNK) == chunk;
+
+  // ---- K / V bytes and scales of this wave's 32 positions: requested before anything else, converted further down ----
+  const size_t k_off = (((size_t)b * hkv + kvh) * max_ctx + p0) * HD;
+  const size_t v_off = ((((size_t)b * hkv + kvh) * (max_ctx / 8) + p0 / 8) * HD) * 8;
+  char8_t kraw[2][4], vraw[8];
+  float k_scale[2] = {1.0f, 1.0f}, v_scale[8];
+  if (wave_live) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) v_scale[e] = vs[(size_t)b * max_ctx + p0 + 8 * c + e];
+#pragma unroll
+    for (int pb = 0; pb < 2; pb++) {
+      k_scale[pb] = ks[(size_t)b * max_ctx + p0 + pb * 16 + r];
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        kraw[pb][j] = *reinterpret_cast<const char8_t *>(kc + k_off + (size_t)(pb * 16 + r) * HD + 32 * c + 8 * j);
+    }
+#pragma unroll
+    for (int t = 0; t < 8; t++) vraw[t] = *reinterpret_cast<const char8_t *>(vc + v_off + ((size_t)c * HD + t * 16 + r) * 8);
+  }
+
+  // ---- rotary embedding of the query heads; the owners also rotate k, find the row scales and append ----
+  {
+    const int h = tid >> 6, i = tid & 63;
+    const SinCos sc = rope_sincos(theta, i, HD, pos);
+    const float sn = sc.sn, cs = sc.cs;
+    if (h < group) {
+      const int head = kvh * group + h;
+      const _Float16 *src = qkv + (size_t)b * row_elems + (size_t)head * HD;
+      const float x0 = (float)src[i], x1 = (float)src[i + HD / 2];
+      _Float16 y0, y1;
+      rope_pair(x0, x1, cs, sn, y0, y1);
+      q_lds[h][i] = y0;
+      q_lds[h][i + HD / 2] = y1;
+      if (chunk == 0) {
+        qrot[((size_t)b * hq + head) * HD + i] = y0;
+        qrot[((size_t)b * hq + head) * HD + i + HD / 2] = y1;
+      }
+    }
+    if (owner) {
+      const _Float16 *row = qkv + (size_t)b * row_elems;
+      float kmax = 0.0f, vmax = 0.0f;
+      for (int slot = h; slot < hkv; slot += 4) {  // pair i of kv head `slot`: the angle is this thread's
+        const _Float16 *src = row + (size_t)(hq + slot) * HD;
+        const float x0 = (float)src[i], x1 = (float)src[i + HD / 2];
+        float y0, y1;
+        rope_pair_f32(x0, x1, cs, sn, y0, y1);
+        krow_lds[slot * HD + i] = y0;
+        krow_lds[slot * HD + i + HD / 2] = y1;
+        kmax = fmaxf(kmax, fmaxf(fabsf(y0), fabsf(y1)));
+      }
+      for (int idx = tid; idx < hkv * HD; idx += 256) vmax = fmaxf(vmax, fabsf((float)row[(size_t)(hq + hkv) * HD + idx]));
+      kmax = block_max_256(kmax, red);
+      vmax = block_max_256(vmax, red);
+      float ksc, kinv, vsc, vinv;
+      kv_row_scale(kmax, &ksc, &kinv);
+      kv_row_scale(vmax, &vsc, &vinv);
+      if (tid == 0) {
+        ks[(size_t)b * max_ctx + pos] = ksc;
+        vs[(size_t)b * max_ctx + pos] = vsc;
+        new_k_scale = ksc;
+      }
+      if (tid < HD) {
+        const int8_t q8 = kv_quant_one(krow_lds[kvh * HD + tid], kinv);
+        kc[(((size_t)b * hkv + kvh) * max_ctx + pos) * HD + tid] = q8;
+        knew[tid] = (_Float16)(float)q8;
+      } else {
+        const int dd = tid - HD;
+        const int8_t q8 = kv_quant_one((float)row[(size_t)(hq + hkv + kvh) * HD + dd], vinv);
+        vc[((((size_t)b * hkv + kvh) * (max_ctx / 8) + pos / 8) * HD + dd) * 8 + (pos & 7)] = q8;
+        vnew[dd] = (_Float16)((float)q8 * vsc);
+      }
+    }
+  }
+  __syncthreads();
+
+  float m_h = -INFINITY, l_h = 0.0f;
+  float o_acc[8];
+#pragma unroll
+  for (int t = 0; t < 8; t++) o_acc[t] = 0.0f;
+
+  if (wave_live) {
+    half8_t qa[4];
+    {
+      const int h = r >> 2;
+      const bool valid = ((r & 3) == 0) && h < group;
+      const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < 4; j++) qa[j] = valid ? *reinterpret_cast<const half8_t *>(&q_lds[h & 3][32 * c + 8 * j]) : z;
+    }
+    // int8 values are exact in fp16: the K scale multiplies the finished score, the V scale goes into the operand
+    // (V is converted after the scores, so that the bytes and the fp16 values of both are never live together)
+    half8_t kf[2][4];
+#pragma unroll
+    for (int pb = 0; pb < 2; pb++)
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) kf[pb][j][e] = (_Float16)(float)kraw[pb][j][e];
+    // the row appended in this launch: the loads above read whatever the cache held before
+    const int rel = pos - p0;
+    const bool patch = owner && rel >= 0 && rel < ATT_POS_PER_WAVE;
+    if (patch) {
+#pragma unroll
+      for (int pb = 0; pb < 2; pb++)
+        if (rel == pb * 16 + r) {
+          k_scale[pb] = new_k_scale;
+#pragma unroll
+          for (int j = 0; j < 4; j++) kf[pb][j] = *reinterpret_cast<const half8_t *>(&knew[32 * c + 8 * j]);
+        }
+    }
+
+    float s[2];
+#pragma unroll
+    for (int pb = 0; pb < 2; pb++) {
+      float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int j = 0; j < 4; j++) d = __builtin_amdgcn_mfma_f32_16x16x32_f16(qa[j], kf[pb][j], d, 0, 0, 0);
+      const int p = p0 + pb * 16 + r;
+      s[pb] = (p < n_ctx) ? d[0] * scale * k_scale[pb] : -INFINITY;
+    }
+    float mx = fmaxf(s[0], s[1]);
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    const float e0 = (s[0] == -INFINITY) ? 0.0f : __expf(s[0] - mx);
+    const float e1 = (s[1] == -INFINITY) ? 0.0f : __expf(s[1] - mx);
+    float sum = e0 + e1;
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    m_h = mx;
+    l_h = sum;
+    if (c < 4) {
+      p_lds[wave][c][r] = (_Float16)e0;
+      p_lds[wave][c][16 + r] = (_Float16)e1;
+    }
+    __builtin_amdgcn_wave_barrier();
+    half8_t vf[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) vf[t][e] = (_Float16)((float)vraw[t][e] * v_scale[e]);
+    if (patch) {
+      const int e_new = rel - 8 * c;
+      if (e_new >= 0 && e_new < 8) {
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+          const _Float16 nv = vnew[t * 16 + r];
+#pragma unroll
+          for (int e = 0; e < 8; e++)
+            if (e == e_new) vf[t][e] = nv;
+        }
+      }
+    }
+    half8_t pa = {0, 0, 0, 0, 0, 0, 0, 0};
+    if ((r & 3) == 0 && (r >> 2) < group) pa = *reinterpret_cast<const half8_t *>(&p_lds[wave][r >> 2][8 * c]);
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      half8_t vv = vf[t];
+      if (p0 + 8 * c >= n_ctx) vv = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      else if (p0 + 8 * c + 8 > n_ctx) {
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+          if (p0 + 8 * c + e >= n_ctx) vv[e] = (_Float16)0.0f;
+      }
+      float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
+      d = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vv, d, 0, 0, 0);
+      o_acc[t] = d[0];
+    }
+  }
+
+  // ---- merge the 4 waves, write this chunk's partial ----
+  if (c < 4) {
+    if (r == 0) {
+      w_m[wave][c] = m_h;
+      w_l[wave][c] = l_h;
+    }
+#pragma unroll
+    for (int t = 0; t < 8; t++) w_o[wave][c][t * 16 + r] = o_acc[t];
+  }
+  __syncthreads();
+  for (int idx = tid; idx < group * HD; idx += blockDim.x) {
+    const int h = idx / HD, dd = idx % HD;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < ATT_WAVES; w++) mx = fmaxf(mx, w_m[w][h]);
+    float l = 0.0f, o = 0.0f;
+#pragma unroll
+    for (int w = 0; w < ATT_WAVES; w++) {
+      const float f = (w_m[w][h] == -INFINITY) ? 0.0f : __expf(w_m[w][h] - mx);
+      l += w_l[w][h] * f;
+      o += w_o[w][h][dd] * f;
+    }
+    const int head = kvh * group + h;
+    float *dst = part + (((size_t)b * hq + head) * max_chunks + chunk) * (HD + 2);
+    dst[2 + dd] = o;
+    if (dd == 0) {
+      dst[0] = mx;
+      dst[1] = l;
+    }
   }
 }
 
@@ -972,6 +1224,24 @@ int32_t launch_attention_i8(const _Float16 *qkv, const int8_t *kc, const float *
   const float scale = 1.0f / sqrtf((float)hd);
   hipLaunchKernelGGL(attn_partial_kernel<true>, dim3(max_chunks, hkv, batch), dim3(256), 0, s, qkv, kc, vc, ks, vs, pos_ptr, hq,
                      hkv, max_ctx, max_chunks, scale, part);
+  YSCV_HIP_TRY(hipGetLastError());
+  hipLaunchKernelGGL(attn_combine_kernel, dim3(hq, batch), dim3(128), 0, s, part, pos_ptr, hq, max_chunks, out);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_attention_fused_i8(const _Float16 *qkv, int8_t *kc, float *ks, int8_t *vc, float *vs, const int32_t *pos_ptr,
+                                  int batch, int hq, int hkv, int hd, float theta, int max_ctx, float *part, _Float16 *qrot,
+                                  _Float16 *out, hipStream_t s) {
+  if (hd != 128) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "attention kernel is built for head_dim 128, got %d", hd);
+  if (hq % hkv != 0 || hq / hkv > 4)
+    return set_error(YSCV_HIP_ERR_UNSUPPORTED, "attention kernel handles 1..4 query heads per kv head");
+  const size_t lds = (size_t)hkv * hd * sizeof(float);
+  if (lds > 32 * 1024) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "int8 cache append: too many kv heads (%d)", hkv);
+  const int max_chunks = max_ctx / ATT_CHUNK;
+  const float scale = 1.0f / sqrtf((float)hd);
+  hipLaunchKernelGGL(attn_fused_i8_kernel, dim3(max_chunks, hkv, batch), dim3(256), lds, s, qkv, kc, ks, vc, vs, pos_ptr, hq, hkv,
+                     max_ctx, max_chunks, scale, theta, part, qrot);
   YSCV_HIP_TRY(hipGetLastError());
   hipLaunchKernelGGL(attn_combine_kernel, dim3(hq, batch), dim3(128), 0, s, part, pos_ptr, hq, max_chunks, out);
   YSCV_HIP_TRY(hipGetLastError());
