@@ -420,11 +420,15 @@ static int32_t finish_setup(yscv_hip_decoder *d) {
     const Context *ctx = nullptr;
     YSCV_TRY(ensure_context(&ctx));
     // (a consuming projection adds up at most 256 partial sums per row, four rows per wave of 512 k)
-    bool ok = d->cfg.d_model % 256 == 0 && d->cfg.d_model <= 4096 && d->fold_norm_wanted &&
-              d->cfg.max_batch <= 4 * ((d->cfg.d_model + 511) / 512);
+    bool ok = d->cfg.d_model % 256 == 0 && d->cfg.d_model <= 4096 && d->fold_norm_wanted;
+    auto consumes = [&](const yscv_hip_int4_weight *w) {
+      if (!w->tiled) return false;
+      const SkinnyPlan plan = plan_int4_skinny(w, d->cfg.max_batch, 1, ctx->num_cus);
+      return plan.ksg == 1 && d->cfg.max_batch <= 4 * plan.waves;
+    };
     for (auto &L : d->layers)
-      for (auto *w : {L.wqkv, L.wgu}) ok = ok && w->tiled && plan_int4_skinny(w, d->cfg.max_batch, 1, ctx->num_cus).ksg == 1;
-    ok = ok && d->lm_head->tiled && plan_int4_skinny(d->lm_head, d->cfg.max_batch, 1, ctx->num_cus).ksg == 1;
+      for (auto *w : {L.wqkv, L.wgu}) ok = ok && consumes(w);
+    ok = ok && consumes(d->lm_head);
     for (auto &L : d->layers) ok = ok && L.wo->tiled && L.wdown->tiled;
     // every projection takes its fp16 activations as they are (no padded copy with a row scale of its own)
     auto direct = [](const yscv_hip_int4_weight *w) { return w->ktp * 128 == w->k; };
