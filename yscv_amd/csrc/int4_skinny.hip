@@ -421,11 +421,11 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
       }
     }
   }
-  // Folded RMSNorm, consumer side: the row factors 1 / (pre * sqrt(sum(h^2) / d + eps)) come from the partial sums the
-  // kernel that wrote the residual left behind and from the power of two it scaled the row with.  Row q is added up by wave q % waves (four consecutive partials per
-  // lane, requested further up together with the activations, then a fixed tree of DPP moves and lane swaps: the
-  // same order in every run); the sixteen factors meet in LDS behind the barrier of the first reduction, which every
-  // use of them follows.
+  // Folded RMSNorm, consumer side: the row factors 1 / (pre * sqrt(sum(h^2) / d + eps)) come from the partial sums
+  // the kernel that wrote the residual left behind and from the power of two it scaled the row with.  Row q is added
+  // up by wave q % waves (four consecutive partials per lane, requested further up together with the activations,
+  // then a fixed tree of DPP moves and lane swaps: the same order in every run); the sixteen factors meet in LDS
+  // behind the barrier of the first reduction, which every use of them follows.
   float *rs_lds = red + (size_t)2 * waves * (UB * NI) * 64;
   if (a.ss_in) {
 #pragma unroll
@@ -605,7 +605,8 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
         if (a.ss_in) rsv = rs_lds[min(mrow, a.m - 1)];
         v *= rsv;
         if (a.epi == EPI_ADD_F32 && a.xg) {
-          // residual update that also feeds the next norm: h_new, its fp16 image times gamma and the row's power of two, and the sum of
+          // residual update that also feeds the next norm: h_new, its fp16 image times gamma and the row's power of
+          // two, and the sum of
           // h_new^2 over the sixteen columns of this block (the lanes r = 0..15 of a lane group), one per row
           float hn = 0.0f;
           if (live) {
