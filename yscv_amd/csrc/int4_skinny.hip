@@ -606,8 +606,8 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
         v *= rsv;
         if (a.epi == EPI_ADD_F32 && a.xg) {
           // residual update that also feeds the next norm: h_new, its fp16 image times gamma and the row's power of
-          // two, and the sum of
-          // h_new^2 over the sixteen columns of this block (the lanes r = 0..15 of a lane group), one per row
+          // two, and the sum of h_new^2 over the sixteen columns of this block (the lanes r = 0..15 of a lane group),
+          // one per row
           float hn = 0.0f;
           if (live) {
             float *hp = reinterpret_cast<float *>(a.y) + (size_t)mrow * a.n + col;
