@@ -505,7 +505,9 @@ __global__ void __launch_bounds__(256) attn_fused_kernel(const _Float16 *__restr
   __shared__ __attribute__((aligned(16))) _Float16 p_lds[ATT_WAVES][4][32];
   __shared__ float w_m[ATT_WAVES][4], w_l[ATT_WAVES][4];
   __shared__ float w_o[ATT_WAVES][4][HD];
-  const int chunk = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  // chunk index slowest: the workgroups of the last, partly filled chunk (a quarter of the loads or less) are the
+  // ones that run while the grid drains
+  const int kvh = blockIdx.x, b = blockIdx.y, chunk = blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, c = lane >> 4;
   const int group = hq / hkv;
@@ -880,7 +882,9 @@ __global__ void __launch_bounds__(256) attn_fused_i8_kernel(const _Float16 *__re
   __shared__ __attribute__((aligned(16))) _Float16 p_lds[ATT_WAVES][4][32];
   __shared__ float w_m[ATT_WAVES][4], w_l[ATT_WAVES][4];
   __shared__ float w_o[ATT_WAVES][4][HD];
-  const int chunk = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  // chunk index slowest: the workgroups of the last, partly filled chunk (a quarter of the loads or less) are the
+  // ones that run while the grid drains
+  const int kvh = blockIdx.x, b = blockIdx.y, chunk = blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, c = lane >> 4;
   const int group = hq / hkv;
@@ -1206,7 +1210,7 @@ int32_t launch_attention_fused(const _Float16 *qkv, _Float16 *kc, _Float16 *vc, 
     return set_error(YSCV_HIP_ERR_UNSUPPORTED, "attention kernel handles 1..4 query heads per kv head");
   const int max_chunks = max_ctx / ATT_CHUNK;
   const float scale = 1.0f / sqrtf((float)hd);
-  hipLaunchKernelGGL(attn_fused_kernel, dim3(max_chunks, hkv, batch), dim3(256), 0, s, qkv, kc, vc, pos_ptr, hq, hkv, max_ctx,
+  hipLaunchKernelGGL(attn_fused_kernel, dim3(hkv, batch, max_chunks), dim3(256), 0, s, qkv, kc, vc, pos_ptr, hq, hkv, max_ctx,
                      max_chunks, scale, theta, part, qrot);
   YSCV_HIP_TRY(hipGetLastError());
   hipLaunchKernelGGL(attn_combine_kernel, dim3(hq, batch), dim3(128), 0, s, part, pos_ptr, hq, max_chunks, out);
@@ -1240,7 +1244,7 @@ int32_t launch_attention_fused_i8(const _Float16 *qkv, int8_t *kc, float *ks, in
   if (lds > 32 * 1024) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "int8 cache append: too many kv heads (%d)", hkv);
   const int max_chunks = max_ctx / ATT_CHUNK;
   const float scale = 1.0f / sqrtf((float)hd);
-  hipLaunchKernelGGL(attn_fused_i8_kernel, dim3(max_chunks, hkv, batch), dim3(256), lds, s, qkv, kc, ks, vc, vs, pos_ptr, hq, hkv,
+  hipLaunchKernelGGL(attn_fused_i8_kernel, dim3(hkv, batch, max_chunks), dim3(256), lds, s, qkv, kc, ks, vc, vs, pos_ptr, hq, hkv,
                      max_ctx, max_chunks, scale, theta, part, qrot);
   YSCV_HIP_TRY(hipGetLastError());
   hipLaunchKernelGGL(attn_combine_kernel, dim3(hq, batch), dim3(128), 0, s, part, pos_ptr, hq, max_chunks, out);
