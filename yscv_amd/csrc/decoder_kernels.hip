@@ -249,13 +249,27 @@ constexpr int ATT_CHUNK = ATT_WAVES * ATT_POS_PER_WAVE;  // 128 positions per wo
 
 // KV8: the cache holds int8 rows with one f32 scale per (batch row, position) for K and for V (KvCache with
 // KvDtype::I8, crates/yscv-onnx/src/runner/kv_cache.rs:45-79: values read back as q * scale).  int8 values are exact in
-// fp16, so the K scale multiplies the finished score and the V scale is folded into the fp16 operand.
-__device__ __forceinline__ half8_t i8x8_to_half8(const int8_t *p, const float *sc8) {
-  typedef int8_t char8_t __attribute__((ext_vector_type(8)));
-  const char8_t v = *reinterpret_cast<const char8_t *>(p);
+// fp16, so both operands carry the bare int8 values: the K scale multiplies the finished score, the V scale the
+// softmax weight of its position before that is rounded to fp16 (one rounding per product, where scaling V itself
+// would round twice).  Eight bytes -> eight fp16 values: b ^ 0x80 is b + 128 as an unsigned byte u, the fp16 with bits
+// 0x6400 | u is 1024 + u, and subtracting 1152 leaves b (two byte permutes and two packed adds per four values).
+typedef int int2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ half8_t i8x8_to_half8(int2_t raw) {
+  const half2_t bias = {(_Float16)(-1152.0f), (_Float16)(-1152.0f)};
   half8_t h;
 #pragma unroll
-  for (int e = 0; e < 8; e++) h[e] = sc8 ? (_Float16)((float)v[e] * sc8[e]) : (_Float16)(float)v[e];
+  for (int w = 0; w < 2; w++) {
+    const uint32_t x = (uint32_t)raw[w] ^ 0x80808080u;
+    // v_perm_b32: result byte i = byte sel[i] of {0x64646464 (bytes 4..7), x (bytes 0..3)}
+    const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u);
+    const uint32_t hi = __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u);
+    const half2_t a = __builtin_bit_cast(half2_t, lo) + bias;
+    const half2_t c = __builtin_bit_cast(half2_t, hi) + bias;
+    h[4 * w + 0] = a[0];
+    h[4 * w + 1] = a[1];
+    h[4 * w + 2] = c[0];
+    h[4 * w + 3] = c[1];
+  }
   return h;
 }
 
@@ -302,21 +316,27 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const _Float16 *__res
     const size_t v_off = ((((size_t)b * hkv + kvh) * (max_ctx / 8) + p0 / 8) * HD) * 8;
     // issue every load of this wave up front: 8 KiB of K, 8 KiB of V (half of that from an int8 cache)
     half8_t kf[2][4], vf[8];
-    float k_scale[2] = {1.0f, 1.0f};
+    float k_scale[2] = {1.0f, 1.0f}, v_scale[2] = {1.0f, 1.0f};  // of position p0 + 16 pb + r
     if constexpr (KV8) {
       const int8_t *kbase = static_cast<const int8_t *>(kc_v) + k_off;
       const int8_t *vbase = static_cast<const int8_t *>(vc_v) + v_off;
-      float v_scale[8];
-#pragma unroll
-      for (int e = 0; e < 8; e++) v_scale[e] = vs[(size_t)b * max_ctx + p0 + 8 * c + e];
+      int2_t kraw[2][4], vraw[8];
 #pragma unroll
       for (int pb = 0; pb < 2; pb++) {
         k_scale[pb] = ks[(size_t)b * max_ctx + p0 + pb * 16 + r];
+        v_scale[pb] = vs[(size_t)b * max_ctx + p0 + pb * 16 + r];
 #pragma unroll
-        for (int j = 0; j < 4; j++) kf[pb][j] = i8x8_to_half8(kbase + (size_t)(pb * 16 + r) * HD + 32 * c + 8 * j, nullptr);
+        for (int j = 0; j < 4; j++)
+          kraw[pb][j] = *reinterpret_cast<const int2_t *>(kbase + (size_t)(pb * 16 + r) * HD + 32 * c + 8 * j);
       }
 #pragma unroll
-      for (int t = 0; t < 8; t++) vf[t] = i8x8_to_half8(vbase + ((size_t)c * HD + t * 16 + r) * 8, v_scale);
+      for (int t = 0; t < 8; t++) vraw[t] = *reinterpret_cast<const int2_t *>(vbase + ((size_t)c * HD + t * 16 + r) * 8);
+#pragma unroll
+      for (int pb = 0; pb < 2; pb++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) kf[pb][j] = i8x8_to_half8(kraw[pb][j]);
+#pragma unroll
+      for (int t = 0; t < 8; t++) vf[t] = i8x8_to_half8(vraw[t]);
     } else {
       const _Float16 *kbase = static_cast<const _Float16 *>(kc_v) + k_off;
       const _Float16 *vbase = static_cast<const _Float16 *>(vc_v) + v_off;
@@ -351,8 +371,9 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const _Float16 *__res
     m_h = mx;
     l_h = sum;
     if (c < 4) {
-      p_lds[wave][c][r] = (_Float16)e0;
-      p_lds[wave][c][16 + r] = (_Float16)e1;
+      // int8 cache: the V scale of the position rides on its weight (a dead position has weight 0 whatever its scale)
+      p_lds[wave][c][r] = KV8 ? (e0 == 0.0f ? (_Float16)0.0f : (_Float16)(e0 * v_scale[0])) : (_Float16)e0;
+      p_lds[wave][c][16 + r] = KV8 ? (e1 == 0.0f ? (_Float16)0.0f : (_Float16)(e1 * v_scale[1])) : (_Float16)e1;
     }
     __builtin_amdgcn_wave_barrier();  // LDS is in order per wave: the reads below see the writes above
     // P operand: MFMA row 4*h = head h, lane (r, c) holds positions 8c .. 8c+7 of this wave's 32
@@ -874,11 +895,10 @@ __global__ void __launch_bounds__(256) attn_fused_i8_kernel(const _Float16 *__re
                                                             int max_ctx, int max_chunks, float scale, float theta,
                                                             float *__restrict__ part, _Float16 *__restrict__ qrot) {
   constexpr int HD = 128;
-  typedef int8_t char8_t __attribute__((ext_vector_type(8)));
   extern __shared__ float krow_lds[];  // owner only: the rotated k row of every kv head, f32
   __shared__ __attribute__((aligned(16))) _Float16 q_lds[4][HD];
-  __shared__ __attribute__((aligned(16))) _Float16 knew[HD], vnew[HD];  // k as its int8 value, v as q * scale
-  __shared__ float red[4], new_k_scale;
+  __shared__ __attribute__((aligned(16))) _Float16 knew[HD], vnew[HD];  // the appended int8 values, as fp16
+  __shared__ float red[4], new_k_scale, new_v_scale;
   __shared__ __attribute__((aligned(16))) _Float16 p_lds[ATT_WAVES][4][32];
   __shared__ float w_m[ATT_WAVES][4], w_l[ATT_WAVES][4];
   __shared__ float w_o[ATT_WAVES][4][HD];
@@ -900,20 +920,19 @@ __global__ void __launch_bounds__(256) attn_fused_i8_kernel(const _Float16 *__re
   // ---- K / V bytes and scales of this wave's 32 positions: requested before anything else, converted further down ----
   const size_t k_off = (((size_t)b * hkv + kvh) * max_ctx + p0) * HD;
   const size_t v_off = ((((size_t)b * hkv + kvh) * (max_ctx / 8) + p0 / 8) * HD) * 8;
-  char8_t kraw[2][4], vraw[8];
-  float k_scale[2] = {1.0f, 1.0f}, v_scale[8];
+  int2_t kraw[2][4], vraw[8];
+  float k_scale[2] = {1.0f, 1.0f}, v_scale[2] = {1.0f, 1.0f};  // of position p0 + 16 pb + r
   if (wave_live) {
-#pragma unroll
-    for (int e = 0; e < 8; e++) v_scale[e] = vs[(size_t)b * max_ctx + p0 + 8 * c + e];
 #pragma unroll
     for (int pb = 0; pb < 2; pb++) {
       k_scale[pb] = ks[(size_t)b * max_ctx + p0 + pb * 16 + r];
+      v_scale[pb] = vs[(size_t)b * max_ctx + p0 + pb * 16 + r];
 #pragma unroll
       for (int j = 0; j < 4; j++)
-        kraw[pb][j] = *reinterpret_cast<const char8_t *>(kc + k_off + (size_t)(pb * 16 + r) * HD + 32 * c + 8 * j);
+        kraw[pb][j] = *reinterpret_cast<const int2_t *>(kc + k_off + (size_t)(pb * 16 + r) * HD + 32 * c + 8 * j);
     }
 #pragma unroll
-    for (int t = 0; t < 8; t++) vraw[t] = *reinterpret_cast<const char8_t *>(vc + v_off + ((size_t)c * HD + t * 16 + r) * 8);
+    for (int t = 0; t < 8; t++) vraw[t] = *reinterpret_cast<const int2_t *>(vc + v_off + ((size_t)c * HD + t * 16 + r) * 8);
   }
 
   // ---- rotary embedding of the query heads; the owners also rotate k, find the row scales and append ----
@@ -956,6 +975,7 @@ __global__ void __launch_bounds__(256) attn_fused_i8_kernel(const _Float16 *__re
         ks[(size_t)b * max_ctx + pos] = ksc;
         vs[(size_t)b * max_ctx + pos] = vsc;
         new_k_scale = ksc;
+        new_v_scale = vsc;
       }
       if (tid < HD) {
         const int8_t q8 = kv_quant_one(krow_lds[kvh * HD + tid], kinv);
@@ -965,7 +985,7 @@ __global__ void __launch_bounds__(256) attn_fused_i8_kernel(const _Float16 *__re
         const int dd = tid - HD;
         const int8_t q8 = kv_quant_one((float)row[(size_t)(hq + hkv + kvh) * HD + dd], vinv);
         vc[((((size_t)b * hkv + kvh) * (max_ctx / 8) + pos / 8) * HD + dd) * 8 + (pos & 7)] = q8;
-        vnew[dd] = (_Float16)((float)q8 * vsc);
+        vnew[dd] = (_Float16)(float)q8;
       }
     }
   }
@@ -985,15 +1005,13 @@ __global__ void __launch_bounds__(256) attn_fused_i8_kernel(const _Float16 *__re
 #pragma unroll
       for (int j = 0; j < 4; j++) qa[j] = valid ? *reinterpret_cast<const half8_t *>(&q_lds[h & 3][32 * c + 8 * j]) : z;
     }
-    // int8 values are exact in fp16: the K scale multiplies the finished score, the V scale goes into the operand
+    // int8 values are exact in fp16: the K scale multiplies the finished score, the V scale the softmax weight
     // (V is converted after the scores, so that the bytes and the fp16 values of both are never live together)
     half8_t kf[2][4];
 #pragma unroll
     for (int pb = 0; pb < 2; pb++)
 #pragma unroll
-      for (int j = 0; j < 4; j++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) kf[pb][j][e] = (_Float16)(float)kraw[pb][j][e];
+      for (int j = 0; j < 4; j++) kf[pb][j] = i8x8_to_half8(kraw[pb][j]);
     // the row appended in this launch: the loads above read whatever the cache held before
     const int rel = pos - p0;
     const bool patch = owner && rel >= 0 && rel < ATT_POS_PER_WAVE;
@@ -1002,6 +1020,7 @@ __global__ void __launch_bounds__(256) attn_fused_i8_kernel(const _Float16 *__re
       for (int pb = 0; pb < 2; pb++)
         if (rel == pb * 16 + r) {
           k_scale[pb] = new_k_scale;
+          v_scale[pb] = new_v_scale;
 #pragma unroll
           for (int j = 0; j < 4; j++) kf[pb][j] = *reinterpret_cast<const half8_t *>(&knew[32 * c + 8 * j]);
         }
@@ -1026,16 +1045,14 @@ __global__ void __launch_bounds__(256) attn_fused_i8_kernel(const _Float16 *__re
     for (int off = 8; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
     m_h = mx;
     l_h = sum;
-    if (c < 4) {
-      p_lds[wave][c][r] = (_Float16)e0;
-      p_lds[wave][c][16 + r] = (_Float16)e1;
+    if (c < 4) {  // the V scale of the position rides on its weight (a dead position has weight 0 whatever its scale)
+      p_lds[wave][c][r] = e0 == 0.0f ? (_Float16)0.0f : (_Float16)(e0 * v_scale[0]);
+      p_lds[wave][c][16 + r] = e1 == 0.0f ? (_Float16)0.0f : (_Float16)(e1 * v_scale[1]);
     }
     __builtin_amdgcn_wave_barrier();
     half8_t vf[8];
 #pragma unroll
-    for (int t = 0; t < 8; t++)
-#pragma unroll
-      for (int e = 0; e < 8; e++) vf[t][e] = (_Float16)((float)vraw[t][e] * v_scale[e]);
+    for (int t = 0; t < 8; t++) vf[t] = i8x8_to_half8(vraw[t]);
     if (patch) {
       const int e_new = rel - 8 * c;
       if (e_new >= 0 && e_new < 8) {
