@@ -360,14 +360,10 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const _Float16 *__res
       const int p = p0 + pb * 16 + r;
       s[pb] = (p < n_ctx) ? d[0] * scale * k_scale[pb] : -INFINITY;
     }
-    float mx = fmaxf(s[0], s[1]);
-#pragma unroll
-    for (int off = 8; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));  // within the 16 lanes of a group
+    const float mx = row_max16(fmaxf(s[0], s[1]));  // over the 16 lanes of a group: DPP moves, no LDS round trips
     const float e0 = (s[0] == -INFINITY) ? 0.0f : __expf(s[0] - mx);
     const float e1 = (s[1] == -INFINITY) ? 0.0f : __expf(s[1] - mx);
-    float sum = e0 + e1;
-#pragma unroll
-    for (int off = 8; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    const float sum = row_sum16(e0 + e1);
     m_h = mx;
     l_h = sum;
     if (c < 4) {
@@ -645,14 +641,10 @@ __global__ void __launch_bounds__(256) attn_fused_kernel(const _Float16 *__restr
       const int p = p0 + pb * 16 + r;
       s[pb] = (p < n_ctx) ? d[0] * scale : -INFINITY;
     }
-    float mx = fmaxf(s[0], s[1]);
-#pragma unroll
-    for (int off = 8; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    const float mx = row_max16(fmaxf(s[0], s[1]));  // over the 16 lanes of a group: DPP moves, no LDS round trips
     const float e0 = (s[0] == -INFINITY) ? 0.0f : __expf(s[0] - mx);
     const float e1 = (s[1] == -INFINITY) ? 0.0f : __expf(s[1] - mx);
-    float sum = e0 + e1;
-#pragma unroll
-    for (int off = 8; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    const float sum = row_sum16(e0 + e1);
     m_h = mx;
     l_h = sum;
     if (c < 4) {
@@ -1035,14 +1027,10 @@ __global__ void __launch_bounds__(256) attn_fused_i8_kernel(const _Float16 *__re
       const int p = p0 + pb * 16 + r;
       s[pb] = (p < n_ctx) ? d[0] * scale * k_scale[pb] : -INFINITY;
     }
-    float mx = fmaxf(s[0], s[1]);
-#pragma unroll
-    for (int off = 8; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    const float mx = row_max16(fmaxf(s[0], s[1]));  // over the 16 lanes of a group: DPP moves, no LDS round trips
     const float e0 = (s[0] == -INFINITY) ? 0.0f : __expf(s[0] - mx);
     const float e1 = (s[1] == -INFINITY) ? 0.0f : __expf(s[1] - mx);
-    float sum = e0 + e1;
-#pragma unroll
-    for (int off = 8; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    const float sum = row_sum16(e0 + e1);
     m_h = mx;
     l_h = sum;
     if (c < 4) {  // the V scale of the position rides on its weight (a dead position has weight 0 whatever its scale)
