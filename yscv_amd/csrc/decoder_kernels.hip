@@ -450,14 +450,14 @@ __global__ void __launch_bounds__(128) attn_combine_kernel(const float *__restri
       pl = src[(size_t)tid * (HD + 2) + 1];
     }
     float mx = pm;
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    mx = wave_max(mx);
     if ((tid & 63) == 0) red_m[tid >> 6] = mx;
     __syncthreads();
     mx = fmaxf(red_m[0], red_m[1]);
     const float f = (pm == -INFINITY) ? 0.0f : __expf(pm - mx);
     if (tid < chunks) wgt[tid] = f;
     float l = pl * f;
-    for (int off = 32; off > 0; off >>= 1) l += __shfl_xor(l, off, 64);
+    l = wave_sum(l);
     if ((tid & 63) == 0) red_l[tid >> 6] = l;
     __syncthreads();
     l = red_l[0] + red_l[1];
@@ -472,7 +472,7 @@ __global__ void __launch_bounds__(128) attn_combine_kernel(const float *__restri
   // maximum over all chunks
   float mx = -INFINITY;
   for (int ch = tid; ch < chunks; ch += 128) mx = fmaxf(mx, src[(size_t)ch * (HD + 2)]);
-  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+  mx = wave_max(mx);
   if ((tid & 63) == 0) red_m[tid >> 6] = mx;
   __syncthreads();
   mx = fmaxf(red_m[0], red_m[1]);
@@ -484,7 +484,7 @@ __global__ void __launch_bounds__(128) attn_combine_kernel(const float *__restri
     if (ch < CAP) wgt[ch] = f;
     l += p[1] * f;
   }
-  for (int off = 32; off > 0; off >>= 1) l += __shfl_xor(l, off, 64);
+  l = wave_sum(l);
   if ((tid & 63) == 0) red_l[tid >> 6] = l;
   __syncthreads();
   l = red_l[0] + red_l[1];
