@@ -444,27 +444,21 @@ __global__ void __launch_bounds__(128) attn_combine_kernel(const float *__restri
     float po[FAST];
 #pragma unroll
     for (int ch = 0; ch < FAST; ch++) po[ch] = src[(size_t)(ch < chunks ? ch : chunks - 1) * (HD + 2) + 2 + tid];
+    // both waves fetch the (maximum, sum) pairs of all chunks, one chunk per lane: each wave then has the merge
+    // statistics without LDS or a barrier, and a chunk's weight reaches every lane as a scalar read of its lane
+    const int ln = tid & 63;
     float pm = -INFINITY, pl = 0.0f;
-    if (tid < chunks) {
-      pm = src[(size_t)tid * (HD + 2)];
-      pl = src[(size_t)tid * (HD + 2) + 1];
+    if (ln < chunks) {
+      pm = src[(size_t)ln * (HD + 2)];
+      pl = src[(size_t)ln * (HD + 2) + 1];
     }
-    float mx = pm;
-    mx = wave_max(mx);
-    if ((tid & 63) == 0) red_m[tid >> 6] = mx;
-    __syncthreads();
-    mx = fmaxf(red_m[0], red_m[1]);
+    const float mx = wave_max(pm);
     const float f = (pm == -INFINITY) ? 0.0f : __expf(pm - mx);
-    if (tid < chunks) wgt[tid] = f;
-    float l = pl * f;
-    l = wave_sum(l);
-    if ((tid & 63) == 0) red_l[tid >> 6] = l;
-    __syncthreads();
-    l = red_l[0] + red_l[1];
+    const float l = wave_sum(pl * f);
     float o = 0.0f;
 #pragma unroll
     for (int ch = 0; ch < FAST; ch++)
-      if (ch < chunks) o += po[ch] * wgt[ch];
+      if (ch < chunks) o += po[ch] * __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), ch));
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
     out[((size_t)b * hq + head) * HD + tid] = (_Float16)(o * inv);
     return;
