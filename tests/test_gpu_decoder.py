@@ -87,6 +87,48 @@ def test_decode_steps_match_numpy(use_graph):
 
 
 @pytest.mark.parametrize("kv_dtype", ["f16", "i8"])
+def test_long_context_matches_numpy(kv_dtype):
+    """4 230 cached positions = 34 chunks of 128: more than the chunk merge takes in its one-pass form (32), so the
+    general merge runs, against the checker; the attention output of the last layer is also held to a float64 softmax
+    over the cache rows the GPU holds."""
+    import math
+
+    rng = np.random.default_rng(4300)
+    cfg = dict(CFG, max_ctx=4352, max_batch=2)
+    dec, ref = _build(rng, cfg, kv_dtype=kv_dtype, symmetric=True)
+    B, prefill = 2, 4230
+    for l in range(cfg["n_layers"]):
+        k = rng.standard_normal((B, prefill, cfg["n_kv_heads"], cfg["head_dim"])).astype(np.float16)
+        v = rng.standard_normal((B, prefill, cfg["n_kv_heads"], cfg["head_dim"])).astype(np.float16)
+        dec.set_kv(l, k, v)
+        ref.set_kv(l, k.astype(np.float32), v.astype(np.float32))
+    tokens = np.array([7, 201], np.int32)
+    dec.reset(tokens, prefill)
+    cur = tokens.copy()
+    nh, nkv, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    for step in range(2):
+        dec.run(1, use_graph=bool(step))
+        got_logits, got_tok = dec.logits(), dec.tokens(step, 1)[0]
+        exp_logits = ref.step(cur, prefill + step)
+        err = np.abs(got_logits - exp_logits).max() / np.abs(exp_logits).max()
+        assert err < 2e-2, (step, err)
+        # the last layer's attention from the GPU's own rotated q against the checker's cache of that layer (which
+        # holds what the int8 mode reads back), in float64
+        qkv, ao = dec.activation("qkv"), dec.activation("attn_out")
+        L = cfg["n_layers"] - 1
+        for b in range(B):
+            q = qkv[b][: nh * hd].reshape(nh, hd).astype(np.float64)
+            kc, vc = ref.kc[L][b].astype(np.float64), ref.vc[L][b].astype(np.float64)
+            for h in range(nh):
+                sc = kc[:, h // (nh // nkv), :] @ q[h] / math.sqrt(hd)
+                pr = np.exp(sc - sc.max())
+                want = (pr / pr.sum()) @ vc[:, h // (nh // nkv), :]
+                got = ao[b].reshape(nh, hd)[h]
+                assert np.abs(got - want).max() <= 1e-2 * np.abs(want).max() + 1e-3, (step, b, h)
+        cur = got_tok.copy()
+
+
+@pytest.mark.parametrize("kv_dtype", ["f16", "i8"])
 @pytest.mark.parametrize("prefill", [5, 127, 128, 133, 250])
 def test_fused_attention_equals_the_separate_rope_append(prefill, kv_dtype):
     """Rotary embedding and cache append inside the attention kernel against the separate rope_append launch in front
