@@ -330,6 +330,29 @@ def _prefill(rng, dec, ref, cfg, B, prefill):
             ref.set_kv(l, k.astype(np.float32), v.astype(np.float32))
 
 
+def test_persistent_decode_at_34_context_chunks():
+    """The single-launch kernel over 4 230 cached positions (each workgroup takes several attention items and several
+    merge heads): against the checker, and against the multi-kernel path from the same state."""
+    rng = np.random.default_rng(4400)
+    cfg = dict(PCFG, max_ctx=4352)
+    dec, ref = _build(rng, cfg, symmetric=True)
+    prefill = 4230
+    _prefill(rng, dec, ref, cfg, 1, prefill)
+    tokens = np.array([7], np.int32)
+    cur = tokens.copy()
+    for step in range(2):
+        dec.reset(cur, prefill + step)
+        dec.run(1, use_graph=True)
+        graph_logits = dec.logits()[0].copy()
+        dec.reset(cur, prefill + step)
+        dec.run(1, persistent=True)
+        got, tok = dec.logits()[0].copy(), dec.tokens(0, 1)[0]
+        exp = ref.step(cur, prefill + step)[0]
+        assert np.abs(got - exp).max() / np.abs(exp).max() < 2e-2, step
+        assert np.abs(got - graph_logits).max() / np.abs(graph_logits).max() < 5e-3, step
+        cur = tok.copy()
+
+
 @pytest.mark.parametrize("prefill", [0, 133, 300])
 def test_persistent_decode_matches_numpy_and_graph_path(prefill):
     import torch
