@@ -87,6 +87,31 @@ def test_decode_steps_match_numpy(use_graph):
 
 
 @pytest.mark.parametrize("kv_dtype", ["f16", "i8"])
+@pytest.mark.parametrize("heads", [(3, 3), (6, 2), (4, 1)], ids=["group1", "group3", "group4"])
+def test_query_heads_per_kv_head(heads, kv_dtype):
+    """1, 3 and 4 query heads per kv head (kv_h = q_h / groups, runner/linear.rs:552-646): the other tests here run 2."""
+    rng = np.random.default_rng(4500 + 10 * heads[0] + heads[1])
+    cfg = dict(CFG, n_heads=heads[0], n_kv_heads=heads[1])
+    dec, ref = _build(rng, cfg, kv_dtype=kv_dtype, symmetric=True)
+    B, prefill = 3, 141
+    for l in range(cfg["n_layers"]):
+        k = rng.standard_normal((B, prefill, cfg["n_kv_heads"], cfg["head_dim"])).astype(np.float16)
+        v = rng.standard_normal((B, prefill, cfg["n_kv_heads"], cfg["head_dim"])).astype(np.float16)
+        dec.set_kv(l, k, v)
+        ref.set_kv(l, k.astype(np.float32), v.astype(np.float32))
+    tokens = np.array([5, 17, 300], np.int32)
+    dec.reset(tokens, prefill)
+    cur = tokens.copy()
+    for step in range(3):
+        dec.run(1, use_graph=bool(step & 1))
+        got_logits, got_tok = dec.logits(), dec.tokens(step, 1)[0]
+        exp_logits = ref.step(cur, prefill + step)
+        err = np.abs(got_logits - exp_logits).max() / np.abs(exp_logits).max()
+        assert err < 2e-2, (step, err)
+        cur = got_tok.copy()
+
+
+@pytest.mark.parametrize("kv_dtype", ["f16", "i8"])
 def test_long_context_matches_numpy(kv_dtype):
     """4 230 cached positions = 34 chunks of 128: more than the chunk merge takes in its one-pass form (32), so the
     general merge runs, against the checker; the attention output of the last layer is also held to a float64 softmax
