@@ -218,14 +218,14 @@ __device__ __forceinline__ float row_max16(float v) {
   return v;
 }
 __device__ __forceinline__ float wave_sum(float v) { return sum_xor16_xor32(row_sum16(v)); }
-__device__ __forceinline__ float wave_max(float v) {
+__device__ __forceinline__ float max_xor16_xor32(float v) {  // max(v, v[lane ^ 16]), then the same over lane ^ 32
   float x, y;
-  v = row_max16(v);
   xor16_pair(v, x, y);
   v = fmaxf(x, y);
   xor32_pair(v, x, y);
   return fmaxf(x, y);
 }
+__device__ __forceinline__ float wave_max(float v) { return max_xor16_xor32(row_max16(v)); }
 
 // The power of two at or below 1 / (4 rms), rms = 1 / inv_rms, kept within 2^-40 .. 2^40 (NormFold, kernels.hpp)
 __device__ __forceinline__ float norm_fold_prescale(float inv_rms) {

@@ -264,8 +264,7 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
             amax_bits = max(amax_bits, max(lo, hi));
           }
       float amax = valid ? __uint_as_float(amax_bits << 16) : 0.0f;
-      amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-      amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+      amax = max_xor16_xor32(amax);
       int e2 = 14;
       if (amax > 0.0f && amax < 3.0e38f) {
         (void)frexpf(amax, &e2);
@@ -309,10 +308,7 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
 #pragma unroll
         for (int u = 0; u < 4; u++) amax = fmaxf(amax, fabsf(raw[e][u]));
       if (!svalid) amax = 0.0f;
-      amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-      amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-      amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
-      amax = fmaxf(amax, __shfl_xor(amax, 8, 64));
+      amax = row_max16(amax);
       int e2 = 14;
       if (amax > 0.0f && amax < 3.0e38f) {
         (void)frexpf(amax, &e2);
@@ -368,8 +364,7 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
           for (int e = 0; e < 4; e++) amax = fmaxf(amax, fmaxf(fabsf(v0[e]), fabsf(v1[e])));
         }
       if (!valid) amax = 0.0f;
-      amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-      amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+      amax = max_xor16_xor32(amax);
       int e2 = 14;
       if (amax > 0.0f && amax < 3.0e38f) {
         (void)frexpf(amax, &e2);
@@ -626,7 +621,7 @@ __global__ void __launch_bounds__(512, 1) int4_skinny_kernel(SkinnyArgs a) {
         }
         if (a.epi == EPI_SWIGLU) {
           // rows 2i / 2i+1 of the weight are gate_i / up_i: neighbours in the wave
-          const float up = __shfl_xor(v, 1, 64);
+          const float up = dpp_move<DPP_XOR1>(v);
           if (live && !(r & 1))
             store_out(a.y, (size_t)mrow * (a.n >> 1) + (col >> 1), silu(v) * up, a.y_dtype);
         } else if (a.epi == EPI_ADD_F32) {
