@@ -582,6 +582,13 @@ def main():
                                        "ms_per_step": round(dt16 / min(args.steps, 64) * 1e3, 4),
                                        "path": "one HIP-graph replay per step",
                                        "skinny_kernel_GB/s": round(w_bytes / n_proj / avg16 / 1e9, 1)}
+            # the batches between the two the metric names, same path (fp16 cache, one graph replay per step)
+            sweep = {}
+            for bsz in (2, 4, 8):
+                dtb, _ = bench_decode(dec, torch, bsz, min(args.steps, 64), 4, stream_ptr)
+                sweep[f"batch{bsz}"] = {"tok/s": round(bsz * min(args.steps, 64) / dtb, 1),
+                                        "ms_per_step": round(dtb / min(args.steps, 64) * 1e3, 4)}
+            extra["decode_batch_sweep"] = sweep
     del dec
     torch.cuda.empty_cache()
     if not args.no_extra and args.batch != 16:
