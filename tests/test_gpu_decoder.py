@@ -111,6 +111,40 @@ def test_query_heads_per_kv_head(heads, kv_dtype):
         cur = got_tok.copy()
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_model_shapes_match_numpy(seed):
+    """Seeded random shapes (widths that fold the norms and widths that do not, 1..4 kv heads with 1..4 query heads each,
+    K-split and unsplit projections, 1..8 sequences, either cache type, any prefill) against the checker, eager and
+    replayed."""
+    rng = np.random.default_rng(4600 + seed)
+    n_kv = int(rng.integers(1, 5))
+    group = int(rng.integers(1, 5))
+    B = int(rng.integers(1, 9))
+    cfg = dict(CFG, d_model=int(rng.choice([256, 384, 512, 768, 1024, 1536])), n_heads=n_kv * group, n_kv_heads=n_kv,
+               d_ff=int(rng.choice([256, 384, 512, 1024, 2048, 4608])), vocab=int(rng.choice([320, 512, 1000])),
+               max_batch=B, max_ctx=384)
+    kv_dtype = "i8" if rng.integers(0, 2) else "f16"
+    prefill = int(rng.integers(0, 300))
+    dec, ref = _build(rng, cfg, kv_dtype=kv_dtype, symmetric=True)
+    if prefill:
+        for l in range(cfg["n_layers"]):
+            k = rng.standard_normal((B, prefill, n_kv, cfg["head_dim"])).astype(np.float16)
+            v = rng.standard_normal((B, prefill, n_kv, cfg["head_dim"])).astype(np.float16)
+            dec.set_kv(l, k, v)
+            ref.set_kv(l, k.astype(np.float32), v.astype(np.float32))
+    tokens = rng.integers(0, cfg["vocab"], B).astype(np.int32)
+    dec.reset(tokens, prefill)
+    cur = tokens.copy()
+    for step in range(3):
+        dec.run(1, use_graph=bool(step & 1))
+        got_logits, got_tok = dec.logits(), dec.tokens(step, 1)[0]
+        exp_logits = ref.step(cur, prefill + step)
+        err = np.abs(got_logits - exp_logits).max() / np.abs(exp_logits).max()
+        assert err < 2e-2, (cfg, kv_dtype, prefill, step, err)
+        cur = got_tok.copy()
+    dec.close()
+
+
 @pytest.mark.parametrize("kv_dtype", ["f16", "i8"])
 def test_long_context_matches_numpy(kv_dtype):
     """4 230 cached positions = 34 chunks of 128: more than the chunk merge takes in its one-pass form (32), so the
