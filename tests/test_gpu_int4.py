@@ -410,6 +410,43 @@ def test_every_output_at_lm_head_shape(K, torch_cuda):
     w.close()
 
 
+def test_every_output_at_the_prefill_shape(K, torch_cuda):
+    """Every element of BASELINE config 3's output (M=2048, K=4096, N=14336, g=128, fp16 scales, zero points 6..10,
+    bf16 in and out) -- the 128-k-group instantiation with explicit zero points and every column range the call is
+    cut into -- against an fp32 product with the dequantised weight on the GPU (tolerance: the bf16 rounding of
+    the output), three calls, bit-identical from call to call.  Also with 2000 rows: a last row tile that is not full."""
+    torch = torch_cuda
+    rng = np.random.default_rng(57)
+    m, k, n, g = 2048, 4096, 14336, 128
+    groups = k // g
+    b = rng.integers(0, 256, n * k // 2, dtype=np.uint8)
+    scales16 = rng.uniform(0.005, 0.02, n * groups).astype(np.float16)
+    zq = rng.integers(6, 11, (n, groups))
+    w = K.PackedInt4Weight(b, scales16, g, n, k, zero_points=pack_zero_points(zq), nibble_format=K.NIBBLE_UNSIGNED)
+    bt = torch.from_numpy(b.reshape(n, k // 2)).cuda()
+    wd = torch.stack(((bt & 15).float(), (bt >> 4).float()), dim=2).reshape(n, groups, g)
+    del bt
+    wd = wd - torch.from_numpy(zq.astype(np.float32)).cuda()[:, :, None]
+    wd = (wd * torch.from_numpy(scales16.reshape(n, groups).astype(np.float32)).cuda()[:, :, None]).reshape(n, k)
+    x_all = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).bfloat16().cuda()
+    for rows in (m, 2000):
+        x = x_all[:rows].contiguous()
+        ref = x.float() @ wd.T
+        bound = float(ref.abs().max()) * 2.0 ** -7
+        first = None
+        for rep in range(3):
+            y = w.matmul(x)
+            assert y.dtype == torch.bfloat16 and tuple(y.shape) == (rows, n)
+            err = float((y.float() - ref).abs().nan_to_num(1e9).max())
+            assert err <= bound, (rows, rep, err, bound)
+            if first is None:
+                first = y
+            else:
+                assert torch.equal(y, first), (rows, rep)
+        del ref
+    w.close()
+
+
 def test_weight_loaded_from_a_file_equals_the_uploaded_one(K, torch_cuda, tmp_path):
     """yscv_hip_int4_weight_load: the on-disk form carries exactly the arguments of the upload call."""
     torch = torch_cuda
