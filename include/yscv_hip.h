@@ -495,11 +495,17 @@ int32_t yscv_hip_decoder_reset(yscv_hip_decoder *d, int32_t batch, int32_t start
  * by one, 1 replays one captured HIP graph per step, 2 runs all n_steps in ONE cooperative launch of the
  * persistent decode kernel (batch 1 only; YSCV_HIP_ERR_UNSUPPORTED with the reason in the error text when
  * the model shape or the device cannot run it), YSCV_HIP_DECODE_AUTO picks 2 where it applies (batch 1, fp16
- * cache, supported shape) and 1 otherwise.  All produce the same tokens.  Fails if the KV cache
- * or the token history would overflow (KvCache::append returns an error in the same situation,
- * kv_cache.rs:160-185). */
+ * cache, supported shape) and 1 otherwise.  Paths 0 and 1 run the same kernels and give the same bits; path 2
+ * rounds its fp16 activations at other points, so its logits agree with theirs to about 1e-4 .. 5e-3 of max|logit|
+ * (each path is within the float bar of the int4 kernels against the reference arithmetic) and a greedy pick can
+ * differ where two logits are that close.  A caller that needs one arithmetic for every batch size names the path
+ * instead of passing AUTO; yscv_hip_decoder_last_path tells which one a call took.  Fails if the KV cache or the
+ * token history would overflow (KvCache::append returns an error in the same situation, kv_cache.rs:160-185). */
 #define YSCV_HIP_DECODE_AUTO 3
 int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_graph, void *stream);
+/* The path the last yscv_hip_decoder_run of this decoder took: 0, 1 or 2 as above, -1 before the first call.
+ * (The reference has one CPU path and no counterpart; this is how a caller of AUTO learns what ran.) */
+int32_t yscv_hip_decoder_last_path(const yscv_hip_decoder *d, int32_t *path);
 /* Measurement aid: enqueue only the int4 projections of n_steps decode steps (same weights, same
  * order, same buffers as a real step, no attention / norm / sampling), so that the projections'
  * share of a step can be timed on its own.  The activations it reads are whatever the buffers hold. */

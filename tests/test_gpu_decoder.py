@@ -13,7 +13,7 @@ CFG = dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, head_dim=128, d_ff=
            max_batch=3, max_ctx=256, max_steps=16, rope_theta=10000.0, rms_eps=1e-5)
 
 
-def _build(rng, cfg, kv_dtype="f16", emb_scale=1.0, symmetric=False):
+def _build(rng, cfg, kv_dtype="f16", emb_scale=1.0, symmetric=False, v_mul=1.0):
     from oracle.decoder_ref import RefDecoder
     from yscv_amd.decoder import Decoder
 
@@ -35,6 +35,8 @@ def _build(rng, cfg, kv_dtype="f16", emb_scale=1.0, symmetric=False):
         for kind, (n, k) in shapes.items():
             p = nibbles(n * k // 2)
             s = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float16)
+            if kind == "v":
+                s = (s.astype(np.float32) * v_mul).astype(np.float16)  # small values: rows of the V cache far below 1
             linears[(l, kind)] = (p, s)
             dec.set_linear(l, kind, p, s, n, k)
         for kind in ("attn", "ffn"):
@@ -189,6 +191,46 @@ def test_long_context_matches_numpy(kv_dtype):
                 got = ao[b].reshape(nh, hd)[h]
                 assert np.abs(got - want).max() <= 1e-2 * np.abs(want).max() + 1e-3, (step, b, h)
         cur = got_tok.copy()
+
+
+@pytest.mark.parametrize("v_mag", [1e-3, 1e-4])
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_int8_cache_with_small_values(v_mag, use_graph):
+    """V rows of absmax 1e-3 .. 1e-4 in the int8 cache (cached rows and the appended one): the per-row scale absmax / 127
+    is then 1e-5 .. 1e-6, far below fp16's normal range, and must not be lost where it meets the softmax weights.  The
+    last layer's attention output against a float64 softmax over the checker's cache (dequantised q * scale in f32, as
+    runner/kv_cache.rs:65-79 reads it back), relative to the output's own magnitude."""
+    import math
+
+    rng = np.random.default_rng(4700 + int(-math.log10(v_mag)))
+    cfg = dict(CFG)
+    dec, ref = _build(rng, cfg, kv_dtype="i8", symmetric=True, v_mul=v_mag)
+    B, prefill = 2, 141
+    for l in range(cfg["n_layers"]):
+        k = rng.standard_normal((B, prefill, cfg["n_kv_heads"], cfg["head_dim"])).astype(np.float16)
+        v = (rng.standard_normal((B, prefill, cfg["n_kv_heads"], cfg["head_dim"])) * v_mag).astype(np.float16)
+        dec.set_kv(l, k, v)
+        ref.set_kv(l, k.astype(np.float32), v.astype(np.float32))
+    tokens = np.array([9, 33], np.int32)
+    dec.reset(tokens, prefill)
+    cur = tokens.copy()
+    nh, nkv, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    for step in range(2):
+        dec.run(1, use_graph=use_graph)
+        ref.step(cur, prefill + step)
+        qkv, ao = dec.activation("qkv"), dec.activation("attn_out")
+        L = cfg["n_layers"] - 1
+        for b in range(B):
+            q = qkv[b][: nh * hd].reshape(nh, hd).astype(np.float64)
+            kc, vc = ref.kc[L][b].astype(np.float64), ref.vc[L][b].astype(np.float64)
+            assert np.abs(vc).max() < 20 * v_mag
+            for h in range(nh):
+                sc = kc[:, h // (nh // nkv), :] @ q[h] / math.sqrt(hd)
+                pr = np.exp(sc - sc.max())
+                want = (pr / pr.sum()) @ vc[:, h // (nh // nkv), :]
+                got = ao[b].reshape(nh, hd)[h]
+                assert np.abs(got - want).max() <= 1e-2 * np.abs(want).max(), (step, b, h, np.abs(got - want).max(), np.abs(want).max())
+        cur = dec.tokens(step, 1)[0].copy()
 
 
 @pytest.mark.parametrize("kv_dtype", ["f16", "i8"])
@@ -477,22 +519,30 @@ def test_single_launch_tags_wrap_around_cleanly():
         assert np.array_equal(dec.logits(), want_logits), back
 
 
-def test_generate_matches_device_greedy_and_stops_at_eos():
+@pytest.mark.parametrize("shape", ["graph", "single_launch"])
+def test_generate_matches_device_greedy_and_stops_at_eos(shape):
     """generate() (generate.rs:58-118) with the decoder as the model: top_k = 1 reproduces the tokens the device picks
-    greedily; an EOS token ends the loop without being stored; the sampling path runs with the default configuration."""
+    greedily; an EOS token ends the loop without being stored; the sampling path runs with the default configuration.
+    Two shapes: one only the multi-kernel path takes, and one (widths in multiples of 1024) that generate() runs on the
+    single-launch kernel, one cooperative launch per prompt token."""
     import numpy as np
 
     from yscv_amd.decoder import Decoder
 
     cfg = dict(n_layers=2, d_model=512, n_heads=4, n_kv_heads=2, head_dim=128, d_ff=1024, vocab=320, group_size=32,
                max_batch=1, max_ctx=256, max_steps=64, rope_theta=10000.0, rms_eps=1e-5)
+    if shape == "single_launch":
+        cfg.update(d_model=1024, n_heads=8, n_kv_heads=2, d_ff=2048)
     dec = Decoder(**cfg)
     dec.init_random(seed=5)
     prompt = [7, 3, 11]
+    assert dec.last_path() == -1
     got = dec.generate(prompt, max_tokens=12, top_k=1, top_p=1.0)
+    assert dec.last_path() == (2 if shape == "single_launch" else 1)
     # the same through the device-side greedy loop: feed the prompt, then let the decoder run on its own picks
     dec.reset(np.array([prompt[0]], np.int32), 0)
     dec.run(1, auto=True)  # the path generate() takes: the fastest one the decoder has
+    assert dec.last_path() == (2 if shape == "single_launch" else 1)
     for p, t in enumerate(prompt[1:], start=1):
         dec.reset(np.array([t], np.int32), p)
         dec.run(1, auto=True)

@@ -7,6 +7,26 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
+class _PoolProbe:
+    """hipMemPoolAttrReservedMemCurrent of device 0's default stream-ordered pool, read through the HIP runtime the
+    library itself is linked against (symbol lookup on its handle reaches its dependencies)."""
+
+    def __init__(self):
+        import ctypes as C
+
+        from yscv_amd import capi
+
+        self.C = C
+        self.hip = capi.lib()._cdll
+        self.pool = C.c_void_p()
+        assert self.hip.hipDeviceGetDefaultMemPool(C.byref(self.pool), 0) == 0
+
+    def reserved(self):
+        v = self.C.c_uint64(0)
+        assert self.hip.hipMemPoolGetAttribute(self.pool, 5, self.C.byref(v)) == 0  # hipMemPoolAttrReservedMemCurrent
+        return int(v.value)
+
+
 def _weight(K, rng, n, k, g, f16_scales):
     b = rng.integers(0, 256, n * k // 2, dtype=np.uint8)
     s = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float16 if f16_scales else np.float32)
@@ -38,6 +58,16 @@ def test_static_scratch_call_equals_the_allocating_call(n, k, g, xdt, f16s, m_fi
             torch.cuda.synchronize()
             assert torch.equal(got[:m], want), (m, odt)
             assert bool((got[m] == 5.0).all())
+            # the property the entry point exists for: a batch of calls leaves the device's free memory and the
+            # stream-ordered pool's reservation where they were (the allocating call takes its scratch from that pool)
+            pool = _PoolProbe()
+            free_before, reserved_before = torch.cuda.mem_get_info()[0], pool.reserved()
+            for _ in range(8):
+                w.matmul_static(x, got[:m])
+            torch.cuda.synchronize()
+            assert torch.cuda.mem_get_info()[0] == free_before, (m, odt)
+            assert pool.reserved() == reserved_before, (m, odt)
+            assert torch.equal(got[:m], want), (m, odt)
     w.close()
 
 

@@ -139,6 +139,7 @@ _SIGNATURES = {
     "yscv_hip_decoder_get_kv": [_vp, _i32, _vp, _vp, _i32, _i32, _i32],
     "yscv_hip_decoder_reset": [_vp, _i32, _i32, _vp],
     "yscv_hip_decoder_run": [_vp, _i32, _i32, _vp],
+    "yscv_hip_decoder_last_path": [_vp, _vp],
     "yscv_hip_decoder_run_projections": [_vp, _i32, _vp],
     "yscv_hip_decoder_read_tokens": [_vp, _i32, _i32, _vp],
     "yscv_hip_decoder_read_logits": [_vp, _vp],

@@ -133,6 +133,7 @@ struct yscv_hip_decoder {
   size_t weight_bytes = 0;
   // persistent single-launch path (batch 1)
   bool persist_ok = false;     // the shape is supported and the buffers exist
+  int last_path = -1;          // path of the last yscv_hip_decoder_run: 0 launches, 1 graph replays, 2 single launch
   PersistModel pm{};
   uint8_t *p_stream = nullptr;
   uint64_t *p_wg_off = nullptr;
@@ -888,6 +889,7 @@ int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_g
                d->cfg.max_steps);
   if (use_graph == YSCV_HIP_DECODE_AUTO)  // the fastest path this decoder has for its batch
     use_graph = (d->batch == 1 && d->persist_ok && d->kv_dtype == YSCV_HIP_KV_F16) ? 2 : 1;
+  d->last_path = use_graph == 2 ? 2 : (use_graph ? 1 : 0);
   if (use_graph == 2) {
     if (d->kv_dtype != YSCV_HIP_KV_F16)
       return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the single-launch decode path reads an fp16 KV cache only");
@@ -1098,6 +1100,12 @@ int32_t yscv_hip_decoder_debug_set_folded_norm(yscv_hip_decoder *d, int32_t on) 
   drop_graph(d);
   d->fold_norm_wanted = on != 0;
   if (d->finalized) YSCV_TRY(finish_setup(d));
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_last_path(const yscv_hip_decoder *d, int32_t *path) {
+  YSCV_REQUIRE(d != nullptr && path != nullptr, "null argument");
+  *path = d->last_path;
   return YSCV_HIP_OK;
 }
 

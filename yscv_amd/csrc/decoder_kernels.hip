@@ -273,6 +273,18 @@ __device__ __forceinline__ half8_t i8x8_to_half8(int2_t raw) {
   return h;
 }
 
+// int8 cache: the value scale of a position rides on its softmax weight, which the second MFMA takes as fp16.  The
+// largest scale among the wave's live positions, rounded up to a power of two S, is taken out first: the weights carry
+// v_scale / S <= 1 (a row of small values, absmax 1e-4 say, would otherwise push them into fp16's subnormals) and the
+// f32 result is multiplied by S.  Returns S; *inv = 1 / S (both exact).
+__device__ __forceinline__ float v_scale_pow2(float v0, float v1, bool live0, bool live1, float *inv) {
+  const float m = row_max16(fmaxf(live0 ? v0 : 0.0f, live1 ? v1 : 0.0f));
+  int e = 0;
+  if (m > 0.0f && m < INFINITY) (void)frexpf(m, &e);  // m = f * 2^e, f in [0.5, 1)
+  *inv = ldexpf(1.0f, -e);
+  return ldexpf(1.0f, e);
+}
+
 template <bool KV8>
 __global__ void __launch_bounds__(256) attn_partial_kernel(const _Float16 *__restrict__ qkv,
                                                            const void *__restrict__ kc_v,
@@ -366,10 +378,12 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const _Float16 *__res
     const float sum = row_sum16(e0 + e1);
     m_h = mx;
     l_h = sum;
+    float vS = 1.0f, vS_inv = 1.0f;
+    if constexpr (KV8) vS = v_scale_pow2(v_scale[0], v_scale[1], p0 + r < n_ctx, p0 + 16 + r < n_ctx, &vS_inv);
     if (c < 4) {
       // int8 cache: the V scale of the position rides on its weight (a dead position has weight 0 whatever its scale)
-      p_lds[wave][c][r] = KV8 ? (e0 == 0.0f ? (_Float16)0.0f : (_Float16)(e0 * v_scale[0])) : (_Float16)e0;
-      p_lds[wave][c][16 + r] = KV8 ? (e1 == 0.0f ? (_Float16)0.0f : (_Float16)(e1 * v_scale[1])) : (_Float16)e1;
+      p_lds[wave][c][r] = KV8 ? (e0 == 0.0f ? (_Float16)0.0f : (_Float16)(e0 * (v_scale[0] * vS_inv))) : (_Float16)e0;
+      p_lds[wave][c][16 + r] = KV8 ? (e1 == 0.0f ? (_Float16)0.0f : (_Float16)(e1 * (v_scale[1] * vS_inv))) : (_Float16)e1;
     }
     __builtin_amdgcn_wave_barrier();  // LDS is in order per wave: the reads below see the writes above
     // P operand: MFMA row 4*h = head h, lane (r, c) holds positions 8c .. 8c+7 of this wave's 32
@@ -388,7 +402,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const _Float16 *__res
       }
       float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
       d = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vv, d, 0, 0, 0);
-      o_acc[t] = d[0];  // lane (r, c): o of head c at d = 16 t + r
+      o_acc[t] = KV8 ? d[0] * vS : d[0];  // lane (r, c): o of head c at d = 16 t + r
     }
   }
 
@@ -1027,9 +1041,11 @@ __global__ void __launch_bounds__(256) attn_fused_i8_kernel(const _Float16 *__re
     const float sum = row_sum16(e0 + e1);
     m_h = mx;
     l_h = sum;
+    float vS_inv = 1.0f;
+    const float vS = v_scale_pow2(v_scale[0], v_scale[1], p0 + r < n_ctx, p0 + 16 + r < n_ctx, &vS_inv);
     if (c < 4) {  // the V scale of the position rides on its weight (a dead position has weight 0 whatever its scale)
-      p_lds[wave][c][r] = e0 == 0.0f ? (_Float16)0.0f : (_Float16)(e0 * v_scale[0]);
-      p_lds[wave][c][16 + r] = e1 == 0.0f ? (_Float16)0.0f : (_Float16)(e1 * v_scale[1]);
+      p_lds[wave][c][r] = e0 == 0.0f ? (_Float16)0.0f : (_Float16)(e0 * (v_scale[0] * vS_inv));
+      p_lds[wave][c][16 + r] = e1 == 0.0f ? (_Float16)0.0f : (_Float16)(e1 * (v_scale[1] * vS_inv));
     }
     __builtin_amdgcn_wave_barrier();
     half8_t vf[8];
@@ -1060,7 +1076,7 @@ __global__ void __launch_bounds__(256) attn_fused_i8_kernel(const _Float16 *__re
       }
       float4_t d = {0.0f, 0.0f, 0.0f, 0.0f};
       d = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vv, d, 0, 0, 0);
-      o_acc[t] = d[0];
+      o_acc[t] = d[0] * vS;
     }
   }
 

@@ -76,6 +76,12 @@ class Decoder:
         mode = 3 if auto else (2 if persistent else int(bool(use_graph)))
         lib().decoder_run(self._h, int(n_steps), mode, C.c_void_p(stream) if stream else None)
 
+    def last_path(self):
+        """yscv_hip_decoder_last_path: 0 kernel launches, 1 graph replays, 2 the single-launch kernel, -1 before any run."""
+        v = C.c_int32(-1)
+        lib().decoder_last_path(self._h, C.byref(v))
+        return int(v.value)
+
     def run_projections(self, n_steps, stream=None):
         lib().decoder_run_projections(self._h, int(n_steps), C.c_void_p(stream) if stream else None)
 
