@@ -409,6 +409,27 @@ int32_t yscv_hip_kv_i8_quantize_rows(const float *src_dev, size_t rows, size_t k
 int32_t yscv_hip_kv_i8_dequantize_rows(const int8_t *data_dev, const float *scales_dev, size_t rows, size_t kv_dim,
                                        float *out_dev, void *stream);
 
+/* ---- the operators between the MatMuls of an LLM graph, on device tensors ------------------------------------
+ * A graph executor that keeps its tensors on the GPU calls these between two projections instead of leaving the
+ * device; layouts and arithmetic are the reference operators', f32 in and out. */
+/* rms_norm_last_dim (crates/yscv-kernels/src/ops/norm.rs:1431-1518): y[row] = x[row] * (1 / sqrt(mean(x[row]^2) + eps))
+ * * gamma over rows of d values; epsilon must be finite and > 0 (InvalidRmsNormEpsilon -> INVALID_ARG). */
+int32_t yscv_hip_rms_norm_dev(const float *x_dev, const float *gamma_dev, size_t rows, size_t d, float eps, float *y_dev,
+                              void *stream);
+/* apply_rotary_embedding (crates/yscv-kernels/src/ops/rope.rs:24-117), in place: q [seq_len][num_q_heads][d_head],
+ * k [seq_len][num_kv_heads][d_head], pair (x[i], x[i + d/2]) rotated by inv_freq[i] * (pos + seq_offset) with
+ * inv_freq[i] = 1 / theta^(2i / d_head).  sin / cos come from the device's math library: tolerance, not bit parity. */
+int32_t yscv_hip_rope_dev(float *q_dev, float *k_dev, size_t num_q_heads, size_t num_kv_heads, size_t d_head, size_t seq_len,
+                          size_t seq_offset, float theta, void *stream);
+/* exec_grouped_query_attention (crates/yscv-onnx/src/runner/linear.rs:552-646): q [batch][seq_q][num_q_heads * d_head],
+ * k / v [batch][seq_k][num_kv_heads * d_head] -> out [batch][seq_q][num_q_heads * d_head]; kv head = q head / groups,
+ * scores * 1 / sqrt(d_head), max-subtracted softmax over all seq_k positions, no mask.  d_head 32, 64, 96 or 128
+ * (UNSUPPORTED otherwise); operands enter the matrix cores as fp16 with f32 accumulation (relative error about 1e-3).
+ * q, k and out must be 16-byte aligned. */
+int32_t yscv_hip_gqa_attention_dev(const float *q_dev, const float *k_dev, const float *v_dev, size_t batch, size_t seq_q,
+                                   size_t seq_k, size_t num_q_heads, size_t num_kv_heads, size_t d_head, float *out_dev,
+                                   void *stream);
+
 /* ---- decode loop (Llama-style decoder, int4 projections, fp16 KV cache) ----------------- */
 
 /* GPU-resident counterpart of the llm-bench decode loop (apps/llm-bench/src/main.rs:403-561:
@@ -422,8 +443,9 @@ typedef struct yscv_hip_decoder_config {
   int32_t n_layers;
   int32_t d_model;
   int32_t n_heads;    /* query heads */
-  int32_t n_kv_heads; /* n_heads / n_kv_heads must be 1..4 */
-  int32_t head_dim;   /* 128 */
+  int32_t n_kv_heads; /* divides n_heads; head_dim 128 with 1..4 query heads per kv head takes the specialised
+                         attention kernels (fp16 or int8 cache, single-launch path), anything else the general one */
+  int32_t head_dim;   /* 32, 64, 96 or 128 */
   int32_t d_ff;
   int32_t vocab;
   int32_t group_size; /* int4 group size of every projection: 32, 64 or a multiple of 128 */
@@ -503,6 +525,21 @@ int32_t yscv_hip_decoder_reset(yscv_hip_decoder *d, int32_t batch, int32_t start
  * token history would overflow (KvCache::append returns an error in the same situation, kv_cache.rs:160-185). */
 #define YSCV_HIP_DECODE_AUTO 3
 int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_graph, void *stream);
+/* The prompt phase of the decode loop (apps/llm-bench/src/main.rs:403-470 times it apart from the decode phase): feeds
+ * n_tokens prompt tokens at positions start_pos .. start_pos + n_tokens - 1 of batch row 0 in ONE pass -- every
+ * projection sees all rows at once (the MFMA GEMM above 16 rows), attention is causal over the cache, which receives
+ * the rotated keys and the values of every position -- and computes the logits of the last position only.  Leaves the
+ * decoder as yscv_hip_decoder_reset(1, start_pos + n_tokens - 1, last token) + one decode step would: batch 1, the
+ * greedy pick as the next input token and as token 0 of the history, position start_pos + n_tokens, step 1.  The
+ * results agree with token-by-token feeding to the float bar of the int4 kernels (the GEMM folds the group scale into
+ * fp16 weights where the decode kernel applies it in fp32).  A decoder with an int8 cache runs the decode step per
+ * position instead.  tokens_host is read before the call returns. */
+int32_t yscv_hip_decoder_prefill(yscv_hip_decoder *d, const int32_t *tokens_host, int32_t n_tokens, int32_t start_pos,
+                                 void *stream);
+/* Optional bias of the fused q / k / v projection of one layer (Qwen-style attention; the reference adds it with
+ * the Add node behind the MatMul): fp16 [(n_heads + 2 n_kv_heads) * head_dim] in q, k, v order, or NULL to remove it.
+ * A decoder with a bias takes the multi-kernel path (the single-launch kernel has none). */
+int32_t yscv_hip_decoder_set_qkv_bias(yscv_hip_decoder *d, int32_t layer, const uint16_t *bias_f16);
 /* The path the last yscv_hip_decoder_run of this decoder took: 0, 1 or 2 as above, -1 before the first call.
  * (The reference has one CPU path and no counterpart; this is how a caller of AUTO learns what ran.) */
 int32_t yscv_hip_decoder_last_path(const yscv_hip_decoder *d, int32_t *path);

@@ -91,7 +91,8 @@ def kv_i8_roundtrip(rows):
 
 
 class RefDecoder:
-    def __init__(self, cfg: dict, linears: dict, norms: dict, emb16, kv_i8: bool = False, round_f16: bool = True):
+    def __init__(self, cfg: dict, linears: dict, norms: dict, emb16, kv_i8: bool = False, round_f16: bool = True,
+                 biases: dict | None = None):
         """linears[(layer, kind)] = (packed, scales16) with kind in q k v o gate up down, and
         linears[('lm_head',)]; norms[(layer, 'attn'|'ffn')], norms[('final',)] f32 gamma.
         kv_i8: the cache stores per-row int8 (KvDtype::I8); the rotated key of a new token is then quantised from its f32
@@ -111,6 +112,9 @@ class RefDecoder:
             n, k = (cfg["vocab"], D) if key == ("lm_head",) else shapes[key[1]]
             self.w[key] = dequant_uint4(p, s, n, k, g)
         self.norms = norms
+        # biases[layer] = f32 [(n_heads + 2 n_kv_heads) * head_dim] in q, k, v order, added to the projections' outputs
+        # (the Add node an exporter places behind the q / k / v MatMuls of a Qwen-style attention block)
+        self.biases = biases or {}
         self.emb = np.asarray(emb16).view(np.float16).astype(np.float32).reshape(cfg["vocab"], D)
         L, B = cfg["n_layers"], cfg["max_batch"]
         self.kc = [[np.zeros((0, cfg["n_kv_heads"], hd), np.float32) for _ in range(B)] for _ in range(L)]
@@ -143,9 +147,15 @@ class RefDecoder:
         h = self.emb[np.asarray(tokens)].astype(np.float32)
         for l in range(c["n_layers"]):
             xn = self._rmsnorm(h, self.norms[(l, "attn")])
-            q = self._r(xn @ self.w[(l, "q")].T).reshape(B, nh, hd)
-            k = self._r(xn @ self.w[(l, "k")].T).reshape(B, nkv, hd)
-            v = self._r(xn @ self.w[(l, "v")].T).reshape(B, nkv, hd)
+            q = self._r(xn @ self.w[(l, "q")].T)
+            k = self._r(xn @ self.w[(l, "k")].T)
+            v = self._r(xn @ self.w[(l, "v")].T)
+            if l in self.biases:
+                bias = np.asarray(self.biases[l], np.float32)
+                q = self._r(q + bias[: nh * hd])
+                k = self._r(k + bias[nh * hd: (nh + nkv) * hd])
+                v = self._r(v + bias[(nh + nkv) * hd:])
+            q, k, v = q.reshape(B, nh, hd), k.reshape(B, nkv, hd), v.reshape(B, nkv, hd)
             ao = np.zeros((B, nh, hd), np.float32)
             qkv = np.zeros((B, (nh + 2 * nkv) * hd), np.float32)
             for b in range(B):

@@ -13,7 +13,7 @@ CFG = dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, head_dim=128, d_ff=
            max_batch=3, max_ctx=256, max_steps=16, rope_theta=10000.0, rms_eps=1e-5)
 
 
-def _build(rng, cfg, kv_dtype="f16", emb_scale=1.0, symmetric=False, v_mul=1.0):
+def _build(rng, cfg, kv_dtype="f16", emb_scale=1.0, symmetric=False, v_mul=1.0, qkv_bias=False):
     from oracle.decoder_ref import RefDecoder
     from yscv_amd.decoder import Decoder
 
@@ -21,7 +21,7 @@ def _build(rng, cfg, kv_dtype="f16", emb_scale=1.0, symmetric=False, v_mul=1.0):
     hq, hkv, ff = cfg["n_heads"] * hd, cfg["n_kv_heads"] * hd, cfg["d_ff"]
     shapes = {"q": (hq, D), "k": (hkv, D), "v": (hkv, D), "o": (D, hq), "gate": (ff, D), "up": (ff, D), "down": (D, ff)}
     dec = Decoder(kv_dtype=kv_dtype, **cfg)
-    linears, norms = {}, {}
+    linears, norms, biases = {}, {}, {}
 
     def nibbles(count):
         # symmetric: nibbles 1..15 only, mean zero after the zero point 8.  Uniform bytes give every projection output a
@@ -43,6 +43,10 @@ def _build(rng, cfg, kv_dtype="f16", emb_scale=1.0, symmetric=False, v_mul=1.0):
             gmm = rng.uniform(0.5, 1.5, D).astype(np.float32)
             norms[(l, kind)] = gmm
             dec.set_norm(l, kind, gmm)
+        if qkv_bias:
+            bias = (rng.standard_normal(hq + 2 * hkv) * 0.5).astype(np.float16)
+            biases[l] = bias.astype(np.float32)
+            dec.set_qkv_bias(l, bias)
     p = nibbles(cfg["vocab"] * D // 2)
     s = rng.uniform(0.005, 0.02, cfg["vocab"] * (D // g)).astype(np.float16)
     linears[("lm_head",)] = (p, s)
@@ -56,7 +60,7 @@ def _build(rng, cfg, kv_dtype="f16", emb_scale=1.0, symmetric=False, v_mul=1.0):
     emb = emb.astype(np.float16)
     dec.set_embedding(emb)
     dec.finalize()
-    ref = RefDecoder(cfg, linears, norms, emb, kv_i8=kv_dtype == "i8")
+    ref = RefDecoder(cfg, linears, norms, emb, kv_i8=kv_dtype == "i8", biases=biases)
     return dec, ref
 
 
@@ -560,4 +564,84 @@ def test_generate_matches_device_greedy_and_stops_at_eos(shape):
     a = dec.generate(prompt, max_tokens=8, temperature=0.8, repetition_penalty=1.3)
     b = dec.generate(prompt, max_tokens=8, temperature=0.8, repetition_penalty=1.3)
     assert a.tolist() == b.tolist() and len(a) == 8 and (a < cfg["vocab"]).all()
+    dec.close()
+
+
+# ---- the reference's own benchmark model, prompt pass, q / k / v bias ------------------------------------------------
+# apps/llm-bench/COMPARISON.md:9-12: 24 layers, hidden 1024, 2 kv heads, head_dim 64 (16 query heads: eight per kv
+# head), a 43-token prompt; the vocabulary and the FFN width are cut down to keep the numpy side short.
+BENCH_MODEL = dict(n_layers=24, d_model=1024, n_heads=16, n_kv_heads=2, head_dim=64, d_ff=2816, vocab=2048, group_size=32,
+                   max_batch=2, max_ctx=256, max_steps=16, rope_theta=1000000.0, rms_eps=1e-6)
+
+
+def test_reference_benchmark_model_decodes_and_prefills():
+    """head_dim 64 with eight query heads per kv head (the general attention kernel) at 24 layers: token-by-token feeding
+    of a 43-token prompt against the checker, then the same prompt through yscv_hip_decoder_prefill: logits of the last
+    prompt position, the cache rows of every position and the decode steps that follow agree with the fed run."""
+    rng = np.random.default_rng(4800)
+    cfg = dict(BENCH_MODEL)
+    dec, ref = _build(rng, cfg, symmetric=True, qkv_bias=True)
+    prompt = rng.integers(0, cfg["vocab"], 43).astype(np.int32)
+    for p, t in enumerate(prompt):
+        dec.reset(np.array([t], np.int32), p)
+        dec.run(1, use_graph=bool(p & 1))
+        exp = ref.step(np.array([t]), p)
+        if p in (0, 1, 20, 42):
+            err = np.abs(dec.logits() - exp).max() / np.abs(exp).max()
+            assert err < LOGIT_TOL, (p, err)
+    fed_logits = dec.logits().copy()
+    fed_kv = [dec.get_kv(l, 1, 0, 43) for l in (0, 11, 23)]
+    fed_tok = int(dec.tokens(0, 1)[0, 0])
+    # continue for three steps on the device's own picks: the trajectory the prefilled decoder must repeat
+    dec.run(3, use_graph=True)
+    fed_next = dec.tokens(0, 4)[:, 0].tolist()
+    fed_logits3 = dec.logits().copy()
+
+    dec2, _ = _build(np.random.default_rng(4800), cfg, symmetric=True, qkv_bias=True)  # same seed: the same model
+    dec2.prefill(prompt)
+    got = dec2.logits()
+    assert np.abs(got - exp).max() / np.abs(exp).max() < LOGIT_TOL
+    # two paths that each meet the bar against the checker (the prompt pass folds the group scales into fp16 weights,
+    # 24 layers deep) are within twice the bar of each other
+    between = np.abs(got - fed_logits).max() / np.abs(fed_logits).max()
+    assert between < 2 * LOGIT_TOL, between
+    assert int(dec2.tokens(0, 1)[0, 0]) == fed_tok or between > 1e-3
+    for (fk, fv), l in zip(fed_kv, (0, 11, 23)):
+        gk, gv = dec2.get_kv(l, 1, 0, 43)
+        assert np.abs(gk.astype(np.float32) - fk.astype(np.float32)).max() <= 2e-2 * np.abs(fk.astype(np.float32)).max(), l
+        assert np.abs(gv.astype(np.float32) - fv.astype(np.float32)).max() <= 2e-2 * np.abs(fv.astype(np.float32)).max(), l
+    dec2.run(3, use_graph=True)
+    if dec2.tokens(0, 4)[:, 0].tolist() == fed_next:  # the same trajectory: the same inputs at every step
+        assert np.abs(dec2.logits() - fed_logits3).max() / np.abs(fed_logits3).max() < 2 * LOGIT_TOL
+    dec.close()
+    dec2.close()
+
+
+@pytest.mark.parametrize("n_prompt,start", [(1, 0), (5, 0), (16, 3), (17, 0), (130, 9)])
+def test_prefill_equals_feeding_at_toy_widths(n_prompt, start):
+    """Prompt lengths on both sides of the skinny / GEMM switch (16 rows) and across a 128-position attention chunk, at a
+    start position other than 0 (a prompt appended to a cache that already holds positions): prefill against the
+    checker fed token by token, head_dim 128."""
+    rng = np.random.default_rng(4900 + n_prompt)
+    cfg = dict(CFG, max_batch=1, max_ctx=256)
+    dec, ref = _build(rng, cfg, symmetric=True)
+    for l in range(cfg["n_layers"]):
+        k = rng.standard_normal((1, start, cfg["n_kv_heads"], cfg["head_dim"])).astype(np.float16)
+        v = rng.standard_normal((1, start, cfg["n_kv_heads"], cfg["head_dim"])).astype(np.float16)
+        if start:
+            dec.set_kv(l, k, v)
+        ref.set_kv(l, k.astype(np.float32), v.astype(np.float32))
+    prompt = rng.integers(0, cfg["vocab"], n_prompt).astype(np.int32)
+    for i, t in enumerate(prompt):
+        exp = ref.step(np.array([t]), start + i)
+    dec.prefill(prompt, start_pos=start)
+    got = dec.logits()
+    assert np.abs(got - exp).max() / np.abs(exp).max() < LOGIT_TOL
+    row = got[0]
+    assert int(dec.tokens(0, 1)[0, 0]) == np.flatnonzero(row == row.max())[-1]
+    # the step after the prompt continues from the cache the prompt pass wrote
+    nxt = dec.tokens(0, 1)[0].copy()
+    dec.run(1, use_graph=True)
+    exp2 = ref.step(nxt, start + n_prompt)
+    assert np.abs(dec.logits() - exp2).max() / np.abs(exp2).max() < LOGIT_TOL
     dec.close()

@@ -140,6 +140,11 @@ _SIGNATURES = {
     "yscv_hip_decoder_reset": [_vp, _i32, _i32, _vp],
     "yscv_hip_decoder_run": [_vp, _i32, _i32, _vp],
     "yscv_hip_decoder_last_path": [_vp, _vp],
+    "yscv_hip_decoder_prefill": [_vp, _vp, _i32, _i32, _vp],
+    "yscv_hip_decoder_set_qkv_bias": [_vp, _i32, _vp],
+    "yscv_hip_rms_norm_dev": [_vp, _vp, _sz, _sz, C.c_float, _vp, _vp],
+    "yscv_hip_rope_dev": [_vp, _vp, _sz, _sz, _sz, _sz, _sz, C.c_float, _vp],
+    "yscv_hip_gqa_attention_dev": [_vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz, _vp, _vp],
     "yscv_hip_decoder_run_projections": [_vp, _i32, _vp],
     "yscv_hip_decoder_read_tokens": [_vp, _i32, _i32, _vp],
     "yscv_hip_decoder_read_logits": [_vp, _vp],

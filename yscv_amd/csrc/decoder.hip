@@ -102,6 +102,7 @@ struct yscv_hip_decoder {
     _Float16 *kc = nullptr, *vc = nullptr;   // fp16 cache
     int8_t *kc8 = nullptr, *vc8 = nullptr;   // int8 cache (kv_dtype I8) ...
     float *ks = nullptr, *vs = nullptr;      // ... with one scale per (batch row, position)
+    _Float16 *qkv_bias = nullptr;            // null, or [(hq + 2 hkv) hd] added to the q / k / v projection
     HostLinear stage[7];  // q k v o gate up down, kept until finalize
   };
   std::vector<Layer> layers;
@@ -113,6 +114,8 @@ struct yscv_hip_decoder {
   _Float16 *xn = nullptr, *qkv = nullptr, *ao = nullptr, *act = nullptr;
   _Float16 *qrot = nullptr;       // rotated query heads of the last fused attention launch (diagnostics)
   bool fused_attn = true;         // rope + append inside the attention kernel
+  bool generic_attn = false;      // head width other than 128 or more than 4 query heads per kv head: the general kernel
+  bool has_bias = false;          // a layer has a q / k / v bias (the single-launch kernel has none)
   // RMSNorm folded into the projections around it (NormFold, kernels.hpp): two buffers of partial sums of squares,
   // written and read in turn, each with the power of two per row that xn's rows were multiplied by
   bool fold_norm = false;         // decided in finish_setup from the shapes
@@ -174,6 +177,7 @@ static void decoder_free(yscv_hip_decoder *d) {
     (void)hipFree(L.vc8);
     (void)hipFree(L.ks);
     (void)hipFree(L.vs);
+    (void)hipFree(L.qkv_bias);
   }
   destroy_int4(d->lm_head);
   (void)hipFree(d->final_norm);
@@ -485,7 +489,13 @@ static int32_t enqueue_step(yscv_hip_decoder *d, int batch, hipStream_t s) {
       YSCV_TRY(launch_rmsnorm(d->h, L.attn_norm, batch, D, c.rms_eps, d->xn, s));
       YSCV_TRY(int4_run_ws(L.wqkv, d->xn, YSCV_HIP_F16, d->qkv, YSCV_HIP_F16, batch, 1, EPI_STORE, d->ws, d->ws_bytes, s));
     }
-    if (d->kv_dtype == YSCV_HIP_KV_I8 && d->fused_attn) {
+    const int qkv_n = (c.n_heads + 2 * c.n_kv_heads) * c.head_dim;
+    if (L.qkv_bias) YSCV_TRY(launch_bias_add_f16(d->qkv, L.qkv_bias, (size_t)batch, (size_t)qkv_n, s));
+    if (d->generic_attn) {
+      YSCV_TRY(launch_rope_append(d->qkv, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_theta, c.max_ctx,
+                                  L.kc, L.vc, s));
+      YSCV_TRY(launch_gqa_cache(d->qkv, L.kc, L.vc, d->pos, batch, 0, c.n_heads, c.n_kv_heads, c.head_dim, c.max_ctx, d->ao, s));
+    } else if (d->kv_dtype == YSCV_HIP_KV_I8 && d->fused_attn) {
       YSCV_TRY(launch_attention_fused_i8(d->qkv, L.kc8, L.ks, L.vc8, L.vs, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim,
                                          c.rope_theta, c.max_ctx, d->attn_part, d->qrot, d->ao, s));
     } else if (d->kv_dtype == YSCV_HIP_KV_I8) {
@@ -563,8 +573,12 @@ int32_t yscv_hip_decoder_create_kv(const yscv_hip_decoder_config *cfg, int32_t k
   const auto &c = *cfg;
   YSCV_REQUIRE(c.n_layers > 0 && c.d_model > 0 && c.n_heads > 0 && c.n_kv_heads > 0 && c.d_ff > 0 && c.vocab > 0,
                "non-positive model dimension");
-  YSCV_REQUIRE(c.head_dim == 128, "head_dim must be 128 (got %d)", c.head_dim);
-  YSCV_REQUIRE(c.n_heads % c.n_kv_heads == 0 && c.n_heads / c.n_kv_heads <= 4, "1..4 query heads per kv head");
+  YSCV_REQUIRE(c.head_dim == 32 || c.head_dim == 64 || c.head_dim == 96 || c.head_dim == 128,
+               "head_dim must be 32, 64, 96 or 128 (got %d)", c.head_dim);
+  YSCV_REQUIRE(c.n_heads % c.n_kv_heads == 0, "the kv heads must divide the query heads (%d over %d)", c.n_heads, c.n_kv_heads);
+  const bool generic_attn = c.head_dim != 128 || c.n_heads / c.n_kv_heads > 4;
+  if (generic_attn && kv_dtype == YSCV_HIP_KV_I8)
+    return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the int8 cache exists for head_dim 128 with 1..4 query heads per kv head");
   YSCV_REQUIRE(c.d_model % 128 == 0 && c.d_ff % 128 == 0 && (c.n_heads * c.head_dim) % 128 == 0,
                "d_model, d_ff and n_heads*head_dim must be multiples of 128");
   YSCV_REQUIRE(c.max_batch >= 1 && c.max_batch <= 16, "max_batch must be 1..16 (skinny kernel)");
@@ -575,6 +589,7 @@ int32_t yscv_hip_decoder_create_kv(const yscv_hip_decoder_config *cfg, int32_t k
   auto *d = new yscv_hip_decoder();
   d->cfg = c;
   d->kv_dtype = kv_dtype;
+  d->generic_attn = generic_attn;
   d->layers.resize(c.n_layers);
   int32_t st = alloc_runtime(d);
   const size_t D = c.d_model;
@@ -888,13 +903,14 @@ int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_g
   YSCV_REQUIRE(step + n_steps <= d->cfg.max_steps, "token history overflow: %d + %d > max_steps %d", step, n_steps,
                d->cfg.max_steps);
   if (use_graph == YSCV_HIP_DECODE_AUTO)  // the fastest path this decoder has for its batch
-    use_graph = (d->batch == 1 && d->persist_ok && d->kv_dtype == YSCV_HIP_KV_F16) ? 2 : 1;
+    use_graph = (d->batch == 1 && d->persist_ok && !d->has_bias && d->kv_dtype == YSCV_HIP_KV_F16) ? 2 : 1;
   d->last_path = use_graph == 2 ? 2 : (use_graph ? 1 : 0);
   if (use_graph == 2) {
     if (d->kv_dtype != YSCV_HIP_KV_F16)
       return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the single-launch decode path reads an fp16 KV cache only");
     if (!d->persist_ok)
       return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the single-launch decode path does not support this model shape");
+    if (d->has_bias) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the single-launch decode path has no q / k / v bias");
     if (d->batch != 1) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "the single-launch decode path runs batch 1 only");
     if (n_steps == 0) return YSCV_HIP_OK;
     // A tag is ((epoch + step) * (layers + 2) + 1 + layer) modulo 2^24.  Before the tag space wraps, the exchange
@@ -1100,6 +1116,102 @@ int32_t yscv_hip_decoder_debug_set_folded_norm(yscv_hip_decoder *d, int32_t on) 
   drop_graph(d);
   d->fold_norm_wanted = on != 0;
   if (d->finalized) YSCV_TRY(finish_setup(d));
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_set_qkv_bias(yscv_hip_decoder *d, int32_t layer, const uint16_t *bias_f16) {
+  YSCV_REQUIRE(d != nullptr, "null decoder");
+  const auto &c = d->cfg;
+  YSCV_REQUIRE(layer >= 0 && layer < c.n_layers, "layer %d out of range", layer);
+  auto &L = d->layers[layer];
+  drop_graph(d);
+  const size_t n = (size_t)(c.n_heads + 2 * c.n_kv_heads) * c.head_dim;
+  if (!bias_f16) {
+    (void)hipFree(L.qkv_bias);
+    L.qkv_bias = nullptr;
+  } else {
+    if (!L.qkv_bias) DEC_HIP(hipMalloc(reinterpret_cast<void **>(&L.qkv_bias), n * 2));
+    DEC_HIP(hipMemcpy(L.qkv_bias, bias_f16, n * 2, hipMemcpyHostToDevice));
+  }
+  d->has_bias = false;
+  for (auto &l : d->layers) d->has_bias = d->has_bias || l.qkv_bias != nullptr;
+  return YSCV_HIP_OK;
+}
+
+// The prompt pass: every projection sees all rows at once (the MFMA GEMM above 16 rows), attention is causal over the
+// cache, and only the last row goes through the final norm and the LM head.
+static int32_t prefill_chunk(yscv_hip_decoder *d, const int32_t *tokens_dev, int rows, int start_pos, bool last, hipStream_t s) {
+  const auto &c = d->cfg;
+  const size_t R = (size_t)rows, D = c.d_model, hq = (size_t)c.n_heads * c.head_dim;
+  const size_t qkv_n = (size_t)(c.n_heads + 2 * c.n_kv_heads) * c.head_dim, ff = c.d_ff;
+  StreamBuf h, t, xn, qkv, ao, gu, act;
+  YSCV_TRY(h.alloc(R * D * 4, s));
+  YSCV_TRY(t.alloc(R * D * 4, s));
+  YSCV_TRY(xn.alloc(R * D * 2, s));
+  YSCV_TRY(qkv.alloc(R * qkv_n * 2, s));
+  YSCV_TRY(ao.alloc(R * hq * 2, s));
+  YSCV_TRY(gu.alloc(R * 2 * ff * 4, s));
+  YSCV_TRY(act.alloc(R * ff * 2, s));
+  YSCV_TRY(launch_embed(tokens_dev, d->emb, rows, (int)D, c.vocab, h.as<float>(), s));
+  for (auto &L : d->layers) {
+    YSCV_TRY(launch_rmsnorm(h.as<float>(), L.attn_norm, rows, (int)D, c.rms_eps, xn.as<_Float16>(), s));
+    YSCV_TRY(int4_run_ws(L.wqkv, xn.p, YSCV_HIP_F16, qkv.p, YSCV_HIP_F16, R, 0, EPI_STORE, nullptr, 0, s));
+    if (L.qkv_bias) YSCV_TRY(launch_bias_add_f16(qkv.as<_Float16>(), L.qkv_bias, R, qkv_n, s));
+    YSCV_TRY(launch_prefill_rope_append(qkv.as<_Float16>(), rows, start_pos, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_theta,
+                                        c.max_ctx, L.kc, L.vc, s));
+    YSCV_TRY(launch_gqa_cache(qkv.as<_Float16>(), L.kc, L.vc, nullptr, rows, start_pos, c.n_heads, c.n_kv_heads, c.head_dim,
+                              c.max_ctx, ao.as<_Float16>(), s));
+    YSCV_TRY(int4_run_ws(L.wo, ao.p, YSCV_HIP_F16, t.p, YSCV_HIP_F32, R, 0, EPI_STORE, nullptr, 0, s));
+    YSCV_TRY(launch_residual_add(h.as<float>(), t.as<float>(), R * D, s));
+    YSCV_TRY(launch_rmsnorm(h.as<float>(), L.ffn_norm, rows, (int)D, c.rms_eps, xn.as<_Float16>(), s));
+    YSCV_TRY(int4_run_ws(L.wgu, xn.p, YSCV_HIP_F16, gu.p, YSCV_HIP_F32, R, 0, EPI_STORE, nullptr, 0, s));
+    YSCV_TRY(launch_swiglu_rows(gu.as<float>(), act.as<_Float16>(), R, ff, s));
+    YSCV_TRY(int4_run_ws(L.wdown, act.p, YSCV_HIP_F16, t.p, YSCV_HIP_F32, R, 0, EPI_STORE, nullptr, 0, s));
+    YSCV_TRY(launch_residual_add(h.as<float>(), t.as<float>(), R * D, s));
+  }
+  if (last) {
+    YSCV_TRY(launch_rmsnorm(h.as<float>() + (R - 1) * D, d->final_norm, 1, (int)D, c.rms_eps, d->xn, s));
+    YSCV_TRY(int4_run_ws(d->lm_head, d->xn, YSCV_HIP_F16, d->logits, YSCV_HIP_F32, 1, 1, EPI_STORE, d->ws, d->ws_bytes, s));
+  }
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_prefill(yscv_hip_decoder *d, const int32_t *tokens_host, int32_t n_tokens, int32_t start_pos,
+                                 void *stream) {
+  YSCV_REQUIRE(d != nullptr && tokens_host != nullptr, "null argument");
+  YSCV_REQUIRE(d->finalized, "decoder weights are not finalized");
+  const auto &c = d->cfg;
+  YSCV_REQUIRE(n_tokens >= 1 && start_pos >= 0, "prefill needs at least one token and a non-negative position");
+  YSCV_REQUIRE((int64_t)start_pos + n_tokens <= c.max_ctx, "KV cache overflow: position %d + %d tokens > max_ctx %d", start_pos,
+               n_tokens, c.max_ctx);
+  for (int32_t i = 0; i < n_tokens; i++)
+    YSCV_REQUIRE(tokens_host[i] >= 0 && tokens_host[i] < c.vocab, "token %d outside the vocabulary (%d)", tokens_host[i], c.vocab);
+  hipStream_t s = as_stream(stream);
+  if (d->kv_dtype != YSCV_HIP_KV_F16) {
+    // the quantised cache appends one row at a time (its row scales cover all kv heads): the prompt goes through the
+    // decode step position by position
+    for (int32_t i = 0; i < n_tokens; i++) {
+      YSCV_TRY(yscv_hip_decoder_reset(d, 1, start_pos + i, tokens_host + i));
+      YSCV_TRY(yscv_hip_decoder_run(d, 1, 1, stream));
+    }
+    return YSCV_HIP_OK;
+  }
+  d->batch = 1;
+  StreamBuf toks;
+  YSCV_TRY(toks.alloc((size_t)n_tokens * 4, s));
+  DEC_HIP(hipMemcpyAsync(toks.p, tokens_host, (size_t)n_tokens * 4, hipMemcpyHostToDevice, s));
+  DEC_HIP(hipStreamSynchronize(s));  // tokens_host is the caller's again
+  constexpr int kChunk = 2048;       // rows per pass: bounds the activation buffers (gate/up in f32: 8 * d_ff bytes per row)
+  for (int32_t r0 = 0; r0 < n_tokens; r0 += kChunk) {
+    const int rows = n_tokens - r0 < kChunk ? n_tokens - r0 : kChunk;
+    YSCV_TRY(prefill_chunk(d, toks.as<int32_t>() + r0, rows, start_pos + r0, r0 + rows == n_tokens, s));
+  }
+  // as after reset(last token, start_pos + n - 1) + one decode step: the pick is the next input, position and step advance
+  hipLaunchKernelGGL(set_counters_kernel, dim3(1), dim3(64), 0, s, d->pos, d->step, start_pos + n_tokens - 1, 0);
+  DEC_HIP(hipGetLastError());
+  YSCV_TRY(launch_argmax(d->logits, 1, c.vocab, d->tokens, d->history, d->step, c.max_steps, s));
+  YSCV_TRY(launch_advance(d->pos, d->step, s));
+  d->last_path = 1;
   return YSCV_HIP_OK;
 }
 

@@ -44,4 +44,15 @@ int32_t launch_argmax(const float *logits, int batch, int vocab, int32_t *tokens
 int32_t launch_advance(int32_t *pos_ptr, int32_t *step_ptr, hipStream_t s);
 int32_t launch_kv_random_fill(_Float16 *buf, size_t n, uint64_t seed, hipStream_t s);
 
+// glue_ops.hip: the general attention kernel over the fp16 cache (any head width that is a multiple of 32 up to 128,
+// any number of query heads per kv head).  pos_ptr != null: `rows` batch rows at the position *pos_ptr (decode);
+// pos_ptr == null: `rows` consecutive positions start_pos .. of batch row 0, causal (prompt pass).
+int32_t launch_gqa_cache(const _Float16 *qkv, const _Float16 *kc, const _Float16 *vc, const int32_t *pos_ptr, int rows,
+                         int start_pos, int hq, int hkv, int hd, int max_ctx, _Float16 *out, hipStream_t s);
+int32_t launch_prefill_rope_append(_Float16 *qkv, int rows, int start_pos, int hq, int hkv, int hd, float theta, int max_ctx,
+                                   _Float16 *kc, _Float16 *vc, hipStream_t s);
+int32_t launch_bias_add_f16(_Float16 *x, const _Float16 *bias, size_t rows, size_t n, hipStream_t s);
+int32_t launch_residual_add(float *h, const float *t, size_t count, hipStream_t s);
+int32_t launch_swiglu_rows(const float *gu, _Float16 *act, size_t rows, size_t ff, hipStream_t s);
+
 }  // namespace yscv

@@ -106,12 +106,16 @@ int32_t yscv_hip_decoder_generate(yscv_hip_decoder *d, const uint32_t *input_ids
   std::vector<uint32_t> tokens(input_ids, input_ids + n_input);
   std::vector<float> logits(vocab);
   uint64_t rng_state = 0xdeadbeefULL;  // generate.rs:68
-  // the prompt goes through the decoder one position at a time; the KV cache then holds positions 0 .. n_input-1
-  for (size_t p = 0; p < n_input; p++) {
-    YSCV_REQUIRE(input_ids[p] < vocab, "prompt token %u outside the vocabulary (%zu)", input_ids[p], vocab);
-    const int32_t tok = (int32_t)input_ids[p];
-    YSCV_TRY(yscv_hip_decoder_reset(d, 1, (int32_t)p, &tok));
-    YSCV_TRY(yscv_hip_decoder_run(d, 1, YSCV_HIP_DECODE_AUTO, nullptr));
+  // the prompt goes through the decoder in one pass (yscv_hip_decoder_prefill: every projection sees all positions at
+  // once); the KV cache then holds positions 0 .. n_input-1 and the logits are those of the last prompt position
+  {
+    std::vector<int32_t> prompt(n_input);
+    for (size_t p = 0; p < n_input; p++) {
+      YSCV_REQUIRE(input_ids[p] < vocab, "prompt token %u outside the vocabulary (%zu)", input_ids[p], vocab);
+      prompt[p] = (int32_t)input_ids[p];
+    }
+    YSCV_REQUIRE(n_input < ((size_t)1 << 31), "prompt too long");
+    YSCV_TRY(yscv_hip_decoder_prefill(d, prompt.data(), (int32_t)n_input, 0, nullptr));
   }
   for (size_t g = 0; g < cfg->max_tokens; g++) {
     YSCV_TRY(yscv_hip_decoder_read_logits(d, logits.data()));

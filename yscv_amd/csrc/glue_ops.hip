@@ -1,0 +1,434 @@
+// The operators between the MatMuls of an exported LLM graph, as stand-alone entry points on device tensors, so
+// that a graph executor stays on the GPU from one projection to the next:
+//   rms_norm   crates/yscv-kernels/src/ops/norm.rs:1431-1518   y = x * (1 / sqrt(mean(x^2) + eps)) * gamma, last axis
+//   rope       crates/yscv-kernels/src/ops/rope.rs:24-117      rotate-half pairs (i, i + d/2), in place on q and k
+//   GroupQueryAttention  crates/yscv-onnx/src/runner/linear.rs:552-646   q [B][Sq][Hq d], k / v [B][Sk][Hkv d],
+//              kv_h = q_h / groups, scores * 1/sqrt(d), max-subtracted softmax, no mask
+// and the general attention kernel behind the last one, which the decoder also uses where its specialised kernels
+// do not apply: any head width that is a multiple of 32 up to 128, any number of query heads per kv head, several
+// query positions per call with a causal limit (prompt ingestion), K / V either as the operator's tensors or as the
+// decoder's fp16 cache.
+//
+// Attention kernel: a workgroup of four waves owns 16 query positions of one head.  Wave w walks the key blocks
+// w, w + 4, ... of 16 positions each:
+//   S^T = K Q^T   rows = positions, columns = queries: hd / 32 x v_mfma_f32_16x16x32_f16, A = 16 cache rows as they lie
+//                 in memory, B = the 16 query rows as they lie in memory; lane (r, c) then holds positions 4c .. 4c+3
+//                 of query r, which is exactly the B operand of the second product
+//   online softmax per query (= per lane column r; the four lane groups c are reduced with two permlane swaps)
+//   O^T += V^T P^T  hd / 16 x v_mfma_f32_16x16x16_f16, A = V^T (the cache keeps eight consecutive positions of one
+//                 channel together, so a lane's four positions are one 8-byte load)
+// and the four waves merge their (max, sum, O) through LDS.  Scores and sums are f32; q, k, v and the softmax weights
+// enter the MFMAs as fp16, like the decoder's own kernels (tolerance-checked against the f32 restatement).
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+#include "int4_common.hpp"
+#include "decoder.hpp"
+#include "kernels.hpp"
+
+namespace yscv {
+
+namespace {
+
+struct GqaArgs {
+  const void *q, *k, *v;
+  void *out;
+  // element strides: q[b * q_b + s * q_s + h * hd + d], same for k (h = kv head) and out; v natural like k, or
+  // v slab: v[b * v_b + kvh * v_h + ((pos / 8) * hd + d) * 8 + pos % 8]
+  long long q_b, q_s, k_b, k_s, k_h, v_b, v_s, v_h, o_b, o_s;
+  int B, Sq, Sk, Hq, Hkv;
+  int causal_base;            // < 0: every query sees all Sk positions; else query s sees positions <= causal_base + s
+  const int32_t *sk_minus_1;  // null, or device word holding Sk - 1 (the decoder's position counter)
+  float scale;
+};
+
+template <typename T>
+__device__ __forceinline__ half8_t load8(const T *p);
+template <>
+__device__ __forceinline__ half8_t load8<_Float16>(const _Float16 *p) {
+  return *reinterpret_cast<const half8_t *>(p);
+}
+template <>
+__device__ __forceinline__ half8_t load8<float>(const float *p) {
+  const float4_t a = *reinterpret_cast<const float4_t *>(p), b = *reinterpret_cast<const float4_t *>(p + 4);
+  return half8_t{(_Float16)a[0], (_Float16)a[1], (_Float16)a[2], (_Float16)a[3],
+                 (_Float16)b[0], (_Float16)b[1], (_Float16)b[2], (_Float16)b[3]};
+}
+template <typename T>
+__device__ __forceinline__ void store4(T *p, float a, float b, float c, float d);
+template <>
+__device__ __forceinline__ void store4<_Float16>(_Float16 *p, float a, float b, float c, float d) {
+  *reinterpret_cast<half4_t *>(p) = half4_t{(_Float16)a, (_Float16)b, (_Float16)c, (_Float16)d};
+}
+template <>
+__device__ __forceinline__ void store4<float>(float *p, float a, float b, float c, float d) {
+  *reinterpret_cast<float4_t *>(p) = float4_t{a, b, c, d};
+}
+
+constexpr int GQA_WAVES = 4;
+
+__device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
+
+template <int HD, typename TQ, typename TKV, typename TO, bool V_SLAB>
+__global__ void __launch_bounds__(64 * GQA_WAVES) gqa_generic_kernel(GqaArgs p) {
+  static_assert(HD % 32 == 0 && HD >= 32 && HD <= 128, "head width (the merge buffer must fit the static LDS limit)");
+  constexpr int KK = HD / 32, DT = HD / 16;
+  __shared__ float m_s[GQA_WAVES][16], l_s[GQA_WAVES][16];
+  __shared__ float o_s[GQA_WAVES][16][HD + 4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, c = lane >> 4;
+  const int q0 = blockIdx.x * 16, h = blockIdx.y, b = blockIdx.z;
+  const int kvh = h / (p.Hq / p.Hkv);
+  const int Sk = p.sk_minus_1 ? *p.sk_minus_1 + 1 : p.Sk;
+  // query r of this tile (rows past the end repeat the last one and are not stored)
+  const int qi = min(q0 + r, p.Sq - 1);
+  const int lim_q = p.causal_base < 0 ? Sk - 1 : min(Sk - 1, p.causal_base + qi);           // last position query r sees
+  const int lim_tile = p.causal_base < 0 ? Sk - 1 : min(Sk - 1, p.causal_base + min(q0 + 15, p.Sq - 1));
+  const int nblocks = lim_tile / 16 + 1;
+
+  const TQ *qrow = static_cast<const TQ *>(p.q) + (size_t)b * p.q_b + (size_t)qi * p.q_s + (size_t)h * HD;
+  half8_t qf[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++) qf[kk] = load8<TQ>(qrow + 32 * kk + 8 * c);
+
+  const TKV *kbase = static_cast<const TKV *>(p.k) + (size_t)b * p.k_b + (size_t)kvh * p.k_h;
+  const TKV *vbase = static_cast<const TKV *>(p.v) + (size_t)b * p.v_b + (size_t)kvh * p.v_h;
+  float m_run = -INFINITY, l_run = 0.0f;
+  float4_t o_acc[DT];
+#pragma unroll
+  for (int t = 0; t < DT; t++) o_acc[t] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+  for (int blk = wave; blk < nblocks; blk += GQA_WAVES) {
+    const int p0 = blk * 16;
+    // ---- S^T: lane (r, c) as A supplies cache row p0 + r, channels 32 kk + 8c .. + 7 (rows past the end repeat the last)
+    const TKV *krow = kbase + (size_t)min(p0 + r, Sk - 1) * p.k_s;
+    float4_t s = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) s = __builtin_amdgcn_mfma_f32_16x16x32_f16(load8<TKV>(krow + 32 * kk + 8 * c), qf[kk], s, 0, 0, 0);
+    // lane (r, c): query r, positions p0 + 4c + e
+    float sv[4], mx = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      sv[e] = (p0 + 4 * c + e <= lim_q) ? s[e] * p.scale : -INFINITY;
+      mx = fmaxf(mx, sv[e]);
+    }
+    mx = max_xor16_xor32(mx);
+    const float m_new = fmaxf(m_run, mx);
+    float pe[4], sum = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      pe[e] = (sv[e] == -INFINITY) ? 0.0f : __expf(sv[e] - m_new);
+      sum += pe[e];
+    }
+    sum = sum_xor16_xor32(sum);
+    const float alpha = (m_run == -INFINITY) ? 0.0f : __expf(m_run - m_new);
+    l_run = l_run * alpha + sum;
+    m_run = m_new;
+    const half4_t pf = {(_Float16)pe[0], (_Float16)pe[1], (_Float16)pe[2], (_Float16)pe[3]};
+    // ---- O^T += V^T P^T: lane (r, c) as A supplies channel 16 t + r at positions p0 + 4c .. + 3
+#pragma unroll
+    for (int t = 0; t < DT; t++) {
+      half4_t vf;
+      if constexpr (V_SLAB) {
+        // positions past the end of the context lie inside the allocated slab and meet weight 0 -- but 0 * NaN would
+        // poison the sum, so they are blanked
+        const _Float16 *vp = reinterpret_cast<const _Float16 *>(vbase) + ((size_t)((p0 + 4 * c) >> 3) * HD + 16 * t + r) * 8 + ((4 * c) & 7);
+        vf = *reinterpret_cast<const half4_t *>(vp);
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (p0 + 4 * c + e >= Sk) vf[e] = (_Float16)0.0f;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int pos = p0 + 4 * c + e;
+          vf[e] = pos < Sk ? (_Float16)vbase[(size_t)pos * p.v_s + 16 * t + r] : (_Float16)0.0f;
+        }
+      }
+      o_acc[t] = o_acc[t] * alpha;
+      o_acc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(vf, pf, o_acc[t], 0, 0, 0);
+    }
+  }
+  // ---- merge the four waves: lane (r, c) holds O^T[16 t + 4c + e][query r]
+  if (c == 0) {
+    m_s[wave][r] = m_run;
+    l_s[wave][r] = l_run;
+  }
+#pragma unroll
+  for (int t = 0; t < DT; t++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) o_s[wave][r][16 * t + 4 * c + e] = o_acc[t][e];
+  __syncthreads();
+  TO *obase = static_cast<TO *>(p.out) + (size_t)b * p.o_b + (size_t)h * HD;
+  for (int idx = tid; idx < 16 * (HD / 4); idx += 64 * GQA_WAVES) {
+    const int qq = idx / (HD / 4), d4 = (idx % (HD / 4)) * 4;
+    if (q0 + qq >= p.Sq) continue;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < GQA_WAVES; w++) M = fmaxf(M, m_s[w][qq]);
+    float L = 0.0f, o[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int w = 0; w < GQA_WAVES; w++) {
+      const float f = (m_s[w][qq] == -INFINITY) ? 0.0f : __expf(m_s[w][qq] - M);
+      L += l_s[w][qq] * f;
+#pragma unroll
+      for (int e = 0; e < 4; e++) o[e] += o_s[w][qq][d4 + e] * f;
+    }
+    const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+    store4<TO>(obase + (size_t)(q0 + qq) * p.o_s + d4, o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv);
+  }
+}
+
+template <typename TQ, typename TKV, typename TO, bool V_SLAB>
+int32_t gqa_launch(const GqaArgs &a, int hd, hipStream_t s) {
+  const dim3 grid((unsigned)((a.Sq + 15) / 16), (unsigned)a.Hq, (unsigned)a.B), block(64 * GQA_WAVES);
+  switch (hd) {
+    case 32: hipLaunchKernelGGL((gqa_generic_kernel<32, TQ, TKV, TO, V_SLAB>), grid, block, 0, s, a); break;
+    case 64: hipLaunchKernelGGL((gqa_generic_kernel<64, TQ, TKV, TO, V_SLAB>), grid, block, 0, s, a); break;
+    case 96: hipLaunchKernelGGL((gqa_generic_kernel<96, TQ, TKV, TO, V_SLAB>), grid, block, 0, s, a); break;
+    case 128: hipLaunchKernelGGL((gqa_generic_kernel<128, TQ, TKV, TO, V_SLAB>), grid, block, 0, s, a); break;
+    default: return set_error(YSCV_HIP_ERR_UNSUPPORTED, "attention: head width %d (supported: 32, 64, 96, 128)", hd);
+  }
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+// ---- RMSNorm over the last axis, f32 in and out ---------------------------------------------------------------
+__global__ void __launch_bounds__(256) rms_norm_f32_kernel(const float *__restrict__ x, const float *__restrict__ gamma, int d,
+                                                           float eps, float *__restrict__ y) {
+  __shared__ float red[4];
+  const float *row = x + (size_t)blockIdx.x * d;
+  float *out = y + (size_t)blockIdx.x * d;
+  float ss = 0.0f;
+  for (int i = threadIdx.x; i < d; i += 256) ss += row[i] * row[i];
+  ss = wave_sum(ss);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  ss = red[0] + red[1] + red[2] + red[3];
+  // rms = sqrt(sum / n + eps); inv_rms = 1 / rms; y = x * inv_rms * gamma (ops/norm.rs:1507-1516, in that order)
+  const float inv_rms = 1.0f / sqrtf(ss / (float)d + eps);
+  for (int i = threadIdx.x; i < d; i += 256) out[i] = row[i] * inv_rms * gamma[i];
+}
+
+// ---- rotate-half RoPE in place on [seq][heads][d] f32 ------------------------------------------------------------
+__global__ void __launch_bounds__(64) rope_f32_kernel(float *__restrict__ x, int heads, int d, int seq_offset, float theta) {
+  const int pos = blockIdx.y, head = blockIdx.x;
+  float *row = x + ((size_t)pos * heads + head) * d;
+  const int half_d = d / 2;
+  const float abs_pos = (float)(pos + seq_offset);
+  for (int i = threadIdx.x; i < half_d; i += 64) {
+    const float inv_freq = 1.0f / powf(theta, 2.0f * (float)i / (float)d);
+    float sn, cs;
+    sincosf(inv_freq * abs_pos, &sn, &cs);
+    const float x0 = row[i], x1 = row[i + half_d];
+    row[i] = x0 * cs - x1 * sn;
+    row[i + half_d] = x0 * sn + x1 * cs;
+  }
+}
+
+
+// ---- small kernels of the prompt pass (rows = consecutive positions of one sequence) ------------------------------
+// RoPE on the q and k heads of every row (row i sits at position start_pos + i), k and v appended to batch row 0 of
+// the cache: the arithmetic of the decode step's rope + append, one launch for all rows.
+__global__ void __launch_bounds__(64) prefill_rope_append_kernel(_Float16 *__restrict__ qkv, int start_pos, int hq, int hkv, int hd,
+                                                                 float theta, int max_ctx, _Float16 *__restrict__ kc,
+                                                                 _Float16 *__restrict__ vc) {
+  const int row = blockIdx.y, slot = blockIdx.x;
+  const int pos = start_pos + row;
+  _Float16 *src = qkv + (size_t)row * (hq + 2 * hkv) * hd + (size_t)slot * hd;
+  const int half_d = hd / 2;
+  if (slot < hq + hkv) {
+    for (int i = threadIdx.x; i < half_d; i += 64) {
+      const float inv_freq = 1.0f / powf(theta, (float)(2 * i) / (float)hd);
+      float sn, cs;
+      sincosf(inv_freq * (float)pos, &sn, &cs);
+      const float x0 = (float)src[i], x1 = (float)src[i + half_d];
+      float f0 = fmaf(x0, cs, -(x1 * sn)), f1 = fmaf(x0, sn, x1 * cs);
+      asm volatile("" : "+v"(f0), "+v"(f1));  // the f32 value exists before it is narrowed (no mixed-precision fma)
+      const _Float16 y0 = (_Float16)f0, y1 = (_Float16)f1;
+      if (slot < hq) {
+        src[i] = y0;
+        src[i + half_d] = y1;
+      } else {
+        _Float16 *dst = kc + ((size_t)(slot - hq) * max_ctx + pos) * hd;
+        dst[i] = y0;
+        dst[i + half_d] = y1;
+      }
+    }
+  } else {
+    _Float16 *dst = vc + (((size_t)(slot - hq - hkv) * (max_ctx / 8) + pos / 8) * hd) * 8 + (pos & 7);
+    for (int i = threadIdx.x; i < hd; i += 64) dst[(size_t)i * 8] = src[i];
+  }
+}
+
+__global__ void bias_add_f16_kernel(_Float16 *__restrict__ x, const _Float16 *__restrict__ bias, size_t rows, size_t n) {
+  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < rows * n; idx += (size_t)gridDim.x * blockDim.x)
+    x[idx] = (_Float16)((float)x[idx] + (float)bias[idx % n]);
+}
+
+__global__ void residual_add_kernel(float *__restrict__ h, const float *__restrict__ t, size_t count) {
+  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < count; idx += (size_t)gridDim.x * blockDim.x) h[idx] += t[idx];
+}
+
+// gu [rows][2 ff] f32 with gate_i, up_i interleaved -> act [rows][ff] fp16 = silu(gate) * up
+__global__ void swiglu_rows_kernel(const float *__restrict__ gu, _Float16 *__restrict__ act, size_t count) {
+  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < count; idx += (size_t)gridDim.x * blockDim.x) {
+    const float g = gu[2 * idx], u = gu[2 * idx + 1];
+    act[idx] = (_Float16)(silu(g) * u);
+  }
+}
+
+unsigned flat_grid(size_t n) {
+  const size_t b = (n + 255) / 256;
+  return (unsigned)(b > 65535 ? 65535 : (b < 1 ? 1 : b));
+}
+
+}  // namespace
+
+int32_t launch_prefill_rope_append(_Float16 *qkv, int rows, int start_pos, int hq, int hkv, int hd, float theta, int max_ctx,
+                                   _Float16 *kc, _Float16 *vc, hipStream_t s) {
+  hipLaunchKernelGGL(prefill_rope_append_kernel, dim3(hq + 2 * hkv, rows), dim3(64), 0, s, qkv, start_pos, hq, hkv, hd, theta, max_ctx,
+                     kc, vc);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+int32_t launch_bias_add_f16(_Float16 *x, const _Float16 *bias, size_t rows, size_t n, hipStream_t s) {
+  hipLaunchKernelGGL(bias_add_f16_kernel, dim3(flat_grid(rows * n)), dim3(256), 0, s, x, bias, rows, n);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+int32_t launch_residual_add(float *h, const float *t, size_t count, hipStream_t s) {
+  hipLaunchKernelGGL(residual_add_kernel, dim3(flat_grid(count)), dim3(256), 0, s, h, t, count);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+int32_t launch_swiglu_rows(const float *gu, _Float16 *act, size_t rows, size_t ff, hipStream_t s) {
+  hipLaunchKernelGGL(swiglu_rows_kernel, dim3(flat_grid(rows * ff)), dim3(256), 0, s, gu, act, rows * ff);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+// Attention of `rows` query rows against the decoder's fp16 cache of one layer.  qkv: [rows][(hq + 2 hkv) hd] with
+// the query heads already rotated; out: [rows][hq hd].
+//   decode (pos_ptr != null): row b is batch row b at the position *pos_ptr, cache rows [0, *pos_ptr];
+//   prompt ingestion (pos_ptr == null): the rows are consecutive positions start_pos .. of batch row 0, row i sees
+//   cache rows [0, start_pos + i].
+int32_t launch_gqa_cache(const _Float16 *qkv, const _Float16 *kc, const _Float16 *vc, const int32_t *pos_ptr, int rows,
+                         int start_pos, int hq, int hkv, int hd, int max_ctx, _Float16 *out, hipStream_t s) {
+  GqaArgs a{};
+  const long long row_elems = (long long)(hq + 2 * hkv) * hd;
+  a.q = qkv;
+  a.k = kc;
+  a.v = vc;
+  a.out = out;
+  a.k_s = hd;
+  a.k_h = (long long)max_ctx * hd;
+  a.v_h = (long long)max_ctx * hd;
+  a.v_s = 0;
+  a.Hq = hq;
+  a.Hkv = hkv;
+  a.scale = 1.0f / sqrtf((float)hd);
+  if (pos_ptr) {
+    a.B = rows;
+    a.Sq = 1;
+    a.Sk = 1;
+    a.sk_minus_1 = pos_ptr;
+    a.causal_base = -1;
+    a.q_b = row_elems;
+    a.q_s = 0;
+    a.k_b = (long long)hkv * max_ctx * hd;
+    a.v_b = a.k_b;
+    a.o_b = (long long)hq * hd;
+    a.o_s = 0;
+  } else {
+    a.B = 1;
+    a.Sq = rows;
+    a.Sk = start_pos + rows;
+    a.sk_minus_1 = nullptr;
+    a.causal_base = start_pos;
+    a.q_b = 0;
+    a.q_s = row_elems;
+    a.k_b = 0;
+    a.v_b = 0;
+    a.o_b = 0;
+    a.o_s = (long long)hq * hd;
+  }
+  return gqa_launch<_Float16, _Float16, _Float16, true>(a, hd, s);
+}
+
+extern "C" {
+
+int32_t yscv_hip_rms_norm_dev(const float *x, const float *gamma, size_t rows, size_t d, float eps, float *y, void *stream) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(x && gamma && y, "null argument");
+  YSCV_REQUIRE(std::isfinite(eps) && eps > 0.0f, "rms_norm: epsilon must be finite and > 0");
+  YSCV_REQUIRE(d > 0 && d < ((size_t)1 << 31) && rows < ((size_t)1 << 31), "rms_norm: bad shape %zu x %zu", rows, d);
+  if (rows == 0) return YSCV_HIP_OK;
+  hipLaunchKernelGGL(rms_norm_f32_kernel, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), x, gamma, (int)d, eps, y);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_rope_dev(float *q, float *k, size_t num_q_heads, size_t num_kv_heads, size_t d_head, size_t seq_len,
+                          size_t seq_offset, float theta, void *stream) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(q && k, "null argument");
+  YSCV_REQUIRE(d_head % 2 == 0 && d_head > 0, "rope: d_head must be even (got %zu)", d_head);
+  YSCV_REQUIRE(seq_len + seq_offset < ((size_t)1 << 24), "rope: position beyond 2^24");
+  YSCV_REQUIRE(seq_len < 65536 && num_q_heads < ((size_t)1 << 31) && num_kv_heads < ((size_t)1 << 31), "rope: shape too large");
+  if (seq_len == 0) return YSCV_HIP_OK;
+  hipStream_t s = as_stream(stream);
+  if (num_q_heads > 0) {
+    hipLaunchKernelGGL(rope_f32_kernel, dim3((unsigned)num_q_heads, (unsigned)seq_len), dim3(64), 0, s, q, (int)num_q_heads, (int)d_head,
+                       (int)seq_offset, theta);
+    YSCV_HIP_TRY(hipGetLastError());
+  }
+  if (num_kv_heads > 0) {
+    hipLaunchKernelGGL(rope_f32_kernel, dim3((unsigned)num_kv_heads, (unsigned)seq_len), dim3(64), 0, s, k, (int)num_kv_heads, (int)d_head,
+                       (int)seq_offset, theta);
+    YSCV_HIP_TRY(hipGetLastError());
+  }
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_gqa_attention_dev(const float *q, const float *k, const float *v, size_t batch, size_t seq_q, size_t seq_k,
+                                   size_t num_q_heads, size_t num_kv_heads, size_t d_head, float *out, void *stream) {
+  YSCV_TRY(ensure_context(nullptr));
+  YSCV_REQUIRE(q && k && v && out, "null argument");
+  YSCV_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0,
+               "GroupQueryAttention: %zu query heads over %zu kv heads", num_q_heads, num_kv_heads);
+  YSCV_REQUIRE(batch < 65536 && num_q_heads < 65536 && seq_q < ((size_t)1 << 24) && seq_k < ((size_t)1 << 24),
+               "GroupQueryAttention: shape too large");
+  YSCV_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(out)) & 15) == 0,
+               "GroupQueryAttention: tensors must be 16-byte aligned");
+  if (batch == 0 || seq_q == 0) return YSCV_HIP_OK;
+  YSCV_REQUIRE(seq_k > 0, "GroupQueryAttention: no key positions");
+  GqaArgs a{};
+  a.q = q;
+  a.k = k;
+  a.v = v;
+  a.out = out;
+  a.q_s = (long long)(num_q_heads * d_head);
+  a.q_b = (long long)seq_q * a.q_s;
+  a.k_s = (long long)(num_kv_heads * d_head);
+  a.k_b = (long long)seq_k * a.k_s;
+  a.k_h = (long long)d_head;
+  a.v_s = a.k_s;
+  a.v_b = a.k_b;
+  a.v_h = a.k_h;
+  a.o_s = a.q_s;
+  a.o_b = a.q_b;
+  a.B = (int)batch;
+  a.Sq = (int)seq_q;
+  a.Sk = (int)seq_k;
+  a.Hq = (int)num_q_heads;
+  a.Hkv = (int)num_kv_heads;
+  a.causal_base = -1;
+  a.sk_minus_1 = nullptr;
+  a.scale = 1.0f / sqrtf((float)d_head);
+  return gqa_launch<float, float, float, false>(a, (int)d_head, as_stream(stream));
+}
+
+}  // extern "C"
+
+}  // namespace yscv

@@ -37,6 +37,16 @@ class Decoder:
         g = np.ascontiguousarray(gamma, np.float32)
         lib().decoder_set_norm(self._h, int(layer), NORMS[kind], _p(g))
 
+    def set_qkv_bias(self, layer, bias16):
+        """Bias of the fused q / k / v projection of one layer: fp16 [(n_heads + 2 n_kv_heads) * head_dim], or None."""
+        if bias16 is None:
+            lib().decoder_set_qkv_bias(self._h, int(layer), None)
+            return
+        b = np.ascontiguousarray(bias16)
+        c = self.cfg
+        assert b.dtype == np.float16 and b.size == (c["n_heads"] + 2 * c["n_kv_heads"]) * c["head_dim"]
+        lib().decoder_set_qkv_bias(self._h, int(layer), _p(b))
+
     def set_embedding(self, table16):
         t = np.ascontiguousarray(table16)
         assert t.dtype == np.float16
@@ -68,6 +78,13 @@ class Decoder:
         t = np.ascontiguousarray(tokens, np.int32)
         self.batch = t.size
         lib().decoder_reset(self._h, int(t.size), int(start_pos), _p(t))
+
+    def prefill(self, tokens, start_pos=0, stream=None):
+        """yscv_hip_decoder_prefill: the prompt in one pass; afterwards batch 1, the pick of the last position is the
+        next input token and token 0 of the history, position start_pos + len(tokens)."""
+        t = np.ascontiguousarray(tokens, np.int32)
+        self.batch = 1
+        lib().decoder_prefill(self._h, _p(t), int(t.size), int(start_pos), C.c_void_p(stream) if stream else None)
 
     def run(self, n_steps, use_graph=True, stream=None, persistent=False, auto=False):
         """use_graph: replay one captured HIP graph per step; persistent: run all steps inside one

@@ -272,3 +272,46 @@ def exec_dynamic_quantize_linear(x):
     sz = torch.empty(2, device=x.device, dtype=torch.float32)
     lib().exec_dynamic_quantize_linear(_p(x), _sz(x.numel()), _p(y), _p(sz[0:1]), _p(sz[1:2]), _stream_ptr())
     return y, sz[0:1], sz[1:2]
+
+
+# ---- the operators between the MatMuls of an LLM graph (device tensors in, device tensors out) ----------------------
+def rms_norm(x, gamma, eps: float):
+    """rms_norm_last_dim (crates/yscv-kernels/src/ops/norm.rs:1431-1518) over the last axis of a CUDA f32 tensor."""
+    import torch
+
+    x = _dev_f32(x, "x")
+    gamma = _dev_f32(gamma, "gamma")
+    d = x.shape[-1]
+    if gamma.ndim != 1 or gamma.shape[0] != d:
+        raise ValueError(f"gamma must be [{d}], got {tuple(gamma.shape)}")
+    y = torch.empty_like(x)
+    lib().rms_norm_dev(_p(x), _p(gamma), _sz(x.numel() // d if d else 0), _sz(d), C.c_float(eps), _p(y), _stream_ptr())
+    return y
+
+
+def apply_rotary_embedding(q, k, num_q_heads: int, num_kv_heads: int, d_head: int, seq_len: int, seq_offset: int, theta: float):
+    """apply_rotary_embedding (crates/yscv-kernels/src/ops/rope.rs:24-117), in place on CUDA f32 tensors
+    q [seq_len][num_q_heads][d_head] and k [seq_len][num_kv_heads][d_head]."""
+    for t, heads, name in ((q, num_q_heads, "q"), (k, num_kv_heads, "k")):
+        if not (t.is_cuda and t.is_contiguous() and t.numel() == seq_len * heads * d_head):
+            raise ValueError(f"{name}: expected a contiguous CUDA tensor of {seq_len} x {heads} x {d_head} values")
+        _dev_f32(t, name)
+    lib().rope_dev(_p(q), _p(k), _sz(num_q_heads), _sz(num_kv_heads), _sz(d_head), _sz(seq_len), _sz(seq_offset), C.c_float(theta),
+                   _stream_ptr())
+
+
+def exec_grouped_query_attention(q, k, v, num_heads: int, kv_num_heads: int | None = None):
+    """exec_grouped_query_attention (crates/yscv-onnx/src/runner/linear.rs:552-646): q [B][Sq][Hq d], k / v [B][Sk][Hkv d]
+    CUDA f32 tensors -> [B][Sq][Hq d]."""
+    import torch
+
+    q, k, v = _dev_f32(q, "q"), _dev_f32(k, "k"), _dev_f32(v, "v")
+    kv_num_heads = num_heads if kv_num_heads is None else kv_num_heads
+    B, Sq, Sk = q.shape[0], q.shape[1], k.shape[1]
+    d_head = q.shape[2] // num_heads
+    if k.shape != (B, Sk, kv_num_heads * d_head) or v.shape != k.shape or q.shape[2] != num_heads * d_head:
+        raise ValueError("GroupQueryAttention: inconsistent shapes")
+    out = torch.empty_like(q)
+    lib().gqa_attention_dev(_p(q), _p(k), _p(v), _sz(B), _sz(Sq), _sz(Sk), _sz(num_heads), _sz(kv_num_heads), _sz(d_head), _p(out),
+                            _stream_ptr())
+    return out
