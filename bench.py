@@ -455,6 +455,58 @@ def extra_kernels(torch, stream_ptr):
     return out
 
 
+def bench_prefill(dec, torch, cfg, n_tokens, params):
+    """The prompt phase llm-bench times apart from the decode phase (apps/llm-bench/src/main.rs:403-470): n_tokens prompt
+    tokens through yscv_hip_decoder_prefill in one pass (MFMA GEMM projections, causal attention, cache filled)."""
+    import numpy as np
+
+    prompt = np.random.default_rng(11).integers(0, cfg["vocab"], n_tokens).astype(np.int32)
+    dec.prefill(prompt)  # warm-up: kernel images, the stream-ordered pool's first allocations
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    reps = 3
+    for _ in range(reps):
+        dec.prefill(prompt)
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / reps
+    fl = 2.0 * (params - cfg["vocab"] * cfg["d_model"]) * n_tokens  # the LM head sees the last row only
+    return {"ms": round(t * 1e3, 2), "prompt_tok/s": round(n_tokens / t, 0), "TFLOP/s_projections": round(fl / t / 1e12, 1),
+            "frac_of_mfma_peak": round(fl / t / 1e12 / MFMA_BF16_PEAK, 4),
+            "note": "host-timed whole call (token upload, per-call scratch from the stream-ordered pool, every launch), "
+                    "one pass over all 32 layers; feeding the same prompt through the decode step takes n x ms_per_step"}
+
+
+def bench_reference_model(torch):
+    """The model the reference publishes its own llm-bench numbers on (apps/llm-bench/COMPARISON.md:9-12: 24 layers,
+    hidden 1024, 2 kv heads of 64, a 43-token prompt, 16 greedy tokens; there on a 12-thread Zen 4 with int4 group 32:
+    prefill 1939 ms, decode 3.53 tok/s), random weights of that shape: head_dim 64 with eight query heads per kv head
+    runs on the general attention kernel."""
+    import numpy as np
+
+    from yscv_amd.decoder import Decoder
+
+    cfg = dict(n_layers=24, d_model=1024, n_heads=16, n_kv_heads=2, head_dim=64, d_ff=2816, vocab=151936, group_size=32,
+               max_batch=1, max_ctx=256, max_steps=32, rope_theta=1000000.0, rms_eps=1e-6)
+    dec = Decoder(**cfg)
+    dec.init_random(seed=3, nibbles=(1, 15))
+    prompt = np.random.default_rng(12).integers(0, cfg["vocab"], 43).astype(np.int32)
+    out = {}
+    for _ in range(2):  # the first round warms up (graph capture, kernel images)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dec.prefill(prompt)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        dec.run(16, auto=True)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        out = {"prefill_ms_43_tokens": round((t1 - t0) * 1e3, 3), "decode_ms_16_tokens": round((t2 - t1) * 1e3, 3),
+               "decode_tok/s": round(16 / (t2 - t1), 1), "decode_path": {1: "one HIP-graph replay per step", 2: "single launch"}[dec.last_path()]}
+    out["note"] = "host-timed like llm-bench (prefill and decode apart); random weights, FFN width 2816 assumed"
+    dec.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -589,8 +641,12 @@ def main():
                 sweep[f"batch{bsz}"] = {"tok/s": round(bsz * min(args.steps, 64) / dtb, 1),
                                         "ms_per_step": round(dtb / min(args.steps, 64) * 1e3, 4)}
             extra["decode_batch_sweep"] = sweep
+    if not args.no_extra:
+        extra["prefill_2048_tokens"] = bench_prefill(dec, torch, cfg, 2048, params)
     del dec
     torch.cuda.empty_cache()
+    if not args.no_extra:
+        extra["reference_bench_model_24L_h1024_16q2kv_hd64"] = bench_reference_model(torch)
     if not args.no_extra and args.batch != 16:
         # the same batch-16 run with the int8 KV cache (llm-bench --kv-dtype i8): half the cache bytes per step
         dec8 = Decoder(kv_dtype="i8", **cfg)
