@@ -81,3 +81,17 @@ def copies_of_inflight_registers(asm_text):
                     vm = [(ln, rs - dst) for ln, rs in vm]
                     lg = [(ln, rs - dst) for ln, rs in lg]
     return found
+
+
+def scratch_bytes_per_kernel(asm_text):
+    """{kernel symbol: scratch bytes per lane} from the resource comments hipcc writes behind every kernel."""
+    out, name = {}, None
+    for l in asm_text.split("\n"):
+        m = re.match(r"^(_Z\w+):", l)
+        if m:
+            name = m.group(1)
+        m = re.match(r"^; ScratchSize: (\d+)", l)
+        if m and name:
+            out[name] = int(m.group(1))
+            name = None
+    return out

@@ -320,6 +320,11 @@ __global__ void __launch_bounds__(I8R_THREADS) i8_gemm_ring_kernel(I8Args p, int
   static_assert(((MT + NT) * KS) % 2 == 0 && S >= 2 && S <= 7 && (S - 1) * PER_WAVE < 64, "vmcnt budget");
   constexpr int RS32 = BN * 4 + 16, RS8 = BN + 16;  // row strides of the C tile in LDS (odd multiples of 16 B)
   static_assert(BM * RS32 <= S * STAGE, "the C tile reuses the ring");
+  // Registers of a compute lane: accumulators, two fragment sets, the epilogue's per-column terms, addresses.  With
+  // eight waves per workgroup a wave has 256; a tile that needs more spills, and this pipeline (literal wait counts,
+  // registers of pending LDS reads named in asm statements) is not written for spill code: a 256 x 128 tile
+  // (MT 8, NT 4) comes to 128 + 96 + 48 + ~16 = 288 and was measured by the compiler at 256 + 29 spilled.
+  static_assert(MT * NT * 4 + 2 * (MT + NT) * 4 + 3 * NT * 4 + 16 <= 256, "tile too large for the register file");
   extern __shared__ __attribute__((aligned(1024))) uint8_t i8_ring[];
   const uint32_t lds0 = (uint32_t)(size_t)i8_ring;
   const int tid = threadIdx.x;
@@ -620,7 +625,7 @@ int32_t launch_i8_gemm(const void *a, int a_is_u8, int a_zp, const yscv_hip_i8_w
     YSCV_TRY(ensure_context(&ctx));
     const size_t big_tiles = ceil_div(m, (size_t)128) * ceil_div(b->n, (size_t)128);
     const bool wide_a = b->k % 128 == 0;  // k-steps come in pairs: A is fetched as whole 128-byte lines
-    if (big_tiles >= (size_t)ctx->num_cus)
+if (big_tiles >= (size_t)ctx->num_cus)
       return wide_a ? launch_ring<4, 4, 2, 4, true>(p, m, b->n, s) : launch_ring<4, 4, 2, 4, false>(p, m, b->n, s);
     return wide_a ? launch_ring<2, 4, 4, 3, true>(p, m, b->n, s) : launch_ring<2, 4, 4, 3, false>(p, m, b->n, s);
   }
