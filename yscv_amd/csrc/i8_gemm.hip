@@ -625,7 +625,7 @@ int32_t launch_i8_gemm(const void *a, int a_is_u8, int a_zp, const yscv_hip_i8_w
     YSCV_TRY(ensure_context(&ctx));
     const size_t big_tiles = ceil_div(m, (size_t)128) * ceil_div(b->n, (size_t)128);
     const bool wide_a = b->k % 128 == 0;  // k-steps come in pairs: A is fetched as whole 128-byte lines
-if (big_tiles >= (size_t)ctx->num_cus)
+    if (big_tiles >= (size_t)ctx->num_cus)
       return wide_a ? launch_ring<4, 4, 2, 4, true>(p, m, b->n, s) : launch_ring<4, 4, 2, 4, false>(p, m, b->n, s);
     return wide_a ? launch_ring<2, 4, 4, 3, true>(p, m, b->n, s) : launch_ring<2, 4, 4, 3, false>(p, m, b->n, s);
   }
