@@ -518,6 +518,9 @@ def main():
     ap.add_argument("--extra-only", action="store_true",
                     help="run only the stand-alone kernels of BASELINE configs 1, 2, 3 and 5 and print their figures "
                          "(the run the rocprofv3 summaries of those kernels are taken from)")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the prompt phase (2048 tokens through yscv_hip_decoder_prefill) and print its figures "
+                         "(the run the rocprofv3 summary of the prompt pass is taken from)")
     ap.add_argument("--graph-path", action="store_true",
                     help="time the multi-kernel path (one HIP-graph replay per step) instead of the single-launch kernel")
     ap.add_argument("--no-check", action="store_true",
@@ -562,6 +565,9 @@ def main():
     dec.fill_kv_random(seed=2)
     w_bytes, params = decode_bytes_per_step(cfg)
     assert dec.weight_bytes() >= w_bytes
+    if args.prefill_only:
+        print(json.dumps({"extra": {"prefill_2048_tokens": bench_prefill(dec, torch, cfg, 2048, params)}}))
+        return
 
     persistent = args.batch == 1 and not args.graph_path
     check = check_single_launch(dec, torch) if persistent and not args.no_check else None

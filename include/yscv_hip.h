@@ -147,12 +147,14 @@ int32_t yscv_hip_int4_gemv(const yscv_hip_int4_weight *w, const void *x_dev, int
 int32_t yscv_hip_int4_gemm(const yscv_hip_int4_weight *w, const void *x_dev, int32_t x_dtype,
                            void *y_dev, int32_t y_dtype, size_t m, void *stream);
 
-/* The skinny kernel (m <= 16) with a fused epilogue -- the "bias / residual / activation fusion" the reference
- * plans for its int4 MatMul (docs/int4-quant-pipeline-plan.md:45-51); the decode loop uses exactly these.
+/* The int4 matmul with a fused epilogue -- the "bias / residual / activation fusion" the reference plans for its
+ * int4 MatMul (docs/int4-quant-pipeline-plan.md:45-51); the decode loop and the prompt pass use exactly these.  Up to
+ * 16 rows on the skinny kernel (any activation type); above 16 rows on the LDS-ring MFMA GEMM, fp16 / bf16
+ * activations only (f32 activations with ADD_F32 or SWIGLU above 16 rows: INVALID_ARG).
  *   STORE    y[m][n] = x W^T                       (same as yscv_hip_int4_gemv)
  *   ADD_F32  y[m][n] += x W^T, y_dtype must be F32   (projection + residual add)
  *   SWIGLU   rows 2i / 2i+1 of W are gate_i / up_i; y[m][n/2] = silu(gate) * up   (n even)
- * Results follow the skinny kernel's summation order, within the int4 tolerance of the unfused call. */
+ * Results follow the summation order of the kernel that runs, within the int4 tolerance of the unfused call. */
 #define YSCV_HIP_EPILOGUE_STORE 0
 #define YSCV_HIP_EPILOGUE_ADD_F32 1
 #define YSCV_HIP_EPILOGUE_SWIGLU 2

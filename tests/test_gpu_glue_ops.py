@@ -77,6 +77,9 @@ def test_rope_matches_the_restatement(ops, hq, hkv, d, seq, offset, theta):
     (2, 17, 300, 6, 2, 128),    # three query heads per kv head, more than one query tile
     (1, 3, 129, 4, 1, 32),
     (1, 2, 65, 3, 3, 96),
+    (1, 150, 170, 8, 2, 64),    # 64 queries and more: one wave per 32 queries, no split over the keys
+    (2, 64, 33, 2, 1, 128),
+    (1, 97, 97, 3, 3, 32),
 ])
 def test_gqa_attention_matches_the_restatement(ops, B, Sq, Sk, hq, hkv, d):
     """runner/linear.rs:552-646 against gqa_attend per query position (every query sees every key position).  The GPU

@@ -552,7 +552,34 @@ def test_fused_epilogues_at_decoder_shapes(oracle, K, torch_cuda, n, k, m):
         err = np.abs(ga - want).max() / np.abs(want).max()
         assert err < (2e-3 if odt == torch.float16 else 1e-3), (odt, err)
     with pytest.raises(Exception, match="m <= 16"):
-        w.matmul_fused(torch.zeros(17, k, device="cuda", dtype=torch.float16), torch.zeros(17, n, device="cuda"), K.EPILOGUE_STORE)
+        w.matmul_fused(torch.zeros(17, k, device="cuda"), torch.zeros(17, n, device="cuda"), K.EPILOGUE_ADD_F32)
+    w.close()
+
+
+@pytest.mark.parametrize("n,k,m", [(4096, 14336, 200), (28672, 4096, 300), (4096, 4096, 17), (1000, 512, 40)])
+def test_fused_epilogues_above_16_rows(K, torch_cuda, n, k, m):
+    """The same epilogues on the LDS-ring GEMM (what the prompt pass runs): every output against the unfused call of the
+    same kernel -- the residual add is one f32 addition on top of it, SwiGLU the same expression on its f32 sums."""
+    torch = torch_cuda
+    rng = np.random.default_rng(1100 + n + k + m)
+    g = 32
+    w = K.PackedInt4Weight(_rand_packed(rng, n, k), rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float16), g, n, k,
+                           nibble_format=K.NIBBLE_UNSIGNED)
+    x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).half().cuda()
+    plain = w.matmul(x, out_dtype=torch.float32)
+    resid = torch.from_numpy((rng.standard_normal((m, n)) * 10).astype(np.float32)).cuda()
+    y = torch.empty(m + 1, n, device="cuda")
+    y[:m] = resid
+    y[m] = 3.0
+    w.matmul_fused(x, y[:m], K.EPILOGUE_ADD_F32)
+    assert torch.equal(y[:m], resid + plain) and bool((y[m] == 3.0).all())
+    want = torch.nn.functional.silu(plain[:, 0::2].double()) * plain[:, 1::2].double()
+    for odt in (torch.float16, torch.float32):
+        act = torch.full((m + 1, n // 2), 7.0, device="cuda", dtype=odt)
+        w.matmul_fused(x, act[:m], K.EPILOGUE_SWIGLU)
+        err = float((act[:m].double() - want).abs().max() / want.abs().max())
+        assert err < (2e-3 if odt == torch.float16 else 1e-5), (odt, err)
+        assert bool((act[m] == 7.0).all())
     w.close()
 
 

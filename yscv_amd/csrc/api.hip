@@ -157,7 +157,9 @@ int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, v
   }
   note_int4_fast();
   Int4Scratch L = int4_scratch_layout(w, x, x_dtype, m, force, ctx->num_cus);
-  if (!L.skinny && epi != EPI_STORE) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "fused epilogues exist for m <= 16 only");
+  // above 16 rows the LDS-ring GEMM (16-bit activations) has the add and SwiGLU epilogues; the exact-scale kernel has none
+  if (!L.skinny && epi != EPI_STORE && !(x_dtype != YSCV_HIP_F32 && nf == nullptr))
+    return set_error(YSCV_HIP_ERR_UNSUPPORTED, "fused epilogues above 16 rows need 16-bit activations");
   // f32 activations that stay on the exact-scale route (f32 scales, or an output the ring GEMM cannot take): up to
   // 128 rows go through the skinny kernel 16 rows at a time.  Each pass streams the weights again, which is still
   // 5-10 x faster than the exact-scale GEMM kernel there: that one keeps a 64 x 256 tile per workgroup and cannot fill
@@ -210,7 +212,7 @@ int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, v
     if (L.skinny)
       st = launch_int4_skinny(w, L.plan, xh, xl, xraw, row_scale, L.k_pad, L.split, y, y_dtype, m, partial, epi, s, nf);
     else
-      st = launch_int4_gemm(w, xh, xl, row_scale, L.k_pad, run_split, y, y_dtype, m, s);
+      st = launch_int4_gemm(w, xh, xl, row_scale, L.k_pad, run_split, y, y_dtype, m, s, epi);
   }
   if (own) {
     hipError_t fe = hipFreeAsync(scratch, s);
@@ -489,8 +491,9 @@ int32_t yscv_hip_int4_matmul_fused(const yscv_hip_int4_weight *w, const void *x_
   YSCV_REQUIRE(epilogue == YSCV_HIP_EPILOGUE_STORE || epilogue == YSCV_HIP_EPILOGUE_ADD_F32 ||
                    epilogue == YSCV_HIP_EPILOGUE_SWIGLU,
                "unknown epilogue %d", epilogue);
-  YSCV_REQUIRE(m <= 16, "fused epilogues run on the skinny kernel: m <= 16, got %zu", m);
-  return int4_run_ws(w, x_dev, x_dtype, y_dev, y_dtype, m, 1, epilogue, nullptr, 0, as_stream(stream));
+  YSCV_REQUIRE(m <= 16 || x_dtype != YSCV_HIP_F32 || epilogue == YSCV_HIP_EPILOGUE_STORE,
+               "fused epilogues with f32 activations run on the skinny kernel: m <= 16, got %zu", m);
+  return int4_run_ws(w, x_dev, x_dtype, y_dev, y_dtype, m, m <= 16 ? 1 : 0, epilogue, nullptr, 0, as_stream(stream));
 }
 
 int32_t yscv_hip_int4_matmul_static(const yscv_hip_int4_weight *w, const void *x_dev, int32_t x_dtype, void *y_dev,

@@ -1144,13 +1144,11 @@ static int32_t prefill_chunk(yscv_hip_decoder *d, const int32_t *tokens_dev, int
   const auto &c = d->cfg;
   const size_t R = (size_t)rows, D = c.d_model, hq = (size_t)c.n_heads * c.head_dim;
   const size_t qkv_n = (size_t)(c.n_heads + 2 * c.n_kv_heads) * c.head_dim, ff = c.d_ff;
-  StreamBuf h, t, xn, qkv, ao, gu, act;
+  StreamBuf h, xn, qkv, ao, act;
   YSCV_TRY(h.alloc(R * D * 4, s));
-  YSCV_TRY(t.alloc(R * D * 4, s));
   YSCV_TRY(xn.alloc(R * D * 2, s));
   YSCV_TRY(qkv.alloc(R * qkv_n * 2, s));
   YSCV_TRY(ao.alloc(R * hq * 2, s));
-  YSCV_TRY(gu.alloc(R * 2 * ff * 4, s));
   YSCV_TRY(act.alloc(R * ff * 2, s));
   YSCV_TRY(launch_embed(tokens_dev, d->emb, rows, (int)D, c.vocab, h.as<float>(), s));
   for (auto &L : d->layers) {
@@ -1161,13 +1159,12 @@ static int32_t prefill_chunk(yscv_hip_decoder *d, const int32_t *tokens_dev, int
                                         c.max_ctx, L.kc, L.vc, s));
     YSCV_TRY(launch_gqa_cache(qkv.as<_Float16>(), L.kc, L.vc, nullptr, rows, start_pos, c.n_heads, c.n_kv_heads, c.head_dim,
                               c.max_ctx, ao.as<_Float16>(), s));
-    YSCV_TRY(int4_run_ws(L.wo, ao.p, YSCV_HIP_F16, t.p, YSCV_HIP_F32, R, 0, EPI_STORE, nullptr, 0, s));
-    YSCV_TRY(launch_residual_add(h.as<float>(), t.as<float>(), R * D, s));
+    // the residual update and SwiGLU ride on the projections' epilogues (both kernels have them: the skinny kernel up to
+    // 16 rows, the LDS-ring GEMM above)
+    YSCV_TRY(int4_run_ws(L.wo, ao.p, YSCV_HIP_F16, h.p, YSCV_HIP_F32, R, 0, EPI_ADD_F32, nullptr, 0, s));
     YSCV_TRY(launch_rmsnorm(h.as<float>(), L.ffn_norm, rows, (int)D, c.rms_eps, xn.as<_Float16>(), s));
-    YSCV_TRY(int4_run_ws(L.wgu, xn.p, YSCV_HIP_F16, gu.p, YSCV_HIP_F32, R, 0, EPI_STORE, nullptr, 0, s));
-    YSCV_TRY(launch_swiglu_rows(gu.as<float>(), act.as<_Float16>(), R, ff, s));
-    YSCV_TRY(int4_run_ws(L.wdown, act.p, YSCV_HIP_F16, t.p, YSCV_HIP_F32, R, 0, EPI_STORE, nullptr, 0, s));
-    YSCV_TRY(launch_residual_add(h.as<float>(), t.as<float>(), R * D, s));
+    YSCV_TRY(int4_run_ws(L.wgu, xn.p, YSCV_HIP_F16, act.p, YSCV_HIP_F16, R, 0, EPI_SWIGLU, nullptr, 0, s));
+    YSCV_TRY(int4_run_ws(L.wdown, act.p, YSCV_HIP_F16, h.p, YSCV_HIP_F32, R, 0, EPI_ADD_F32, nullptr, 0, s));
   }
   if (last) {
     YSCV_TRY(launch_rmsnorm(h.as<float>() + (R - 1) * D, d->final_norm, 1, (int)D, c.rms_eps, d->xn, s));
@@ -1201,7 +1198,7 @@ int32_t yscv_hip_decoder_prefill(yscv_hip_decoder *d, const int32_t *tokens_host
   YSCV_TRY(toks.alloc((size_t)n_tokens * 4, s));
   DEC_HIP(hipMemcpyAsync(toks.p, tokens_host, (size_t)n_tokens * 4, hipMemcpyHostToDevice, s));
   DEC_HIP(hipStreamSynchronize(s));  // tokens_host is the caller's again
-  constexpr int kChunk = 2048;       // rows per pass: bounds the activation buffers (gate/up in f32: 8 * d_ff bytes per row)
+  constexpr int kChunk = 4096;       // rows per pass: bounds the activation buffers
   for (int32_t r0 = 0; r0 < n_tokens; r0 += kChunk) {
     const int rows = n_tokens - r0 < kChunk ? n_tokens - r0 : kChunk;
     YSCV_TRY(prefill_chunk(d, toks.as<int32_t>() + r0, rows, start_pos + r0, r0 + rows == n_tokens, s));

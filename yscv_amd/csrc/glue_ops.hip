@@ -99,13 +99,38 @@ __global__ void __launch_bounds__(64 * GQA_WAVES) gqa_generic_kernel(GqaArgs p) 
 #pragma unroll
   for (int t = 0; t < DT; t++) o_acc[t] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
+  // operands of one key block: 16 cache rows as the A operand of S^T (lane (r, c): row p0 + r, channels 32 kk + 8c .. + 7;
+  // rows past the end repeat the last one) and V^T as the A operand of the second product (lane (r, c): channel
+  // 16 t + r at positions p0 + 4c .. + 3).  The next block's are requested before this block's arithmetic.
+  auto load_block = [&](int blk, half8_t (&kf)[KK], half4_t (&vf)[DT]) {
+    const int p0 = blk * 16;
+    const TKV *krow = kbase + (size_t)min(p0 + r, Sk - 1) * p.k_s;
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) kf[kk] = load8<TKV>(krow + 32 * kk + 8 * c);
+#pragma unroll
+    for (int t = 0; t < DT; t++) {
+      if constexpr (V_SLAB) {
+        const _Float16 *vp = reinterpret_cast<const _Float16 *>(vbase) + ((size_t)((p0 + 4 * c) >> 3) * HD + 16 * t + r) * 8 + ((4 * c) & 7);
+        vf[t] = *reinterpret_cast<const half4_t *>(vp);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int pos = min(p0 + 4 * c + e, Sk - 1);
+          vf[t][e] = (_Float16)vbase[(size_t)pos * p.v_s + 16 * t + r];
+        }
+      }
+    }
+  };
+  half8_t kf[KK], kn[KK];
+  half4_t vf[DT], vn[DT];
+  if (wave < nblocks) load_block(wave, kf, vf);
   for (int blk = wave; blk < nblocks; blk += GQA_WAVES) {
     const int p0 = blk * 16;
-    // ---- S^T: lane (r, c) as A supplies cache row p0 + r, channels 32 kk + 8c .. + 7 (rows past the end repeat the last)
-    const TKV *krow = kbase + (size_t)min(p0 + r, Sk - 1) * p.k_s;
+    const bool more = blk + GQA_WAVES < nblocks;  // uniform in the wave
+    if (more) load_block(blk + GQA_WAVES, kn, vn);
     float4_t s = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int kk = 0; kk < KK; kk++) s = __builtin_amdgcn_mfma_f32_16x16x32_f16(load8<TKV>(krow + 32 * kk + 8 * c), qf[kk], s, 0, 0, 0);
+    for (int kk = 0; kk < KK; kk++) s = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kk], qf[kk], s, 0, 0, 0);
     // lane (r, c): query r, positions p0 + 4c + e
     float sv[4], mx = -INFINITY;
 #pragma unroll
@@ -126,27 +151,22 @@ __global__ void __launch_bounds__(64 * GQA_WAVES) gqa_generic_kernel(GqaArgs p) 
     l_run = l_run * alpha + sum;
     m_run = m_new;
     const half4_t pf = {(_Float16)pe[0], (_Float16)pe[1], (_Float16)pe[2], (_Float16)pe[3]};
-    // ---- O^T += V^T P^T: lane (r, c) as A supplies channel 16 t + r at positions p0 + 4c .. + 3
 #pragma unroll
     for (int t = 0; t < DT; t++) {
-      half4_t vf;
-      if constexpr (V_SLAB) {
-        // positions past the end of the context lie inside the allocated slab and meet weight 0 -- but 0 * NaN would
-        // poison the sum, so they are blanked
-        const _Float16 *vp = reinterpret_cast<const _Float16 *>(vbase) + ((size_t)((p0 + 4 * c) >> 3) * HD + 16 * t + r) * 8 + ((4 * c) & 7);
-        vf = *reinterpret_cast<const half4_t *>(vp);
+      // positions past the end of the context meet weight 0 -- but 0 * NaN would poison the sum (the slab may hold
+      // anything there), so they are blanked
+      half4_t vv = vf[t];
 #pragma unroll
-        for (int e = 0; e < 4; e++)
-          if (p0 + 4 * c + e >= Sk) vf[e] = (_Float16)0.0f;
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          const int pos = p0 + 4 * c + e;
-          vf[e] = pos < Sk ? (_Float16)vbase[(size_t)pos * p.v_s + 16 * t + r] : (_Float16)0.0f;
-        }
-      }
+      for (int e = 0; e < 4; e++)
+        if (p0 + 4 * c + e >= Sk) vv[e] = (_Float16)0.0f;
       o_acc[t] = o_acc[t] * alpha;
-      o_acc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(vf, pf, o_acc[t], 0, 0, 0);
+      o_acc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(vv, pf, o_acc[t], 0, 0, 0);
+    }
+    if (more) {
+#pragma unroll
+      for (int kk = 0; kk < KK; kk++) kf[kk] = kn[kk];
+#pragma unroll
+      for (int t = 0; t < DT; t++) vf[t] = vn[t];
     }
   }
   // ---- merge the four waves: lane (r, c) holds O^T[16 t + 4c + e][query r]
@@ -179,8 +199,142 @@ __global__ void __launch_bounds__(64 * GQA_WAVES) gqa_generic_kernel(GqaArgs p) 
   }
 }
 
+// Many query positions (prompt pass, or the operator with a long seq_q): a wave owns 32 consecutive queries of one
+// head and walks every key block itself -- each K / V load then feeds two query tiles, and nothing is merged at the
+// end.  A workgroup's four waves take neighbouring query ranges of the same head, so their K / V requests meet in
+// the CU's cache.  Same arithmetic per (query, position) as gqa_generic_kernel.
+template <int HD, typename TQ, typename TKV, typename TO, bool V_SLAB>
+__global__ void __launch_bounds__(64 * GQA_WAVES) gqa_rows_kernel(GqaArgs p) {
+  static_assert(HD % 32 == 0 && HD >= 32 && HD <= 128, "head width");
+  constexpr int KK = HD / 32, DT = HD / 16, QT = 2;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, c = lane >> 4;
+  const int q0 = (blockIdx.x * GQA_WAVES + wave) * 16 * QT, h = blockIdx.y, b = blockIdx.z;
+  if (q0 >= p.Sq) return;  // no barrier in this kernel
+  const int kvh = h / (p.Hq / p.Hkv);
+  const int Sk = p.Sk;
+  int qi[QT], lim_q[QT];
+  half8_t qf[QT][KK];
+#pragma unroll
+  for (int u = 0; u < QT; u++) {
+    qi[u] = min(q0 + 16 * u + r, p.Sq - 1);
+    lim_q[u] = p.causal_base < 0 ? Sk - 1 : min(Sk - 1, p.causal_base + qi[u]);
+    const TQ *qrow = static_cast<const TQ *>(p.q) + (size_t)b * p.q_b + (size_t)qi[u] * p.q_s + (size_t)h * HD;
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) qf[u][kk] = load8<TQ>(qrow + 32 * kk + 8 * c);
+  }
+  const int lim_wave = p.causal_base < 0 ? Sk - 1 : min(Sk - 1, p.causal_base + min(q0 + 16 * QT - 1, p.Sq - 1));
+  const int nblocks = lim_wave / 16 + 1;
+  const TKV *kbase = static_cast<const TKV *>(p.k) + (size_t)b * p.k_b + (size_t)kvh * p.k_h;
+  const TKV *vbase = static_cast<const TKV *>(p.v) + (size_t)b * p.v_b + (size_t)kvh * p.v_h;
+  float m_run[QT], l_run[QT];
+  float4_t o_acc[QT][DT];
+#pragma unroll
+  for (int u = 0; u < QT; u++) {
+    m_run[u] = -INFINITY;
+    l_run[u] = 0.0f;
+#pragma unroll
+    for (int t = 0; t < DT; t++) o_acc[u][t] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  }
+  auto load_block = [&](int blk, half8_t (&kf)[KK], half4_t (&vf)[DT]) {
+    const int p0 = blk * 16;
+    const TKV *krow = kbase + (size_t)min(p0 + r, Sk - 1) * p.k_s;
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) kf[kk] = load8<TKV>(krow + 32 * kk + 8 * c);
+#pragma unroll
+    for (int t = 0; t < DT; t++) {
+      if constexpr (V_SLAB) {
+        const _Float16 *vp = reinterpret_cast<const _Float16 *>(vbase) + ((size_t)((p0 + 4 * c) >> 3) * HD + 16 * t + r) * 8 + ((4 * c) & 7);
+        vf[t] = *reinterpret_cast<const half4_t *>(vp);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int pos = min(p0 + 4 * c + e, Sk - 1);
+          vf[t][e] = (_Float16)vbase[(size_t)pos * p.v_s + 16 * t + r];
+        }
+      }
+    }
+  };
+  half8_t kf[KK], kn[KK];
+  half4_t vf[DT], vn[DT];
+  load_block(0, kf, vf);
+  for (int blk = 0; blk < nblocks; blk++) {
+    const int p0 = blk * 16;
+    const bool more = blk + 1 < nblocks;
+    if (more) load_block(blk + 1, kn, vn);
+    half4_t vv[DT];
+#pragma unroll
+    for (int t = 0; t < DT; t++) {
+      vv[t] = vf[t];
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        if (p0 + 4 * c + e >= Sk) vv[t][e] = (_Float16)0.0f;  // 0 * NaN would poison the sum
+    }
+#pragma unroll
+    for (int u = 0; u < QT; u++) {
+      float4_t s = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int kk = 0; kk < KK; kk++) s = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kk], qf[u][kk], s, 0, 0, 0);
+      float sv[4], mx = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        sv[e] = (p0 + 4 * c + e <= lim_q[u]) ? s[e] * p.scale : -INFINITY;
+        mx = fmaxf(mx, sv[e]);
+      }
+      mx = max_xor16_xor32(mx);
+      const float m_new = fmaxf(m_run[u], mx);
+      float pe[4], sum = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        pe[e] = (sv[e] == -INFINITY) ? 0.0f : __expf(sv[e] - m_new);
+        sum += pe[e];
+      }
+      sum = sum_xor16_xor32(sum);
+      const float alpha = (m_run[u] == -INFINITY) ? 0.0f : __expf(m_run[u] - m_new);
+      l_run[u] = l_run[u] * alpha + sum;
+      m_run[u] = m_new;
+      const half4_t pf = {(_Float16)pe[0], (_Float16)pe[1], (_Float16)pe[2], (_Float16)pe[3]};
+#pragma unroll
+      for (int t = 0; t < DT; t++) {
+        o_acc[u][t] = o_acc[u][t] * alpha;
+        o_acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x16f16(vv[t], pf, o_acc[u][t], 0, 0, 0);
+      }
+    }
+    if (more) {
+#pragma unroll
+      for (int kk = 0; kk < KK; kk++) kf[kk] = kn[kk];
+#pragma unroll
+      for (int t = 0; t < DT; t++) vf[t] = vn[t];
+    }
+  }
+  // lane (r, c) holds O^T[16 t + 4c + e][query r] of each query tile: four consecutive channels per store
+  TO *obase = static_cast<TO *>(p.out) + (size_t)b * p.o_b + (size_t)h * HD;
+#pragma unroll
+  for (int u = 0; u < QT; u++) {
+    if (q0 + 16 * u + r >= p.Sq) continue;
+    const float inv = l_run[u] > 0.0f ? 1.0f / l_run[u] : 0.0f;
+    TO *orow = obase + (size_t)(q0 + 16 * u + r) * p.o_s;
+#pragma unroll
+    for (int t = 0; t < DT; t++)
+      store4<TO>(orow + 16 * t + 4 * c, o_acc[u][t][0] * inv, o_acc[u][t][1] * inv, o_acc[u][t][2] * inv, o_acc[u][t][3] * inv);
+  }
+}
+
 template <typename TQ, typename TKV, typename TO, bool V_SLAB>
 int32_t gqa_launch(const GqaArgs &a, int hd, hipStream_t s) {
+  // many queries and a host-known context: one wave per 32 queries, no split over the keys
+  if (a.Sq >= 64 && a.sk_minus_1 == nullptr) {
+    const dim3 grid((unsigned)((a.Sq + 32 * GQA_WAVES - 1) / (32 * GQA_WAVES)), (unsigned)a.Hq, (unsigned)a.B), block(64 * GQA_WAVES);
+    switch (hd) {
+      case 32: hipLaunchKernelGGL((gqa_rows_kernel<32, TQ, TKV, TO, V_SLAB>), grid, block, 0, s, a); break;
+      case 64: hipLaunchKernelGGL((gqa_rows_kernel<64, TQ, TKV, TO, V_SLAB>), grid, block, 0, s, a); break;
+      case 96: hipLaunchKernelGGL((gqa_rows_kernel<96, TQ, TKV, TO, V_SLAB>), grid, block, 0, s, a); break;
+      case 128: hipLaunchKernelGGL((gqa_rows_kernel<128, TQ, TKV, TO, V_SLAB>), grid, block, 0, s, a); break;
+      default: return set_error(YSCV_HIP_ERR_UNSUPPORTED, "attention: head width %d (supported: 32, 64, 96, 128)", hd);
+    }
+    YSCV_HIP_TRY(hipGetLastError());
+    return YSCV_HIP_OK;
+  }
   const dim3 grid((unsigned)((a.Sq + 15) / 16), (unsigned)a.Hq, (unsigned)a.B), block(64 * GQA_WAVES);
   switch (hd) {
     case 32: hipLaunchKernelGGL((gqa_generic_kernel<32, TQ, TKV, TO, V_SLAB>), grid, block, 0, s, a); break;

@@ -30,6 +30,7 @@ namespace yscv {
 namespace {
 
 __device__ const float kOne = 1.0f;  // stands in for an absent row-scale vector
+__device__ __forceinline__ float ring_silu(float g) { return g / (1.0f + __expf(-g)); }
 
 typedef __attribute__((address_space(3))) void lds_void;
 #define G4_AS1(ptr) ((const void __attribute__((address_space(1))) *)(ptr))
@@ -47,6 +48,7 @@ struct RingArgs {
   int chunks, chunk_div;
   int k_pad;
   int y_dtype;
+  int epi;         // EPI_STORE, EPI_ADD_F32 (y f32, y += product) or EPI_SWIGLU (y [m][n / 2] = silu(gate) * up, columns 2i / 2i+1)
 };
 
 template <int N>
@@ -457,7 +459,20 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
       if (row >= p.m || col >= p.n) continue;
       const float4_t v = *reinterpret_cast<const float4_t *>(g4_ring + lrow * RS + ch * 16);
       const size_t o = (size_t)row * p.ldy + col;
-      if (vec) {
+      if (p.epi == EPI_SWIGLU) {
+        // columns col .. col + 3 are gate, up, gate, up of two channels (n is even, col a multiple of 4)
+        const size_t oh = (size_t)row * (p.ldy >> 1) + (col >> 1);
+        store_out(p.y, oh, ring_silu(v[0]) * v[1], p.y_dtype);
+        if (col + 2 < p.n) store_out(p.y, oh + 1, ring_silu(v[2]) * v[3], p.y_dtype);
+      } else if (p.epi == EPI_ADD_F32) {
+        float *dst = reinterpret_cast<float *>(p.y) + o;  // every element has one writer in a launch
+        if (vec) {
+          *reinterpret_cast<float4_t *>(dst) = *reinterpret_cast<const float4_t *>(dst) + v;
+        } else {
+          for (int e = 0; e < 4; e++)
+            if (col + e < p.n) dst[e] += v[e];
+        }
+      } else if (vec) {
         if (p.y_dtype == YSCV_HIP_F32) {
           *reinterpret_cast<float4_t *>(reinterpret_cast<float *>(p.y) + o) = v;
         } else if (p.y_dtype == YSCV_HIP_F16) {
@@ -520,8 +535,11 @@ bool int4_gemm_ring_eligible(const yscv_hip_int4_weight *w, const _Float16 *xh, 
 }
 
 int32_t launch_int4_gemm_ring(const yscv_hip_int4_weight *w, const _Float16 *xh, const float *row_scale, size_t k_pad,
-                              void *y, int y_dtype, size_t m, hipStream_t s) {
+                              void *y, int y_dtype, size_t m, hipStream_t s, int epi) {
+  if (epi == EPI_ADD_F32 && y_dtype != YSCV_HIP_F32) return set_error(YSCV_HIP_ERR_INVALID_ARG, "the add epilogue updates an f32 tensor");
+  if (epi == EPI_SWIGLU && (w->n & 1)) return set_error(YSCV_HIP_ERR_INVALID_ARG, "SwiGLU epilogue needs an even row count");
   RingArgs a;
+  a.epi = epi;
   a.tiles = w->tiles;
   a.tscales = w->tscales;
   a.tzps = w->has_zp ? w->tzps : nullptr;

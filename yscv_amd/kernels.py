@@ -292,7 +292,8 @@ class PackedInt4Weight:
         return out
 
     def matmul_fused(self, x, out, epilogue: int):
-        """yscv_hip_int4_matmul_fused: skinny kernel (m <= 16) with the epilogue fused.  EPILOGUE_ADD_F32 adds into the
+        """yscv_hip_int4_matmul_fused: the int4 matmul with the epilogue fused (skinny kernel up to 16 rows, the LDS-ring GEMM
+        above with 16-bit activations).  EPILOGUE_ADD_F32 adds into the
         f32 tensor `out` [m, m_w]; EPILOGUE_SWIGLU writes silu(gate) * up into `out` [m, m_w / 2]."""
         assert x.is_cuda and out.is_cuda and x.shape[-1] == self.k
         x = x.contiguous()
