@@ -209,7 +209,8 @@ __global__ void __launch_bounds__(64 * GQA_WAVES) gqa_rows_kernel(GqaArgs p) {
   constexpr int KK = HD / 32, DT = HD / 16, QT = 2;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, c = lane >> 4;
-  const int q0 = (blockIdx.x * GQA_WAVES + wave) * 16 * QT, h = blockIdx.y, b = blockIdx.z;
+  // late query ranges see the most keys: they are dispatched first, so that the grid does not end on its longest workgroups
+  const int q0 = (((int)gridDim.x - 1 - (int)blockIdx.x) * GQA_WAVES + wave) * 16 * QT, h = blockIdx.y, b = blockIdx.z;
   if (q0 >= p.Sq) return;  // no barrier in this kernel
   const int kvh = h / (p.Hq / p.Hkv);
   const int Sk = p.Sk;
