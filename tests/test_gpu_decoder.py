@@ -647,3 +647,44 @@ def test_prefill_equals_feeding_at_toy_widths(n_prompt, start):
     exp2 = ref.step(nxt, start + n_prompt)
     assert np.abs(dec.logits() - exp2).max() / np.abs(exp2).max() < LOGIT_TOL
     dec.close()
+
+
+@pytest.mark.parametrize("hd,nh,nkv,n_prompt,start", [
+    (128, 4, 1, 150, 0),   # four query heads per kv head: the four waves of a workgroup are the four heads
+    (64, 8, 1, 97, 5),     # eight per kv head: two workgroups per kv head; the prompt ends inside a 32-query range
+    (64, 4, 2, 200, 0),    # two per kv head: two heads x two query ranges per workgroup
+    (32, 4, 4, 161, 30),   # one per kv head: four query ranges per workgroup, the last one past the prompt's end
+    (96, 12, 4, 70, 0),    # three per kv head (neither four nor two divides it): one head per workgroup; 96-wide rows
+])
+def test_prefill_of_long_prompts_across_head_shapes(hd, nh, nkv, n_prompt, start):
+    """Prompts of 64 rows and more go through the attention kernel that shares a stage of K / V between the four waves
+    of a workgroup; how heads and query ranges are spread over the waves depends on the heads per kv head.  Logits of
+    the last prompt position (which, through the second layer's K / V, depend on the first layer's attention output at
+    every position) against the checker fed token by token, and the cache the pass leaves behind through one more
+    decode step."""
+    rng = np.random.default_rng(5000 + hd + nh)
+    cfg = dict(CFG, n_heads=nh, n_kv_heads=nkv, head_dim=hd, d_model=256, max_batch=1, max_ctx=256)
+    dec, ref = _build(rng, cfg, symmetric=True)
+    if start:
+        for l in range(cfg["n_layers"]):
+            k = rng.standard_normal((1, start, nkv, hd)).astype(np.float16)
+            v = rng.standard_normal((1, start, nkv, hd)).astype(np.float16)
+            dec.set_kv(l, k, v)
+            ref.set_kv(l, k.astype(np.float32), v.astype(np.float32))
+    prompt = rng.integers(0, cfg["vocab"], n_prompt).astype(np.int32)
+    for i, t in enumerate(prompt):
+        exp = ref.step(np.array([t]), start + i)
+    dec.prefill(prompt, start_pos=start)
+    got = dec.logits()
+    assert np.abs(got - exp).max() / np.abs(exp).max() < LOGIT_TOL
+    # every cache row the pass wrote, first and second layer
+    for l in range(cfg["n_layers"]):
+        gk, gv = dec.get_kv(l, 1, 0, start + n_prompt)
+        ek, ev = ref.kc[l][0], ref.vc[l][0]
+        assert np.abs(gk.astype(np.float32) - ek).max() <= 1e-2 * np.abs(ek).max(), l
+        assert np.abs(gv.astype(np.float32) - ev).max() <= 1e-2 * np.abs(ev).max(), l
+    nxt = dec.tokens(0, 1)[0].copy()
+    dec.run(1, use_graph=True)
+    exp2 = ref.step(nxt, start + n_prompt)
+    assert np.abs(dec.logits() - exp2).max() / np.abs(exp2).max() < LOGIT_TOL
+    dec.close()

@@ -321,6 +321,219 @@ __global__ void __launch_bounds__(64 * GQA_WAVES) gqa_rows_kernel(GqaArgs p) {
   }
 }
 
+// Prompt pass over the decoder's fp16 cache: the four waves of a workgroup take the same key range -- query heads
+// that share a kv head (as many of them as divide four), else neighbouring 32-query ranges of one head -- so a
+// stage of 32 cache positions is fetched once per workgroup into LDS (K rows with their 16-byte pieces XOR-swizzled
+// so that the 16 rows a fragment read touches fall into 16 different bank groups; V as its slabs lie in memory) and
+// read from there by all four: a quarter of the L2 traffic of gqa_rows_kernel, which is what bounds that kernel at
+// prompt lengths in the thousands.  Two stage buffers: the next stage's pieces are requested into registers before
+// this stage's arithmetic and written to the other buffer behind it, one barrier per stage.  Arithmetic per
+// (query, position) as in gqa_generic_kernel; the running output is rescaled only where some query's maximum moved
+// (a factor of exactly one otherwise).
+template <int HD>
+__global__ void __launch_bounds__(64 * GQA_WAVES, 2) gqa_shared_kv_kernel(GqaArgs p, int hw_log2) {
+  static_assert(HD % 32 == 0 && HD >= 32 && HD <= 128, "head width");
+  constexpr int KK = HD / 32, DT = HD / 16, QT = 2, KB = 32;  // KB: cache positions per stage
+  constexpr int CPR = HD / 8;                                  // 16-byte pieces of a K row
+  constexpr int PITCH = HD > 64 ? 16 : (HD > 32 ? 8 : 4);      // row pitch in pieces (a power of two)
+  constexpr int RPW = 16 / PITCH;                              // rows per 256 bytes
+  constexpr int K_BYTES = KB * PITCH * 16, V_BYTES = (KB / 8) * HD * 16, ST_BYTES = K_BYTES + V_BYTES;
+  constexpr int K_PIECES = KB * CPR, V_PIECES = (KB / 8) * HD;
+  constexpr int THREADS = 64 * GQA_WAVES;
+  constexpr int K_LD = (K_PIECES + THREADS - 1) / THREADS, V_LD = (V_PIECES + THREADS - 1) / THREADS;
+  __shared__ __attribute__((aligned(16))) uint8_t stage[2 * ST_BYTES];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, c = lane >> 4;
+  const int hw = 1 << hw_log2, qw = GQA_WAVES >> hw_log2;  // heads x query ranges of a workgroup
+  const int group = p.Hq / p.Hkv, chunks = group >> hw_log2;
+  const int kvh = (int)blockIdx.x / chunks, b = blockIdx.z;
+  const int h = kvh * group + ((int)blockIdx.x % chunks) * hw + (wave & (hw - 1));
+  // Workgroups start in the order of blockIdx.y.  The first half takes the late query ranges (most positions), the
+  // second half the early ones in rising order: two workgroups that start half a grid apart, and so tend to share
+  // a CU, carry about the same work together as any other such pair.
+  const int T = gridDim.y, first_half = (T + 1) / 2;
+  const int tile = (int)blockIdx.y < first_half ? T - 1 - (int)blockIdx.y : (int)blockIdx.y - first_half;
+  const int q0 = (tile * qw + (wave >> hw_log2)) * 16 * QT;
+  const bool active = q0 < p.Sq;
+  const int Sk = p.Sk;
+  int qi[QT], lim_q[QT];
+  half8_t qf[QT][KK];
+#pragma unroll
+  for (int u = 0; u < QT; u++) {
+    qi[u] = min(q0 + 16 * u + r, p.Sq - 1);
+    lim_q[u] = p.causal_base < 0 ? Sk - 1 : min(Sk - 1, p.causal_base + qi[u]);
+    const _Float16 *qrow = static_cast<const _Float16 *>(p.q) + (size_t)b * p.q_b + (size_t)qi[u] * p.q_s + (size_t)h * HD;
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) qf[u][kk] = load8<_Float16>(qrow + 32 * kk + 8 * c);
+  }
+  const int lim_wave = p.causal_base < 0 ? Sk - 1 : min(Sk - 1, p.causal_base + min(q0 + 16 * QT - 1, p.Sq - 1));
+  const int lim_first = p.causal_base < 0 ? Sk - 1 : min(Sk - 1, p.causal_base + min(q0, p.Sq - 1));  // what the wave's first query sees
+  const int q_last = min((tile + 1) * qw * 16 * QT, p.Sq) - 1;  // last query of the workgroup
+  const int lim_wg = p.causal_base < 0 ? Sk - 1 : min(Sk - 1, p.causal_base + q_last);
+  const int nstages = lim_wg / KB + 1;
+  const _Float16 *kbase = static_cast<const _Float16 *>(p.k) + (size_t)b * p.k_b + (size_t)kvh * p.k_h;
+  const _Float16 *vbase = static_cast<const _Float16 *>(p.v) + (size_t)b * p.v_b + (size_t)kvh * p.v_h;
+  float m_run[QT], l_run[QT];
+  float4_t o_acc[QT][DT];
+#pragma unroll
+  for (int u = 0; u < QT; u++) {
+    m_run[u] = -INFINITY;
+    l_run[u] = 0.0f;
+#pragma unroll
+    for (int t = 0; t < DT; t++) o_acc[u][t] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  }
+  // piece idx of a stage's K: row idx / CPR, piece idx % CPR; of its V: slab idx / HD, channel idx % HD.  Rows and
+  // slabs past the end of the context repeat the last one (never used: their positions are masked)
+  auto fetch = [&](int st, uint4_t (&kr)[K_LD], uint4_t (&vr)[V_LD]) {
+#pragma unroll
+    for (int j = 0; j < K_LD; j++) {
+      const int idx = tid + THREADS * j;
+      if (K_PIECES % THREADS == 0 || idx < K_PIECES) {
+        const int pos = min(st * KB + idx / CPR, Sk - 1);
+        kr[j] = *reinterpret_cast<const uint4_t *>(kbase + (size_t)pos * p.k_s + (idx % CPR) * 8);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < V_LD; j++) {
+      const int idx = tid + THREADS * j;
+      if (V_PIECES % THREADS == 0 || idx < V_PIECES) {
+        const int slab = min(st * (KB / 8) + idx / HD, (Sk - 1) >> 3);
+        vr[j] = *reinterpret_cast<const uint4_t *>(vbase + ((size_t)slab * HD + idx % HD) * 8);
+      }
+    }
+  };
+  auto stash = [&](int buf, const uint4_t (&kr)[K_LD], const uint4_t (&vr)[V_LD]) {
+    uint8_t *base = stage + buf * ST_BYTES;
+#pragma unroll
+    for (int j = 0; j < K_LD; j++) {
+      const int idx = tid + THREADS * j;
+      if (K_PIECES % THREADS == 0 || idx < K_PIECES) {
+        const int row = idx / CPR, piece = idx % CPR;
+        *reinterpret_cast<uint4_t *>(base + (row * PITCH + (piece ^ ((((row >> 3) & 3) * 4 + (row & 3)) / RPW))) * 16) = kr[j];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < V_LD; j++) {
+      const int idx = tid + THREADS * j;
+      if (V_PIECES % THREADS == 0 || idx < V_PIECES) *reinterpret_cast<uint4_t *>(base + K_BYTES + idx * 16) = vr[j];
+    }
+  };
+  auto compute = [&](int st) {
+    const uint8_t *base = stage + (st & 1) * ST_BYTES;
+    const int p0 = st * KB;
+    if (active && p0 <= lim_wave) {  // uniform in the wave
+      // Two S^T tiles per stage.  Row rho of tile j is stage position 8 (rho / 4) + 4 j + rho % 4, so lane (r, c)
+      // ends up with the weights of positions 8c .. 8c+7 (tile 0: the first four, tile 1: the last four): one 16-byte
+      // slab piece of V^T per channel, and the B operand of one 32-deep MFMA.
+      half8_t kf[2][KK], vv[DT];
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        const int row = 8 * (r >> 2) + 4 * j + (r & 3);
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++)
+          kf[j][kk] = *reinterpret_cast<const half8_t *>(base + (row * PITCH + ((4 * kk + c) ^ (r / RPW))) * 16);
+      }
+#pragma unroll
+      for (int t = 0; t < DT; t++) vv[t] = *reinterpret_cast<const half8_t *>(base + K_BYTES + (c * HD + 16 * t + r) * 16);
+      if (p0 + KB > Sk) {  // 0 * NaN would poison the sum: positions past the context are blanked
+#pragma unroll
+        for (int t = 0; t < DT; t++)
+#pragma unroll
+          for (int e = 0; e < 8; e++)
+            if (p0 + 8 * c + e >= Sk) vv[t][e] = (_Float16)0.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < QT; u++) {
+        float4_t s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) {
+          s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[0][kk], qf[u][kk], s0, 0, 0, 0);
+          s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[1][kk], qf[u][kk], s1, 0, 0, 0);
+        }
+        float sv[8], mx = -INFINITY, pe[8], sum = 0.0f, m_new;
+        if (p0 + KB - 1 <= lim_first) {  // uniform in the wave: every query of the wave sees the whole stage
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            sv[e] = (e < 4 ? s0[e & 3] : s1[e & 3]) * p.scale;
+            mx = fmaxf(mx, sv[e]);
+          }
+          m_new = fmaxf(m_run[u], max_xor16_xor32(mx));
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            pe[e] = __expf(sv[e] - m_new);
+            sum += pe[e];
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            const float raw = (e < 4 ? s0[e & 3] : s1[e & 3]) * p.scale;
+            sv[e] = (p0 + 8 * c + e <= lim_q[u]) ? raw : -INFINITY;
+            mx = fmaxf(mx, sv[e]);
+          }
+          m_new = fmaxf(m_run[u], max_xor16_xor32(mx));
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            pe[e] = (sv[e] == -INFINITY) ? 0.0f : __expf(sv[e] - m_new);
+            sum += pe[e];
+          }
+        }
+        sum = sum_xor16_xor32(sum);
+        const float alpha = (m_run[u] == -INFINITY) ? 0.0f : __expf(m_run[u] - m_new);
+        l_run[u] = l_run[u] * alpha + sum;
+        m_run[u] = m_new;
+        const half8_t pf = {(_Float16)pe[0], (_Float16)pe[1], (_Float16)pe[2], (_Float16)pe[3],
+                            (_Float16)pe[4], (_Float16)pe[5], (_Float16)pe[6], (_Float16)pe[7]};
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+          for (int t = 0; t < DT; t++) o_acc[u][t] = o_acc[u][t] * alpha;
+        }
+#pragma unroll
+        for (int t = 0; t < DT; t++) o_acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vv[t], pf, o_acc[u][t], 0, 0, 0);
+      }
+    }
+  };
+  uint4_t kr[K_LD], vr[V_LD];
+  fetch(0, kr, vr);
+  stash(0, kr, vr);
+  __syncthreads();
+  for (int st = 0; st < nstages; st++) {
+    const bool more = st + 1 < nstages;  // uniform in the workgroup
+    if (more) fetch(st + 1, kr, vr);
+    compute(st);
+    if (more) stash((st + 1) & 1, kr, vr);
+    __syncthreads();
+  }
+  if (!active) return;
+  _Float16 *obase = static_cast<_Float16 *>(p.out) + (size_t)b * p.o_b + (size_t)h * HD;
+#pragma unroll
+  for (int u = 0; u < QT; u++) {
+    if (q0 + 16 * u + r >= p.Sq) continue;
+    const float inv = l_run[u] > 0.0f ? 1.0f / l_run[u] : 0.0f;
+    _Float16 *orow = obase + (size_t)(q0 + 16 * u + r) * p.o_s;
+#pragma unroll
+    for (int t = 0; t < DT; t++)
+      store4<_Float16>(orow + 16 * t + 4 * c, o_acc[u][t][0] * inv, o_acc[u][t][1] * inv, o_acc[u][t][2] * inv, o_acc[u][t][3] * inv);
+  }
+}
+
+// heads of one kv group that share a workgroup of gqa_shared_kv_kernel: the largest of 4, 2, 1 that divides the group
+inline int shared_kv_hw_log2(int group) { return group % 4 == 0 ? 2 : (group % 2 == 0 ? 1 : 0); }
+
+int32_t gqa_launch_shared_kv(const GqaArgs &a, int hd, hipStream_t s) {
+  const int hw_log2 = shared_kv_hw_log2(a.Hq / a.Hkv);
+  const int q_per_wg = 32 * (GQA_WAVES >> hw_log2);
+  const dim3 grid((unsigned)(a.Hq >> hw_log2), (unsigned)((a.Sq + q_per_wg - 1) / q_per_wg), (unsigned)a.B), block(64 * GQA_WAVES);
+  switch (hd) {
+    case 32: hipLaunchKernelGGL((gqa_shared_kv_kernel<32>), grid, block, 0, s, a, hw_log2); break;
+    case 64: hipLaunchKernelGGL((gqa_shared_kv_kernel<64>), grid, block, 0, s, a, hw_log2); break;
+    case 96: hipLaunchKernelGGL((gqa_shared_kv_kernel<96>), grid, block, 0, s, a, hw_log2); break;
+    case 128: hipLaunchKernelGGL((gqa_shared_kv_kernel<128>), grid, block, 0, s, a, hw_log2); break;
+    default: return set_error(YSCV_HIP_ERR_UNSUPPORTED, "attention: head width %d (supported: 32, 64, 96, 128)", hd);
+  }
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
 template <typename TQ, typename TKV, typename TO, bool V_SLAB>
 int32_t gqa_launch(const GqaArgs &a, int hd, hipStream_t s) {
   // many queries and a host-known context: one wave per 32 queries, no split over the keys
@@ -508,6 +721,9 @@ int32_t launch_gqa_cache(const _Float16 *qkv, const _Float16 *kc, const _Float16
     a.o_b = 0;
     a.o_s = (long long)hq * hd;
   }
+  // prompt mode with enough rows: the kernel that stages K / V in LDS for four waves (its K rows must be contiguous
+  // 16-byte pieces, which the cache's are)
+  if (!pos_ptr && rows >= 64 && (max_ctx & 7) == 0) return gqa_launch_shared_kv(a, hd, s);
   return gqa_launch<_Float16, _Float16, _Float16, true>(a, hd, s);
 }
 
