@@ -534,8 +534,9 @@ int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_g
  * decoder as yscv_hip_decoder_reset(1, start_pos + n_tokens - 1, last token) + one decode step would: batch 1, the
  * greedy pick as the next input token and as token 0 of the history, position start_pos + n_tokens, step 1.  The
  * results agree with token-by-token feeding to the float bar of the int4 kernels (the GEMM folds the group scale into
- * fp16 weights where the decode kernel applies it in fp32).  A decoder with an int8 cache runs the decode step per
- * position instead.  tokens_host is read before the call returns. */
+ * fp16 weights where the decode kernel applies it in fp32).  With an int8 cache every row is quantised as the decode
+ * step quantises it (scales over all kv heads of the position) and attention reads what the cache returns for each
+ * position, q * scale of its row, earlier positions included.  tokens_host is read before the call returns. */
 int32_t yscv_hip_decoder_prefill(yscv_hip_decoder *d, const int32_t *tokens_host, int32_t n_tokens, int32_t start_pos,
                                  void *stream);
 /* Optional bias of the fused q / k / v projection of one layer (Qwen-style attention; the reference adds it with

@@ -619,20 +619,22 @@ def test_reference_benchmark_model_decodes_and_prefills():
     dec2.close()
 
 
-@pytest.mark.parametrize("n_prompt,start", [(1, 0), (5, 0), (16, 3), (17, 0), (130, 9)])
-def test_prefill_equals_feeding_at_toy_widths(n_prompt, start):
+@pytest.mark.parametrize("n_prompt,start,kv_dtype", [(1, 0, "f16"), (5, 0, "f16"), (16, 3, "f16"), (17, 0, "f16"), (130, 9, "f16"),
+                                                     (1, 0, "i8"), (5, 2, "i8"), (17, 0, "i8"), (130, 9, "i8")])
+def test_prefill_equals_feeding_at_toy_widths(n_prompt, start, kv_dtype):
     """Prompt lengths on both sides of the skinny / GEMM switch (16 rows) and across a 128-position attention chunk, at a
     start position other than 0 (a prompt appended to a cache that already holds positions): prefill against the
-    checker fed token by token, head_dim 128."""
+    checker fed token by token, head_dim 128.  With the int8 cache the pass quantises every appended row (scales over
+    all kv heads of the position) and attends over what the cache returns, earlier positions included."""
     rng = np.random.default_rng(4900 + n_prompt)
     cfg = dict(CFG, max_batch=1, max_ctx=256)
-    dec, ref = _build(rng, cfg, symmetric=True)
+    dec, ref = _build(rng, cfg, kv_dtype=kv_dtype, symmetric=True)
     for l in range(cfg["n_layers"]):
         k = rng.standard_normal((1, start, cfg["n_kv_heads"], cfg["head_dim"])).astype(np.float16)
         v = rng.standard_normal((1, start, cfg["n_kv_heads"], cfg["head_dim"])).astype(np.float16)
         if start:
             dec.set_kv(l, k, v)
-        ref.set_kv(l, k.astype(np.float32), v.astype(np.float32))
+            ref.set_kv(l, k.astype(np.float32), v.astype(np.float32))
     prompt = rng.integers(0, cfg["vocab"], n_prompt).astype(np.int32)
     for i, t in enumerate(prompt):
         exp = ref.step(np.array([t]), start + i)

@@ -1150,15 +1150,30 @@ static int32_t prefill_chunk(yscv_hip_decoder *d, const int32_t *tokens_dev, int
   YSCV_TRY(qkv.alloc(R * qkv_n * 2, s));
   YSCV_TRY(ao.alloc(R * hq * 2, s));
   YSCV_TRY(act.alloc(R * ff * 2, s));
+  const bool i8 = d->kv_dtype == YSCV_HIP_KV_I8;
+  const int t_ctx = (start_pos + rows + 31) / 32 * 32;
+  StreamBuf tk, tv;
+  if (i8) {
+    YSCV_TRY(tk.alloc((size_t)c.n_kv_heads * t_ctx * c.head_dim * 2, s));
+    YSCV_TRY(tv.alloc((size_t)c.n_kv_heads * t_ctx * c.head_dim * 2, s));
+  }
   YSCV_TRY(launch_embed(tokens_dev, d->emb, rows, (int)D, c.vocab, h.as<float>(), s));
   for (auto &L : d->layers) {
     YSCV_TRY(launch_rmsnorm(h.as<float>(), L.attn_norm, rows, (int)D, c.rms_eps, xn.as<_Float16>(), s));
     YSCV_TRY(int4_run_ws(L.wqkv, xn.p, YSCV_HIP_F16, qkv.p, YSCV_HIP_F16, R, 0, EPI_STORE, nullptr, 0, s));
     if (L.qkv_bias) YSCV_TRY(launch_bias_add_f16(qkv.as<_Float16>(), L.qkv_bias, R, qkv_n, s));
-    YSCV_TRY(launch_prefill_rope_append(qkv.as<_Float16>(), rows, start_pos, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_theta,
-                                        c.max_ctx, L.kc, L.vc, s));
-    YSCV_TRY(launch_gqa_cache(qkv.as<_Float16>(), L.kc, L.vc, nullptr, rows, start_pos, c.n_heads, c.n_kv_heads, c.head_dim,
-                              c.max_ctx, ao.as<_Float16>(), s));
+    if (i8) {
+      // the quantised append, and attention over what the int8 cache returns for every position so far (fp16 scratch)
+      YSCV_TRY(launch_prefill_rope_append_i8(qkv.as<_Float16>(), rows, start_pos, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_theta,
+                                             c.max_ctx, L.kc8, L.ks, L.vc8, L.vs, t_ctx, tk.as<_Float16>(), tv.as<_Float16>(), s));
+      YSCV_TRY(launch_gqa_cache(qkv.as<_Float16>(), tk.as<_Float16>(), tv.as<_Float16>(), nullptr, rows, start_pos, c.n_heads,
+                                c.n_kv_heads, c.head_dim, t_ctx, ao.as<_Float16>(), s));
+    } else {
+      YSCV_TRY(launch_prefill_rope_append(qkv.as<_Float16>(), rows, start_pos, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_theta,
+                                          c.max_ctx, L.kc, L.vc, s));
+      YSCV_TRY(launch_gqa_cache(qkv.as<_Float16>(), L.kc, L.vc, nullptr, rows, start_pos, c.n_heads, c.n_kv_heads, c.head_dim,
+                                c.max_ctx, ao.as<_Float16>(), s));
+    }
     // the residual update and SwiGLU ride on the projections' epilogues (both kernels have them: the skinny kernel up to
     // 16 rows, the LDS-ring GEMM above)
     YSCV_TRY(int4_run_ws(L.wo, ao.p, YSCV_HIP_F16, h.p, YSCV_HIP_F32, R, 0, EPI_ADD_F32, nullptr, 0, s));
@@ -1184,15 +1199,6 @@ int32_t yscv_hip_decoder_prefill(yscv_hip_decoder *d, const int32_t *tokens_host
   for (int32_t i = 0; i < n_tokens; i++)
     YSCV_REQUIRE(tokens_host[i] >= 0 && tokens_host[i] < c.vocab, "token %d outside the vocabulary (%d)", tokens_host[i], c.vocab);
   hipStream_t s = as_stream(stream);
-  if (d->kv_dtype != YSCV_HIP_KV_F16) {
-    // the quantised cache appends one row at a time (its row scales cover all kv heads): the prompt goes through the
-    // decode step position by position
-    for (int32_t i = 0; i < n_tokens; i++) {
-      YSCV_TRY(yscv_hip_decoder_reset(d, 1, start_pos + i, tokens_host + i));
-      YSCV_TRY(yscv_hip_decoder_run(d, 1, 1, stream));
-    }
-    return YSCV_HIP_OK;
-  }
   d->batch = 1;
   StreamBuf toks;
   YSCV_TRY(toks.alloc((size_t)n_tokens * 4, s));

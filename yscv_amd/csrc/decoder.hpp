@@ -29,6 +29,12 @@ int32_t launch_attention_fused(const _Float16 *qkv, _Float16 *kc, _Float16 *vc, 
 // one f32 scale per (batch row, position) for each of them
 int32_t launch_rope_append_i8(_Float16 *qkv, const int32_t *pos_ptr, int batch, int hq, int hkv, int hd, float theta,
                               int max_ctx, int8_t *kc, float *ks, int8_t *vc, float *vs, hipStream_t s);
+// prompt pass: positions start_pos .. start_pos + rows - 1 of batch row 0 rotated, quantised and appended; tk / tv
+// (fp16, laid out like the fp16 cache with t_ctx positions) receive what the int8 cache returns for positions
+// 0 .. start_pos + rows - 1
+int32_t launch_prefill_rope_append_i8(_Float16 *qkv, int rows, int start_pos, int hq, int hkv, int hd, float theta, int max_ctx,
+                                      int8_t *kc, float *ks, int8_t *vc, float *vs, int t_ctx, _Float16 *tk, _Float16 *tv,
+                                      hipStream_t s);
 int32_t launch_kv_relayout_i8(const _Float16 *k_nat, const _Float16 *v_nat, int batch, int npos, int hkv, int hd, int max_ctx,
                               int8_t *kc, float *ks, int8_t *vc, float *vs, hipStream_t s);
 int32_t launch_attention_i8(const _Float16 *qkv, const int8_t *kc, const float *ks, const int8_t *vc, const float *vs,

@@ -884,6 +884,81 @@ __global__ void __launch_bounds__(256) rope_append_i8_kernel(_Float16 *__restric
   }
 }
 
+// Prompt pass on the int8 cache: the same rotation, row scales and quantisation for `rows` consecutive positions of
+// batch row 0 (one workgroup per position), and what the cache now returns for each appended value (q * scale of its
+// row, LayerStorage::dequantise_to_vec, crates/yscv-onnx/src/runner/kv_cache.rs:64-79) as fp16 in a scratch K / V
+// pair laid out like the fp16 cache with t_ctx positions: the prompt's attention reads that pair.
+__global__ void __launch_bounds__(256) prefill_rope_append_i8_kernel(_Float16 *__restrict__ qkv, int start_pos, int hq, int hkv,
+                                                                     float theta, int max_ctx, int8_t *__restrict__ kc,
+                                                                     float *__restrict__ ks, int8_t *__restrict__ vc,
+                                                                     float *__restrict__ vs, int t_ctx, _Float16 *__restrict__ tk,
+                                                                     _Float16 *__restrict__ tv) {
+  constexpr int HD = 128, HALF = 64;
+  extern __shared__ float kv_lds[];
+  __shared__ float red[4];
+  const int tid = threadIdx.x;
+  const int pos = start_pos + (int)blockIdx.x;
+  const int kv_dim = hkv * HD;
+  float *kbuf = kv_lds, *vbuf = kv_lds + kv_dim;
+  _Float16 *row = qkv + (size_t)blockIdx.x * (hq + 2 * hkv) * HD;
+  float kmax = 0.0f, vmax = 0.0f;
+  for (int idx = tid; idx < (hq + hkv) * HALF; idx += 256) {
+    const int slot = idx / HALF, i = idx % HALF;
+    const SinCos sc = rope_sincos(theta, i, HD, pos);
+    _Float16 *src = row + (size_t)slot * HD;
+    const float x0 = (float)src[i], x1 = (float)src[i + HALF];
+    float y0, y1;
+    rope_pair_f32(x0, x1, sc.cs, sc.sn, y0, y1);
+    if (slot < hq) {
+      src[i] = f16_of_f32(y0);
+      src[i + HALF] = f16_of_f32(y1);
+    } else {
+      kbuf[(slot - hq) * HD + i] = y0;
+      kbuf[(slot - hq) * HD + i + HALF] = y1;
+      kmax = fmaxf(kmax, fmaxf(fabsf(y0), fabsf(y1)));
+    }
+  }
+  for (int idx = tid; idx < kv_dim; idx += 256) {
+    const float v = (float)row[(size_t)(hq + hkv) * HD + idx];
+    vbuf[idx] = v;
+    vmax = fmaxf(vmax, fabsf(v));
+  }
+  __syncthreads();
+  kmax = block_max_256(kmax, red);
+  vmax = block_max_256(vmax, red);
+  float k_scale, k_inv, v_scale, v_inv;
+  kv_row_scale(kmax, &k_scale, &k_inv);
+  kv_row_scale(vmax, &v_scale, &v_inv);
+  if (tid == 0) {
+    ks[pos] = k_scale;
+    vs[pos] = v_scale;
+  }
+  for (int idx = tid; idx < kv_dim; idx += 256) {
+    const int kvh = idx / HD, i = idx % HD;
+    const int8_t kq = kv_quant_one(kbuf[idx], k_inv), vq = kv_quant_one(vbuf[idx], v_inv);
+    kc[((size_t)kvh * max_ctx + pos) * HD + i] = kq;
+    vc[(((size_t)kvh * (max_ctx / 8) + pos / 8) * HD + i) * 8 + (pos & 7)] = vq;
+    tk[((size_t)kvh * t_ctx + pos) * HD + i] = (_Float16)((float)kq * k_scale);
+    tv[(((size_t)kvh * (t_ctx / 8) + pos / 8) * HD + i) * 8 + (pos & 7)] = (_Float16)((float)vq * v_scale);
+  }
+}
+
+// positions 0 .. npos-1 of batch row 0 of the int8 cache, dequantised into the scratch pair of the prompt pass
+__global__ void __launch_bounds__(256) kv_dequant_i8_kernel(const int8_t *__restrict__ kc, const float *__restrict__ ks,
+                                                            const int8_t *__restrict__ vc, const float *__restrict__ vs, int hkv,
+                                                            int max_ctx, int t_ctx, _Float16 *__restrict__ tk,
+                                                            _Float16 *__restrict__ tv) {
+  constexpr int HD = 128;
+  const int pos = blockIdx.x;
+  const float k_scale = ks[pos], v_scale = vs[pos];
+  for (int idx = threadIdx.x; idx < hkv * HD; idx += 256) {
+    const int kvh = idx / HD, i = idx % HD;
+    tk[((size_t)kvh * t_ctx + pos) * HD + i] = (_Float16)((float)kc[((size_t)kvh * max_ctx + pos) * HD + i] * k_scale);
+    tv[(((size_t)kvh * (t_ctx / 8) + pos / 8) * HD + i) * 8 + (pos & 7)] =
+        (_Float16)((float)vc[(((size_t)kvh * (max_ctx / 8) + pos / 8) * HD + i) * 8 + (pos & 7)] * v_scale);
+  }
+}
+
 // ---- rotary embedding + int8 cache append + attention partials in ONE launch (int8 cache) ---------------------------
 // rope_append_i8_kernel -> attn_partial_kernel<true> without the kernel boundary, as attn_fused_kernel does it for the
 // fp16 cache.  The scale of an int8 row spans all kv heads of the position, so each of the Hkv workgroups whose chunk
@@ -1273,6 +1348,23 @@ int32_t launch_rope_append_i8(_Float16 *qkv, const int32_t *pos_ptr, int batch, 
   const size_t lds = (size_t)2 * hkv * hd * sizeof(float);
   if (lds > 48 * 1024) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "int8 cache append: too many kv heads (%d)", hkv);
   hipLaunchKernelGGL(rope_append_i8_kernel, dim3(batch), dim3(256), lds, s, qkv, pos_ptr, hq, hkv, theta, max_ctx, kc, ks, vc, vs);
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
+int32_t launch_prefill_rope_append_i8(_Float16 *qkv, int rows, int start_pos, int hq, int hkv, int hd, float theta, int max_ctx,
+                                      int8_t *kc, float *ks, int8_t *vc, float *vs, int t_ctx, _Float16 *tk, _Float16 *tv,
+                                      hipStream_t s) {
+  if (hd != 128) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "int8 cache append is built for head_dim 128, got %d", hd);
+  const size_t lds = (size_t)2 * hkv * hd * sizeof(float);
+  if (lds > 48 * 1024) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "int8 cache append: too many kv heads (%d)", hkv);
+  if (t_ctx % 8 != 0 || t_ctx < start_pos + rows) return set_error(YSCV_HIP_ERR_INVALID_ARG, "scratch K / V: %d positions", t_ctx);
+  if (start_pos > 0) {
+    hipLaunchKernelGGL(kv_dequant_i8_kernel, dim3(start_pos), dim3(256), 0, s, kc, ks, vc, vs, hkv, max_ctx, t_ctx, tk, tv);
+    YSCV_HIP_TRY(hipGetLastError());
+  }
+  hipLaunchKernelGGL(prefill_rope_append_i8_kernel, dim3(rows), dim3(256), lds, s, qkv, start_pos, hq, hkv, theta, max_ctx, kc, ks,
+                     vc, vs, t_ctx, tk, tv);
   YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
 }
