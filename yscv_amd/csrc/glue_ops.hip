@@ -597,35 +597,62 @@ __global__ void __launch_bounds__(64) rope_f32_kernel(float *__restrict__ x, int
 
 // ---- small kernels of the prompt pass (rows = consecutive positions of one sequence) ------------------------------
 // RoPE on the q and k heads of every row (row i sits at position start_pos + i), k and v appended to batch row 0 of
-// the cache: the arithmetic of the decode step's rope + append, one launch for all rows.
-__global__ void __launch_bounds__(64) prefill_rope_append_kernel(_Float16 *__restrict__ qkv, int start_pos, int hq, int hkv, int hd,
-                                                                 float theta, int max_ctx, _Float16 *__restrict__ kc,
-                                                                 _Float16 *__restrict__ vc) {
-  const int row = blockIdx.y, slot = blockIdx.x;
-  const int pos = start_pos + row;
-  _Float16 *src = qkv + (size_t)row * (hq + 2 * hkv) * hd + (size_t)slot * hd;
+// the cache: the arithmetic of the decode step's rope + append, one launch for all rows.  A workgroup takes the (up
+// to eight) rows whose positions share one 8-position slab of the V layout: the angle of a pair is worked out once per
+// position for all heads, and the values of a channel at the slab's positions leave as one 16-byte store where the
+// whole slab is new.
+__global__ void __launch_bounds__(256) prefill_rope_append_kernel(_Float16 *__restrict__ qkv, int rows, int start_pos, int hq, int hkv,
+                                                                  int hd, float theta, int max_ctx, _Float16 *__restrict__ kc,
+                                                                  _Float16 *__restrict__ vc) {
+  const int tid = threadIdx.x;
+  const int slab = start_pos / 8 + (int)blockIdx.x;
+  const int p_lo = max(start_pos, slab * 8), p_hi = min(start_pos + rows, slab * 8 + 8);  // positions [p_lo, p_hi)
+  const size_t row_elems = (size_t)(hq + 2 * hkv) * hd;
   const int half_d = hd / 2;
-  if (slot < hq + hkv) {
-    for (int i = threadIdx.x; i < half_d; i += 64) {
-      const float inv_freq = 1.0f / powf(theta, (float)(2 * i) / (float)hd);
-      float sn, cs;
-      sincosf(inv_freq * (float)pos, &sn, &cs);
-      const float x0 = (float)src[i], x1 = (float)src[i + half_d];
-      float f0 = fmaf(x0, cs, -(x1 * sn)), f1 = fmaf(x0, sn, x1 * cs);
+  // the angle of pair i at each of the slab's positions, once for all heads
+  __shared__ float cs_s[8][64], sn_s[8][64];
+  const int n_pos = p_hi - p_lo;
+  for (int idx = tid; idx < n_pos * half_d; idx += 256) {
+    const int e = idx / half_d, i = idx % half_d;
+    const float inv_freq = 1.0f / powf(theta, (float)(2 * i) / (float)hd);
+    sincosf(inv_freq * (float)(p_lo + e), &sn_s[e][i], &cs_s[e][i]);
+  }
+  __syncthreads();
+  const int slots = hq + hkv, vecs = half_d / 8;  // eight pairs per item: 16-byte loads and stores
+#pragma unroll 2
+  for (int item = tid; item < n_pos * slots * vecs; item += 256) {
+    const int i0 = (item % vecs) * 8, slot = (item / vecs) % slots, e = item / (vecs * slots);
+    const int pos = p_lo + e;
+    _Float16 *src = qkv + (size_t)(pos - start_pos) * row_elems + (size_t)slot * hd;
+    const half8_t x0 = *reinterpret_cast<const half8_t *>(src + i0), x1 = *reinterpret_cast<const half8_t *>(src + i0 + half_d);
+    half8_t y0, y1;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const float cs = cs_s[e][i0 + j], sn = sn_s[e][i0 + j];
+      const float a = (float)x0[j], b = (float)x1[j];
+      float f0 = fmaf(a, cs, -(b * sn)), f1 = fmaf(a, sn, b * cs);
       asm volatile("" : "+v"(f0), "+v"(f1));  // the f32 value exists before it is narrowed (no mixed-precision fma)
-      const _Float16 y0 = (_Float16)f0, y1 = (_Float16)f1;
-      if (slot < hq) {
-        src[i] = y0;
-        src[i + half_d] = y1;
-      } else {
-        _Float16 *dst = kc + ((size_t)(slot - hq) * max_ctx + pos) * hd;
-        dst[i] = y0;
-        dst[i + half_d] = y1;
-      }
+      y0[j] = (_Float16)f0;
+      y1[j] = (_Float16)f1;
     }
-  } else {
-    _Float16 *dst = vc + (((size_t)(slot - hq - hkv) * (max_ctx / 8) + pos / 8) * hd) * 8 + (pos & 7);
-    for (int i = threadIdx.x; i < hd; i += 64) dst[(size_t)i * 8] = src[i];
+    _Float16 *dst = slot < hq ? src : kc + ((size_t)(slot - hq) * max_ctx + pos) * hd;
+    *reinterpret_cast<half8_t *>(dst + i0) = y0;
+    *reinterpret_cast<half8_t *>(dst + i0 + half_d) = y1;
+  }
+  // v: channel ch of kv head kvh at the slab's positions
+  const _Float16 *vsrc = qkv + (size_t)(hq + hkv) * hd;
+  const bool whole = p_hi - p_lo == 8;
+  for (int idx = tid; idx < hkv * hd; idx += 256) {
+    const int kvh = idx / hd, ch = idx % hd;
+    _Float16 *dst = vc + (((size_t)kvh * (max_ctx / 8) + slab) * hd + ch) * 8;
+    if (whole) {
+      half8_t v;
+#pragma unroll
+      for (int e = 0; e < 8; e++) v[e] = vsrc[(size_t)(p_lo - start_pos + e) * row_elems + idx];
+      *reinterpret_cast<half8_t *>(dst) = v;
+    } else {
+      for (int pos = p_lo; pos < p_hi; pos++) dst[pos & 7] = vsrc[(size_t)(pos - start_pos) * row_elems + idx];
+    }
   }
 }
 
@@ -655,8 +682,10 @@ unsigned flat_grid(size_t n) {
 
 int32_t launch_prefill_rope_append(_Float16 *qkv, int rows, int start_pos, int hq, int hkv, int hd, float theta, int max_ctx,
                                    _Float16 *kc, _Float16 *vc, hipStream_t s) {
-  hipLaunchKernelGGL(prefill_rope_append_kernel, dim3(hq + 2 * hkv, rows), dim3(64), 0, s, qkv, start_pos, hq, hkv, hd, theta, max_ctx,
-                     kc, vc);
+  if (hd > 128 || hd % 16 != 0) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "rope + append: head width %d", hd);
+  const int slabs = (start_pos + rows - 1) / 8 - start_pos / 8 + 1;
+  hipLaunchKernelGGL(prefill_rope_append_kernel, dim3(slabs), dim3(256), 0, s, qkv, rows, start_pos, hq, hkv, hd, theta, max_ctx, kc,
+                     vc);
   YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
 }
