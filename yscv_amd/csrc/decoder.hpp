@@ -58,7 +58,5 @@ int32_t launch_gqa_cache(const _Float16 *qkv, const _Float16 *kc, const _Float16
 int32_t launch_prefill_rope_append(_Float16 *qkv, int rows, int start_pos, int hq, int hkv, int hd, float theta, int max_ctx,
                                    _Float16 *kc, _Float16 *vc, hipStream_t s);
 int32_t launch_bias_add_f16(_Float16 *x, const _Float16 *bias, size_t rows, size_t n, hipStream_t s);
-int32_t launch_residual_add(float *h, const float *t, size_t count, hipStream_t s);
-int32_t launch_swiglu_rows(const float *gu, _Float16 *act, size_t rows, size_t ff, hipStream_t s);
 
 }  // namespace yscv

@@ -9,7 +9,11 @@
 // query positions per call with a causal limit (prompt ingestion), K / V either as the operator's tensors or as the
 // decoder's fp16 cache.
 //
-// Attention kernel: a workgroup of four waves owns 16 query positions of one head.  Wave w walks the key blocks
+// Three forms of the attention kernel share the arithmetic below: gqa_generic_kernel (a workgroup owns 16 queries of
+// one head, the key blocks are split over its waves: decode and short query counts), gqa_rows_kernel (a wave owns 32
+// queries and walks every key block: the operator from 64 queries on) and gqa_shared_kv_kernel (the prompt pass over
+// the decoder's cache: the waves of a workgroup share each stage of K / V through LDS).
+// gqa_generic_kernel: a workgroup of four waves owns 16 query positions of one head.  Wave w walks the key blocks
 // w, w + 4, ... of 16 positions each:
 //   S^T = K Q^T   rows = positions, columns = queries: hd / 32 x v_mfma_f32_16x16x32_f16, A = 16 cache rows as they lie
 //                 in memory, B = the 16 query rows as they lie in memory; lane (r, c) then holds positions 4c .. 4c+3
@@ -67,8 +71,6 @@ __device__ __forceinline__ void store4<float>(float *p, float a, float b, float 
 }
 
 constexpr int GQA_WAVES = 4;
-
-__device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
 
 template <int HD, typename TQ, typename TKV, typename TO, bool V_SLAB>
 __global__ void __launch_bounds__(64 * GQA_WAVES) gqa_generic_kernel(GqaArgs p) {
@@ -661,18 +663,6 @@ __global__ void bias_add_f16_kernel(_Float16 *__restrict__ x, const _Float16 *__
     x[idx] = (_Float16)((float)x[idx] + (float)bias[idx % n]);
 }
 
-__global__ void residual_add_kernel(float *__restrict__ h, const float *__restrict__ t, size_t count) {
-  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < count; idx += (size_t)gridDim.x * blockDim.x) h[idx] += t[idx];
-}
-
-// gu [rows][2 ff] f32 with gate_i, up_i interleaved -> act [rows][ff] fp16 = silu(gate) * up
-__global__ void swiglu_rows_kernel(const float *__restrict__ gu, _Float16 *__restrict__ act, size_t count) {
-  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < count; idx += (size_t)gridDim.x * blockDim.x) {
-    const float g = gu[2 * idx], u = gu[2 * idx + 1];
-    act[idx] = (_Float16)(silu(g) * u);
-  }
-}
-
 unsigned flat_grid(size_t n) {
   const size_t b = (n + 255) / 256;
   return (unsigned)(b > 65535 ? 65535 : (b < 1 ? 1 : b));
@@ -691,16 +681,6 @@ int32_t launch_prefill_rope_append(_Float16 *qkv, int rows, int start_pos, int h
 }
 int32_t launch_bias_add_f16(_Float16 *x, const _Float16 *bias, size_t rows, size_t n, hipStream_t s) {
   hipLaunchKernelGGL(bias_add_f16_kernel, dim3(flat_grid(rows * n)), dim3(256), 0, s, x, bias, rows, n);
-  YSCV_HIP_TRY(hipGetLastError());
-  return YSCV_HIP_OK;
-}
-int32_t launch_residual_add(float *h, const float *t, size_t count, hipStream_t s) {
-  hipLaunchKernelGGL(residual_add_kernel, dim3(flat_grid(count)), dim3(256), 0, s, h, t, count);
-  YSCV_HIP_TRY(hipGetLastError());
-  return YSCV_HIP_OK;
-}
-int32_t launch_swiglu_rows(const float *gu, _Float16 *act, size_t rows, size_t ff, hipStream_t s) {
-  hipLaunchKernelGGL(swiglu_rows_kernel, dim3(flat_grid(rows * ff)), dim3(256), 0, s, gu, act, rows * ff);
   YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
 }
