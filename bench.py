@@ -521,6 +521,8 @@ def main():
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the prompt phase (2048 tokens through yscv_hip_decoder_prefill) and print its figures "
                          "(the run the rocprofv3 summary of the prompt pass is taken from)")
+    ap.add_argument("--prefill-tokens", type=int, nargs="+", default=[2048],
+                    help="prompt lengths for --prefill-only (default 2048; several lengths give one entry each)")
     ap.add_argument("--graph-path", action="store_true",
                     help="time the multi-kernel path (one HIP-graph replay per step) instead of the single-launch kernel")
     ap.add_argument("--no-check", action="store_true",
@@ -566,7 +568,7 @@ def main():
     w_bytes, params = decode_bytes_per_step(cfg)
     assert dec.weight_bytes() >= w_bytes
     if args.prefill_only:
-        print(json.dumps({"extra": {"prefill_2048_tokens": bench_prefill(dec, torch, cfg, 2048, params)}}))
+        print(json.dumps({"extra": {"prefill_%d_tokens" % n: bench_prefill(dec, torch, cfg, n, params) for n in args.prefill_tokens}}))
         return
 
     persistent = args.batch == 1 and not args.graph_path

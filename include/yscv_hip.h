@@ -164,8 +164,10 @@ int32_t yscv_hip_int4_matmul_fused(const yscv_hip_int4_weight *w, const void *x_
 /* Same as yscv_hip_int4_matmul, but every byte of device scratch comes from the caller, so
  * the call allocates nothing (the reference allocates its output per call,
  * linear.rs:237; there is no scratch to compare with).  workspace_dev must be 256-byte
- * aligned and at least yscv_hip_int4_workspace_bytes(w, m, x_dtype) long (0 for fp16
- * activations whose K is a multiple of 128 and fits one workgroup's K range). */
+ * aligned and at least yscv_hip_int4_workspace_bytes(w, m, x_dtype) long: the prepared
+ * activations, the partial sums of the skinny kernel's grid-level K split and, above 16 rows,
+ * those of the GEMM's K split (shapes with fewer output tiles than half the CUs); 0 for fp16
+ * activations whose K is a multiple of 128 when neither kernel splits K across workgroups. */
 int32_t yscv_hip_int4_workspace_bytes(const yscv_hip_int4_weight *w, size_t m, int32_t x_dtype,
                                       size_t *bytes);
 int32_t yscv_hip_int4_matmul_ws(const yscv_hip_int4_weight *w, const void *x_dev, int32_t x_dtype,

@@ -95,6 +95,7 @@ struct Int4Scratch {
   size_t k_pad;
   SkinnyPlan plan;
   size_t xh_bytes, rs_bytes, part_bytes, total;
+  size_t opt_bytes;  // behind `total`: the K-split partials of the LDS-ring GEMM (0 when that launch is not split)
 };
 
 // f32 activations on the exact-scale route with 16 < m <= this many rows run as 16-row skinny calls
@@ -113,6 +114,7 @@ static Int4Scratch int4_scratch_layout(const yscv_hip_int4_weight *w, const void
   L.rs_bytes = L.direct ? 0 : round_up(m * sizeof(float), 256);
   L.part_bytes = L.skinny ? round_up(L.plan.partial_bytes, 256) : 0;
   L.total = L.xh_bytes * L.split + L.rs_bytes + L.part_bytes;
+  L.opt_bytes = L.skinny ? 0 : round_up(int4_gemm_ring_partial_bytes(w, m, num_cus), 256);
   if (!L.skinny && force == 0 && x_dtype == YSCV_HIP_F32 && m <= kChunkedSkinnyMaxRows) {
     // this call may run as 16-row skinny calls (see int4_run_ws): the scratch must cover one of those too
     const Int4Scratch c = int4_scratch_layout(w, x, x_dtype, 16, 1, num_cus);
@@ -131,7 +133,7 @@ int32_t int4_workspace_bytes(const yscv_hip_int4_weight *w, size_t m, int x_dtyp
   }
   // a 16-byte aligned pointer stands in for the activation: alignment is checked again at run time
   Int4Scratch L = int4_scratch_layout(w, reinterpret_cast<const void *>(uintptr_t(256)), x_dtype, m, force, ctx->num_cus);
-  *bytes = L.total;
+  *bytes = L.total + L.opt_bytes;
   return YSCV_HIP_OK;
 }
 
@@ -179,15 +181,20 @@ int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, v
   }
   char *scratch = static_cast<char *>(ws);
   bool own = false;
-  if (L.total > 0) {
+  size_t have = ws_bytes;
+  if (L.total + L.opt_bytes > 0) {
     if (scratch) {
-      YSCV_REQUIRE(ws_bytes >= L.total, "workspace too small: %zu < %zu bytes", ws_bytes, L.total);
+      YSCV_REQUIRE(ws_bytes >= L.total + L.opt_bytes, "workspace too small: %zu < %zu bytes", ws_bytes, L.total + L.opt_bytes);
       YSCV_REQUIRE((reinterpret_cast<uintptr_t>(scratch) & 255) == 0, "workspace must be 256-byte aligned");
     } else {
-      YSCV_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&scratch), L.total, s));
+      have = L.total + L.opt_bytes;
+      YSCV_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&scratch), have, s));
       own = true;
     }
   }
+  // the GEMM's K-split partials sit behind everything else
+  float *gemm_partial = (scratch != nullptr && L.opt_bytes > 0 && have >= L.total + L.opt_bytes)
+                            ? reinterpret_cast<float *>(scratch + L.total) : nullptr;
   const void *xraw = (L.direct && x_dtype != YSCV_HIP_F16) ? x : nullptr;
   const _Float16 *xh = L.direct ? static_cast<const _Float16 *>(x) : reinterpret_cast<_Float16 *>(scratch);
   _Float16 *xl = (!L.direct && L.split == 2) ? reinterpret_cast<_Float16 *>(scratch + L.xh_bytes) : nullptr;
@@ -212,7 +219,7 @@ int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, v
     if (L.skinny)
       st = launch_int4_skinny(w, L.plan, xh, xl, xraw, row_scale, L.k_pad, L.split, y, y_dtype, m, partial, epi, s, nf);
     else
-      st = launch_int4_gemm(w, xh, xl, row_scale, L.k_pad, run_split, y, y_dtype, m, s, epi);
+      st = launch_int4_gemm(w, xh, xl, row_scale, L.k_pad, run_split, y, y_dtype, m, s, epi, gemm_partial, L.opt_bytes);
   }
   if (own) {
     hipError_t fe = hipFreeAsync(scratch, s);
@@ -507,10 +514,10 @@ int32_t yscv_hip_int4_matmul_static(const yscv_hip_int4_weight *w, const void *x
   if (ws == nullptr) return set_error(YSCV_HIP_ERR_DEVICE, "the static scratch of device %d was never resolved", ctx->device);
   if (w->tiled) {
     const Int4Scratch L = int4_scratch_layout(w, x_dev, x_dtype, m, 0, ctx->num_cus);
-    if (L.total > (size_t)YSCV_HIP_STATIC_SCRATCH_BYTES)
+    if (L.total + L.opt_bytes > (size_t)YSCV_HIP_STATIC_SCRATCH_BYTES)
       return set_error(YSCV_HIP_ERR_INVALID_ARG,
                        "this call needs %zu bytes of scratch, the static scratch holds %zu: use yscv_hip_int4_matmul_ws",
-                       L.total, (size_t)YSCV_HIP_STATIC_SCRATCH_BYTES);
+                       L.total + L.opt_bytes, (size_t)YSCV_HIP_STATIC_SCRATCH_BYTES);
   }
   return int4_run_ws(w, x_dev, x_dtype, y_dev, y_dtype, m, 0, EPI_STORE, ws, YSCV_HIP_STATIC_SCRATCH_BYTES, as_stream(stream));
 }

@@ -1157,10 +1157,20 @@ static int32_t prefill_chunk(yscv_hip_decoder *d, const int32_t *tokens_dev, int
     YSCV_TRY(tk.alloc((size_t)c.n_kv_heads * t_ctx * c.head_dim * 2, s));
     YSCV_TRY(tv.alloc((size_t)c.n_kv_heads * t_ctx * c.head_dim * 2, s));
   }
+  // one scratch for all projections of the pass (prepared activations are not needed: the rows are fp16 already; what
+  // remains are the K-split partial sums of the short-prompt shapes)
+  size_t ws_bytes = 0;
+  for (const yscv_hip_int4_weight *w : {d->layers[0].wqkv, d->layers[0].wo, d->layers[0].wgu, d->layers[0].wdown}) {
+    size_t b = 0;
+    YSCV_TRY(int4_workspace_bytes(w, R, YSCV_HIP_F16, 0, &b));
+    ws_bytes = b > ws_bytes ? b : ws_bytes;
+  }
+  StreamBuf pws;
+  if (ws_bytes > 0) YSCV_TRY(pws.alloc(ws_bytes, s));
   YSCV_TRY(launch_embed(tokens_dev, d->emb, rows, (int)D, c.vocab, h.as<float>(), s));
   for (auto &L : d->layers) {
     YSCV_TRY(launch_rmsnorm(h.as<float>(), L.attn_norm, rows, (int)D, c.rms_eps, xn.as<_Float16>(), s));
-    YSCV_TRY(int4_run_ws(L.wqkv, xn.p, YSCV_HIP_F16, qkv.p, YSCV_HIP_F16, R, 0, EPI_STORE, nullptr, 0, s));
+    YSCV_TRY(int4_run_ws(L.wqkv, xn.p, YSCV_HIP_F16, qkv.p, YSCV_HIP_F16, R, 0, EPI_STORE, pws.p, ws_bytes, s));
     if (L.qkv_bias) YSCV_TRY(launch_bias_add_f16(qkv.as<_Float16>(), L.qkv_bias, R, qkv_n, s));
     if (i8) {
       // the quantised append, and attention over what the int8 cache returns for every position so far (fp16 scratch)
@@ -1176,10 +1186,10 @@ static int32_t prefill_chunk(yscv_hip_decoder *d, const int32_t *tokens_dev, int
     }
     // the residual update and SwiGLU ride on the projections' epilogues (both kernels have them: the skinny kernel up to
     // 16 rows, the LDS-ring GEMM above)
-    YSCV_TRY(int4_run_ws(L.wo, ao.p, YSCV_HIP_F16, h.p, YSCV_HIP_F32, R, 0, EPI_ADD_F32, nullptr, 0, s));
+    YSCV_TRY(int4_run_ws(L.wo, ao.p, YSCV_HIP_F16, h.p, YSCV_HIP_F32, R, 0, EPI_ADD_F32, pws.p, ws_bytes, s));
     YSCV_TRY(launch_rmsnorm(h.as<float>(), L.ffn_norm, rows, (int)D, c.rms_eps, xn.as<_Float16>(), s));
-    YSCV_TRY(int4_run_ws(L.wgu, xn.p, YSCV_HIP_F16, act.p, YSCV_HIP_F16, R, 0, EPI_SWIGLU, nullptr, 0, s));
-    YSCV_TRY(int4_run_ws(L.wdown, act.p, YSCV_HIP_F16, h.p, YSCV_HIP_F32, R, 0, EPI_ADD_F32, nullptr, 0, s));
+    YSCV_TRY(int4_run_ws(L.wgu, xn.p, YSCV_HIP_F16, act.p, YSCV_HIP_F16, R, 0, EPI_SWIGLU, pws.p, ws_bytes, s));
+    YSCV_TRY(int4_run_ws(L.wdown, act.p, YSCV_HIP_F16, h.p, YSCV_HIP_F32, R, 0, EPI_ADD_F32, pws.p, ws_bytes, s));
   }
   if (last) {
     YSCV_TRY(launch_rmsnorm(h.as<float>() + (R - 1) * D, d->final_norm, 1, (int)D, c.rms_eps, d->xn, s));

@@ -622,7 +622,8 @@ __global__ void __launch_bounds__(256) prefill_rope_append_kernel(_Float16 *__re
   __syncthreads();
   const int slots = hq + hkv, vecs = half_d / 8;  // eight pairs per item: 16-byte loads and stores
 #pragma unroll 2
-  for (int item = tid; item < n_pos * slots * vecs; item += 256) {
+  // blockIdx.y takes every gridDim.y-th item of the slab (short prompts have few slabs and would leave the CUs idle)
+  for (int item = tid + 256 * (int)blockIdx.y; item < n_pos * slots * vecs; item += 256 * (int)gridDim.y) {
     const int i0 = (item % vecs) * 8, slot = (item / vecs) % slots, e = item / (vecs * slots);
     const int pos = p_lo + e;
     _Float16 *src = qkv + (size_t)(pos - start_pos) * row_elems + (size_t)slot * hd;
@@ -644,7 +645,7 @@ __global__ void __launch_bounds__(256) prefill_rope_append_kernel(_Float16 *__re
   // v: channel ch of kv head kvh at the slab's positions
   const _Float16 *vsrc = qkv + (size_t)(hq + hkv) * hd;
   const bool whole = p_hi - p_lo == 8;
-  for (int idx = tid; idx < hkv * hd; idx += 256) {
+  for (int idx = tid + 256 * (int)blockIdx.y; idx < hkv * hd; idx += 256 * (int)gridDim.y) {
     const int kvh = idx / hd, ch = idx % hd;
     _Float16 *dst = vc + (((size_t)kvh * (max_ctx / 8) + slab) * hd + ch) * 8;
     if (whole) {
@@ -674,8 +675,10 @@ int32_t launch_prefill_rope_append(_Float16 *qkv, int rows, int start_pos, int h
                                    _Float16 *kc, _Float16 *vc, hipStream_t s) {
   if (hd > 128 || hd % 16 != 0) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "rope + append: head width %d", hd);
   const int slabs = (start_pos + rows - 1) / 8 - start_pos / 8 + 1;
-  hipLaunchKernelGGL(prefill_rope_append_kernel, dim3(slabs), dim3(256), 0, s, qkv, rows, start_pos, hq, hkv, hd, theta, max_ctx, kc,
-                     vc);
+  int parts = 512 / slabs;  // about two workgroups per CU
+  parts = parts < 1 ? 1 : (parts > 16 ? 16 : parts);
+  hipLaunchKernelGGL(prefill_rope_append_kernel, dim3(slabs, parts), dim3(256), 0, s, qkv, rows, start_pos, hq, hkv, hd, theta, max_ctx,
+                     kc, vc);
   YSCV_HIP_TRY(hipGetLastError());
   return YSCV_HIP_OK;
 }

@@ -252,12 +252,12 @@ static int32_t gemm_launch_gm(const GemmArgs &a, int gm, bool sf16, hipStream_t 
 
 int32_t launch_int4_gemm(const yscv_hip_int4_weight *w, const _Float16 *xh, const _Float16 *xl,
                          const float *row_scale, size_t k_pad, int split, void *y, int y_dtype, size_t m,
-                         hipStream_t s, int epi) {
+                         hipStream_t s, int epi, float *partial, size_t partial_bytes) {
   if (!w->tiled) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "int4 GEMM kernel needs the tiled layout");
   // 16-bit activations: the LDS-ring kernel from the first row count the skinny kernel does not take (rows are
   // padded to its 128-row tile; with few rows the weights are still streamed exactly once)
   if (m > 16 && int4_gemm_ring_eligible(w, xh, y, y_dtype, split, m, k_pad))
-    return launch_int4_gemm_ring(w, xh, row_scale, k_pad, y, y_dtype, m, s, epi);
+    return launch_int4_gemm_ring(w, xh, row_scale, k_pad, y, y_dtype, m, s, epi, partial, partial_bytes);
   if (epi != EPI_STORE) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "fused epilogues above 16 rows exist for the LDS-ring GEMM only");
   GemmArgs a;
   a.tiles = w->tiles;

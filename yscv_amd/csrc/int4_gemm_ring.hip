@@ -49,6 +49,10 @@ struct RingArgs {
   int k_pad;
   int y_dtype;
   int epi;         // EPI_STORE, EPI_ADD_F32 (y f32, y += product) or EPI_SWIGLU (y [m][n / 2] = silu(gate) * up, columns 2i / 2i+1)
+  // K split (shapes with fewer tiles than CUs): the workgroups of split j multiply 128-k tiles j * kt_per .. and
+  // stores its f32 products to partial[j][m][n]; ring_finalize_kernel adds the splits in order and applies `epi`
+  float *partial;  // null: no split
+  int kt_per, splits;  // splits == 1 and kt_per == kt without a split
 };
 
 template <int N>
@@ -210,14 +214,20 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
   // XCD-aware tile numbering: the grid of tiles is cut into super-blocks of 32 tiles, 2^sbm_log2 (at most 8) along
   // m; workgroup ids that share an XCD (id mod 8) walk through one super-block at a time, so the 32 workgroups an
   // XCD runs together share row panels of A and column panels of B in its L2.
+  // With a K split the (super-block, split) pairs are numbered the same way: the splits of one super-block land on
+  // different XCDs (a shape with a single super-block would otherwise keep all its workgroups on one).
   const int sbm = 1 << sbm_log2, sbn = 32 >> sbm_log2;
   const int sb_m = (tiles_m + sbm - 1) >> sbm_log2;
+  const int sb_count = sb_m * ((tiles_n + sbn - 1) / sbn);
   const int j_in_xcd = (int)(blockIdx.x >> 3);
-  const int sb = (j_in_xcd >> 5) * 8 + (int)(blockIdx.x & 7);
+  const int pair = (j_in_xcd >> 5) * 8 + (int)(blockIdx.x & 7);
+  const int sb = pair % sb_count, ksplit = pair / sb_count;
   const int tm = (sb % sb_m) * sbm + (j_in_xcd & (sbm - 1)), tn = (sb / sb_m) * sbn + ((j_in_xcd & 31) >> sbm_log2);
-  if (tm >= tiles_m || tn >= tiles_n) return;
+  if (tm >= tiles_m || tn >= tiles_n || ksplit >= p.splits) return;
   const int m0 = tm * BM, n0 = p.col0 + tn * BN;
-  const int nstages = p.kt * (4 / KS);
+  const int kt_lo = ksplit * p.kt_per;
+  const int kt_n = min(p.kt - kt_lo, p.kt_per);
+  const int nstages = kt_n * (4 / KS), st_base = kt_lo * (4 / KS);  // this workgroup's stages are st_base + 0 .. nstages - 1
 
   float4_t acc[MT][NT];  // MMA waves only; the producers never touch it
   const int wm = (wave >> 1) & 1, wn = wave & 1;
@@ -261,8 +271,9 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
 
     Tile wr[SA / 2][WT];  // weight registers of the even stages in flight
     // stage st goes to activation slot / register set ri = st mod SA; par = st & 1 picks the words of the tile
-    auto issue_stage = [&](int st, auto ric, auto parc) {
+    auto issue_stage = [&](int st_local, auto ric, auto parc) {
       constexpr int ri = decltype(ric)::value, par = decltype(parc)::value;
+      const int st = st_base + st_local;
       if constexpr (par == 0) {
         const int kt = st >> 1;
         const int chunk = GM == GM128 ? kt / p.chunk_div : kt;
@@ -459,7 +470,15 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
       if (row >= p.m || col >= p.n) continue;
       const float4_t v = *reinterpret_cast<const float4_t *>(g4_ring + lrow * RS + ch * 16);
       const size_t o = (size_t)row * p.ldy + col;
-      if (p.epi == EPI_SWIGLU) {
+      if (p.partial) {
+        float *dst = p.partial + ((size_t)ksplit * p.m + row) * p.n + col;
+        if (vec) {
+          *reinterpret_cast<float4_t *>(dst) = v;
+        } else {
+          for (int e = 0; e < 4; e++)
+            if (col + e < p.n) dst[e] = v[e];
+        }
+      } else if (p.epi == EPI_SWIGLU) {
         // columns col .. col + 3 are gate, up, gate, up of two channels (n is even, col a multiple of 4)
         const size_t oh = (size_t)row * (p.ldy >> 1) + (col >> 1);
         store_out(p.y, oh, ring_silu(v[0]) * v[1], p.y_dtype);
@@ -492,6 +511,40 @@ __global__ void __launch_bounds__(256 + 64 * NP) int4_gemm_ring_kernel(RingArgs 
   }
 }
 
+// Adds the K splits of a launch in a fixed order and applies the epilogue: four columns per thread.
+__global__ void __launch_bounds__(256) ring_finalize_kernel(const float *__restrict__ partial, int splits, int m, int n, void *y,
+                                                            int y_dtype, int epi, int ldy) {
+  const int chunks = (n + 3) / 4;
+  const size_t total = (size_t)m * chunks;
+  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const int row = (int)(idx / chunks), col = (int)(idx % chunks) * 4;
+    const bool whole = col + 4 <= n && (n & 3) == 0;
+    float4_t v = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int j = 0; j < splits; j++) {
+      const float *src = partial + ((size_t)j * m + row) * n + col;
+      if (whole) {
+        v += *reinterpret_cast<const float4_t *>(src);
+      } else {
+        for (int e = 0; e < 4; e++)
+          if (col + e < n) v[e] += src[e];
+      }
+    }
+    const size_t o = (size_t)row * ldy + col;
+    if (epi == EPI_SWIGLU) {
+      const size_t oh = (size_t)row * (ldy >> 1) + (col >> 1);
+      store_out(y, oh, ring_silu(v[0]) * v[1], y_dtype);
+      if (col + 2 < n) store_out(y, oh + 1, ring_silu(v[2]) * v[3], y_dtype);
+    } else if (epi == EPI_ADD_F32) {
+      float *dst = reinterpret_cast<float *>(y) + o;
+      for (int e = 0; e < 4; e++)
+        if (col + e < n) dst[e] += v[e];
+    } else {
+      for (int e = 0; e < 4; e++)
+        if (col + e < n) store_out(y, o + e, v[e], y_dtype);
+    }
+  }
+}
+
 template <int MT, int NT, int KS, int SA, int NP, int GM, bool SF16>
 int32_t ring_launch_one(const RingArgs &a, hipStream_t s) {
   constexpr int LDS = 2 * MT * KS * 1024 * SA + 2 * 2 * NT * KS * 1024;
@@ -508,9 +561,16 @@ int32_t ring_launch_one(const RingArgs &a, hipStream_t s) {
   while (sbm_log2 > 0 && (1 << sbm_log2) > tiles_m) sbm_log2--;
   const int sbm = 1 << sbm_log2, sbn = 32 >> sbm_log2;
   const int super_blocks = ((tiles_m + sbm - 1) / sbm) * ((tiles_n + sbn - 1) / sbn);
-  const unsigned grid = (unsigned)((super_blocks + 7) / 8) * 8 * 32;
+  const unsigned splits = (unsigned)a.splits;
+  const unsigned grid = (unsigned)((super_blocks * splits + 7) / 8) * 8 * 32;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256 + 64 * NP), LDS, s, a, tiles_m, tiles_n, sbm_log2);
   YSCV_HIP_TRY(hipGetLastError());
+  if (a.partial) {
+    const size_t work = (size_t)a.m * ((a.n + 3) / 4);
+    const unsigned fb = (unsigned)std::min<size_t>((work + 255) / 256, 4096);
+    hipLaunchKernelGGL(ring_finalize_kernel, dim3(fb), dim3(256), 0, s, a.partial, (int)splits, a.m, a.n, a.y, a.y_dtype, a.epi, a.ldy);
+    YSCV_HIP_TRY(hipGetLastError());
+  }
   return YSCV_HIP_OK;
 }
 
@@ -534,8 +594,105 @@ bool int4_gemm_ring_eligible(const yscv_hip_int4_weight *w, const _Float16 *xh, 
   return (reinterpret_cast<uintptr_t>(y) & (align - 1)) == 0;
 }
 
+namespace {
+
+// Tile shapes: 0 = 128 x 128, 1 = 128 x 256, 2 = 256 x 128 (m > 128), 3 = 32 x 128 (m <= 32), 4 = 64 x 128 (m <= 64)
+struct RingPlan {
+  int one;           // shape of the launch, or of the first of two launches
+  int second;        // < 0: one launch; else the shape of the launch that takes the columns from split_col on
+  size_t split_col;
+  int splits, kt_per;  // K split of a single launch (splits == 1: none)
+};
+
+RingPlan ring_plan(size_t m, size_t n, size_t kt, size_t cus) {
+  RingPlan pl{0, -1, 0, 1, (int)kt};
+  size_t tiles;
+  if (m <= 32) {
+    // The tile height follows m: the MFMA work of a workgroup, and with it the time a weight tile stays in LDS, is
+    // proportional to the tile's rows whether they exist or not, so a short m streams the weights faster on a
+    // 32- or 64-row tile.
+    pl.one = 3;
+    tiles = ceil_div(n, (size_t)128);
+  } else if (m <= 64) {
+    pl.one = 4;
+    tiles = ceil_div(n, (size_t)128);
+  } else {
+    // Larger tiles: 128 x 256 (a third fewer fragment reads per MFMA) and 256 x 128 (the same, and every decoded
+    // weight feeds twice as many MFMAs).  A workgroup needs about 1.72 / 1.63 times as long for them as for a
+    // 128 x 128 tile; they pay when the tiles come in rounds over the CUs and the larger ones need sufficiently fewer
+    // rounds.  When the last round of the best shape would leave most CUs idle, the columns of its whole rounds go to
+    // one launch and the rest to a second one with the shape that suits the rest (config 3: three rounds of
+    // 256 x 128 tiles, then one round of 128 x 128 tiles, instead of three and a half rounds).
+    struct Shape {
+      size_t bm, bn, cost;
+      int code;
+    };
+    // cost: time of one tile in hundredths of a 128 x 128 tile's (measured on K 4096: 40 us; the 64-row tile 30 us).
+    // The 64-row tile decodes every weight twice as often per MFMA; it pays where it fills CUs that the taller tiles
+    // would leave idle (512 rows against N 4096: 256 tiles instead of 128).
+    const Shape shapes[4] = {{128, 128, 100, 0}, {128, 256, 172, 1}, {256, 128, 163, 2}, {64, 128, 75, 4}};
+    // best single shape for columns [c0, n): cost of its rounds over the CUs
+    auto best_single = [&](size_t c0, int *which, size_t *tiles_out) {
+      size_t best = (size_t)-1;
+      for (int i = 0; i < 4; i++) {
+        if (i == 2 && m <= 128) continue;
+        const size_t t = ceil_div(m, shapes[i].bm) * ceil_div(n - c0, shapes[i].bn);
+        const size_t cost = ceil_div(t, cus) * shapes[i].cost;
+        if (cost < best) {
+          best = cost;
+          *which = shapes[i].code;
+          *tiles_out = t;
+        }
+      }
+      return best;
+    };
+    size_t best = best_single(0, &pl.one, &tiles);
+    const size_t launch_cost = 10;  // a second launch: about a tenth of a tile time
+    for (int i = 0; i < 3; i++) {
+      if (i == 2 && m <= 128) continue;
+      const size_t tm = ceil_div(m, shapes[i].bm), tn = ceil_div(n, shapes[i].bn);
+      const size_t rounds = tm * tn / cus;    // whole rounds
+      const size_t cols = rounds * cus / tm;  // whole tile columns inside them
+      if (rounds == 0 || cols == 0 || cols >= tn) continue;
+      int rest = 0;
+      size_t rest_tiles = 0;
+      const size_t cost =
+          ceil_div(tm * cols, cus) * shapes[i].cost + best_single(cols * shapes[i].bn, &rest, &rest_tiles) + launch_cost;
+      if (cost < best) {
+        best = cost;
+        pl.one = shapes[i].code;
+        pl.second = rest;
+        pl.split_col = cols * shapes[i].bn;
+      }
+    }
+    if (pl.second >= 0) return pl;
+  }
+  // K split: a shape whose tiles cover at most half the CUs is cut along k into up to one workgroup per CU, each with
+  // at least four 128-k tiles (eight stages), as long as the f32 partial sums stay within 8 MB (they travel in the
+  // caller's workspace; yscv_hip_int4_matmul_static keeps them next to 16 MB of prepared activations)
+  if (tiles * 2 <= cus && kt >= 8) {
+    size_t ks = cus / tiles;
+    if (ks > kt / 4) ks = kt / 4;
+    if (ks > 16) ks = 16;
+    while (ks >= 2 && ks * m * n * sizeof(float) > ((size_t)8 << 20)) ks--;
+    if (ks >= 2) {
+      pl.kt_per = (int)ceil_div(kt, ks);
+      pl.splits = (int)ceil_div(kt, (size_t)pl.kt_per);
+    }
+  }
+  return pl;
+}
+
+}  // namespace
+
+size_t int4_gemm_ring_partial_bytes(const yscv_hip_int4_weight *w, size_t m, int num_cus) {
+  if (!w->tiled || m <= 16) return 0;
+  const RingPlan pl = ring_plan(m, w->n, w->kt, (size_t)(num_cus > 0 ? num_cus : 256));
+  return pl.splits > 1 ? (size_t)pl.splits * m * w->n * sizeof(float) : 0;
+}
+
 int32_t launch_int4_gemm_ring(const yscv_hip_int4_weight *w, const _Float16 *xh, const float *row_scale, size_t k_pad,
-                              void *y, int y_dtype, size_t m, hipStream_t s, int epi) {
+                              void *y, int y_dtype, size_t m, hipStream_t s, int epi, float *partial, size_t partial_bytes) {
   if (epi == EPI_ADD_F32 && y_dtype != YSCV_HIP_F32) return set_error(YSCV_HIP_ERR_INVALID_ARG, "the add epilogue updates an f32 tensor");
   if (epi == EPI_SWIGLU && (w->n & 1)) return set_error(YSCV_HIP_ERR_INVALID_ARG, "SwiGLU epilogue needs an even row count");
   RingArgs a;
@@ -557,70 +714,34 @@ int32_t launch_int4_gemm_ring(const yscv_hip_int4_weight *w, const _Float16 *xh,
   a.chunk_div = w->gm == GM128 ? (int)(w->g / 128) : 1;
   a.k_pad = (int)k_pad;
   a.y_dtype = y_dtype;
+  a.partial = nullptr;
+  a.kt_per = (int)w->kt;
+  a.splits = 1;
   const bool sf16 = w->scale_dtype == YSCV_HIP_F16;
-  // The tile height follows m: the MFMA work of a workgroup, and with it the time a weight tile stays in LDS, is
-  // proportional to the tile's rows whether they exist or not, so a short m streams the weights faster on a
-  // 32- or 64-row tile.
-  if (m <= 32) return ring_launch_gm<1, 4, 2, 6, 4>(a, w->gm, sf16, s);
-  if (m <= 64) return ring_launch_gm<2, 4, 2, 6, 8>(a, w->gm, sf16, s);
-  // Larger tiles: 128 x 256 (a third fewer fragment reads per MFMA) and 256 x 128 (the same, and every decoded
-  // weight feeds twice as many MFMAs).  A workgroup needs about 1.72 / 1.63 times as long for them as for a
-  // 128 x 128 tile; they pay when the tiles come in rounds over the CUs and the larger ones need sufficiently fewer
-  // rounds.  When the last round of the best shape would leave most CUs idle, the columns of its whole rounds go to
-  // one launch and the rest to a second one with the shape that suits the rest (config 3: three rounds of
-  // 256 x 128 tiles, then one round of 128 x 128 tiles, instead of three and a half rounds).
   const Context *ctx = nullptr;
   YSCV_TRY(ensure_context(&ctx));
-  const size_t cus = (size_t)(ctx->num_cus > 0 ? ctx->num_cus : 256);
-  struct Shape {
-    size_t bm, bn, cost;
-  };
-  const Shape shapes[3] = {{128, 128, 100}, {128, 256, 172}, {256, 128, 163}};
-  auto launch_shape = [&](int which, RingArgs r) {
-    if (which == 2) return ring_launch_gm<8, 4, 2, 4, 4>(r, w->gm, sf16, s);
-    if (which == 1) return ring_launch_gm<4, 8, 2, 4, 4>(r, w->gm, sf16, s);
-    return ring_launch_gm<4, 4, 2, 6, 8>(r, w->gm, sf16, s);
-  };
-  // best single shape for columns [c0, n): cost in hundredths of a 128 x 128 tile time
-  auto best_single = [&](size_t c0, int *which) {
-    size_t best = (size_t)-1;
-    for (int i = 0; i < 3; i++) {
-      if (i == 2 && m <= 128) continue;
-      const size_t tiles = ceil_div(m, shapes[i].bm) * ceil_div((size_t)w->n - c0, shapes[i].bn);
-      const size_t cost = ceil_div(tiles, cus) * shapes[i].cost;
-      if (cost < best) {
-        best = cost;
-        *which = i;
-      }
-    }
-    return best;
-  };
-  int one = 0;
-  size_t best = best_single(0, &one);
-  int first = -1, second = 0;
-  size_t split_col = 0;
-  const size_t launch_cost = 10;  // a second launch: about a tenth of a tile time
-  for (int i = 0; i < 3; i++) {
-    if (i == 2 && m <= 128) continue;
-    const size_t tm = ceil_div(m, shapes[i].bm), tn = ceil_div((size_t)w->n, shapes[i].bn);
-    const size_t rounds = tm * tn / cus;                // whole rounds
-    const size_t cols = rounds * cus / tm;              // whole tile columns inside them
-    if (rounds == 0 || cols == 0 || cols >= tn) continue;
-    int rest = 0;
-    const size_t cost = ceil_div(tm * cols, cus) * shapes[i].cost + best_single(cols * shapes[i].bn, &rest) + launch_cost;
-    if (cost < best) {
-      best = cost;
-      first = i;
-      second = rest;
-      split_col = cols * shapes[i].bn;
-    }
+  const RingPlan pl = ring_plan(m, w->n, w->kt, (size_t)(ctx->num_cus > 0 ? ctx->num_cus : 256));
+  if (pl.splits > 1 && partial != nullptr && partial_bytes >= (size_t)pl.splits * m * w->n * sizeof(float) &&
+      (reinterpret_cast<uintptr_t>(partial) & 15) == 0) {
+    a.partial = partial;
+    a.kt_per = pl.kt_per;
+    a.splits = pl.splits;
   }
-  if (first < 0) return launch_shape(one, a);
+  auto launch_shape = [&](int which, const RingArgs &r) {
+    switch (which) {
+      case 4: return ring_launch_gm<2, 4, 2, 6, 8>(r, w->gm, sf16, s);
+      case 3: return ring_launch_gm<1, 4, 2, 6, 4>(r, w->gm, sf16, s);
+      case 2: return ring_launch_gm<8, 4, 2, 4, 4>(r, w->gm, sf16, s);
+      case 1: return ring_launch_gm<4, 8, 2, 4, 4>(r, w->gm, sf16, s);
+      default: return ring_launch_gm<4, 4, 2, 6, 8>(r, w->gm, sf16, s);
+    }
+  };
+  if (pl.second < 0) return launch_shape(pl.one, a);
   RingArgs a1 = a, a2 = a;
-  a1.n = (int)split_col;
-  a2.col0 = (int)split_col;
-  YSCV_TRY(launch_shape(first, a1));
-  return launch_shape(second, a2);
+  a1.n = (int)pl.split_col;
+  a2.col0 = (int)pl.split_col;
+  YSCV_TRY(launch_shape(pl.one, a1));
+  return launch_shape(pl.second, a2);
 }
 
 }  // namespace yscv

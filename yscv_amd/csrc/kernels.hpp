@@ -101,15 +101,20 @@ int32_t launch_int4_generic(const yscv_hip_int4_weight *w, const void *x, int x_
                             int y_dtype, size_t m, hipStream_t s);
 int32_t launch_int4_gemm(const yscv_hip_int4_weight *w, const _Float16 *xh, const _Float16 *xl,
                          const float *row_scale, size_t k_pad, int split, void *y, int y_dtype,
-                         size_t m, hipStream_t s, int epi = EPI_STORE);
+                         size_t m, hipStream_t s, int epi = EPI_STORE, float *partial = nullptr, size_t partial_bytes = 0);
 
 // LDS-ring GEMM for fp16-prepared activations (split == 1)
 bool int4_gemm_ring_eligible(const yscv_hip_int4_weight *w, const _Float16 *xh, const void *y, int y_dtype, int split, size_t m,
                              size_t k_pad);
 // epi: EPI_STORE; EPI_ADD_F32 (y f32 [m][n], y += product); EPI_SWIGLU (weight rows 2i / 2i+1 = gate_i / up_i,
 // y [m][n / 2] = silu(gate) * up)
+// partial: optional scratch of int4_gemm_ring_partial_bytes() bytes (16-byte aligned).  With it, a shape whose tiles
+// cover at most half the CUs is also cut along k (f32 partial products, added in a fixed order by a second kernel);
+// without it the launch runs unsplit.
 int32_t launch_int4_gemm_ring(const yscv_hip_int4_weight *w, const _Float16 *xh, const float *row_scale, size_t k_pad,
-                              void *y, int y_dtype, size_t m, hipStream_t s, int epi = EPI_STORE);
+                              void *y, int y_dtype, size_t m, hipStream_t s, int epi = EPI_STORE, float *partial = nullptr,
+                              size_t partial_bytes = 0);
+size_t int4_gemm_ring_partial_bytes(const yscv_hip_int4_weight *w, size_t m, int num_cus);
 
 // Whole int4 call (activation preparation + kernel) with caller-provided scratch; ws may be null.
 int32_t int4_workspace_bytes(const yscv_hip_int4_weight *w, size_t m, int x_dtype, int force, size_t *bytes);
