@@ -631,3 +631,50 @@ def test_random_shapes_every_output(K, torch_cuda):
         assert torch.equal(w.matmul(x), y), tag
         w.close()
         del wd, ref
+
+
+@pytest.mark.parametrize("m,n,k,g,has_zp", [
+    (17, 4096, 4096, 32, False),    # one 32-row tile row, 32 tiles: split eight ways
+    (40, 1001, 2048, 64, True),     # ragged N (scalar stores of the partial sums), zero points
+    (64, 6144, 4096, 32, False),    # the q/k/v projection of a 64-token prompt
+    (100, 4096, 14336, 128, True),  # the down projection of a 100-token prompt: 64-row tiles, long K
+    (200, 512, 4096, 32, False),    # few columns
+    (256, 4096, 4096, 128, False),  # 64-row tiles preferred to 128-row ones, split in two
+    (512, 4096, 4096, 32, False),   # 64-row tiles fill the CUs without a split
+])
+def test_k_split_shapes_every_output(K, torch_cuda, m, n, k, g, has_zp):
+    """Shapes with fewer output tiles than half the CUs: the LDS-ring GEMM is cut along K as well, the splits' f32
+    partial sums go through the workspace and a second kernel adds them in a fixed order and applies the epilogue.
+    Every output of the plain call against an fp32 product on the GPU, twice with the same bits, the same bits with a
+    caller's workspace (nothing written past the announced size), and both fused epilogues against the plain result."""
+    torch = torch_cuda
+    rng = np.random.default_rng(7000 + m + n)
+    b = rng.integers(0, 256, n * k // 2, dtype=np.uint8)
+    scales = rng.uniform(0.005, 0.02, n * (k // g)).astype(np.float16)
+    zq = rng.integers(5, 12, (n, k // g)) if has_zp else None
+    w = K.PackedInt4Weight(b, scales, g, n, k, zero_points=pack_zero_points(zq) if has_zp else None,
+                           nibble_format=K.NIBBLE_UNSIGNED)
+    wd = _dequant_on_gpu(torch, b, scales, n, k, g, zq)
+    x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).half().cuda()
+    ref = x.float() @ wd.T
+    y = w.matmul(x, out_dtype=torch.float32)
+    err, top = float((y - ref).abs().nan_to_num(1e9).max()), float(ref.abs().max())
+    assert err <= top * 1e-3 + 1e-6, (err, top)
+    assert torch.equal(w.matmul(x, out_dtype=torch.float32), y)
+    need = w.workspace_bytes(m, torch.float16)
+    ws = torch.full((need + 256,), 0xA5, dtype=torch.uint8, device="cuda")
+    assert torch.equal(w.matmul(x, out_dtype=torch.float32, workspace=ws[: max(need, 1)]), y)
+    assert bool((ws[need:] == 0xA5).all())
+    resid = torch.from_numpy((rng.standard_normal((m, n)) * 10).astype(np.float32)).cuda()
+    acc = torch.empty(m + 1, n, device="cuda")
+    acc[:m] = resid
+    acc[m] = 3.0
+    w.matmul_fused(x, acc[:m], K.EPILOGUE_ADD_F32)
+    assert torch.equal(acc[:m], resid + y) and bool((acc[m] == 3.0).all())
+    if n % 2 == 0:
+        want = torch.nn.functional.silu(y[:, 0::2].double()) * y[:, 1::2].double()
+        act = torch.full((m + 1, n // 2), 7.0, device="cuda", dtype=torch.float32)
+        w.matmul_fused(x, act[:m], K.EPILOGUE_SWIGLU)
+        assert float((act[:m].double() - want).abs().max() / want.abs().max()) < 1e-5
+        assert bool((act[m] == 7.0).all())
+    w.close()
