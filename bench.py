@@ -651,6 +651,10 @@ def main():
             extra["decode_batch_sweep"] = sweep
     if not args.no_extra:
         extra["prefill_2048_tokens"] = bench_prefill(dec, torch, cfg, 2048, params)
+        # shorter prompts (llm-bench's own prompt has 43 tokens): below ~512 rows the projections have fewer output
+        # tiles than CUs and the GEMM is cut along K as well
+        extra["prefill_short_prompts"] = {"%d_tokens" % n_tok: {kk: vv for kk, vv in bench_prefill(dec, torch, cfg, n_tok, params).items()
+                                                                if kk in ("ms", "prompt_tok/s")} for n_tok in (43, 128, 512)}
     del dec
     torch.cuda.empty_cache()
     if not args.no_extra:

@@ -667,16 +667,29 @@ RingPlan ring_plan(size_t m, size_t n, size_t kt, size_t cus) {
     }
     if (pl.second >= 0) return pl;
   }
-  // K split: a shape whose tiles cover at most half the CUs is cut along k into up to one workgroup per CU, each with
-  // at least four 128-k tiles (eight stages), as long as the f32 partial sums stay within 8 MB (they travel in the
-  // caller's workspace; yscv_hip_int4_matmul_static keeps them next to 16 MB of prepared activations)
+  // K split: a shape whose tiles cover at most half the CUs is cut along k, each part with at least four 128-k tiles
+  // (eight stages), as long as the f32 partial sums stay within 8 MB (they travel in the caller's workspace;
+  // yscv_hip_int4_matmul_static keeps them next to 16 MB of prepared activations).  The workgroups of one
+  // (super-block, split) pair share an XCD, eight pairs run side by side: the number of splits is the one with the
+  // shortest estimated time, rounds of eight pairs x (a part's k-tiles at 0.9 us each + 5 us to start and end a
+  // workgroup), + 5 us for the kernel that adds the parts.
   if (tiles * 2 <= cus && kt >= 8) {
-    size_t ks = cus / tiles;
-    if (ks > kt / 4) ks = kt / 4;
-    if (ks > 16) ks = 16;
-    while (ks >= 2 && ks * m * n * sizeof(float) > ((size_t)8 << 20)) ks--;
-    if (ks >= 2) {
-      pl.kt_per = (int)ceil_div(kt, ks);
+    const size_t bm = pl.one == 3 ? 32 : (pl.one == 4 ? 64 : (pl.one == 2 ? 256 : 128)), bn = pl.one == 1 ? 256 : 128;
+    const size_t tiles_m = ceil_div(m, bm), tiles_n = ceil_div(n, bn);
+    size_t sbm = 8;
+    while (sbm > 1 && sbm > tiles_m) sbm >>= 1;
+    const size_t sb = ceil_div(tiles_m, sbm) * ceil_div(tiles_n, 32 / sbm);
+    size_t best_ks = 1, best_t = ceil_div(sb, (size_t)8) * (kt * 18 + 100);  // units of 0.05 us
+    for (size_t ks = 2; ks <= 16 && ks <= kt / 4; ks++) {
+      if (ks * m * n * sizeof(float) > ((size_t)8 << 20)) break;
+      const size_t t = ceil_div(sb * ks, (size_t)8) * (ceil_div(kt, ks) * 18 + 100) + 100;
+      if (t < best_t) {
+        best_t = t;
+        best_ks = ks;
+      }
+    }
+    if (best_ks >= 2) {
+      pl.kt_per = (int)ceil_div(kt, best_ks);
       pl.splits = (int)ceil_div(kt, (size_t)pl.kt_per);
     }
   }
