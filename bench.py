@@ -417,7 +417,7 @@ def extra_kernels(torch, stream_ptr):
         sweep["m%d" % m] = {"us": round(t * 1e6, 1), "weight_GB/s": round(wbytes / t / 1e9, 0),
                             "frac_of_hbm_peak": round(wbytes / t / 1e9 / HBM_PEAK_GBS, 3),
                             "TFLOP/s": round(fl / t / 1e12, 1), "frac_of_mfma_peak": round(fl / t / 1e12 / MFMA_BF16_PEAK, 4),
-                            "kernel": "int4_skinny_kernel" if m <= 16 else "int4_gemm_ring_kernel"}
+                            "kernel": "int4_skinny_kernel" if m <= 16 else ("int4_mid_kernel" if m <= 32 else "int4_gemm_ring_kernel")}
     out["config5_lm_head_sweep_k4096_n128256"] = sweep
 
     # where the skinny kernel hands over to the MFMA GEMM: both kernels on either side of m = 16 (event-timed eager
@@ -449,8 +449,9 @@ def extra_kernels(torch, stream_ptr):
         "m17_gemm_us": round(teager(lambda: w.matmul(x17, out=y17, mode="gemm")) * 1e6, 1),
         "m32_two_skinny_passes_us": round(teager(two_passes) * 1e6, 1),
         "m32_gemm_us": round(teager(lambda: w.matmul(x32, out=y32, mode="gemm")) * 1e6, 1),
-        "note": "yscv_hip_int4_matmul switches at m = 16: one skinny pass up to 16 rows, above that the LDS-ring MFMA GEMM, "
-                "whose smallest tile has 32 rows (m = 17 costs what m = 32 costs)"}
+        "note": "yscv_hip_int4_matmul switches at m = 16: one skinny pass up to 16 rows, 17 .. 32 rows on the kernel that keeps "
+                "all rows' activations in registers (int4_mid.hip; the forced GEMM mode takes it too), above that the "
+                "LDS-ring MFMA GEMM"}
     w.close()
     return out
 

@@ -114,7 +114,17 @@ static Int4Scratch int4_scratch_layout(const yscv_hip_int4_weight *w, const void
   L.rs_bytes = L.direct ? 0 : round_up(m * sizeof(float), 256);
   L.part_bytes = L.skinny ? round_up(L.plan.partial_bytes, 256) : 0;
   L.total = L.xh_bytes * L.split + L.rs_bytes + L.part_bytes;
-  L.opt_bytes = L.skinny ? 0 : round_up(int4_gemm_ring_partial_bytes(w, m, num_cus), 256);
+  // partial sums of whichever kernel takes the rows above 16: the register-resident one up to 32 rows where its
+  // parts fit the cap, else the LDS-ring GEMM's K split
+  if (L.skinny) {
+    L.opt_bytes = 0;
+  } else if (m <= 32 && int4_mid_partial_bytes(w, m) <= kMidPartialCap) {
+    const size_t ring = int4_gemm_ring_partial_bytes(w, m, num_cus);  // the ring takes over if the mid kernel cannot (alignment)
+    const size_t mid = int4_mid_partial_bytes(w, m);
+    L.opt_bytes = round_up(mid > ring ? mid : ring, 256);
+  } else {
+    L.opt_bytes = round_up(int4_gemm_ring_partial_bytes(w, m, num_cus), 256);
+  }
   if (!L.skinny && force == 0 && x_dtype == YSCV_HIP_F32 && m <= kChunkedSkinnyMaxRows) {
     // this call may run as 16-row skinny calls (see int4_run_ws): the scratch must cover one of those too
     const Int4Scratch c = int4_scratch_layout(w, x, x_dtype, 16, 1, num_cus);

@@ -256,6 +256,12 @@ int32_t launch_int4_gemm(const yscv_hip_int4_weight *w, const _Float16 *xh, cons
   if (!w->tiled) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "int4 GEMM kernel needs the tiled layout");
   // 16-bit activations: the LDS-ring kernel from the first row count the skinny kernel does not take (rows are
   // padded to its 128-row tile; with few rows the weights are still streamed exactly once)
+  // 17 .. 32 rows: the register-resident kernel of int4_mid.hip where its partial sums (if any) have their scratch
+  if (m > 16 && m <= 32 && int4_mid_eligible(w, xh, y, y_dtype, split, m, k_pad, kMidPartialCap)) {
+    const size_t need = int4_mid_partial_bytes(w, m);
+    if (need == 0 || (partial != nullptr && partial_bytes >= need))
+      return launch_int4_mid(w, xh, row_scale, k_pad, y, y_dtype, m, s, epi, partial, partial_bytes);
+  }
   if (m > 16 && int4_gemm_ring_eligible(w, xh, y, y_dtype, split, m, k_pad))
     return launch_int4_gemm_ring(w, xh, row_scale, k_pad, y, y_dtype, m, s, epi, partial, partial_bytes);
   if (epi != EPI_STORE) return set_error(YSCV_HIP_ERR_UNSUPPORTED, "fused epilogues above 16 rows exist for the LDS-ring GEMM only");

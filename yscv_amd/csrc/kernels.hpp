@@ -116,6 +116,16 @@ int32_t launch_int4_gemm_ring(const yscv_hip_int4_weight *w, const _Float16 *xh,
                               size_t partial_bytes = 0);
 size_t int4_gemm_ring_partial_bytes(const yscv_hip_int4_weight *w, size_t m, int num_cus);
 
+// 17 .. 32 rows (int4_mid.hip): K split over the waves with all rows' activations in registers, the weights streamed
+// once.  With K > 4096 K is also cut into parts over workgroups whose f32 partial sums need
+// int4_mid_partial_bytes() of scratch; the kernel is used where that stays within kMidPartialCap.
+constexpr size_t kMidPartialCap = (size_t)16 << 20;
+size_t int4_mid_partial_bytes(const yscv_hip_int4_weight *w, size_t m);
+bool int4_mid_eligible(const yscv_hip_int4_weight *w, const _Float16 *xh, const void *y, int y_dtype, int split, size_t m,
+                       size_t k_pad, size_t max_partial_bytes);
+int32_t launch_int4_mid(const yscv_hip_int4_weight *w, const _Float16 *xh, const float *row_scale, size_t k_pad, void *y,
+                        int y_dtype, size_t m, hipStream_t s, int epi, float *partial, size_t partial_bytes);
+
 // Whole int4 call (activation preparation + kernel) with caller-provided scratch; ws may be null.
 int32_t int4_workspace_bytes(const yscv_hip_int4_weight *w, size_t m, int x_dtype, int force, size_t *bytes);
 int32_t int4_run_ws(const yscv_hip_int4_weight *w, const void *x, int x_dtype, void *y, int y_dtype, size_t m,
