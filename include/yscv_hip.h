@@ -138,8 +138,9 @@ int32_t yscv_hip_int4_weight_dims(const yscv_hip_int4_weight *w, size_t *n, size
  * exec_matmul does (crates/yscv-onnx/src/runner/linear.rs:228-278: per-row GEMV
  * below a threshold, GEMM above); `_gemv` forces the skinny kernel (m <= 16,
  * replaces packed_int4_gemv_dispatch, int4_matmul.rs:310-377, called once per row)
- * and `_gemm` the tiled MFMA kernel (replaces packed_int4_gemm_dispatch,
- * int4_matmul.rs:548-605). */
+ * and `_gemm` the kernels for more rows (replaces packed_int4_gemm_dispatch,
+ * int4_matmul.rs:548-605): with 16-bit activations a weight-streaming kernel that keeps all
+ * rows' activations in registers up to 32 rows, the LDS-ring MFMA GEMM above. */
 int32_t yscv_hip_int4_matmul(const yscv_hip_int4_weight *w, const void *x_dev, int32_t x_dtype,
                              void *y_dev, int32_t y_dtype, size_t m, void *stream);
 int32_t yscv_hip_int4_gemv(const yscv_hip_int4_weight *w, const void *x_dev, int32_t x_dtype,
@@ -149,8 +150,9 @@ int32_t yscv_hip_int4_gemm(const yscv_hip_int4_weight *w, const void *x_dev, int
 
 /* The int4 matmul with a fused epilogue -- the "bias / residual / activation fusion" the reference plans for its
  * int4 MatMul (docs/int4-quant-pipeline-plan.md:45-51); the decode loop and the prompt pass use exactly these.  Up to
- * 16 rows on the skinny kernel (any activation type); above 16 rows on the LDS-ring MFMA GEMM, fp16 / bf16
- * activations only (f32 activations with ADD_F32 or SWIGLU above 16 rows: INVALID_ARG).
+ * 16 rows on the skinny kernel (any activation type); above 16 rows on the kernels for more rows (17 .. 32: the
+ * register-resident streaming kernel, more: the LDS-ring MFMA GEMM), fp16 / bf16 activations only (f32 activations
+ * with ADD_F32 or SWIGLU above 16 rows: INVALID_ARG).
  *   STORE    y[m][n] = x W^T                       (same as yscv_hip_int4_gemv)
  *   ADD_F32  y[m][n] += x W^T, y_dtype must be F32   (projection + residual add)
  *   SWIGLU   rows 2i / 2i+1 of W are gate_i / up_i; y[m][n/2] = silu(gate) * up   (n even)
