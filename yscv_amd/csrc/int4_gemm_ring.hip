@@ -668,8 +668,9 @@ RingPlan ring_plan(size_t m, size_t n, size_t kt, size_t cus) {
     if (pl.second >= 0) return pl;
   }
   // K split: a shape whose tiles cover at most half the CUs is cut along k, each part with at least four 128-k tiles
-  // (eight stages), as long as the f32 partial sums stay within 8 MB (they travel in the caller's workspace;
-  // yscv_hip_int4_matmul_static keeps them next to 16 MB of prepared activations).  The workgroups of one
+  // (eight stages), as long as the f32 partial sums stay within 16 MB and, together with a prepared fp16 copy of the
+  // activations, within 31 MB (they travel in the caller's workspace; yscv_hip_int4_matmul_static has 32 MB for
+  // both).  The workgroups of one
   // (super-block, split) pair share an XCD, eight pairs run side by side: the number of splits is the one with the
   // shortest estimated time, rounds of eight pairs x (a part's k-tiles at 0.9 us each + 5 us to start and end a
   // workgroup), + 5 us for the kernel that adds the parts.
@@ -680,8 +681,11 @@ RingPlan ring_plan(size_t m, size_t n, size_t kt, size_t cus) {
     while (sbm > 1 && sbm > tiles_m) sbm >>= 1;
     const size_t sb = ceil_div(tiles_m, sbm) * ceil_div(tiles_n, 32 / sbm);
     size_t best_ks = 1, best_t = ceil_div(sb, (size_t)8) * (kt * 18 + 100);  // units of 0.05 us
+    const size_t x_bytes = m * kt * 128 * sizeof(_Float16);
+    const size_t room = x_bytes >= ((size_t)31 << 20) ? 0 : ((size_t)31 << 20) - x_bytes;
+    const size_t cap = room < ((size_t)16 << 20) ? room : ((size_t)16 << 20);
     for (size_t ks = 2; ks <= 16 && ks <= kt / 4; ks++) {
-      if (ks * m * n * sizeof(float) > ((size_t)8 << 20)) break;
+      if (ks * m * n * sizeof(float) > cap) break;
       const size_t t = ceil_div(sb * ks, (size_t)8) * (ceil_div(kt, ks) * 18 + 100) + 100;
       if (t < best_t) {
         best_t = t;
