@@ -297,9 +297,13 @@ def measured_peaks(torch):
     torch.cuda.synchronize()
     r, f, i = C.c_double(), C.c_double(), C.c_double()
     capi.lib().measure_peaks(C.byref(r), C.byref(f), C.byref(i))
+    l2, far = C.c_double(), C.c_double()
+    capi.lib().measure_fill(C.byref(l2), C.byref(far))  # operand path of the GEMMs: LDS-direct loads, per CU
     return {"hbm_read_GB/s": round(r.value, 1), "frac_of_8TB/s": round(r.value / HBM_PEAK_GBS, 3),
             "mfma_f16_TFLOP/s": round(f.value, 1), "frac_of_2.5PFLOP/s": round(f.value / 2500.0, 3),
-            "mfma_i8_TOP/s": round(i.value, 1), "frac_of_5POP/s": round(i.value / 5000.0, 3)}
+            "mfma_i8_TOP/s": round(i.value, 1), "frac_of_5POP/s": round(i.value / 5000.0, 3),
+            "lds_direct_fill_from_L2_GB/s_per_CU": round(l2.value, 1),
+            "lds_direct_fill_from_16MiB_region_GB/s_per_CU": round(far.value, 1)}
 
 
 def extra_kernels(torch, stream_ptr):

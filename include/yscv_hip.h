@@ -79,6 +79,12 @@ int32_t yscv_hip_device_info(char *buf, size_t buf_len);
  * its microbenchmark relates the dispatch kernels to its own scalar loops ("SIMD speedup vs scalar",
  * apps/llm-bench/src/bin/kernel_bench.rs:187), not to a machine peak. */
 int32_t yscv_hip_measure_peaks(double *hbm_read_gbs, double *mfma_f16_tflops, double *mfma_i8_tops);
+/* Calibration of the operand path of the GEMM kernels: GB/s ONE CU takes in through LDS-direct loads
+ * (global_load_lds_dwordx4, 1 KiB per wave and instruction, eight in flight per wave, all CUs at once) from a 1 MiB
+ * region that every workgroup reads -- it stays in every XCD's L2, so this is the L2 -> CU path alone -- and from a
+ * 16 MiB region, more than one XCD's L2 holds.  A tile of (bm + bn) rows needs (bm + bn) * K operand bytes per
+ * workgroup whatever the matrix instruction; this figure prices that.  No counterpart in the reference. */
+int32_t yscv_hip_measure_fill(double *l2_gbs_per_cu, double *beyond_l2_gbs_per_cu);
 /* Calibration: one launch of a kernel that does nothing (one 512-thread workgroup per CU) on `stream`.  A benchmark
  * that times many of them, back to back or as the nodes of a graph, gets the floor under the duration of any kernel
  * (what a single short GEMV cannot go below).  No counterpart in the reference. */

@@ -117,6 +117,10 @@ def test_measured_peaks_are_plausible(K):
     assert 3000.0 < r.value <= 8000.0, r.value
     assert 1000.0 < f.value <= 2500.0, f.value
     assert 2000.0 < i.value <= 5000.0, i.value
+    # yscv_hip_measure_fill: what one CU takes in through LDS-direct loads, from L2 and from behind it
+    l2, far = C.c_double(), C.c_double()
+    capi.lib().measure_fill(C.byref(l2), C.byref(far))
+    assert 20.0 < far.value <= l2.value * 1.05 and l2.value < 270.0, (l2.value, far.value)  # 64 B per clock = 154 GB/s at 2.4 GHz
 
 
 def test_quantize_f32_to_int4_bit_exact(oracle, K):

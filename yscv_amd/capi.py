@@ -68,6 +68,7 @@ _SIGNATURES = {
     "yscv_hip_shutdown": [],
     "yscv_hip_device_info": [C.c_char_p, _sz],
     "yscv_hip_measure_peaks": [C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_double)],
+    "yscv_hip_measure_fill": [C.POINTER(C.c_double), C.POINTER(C.c_double)],
     "yscv_hip_launch_empty": [_vp],
     "yscv_hip_malloc": [C.POINTER(_vp), _sz],
     "yscv_hip_free": [_vp],

@@ -2,6 +2,8 @@
 // in registers.  The rooflines in the benchmark are priced against the published peaks (8 TB/s, 2.5 PFLOP/s fp16,
 // 5 POP/s int8); these figures say how much of a published peak any kernel can reach on the machine at hand (the
 // clock under a full MFMA load is below the nominal one).  No counterpart in the reference.
+#include <mutex>
+
 #include "common.hpp"
 #include "int4_common.hpp"
 
@@ -53,6 +55,28 @@ __global__ void __launch_bounds__(512) peak_mfma_kernel(int iters, uint32_t *out
     for (int i = 0; i < NACC; i++) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
   }
   if (s == 123.456f) out[0] = 1;
+}
+
+// Operand fill probe: every workgroup (8 waves) streams `bytes_per_wg` out of a region of `region` bytes into LDS
+// with LDS-direct loads, 1 KiB per wave and instruction, eight instructions in flight per wave -- the path and the
+// granularity of the GEMM kernels' operand rings.  Workgroup w starts `stride` bytes after workgroup w - 1.
+__global__ void __launch_bounds__(512) peak_fill_kernel(const char *__restrict__ base, size_t region, size_t bytes_per_wg,
+                                                        size_t stride) {
+  extern __shared__ __attribute__((aligned(1024))) char fill_lds[];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const size_t start = ((size_t)blockIdx.x * stride) % region;
+  const size_t iters = bytes_per_wg / 8192;  // an iteration: 8 waves x 1 KiB
+  const uint32_t lds0 = (uint32_t)(size_t)fill_lds;
+  for (size_t it = 0; it < iters; it += 8) {
+#pragma unroll
+    for (int d = 0; d < 8; d++) {
+      const char *p = base + (start + (it + d) * 8192 + (size_t)wave * 1024 + lane * 16) % region;
+      const uint32_t dst = lds0 + (uint32_t)((d * 8 + wave) * 1024);
+      // m0: reserved, never allocated by the compiler; nothing else in this kernel reads it
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(p) : "memory");
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
 }
 
 struct Events {
@@ -129,6 +153,43 @@ extern "C" int32_t yscv_hip_measure_peaks(double *hbm_read_gbs, double *mfma_f16
     // 16x16x32 f16: 16384 flop; 16x16x64 i8: 32768 op
     if (kind == 0) *mfma_f16_tflops = mfmas * 16384.0 / (best * 1e-3) / 1e12;
     else *mfma_i8_tops = mfmas * 32768.0 / (best * 1e-3) / 1e12;
+  }
+  return YSCV_HIP_OK;
+}
+
+// What one CU takes in through LDS-direct loads: from a 1 MiB region every workgroup reads (it stays in every XCD's
+// L2: the L2 -> CU path alone) and from a 16 MiB region (more than an XCD's L2 holds: what lies behind it).
+extern "C" int32_t yscv_hip_measure_fill(double *l2_gbs_per_cu, double *beyond_l2_gbs_per_cu) {
+  const Context *ctx = nullptr;
+  YSCV_TRY(ensure_context(&ctx));
+  YSCV_REQUIRE(l2_gbs_per_cu && beyond_l2_gbs_per_cu, "null argument");
+  Events ev;
+  YSCV_HIP_TRY(hipEventCreate(&ev.a));
+  YSCV_HIP_TRY(hipEventCreate(&ev.b));
+  DevBuf buf;
+  const size_t bytes = (size_t)16 << 20, per_wg = (size_t)8 << 20;
+  YSCV_TRY(buf.alloc(bytes));
+  YSCV_HIP_TRY(hipMemset(buf.p, 1, bytes));
+  const int wgs = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(once, [] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(peak_fill_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+  });
+  YSCV_HIP_TRY(attr_err);
+  for (int kind = 0; kind < 2; kind++) {
+    const size_t region = kind == 0 ? (size_t)1 << 20 : bytes, stride = kind == 0 ? 8192 : 65536;
+    float ms = 0.0f, best = 1e30f;
+    for (int rep = 0; rep < 4; rep++) {
+      YSCV_HIP_TRY(hipEventRecord(ev.a, nullptr));
+      hipLaunchKernelGGL(peak_fill_kernel, dim3(wgs), dim3(512), 65536, nullptr, buf.as<char>(), region, per_wg, stride);
+      YSCV_HIP_TRY(hipGetLastError());
+      YSCV_HIP_TRY(hipEventRecord(ev.b, nullptr));
+      YSCV_HIP_TRY(hipEventSynchronize(ev.b));
+      YSCV_HIP_TRY(hipEventElapsedTime(&ms, ev.a, ev.b));
+      if (rep > 0 && ms < best) best = ms;
+    }
+    (kind == 0 ? *l2_gbs_per_cu : *beyond_l2_gbs_per_cu) = (double)per_wg / (best * 1e-3) / 1e9;
   }
   return YSCV_HIP_OK;
 }
