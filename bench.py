@@ -386,7 +386,12 @@ def extra_kernels(torch, stream_ptr):
     ops = 2.0 * m * k * n
     out["config2_int8_m512_k4096_n4096"] = {"us_i32": round(t * 1e6, 2), "TOP/s_i32": round(ops / t / 1e12, 1),
                                             "us_fused_requant": round(t2 * 1e6, 2), "TOP/s_fused_requant": round(ops / t2 / 1e12, 1),
-                                            "frac_of_i8_mfma_peak": round(ops / t / 1e12 / MFMA_I8_PEAK, 4)}
+                                            "frac_of_i8_mfma_peak": round(ops / t / 1e12 / MFMA_I8_PEAK, 4),
+                                            # one 64 x 128 tile per CU: (64 + 128) * K operand bytes through LDS-direct loads
+                                            "operand_KB_per_CU": round((64 + 128) * k / 1024.0, 0),
+                                            "operand_fill_GB/s_per_CU_whole_kernel": round((64 + 128) * k / t / 1e9, 1),
+                                            "note": "compare with extra.measured_peaks.lds_direct_fill_from_L2_GB/s_per_CU: the tiling "
+                                                    "that fills 256 CUs with 512 x 4096 outputs is bound by the L2 -> LDS path"}
     del pb
     # config 3: int4 prefill M2048 K4096 N14336 g128, zero points 6..10, bf16
     m, k, n, g = 2048, 4096, 14336, 128
