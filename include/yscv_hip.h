@@ -549,6 +549,12 @@ int32_t yscv_hip_decoder_run(yscv_hip_decoder *d, int32_t n_steps, int32_t use_g
  * position, q * scale of its row, earlier positions included.  tokens_host is read before the call returns. */
 int32_t yscv_hip_decoder_prefill(yscv_hip_decoder *d, const int32_t *tokens_host, int32_t n_tokens, int32_t start_pos,
                                  void *stream);
+/* Rows of the prompt that yscv_hip_decoder_prefill takes through the layers in one pass (default 4096).  A longer
+ * prompt runs as several passes, each appending to the cache the earlier ones wrote; the per-call scratch (activations of
+ * one pass: rows x (3 d_model + q/k/v width + n_heads head_dim + d_ff) x 2 bytes and up) scales with this number, the
+ * results do not depend on it beyond the float tolerance.  No counterpart in the reference (its prompt phase feeds
+ * the whole prompt at once, apps/llm-bench/src/main.rs:403-470). */
+int32_t yscv_hip_decoder_set_prefill_rows(yscv_hip_decoder *d, int32_t rows);
 /* Optional bias of the fused q / k / v projection of one layer (Qwen-style attention; the reference adds it with
  * the Add node behind the MatMul): fp16 [(n_heads + 2 n_kv_heads) * head_dim] in q, k, v order, or NULL to remove it.
  * A decoder with a bias takes the multi-kernel path (the single-launch kernel has none). */

@@ -690,3 +690,32 @@ def test_prefill_of_long_prompts_across_head_shapes(hd, nh, nkv, n_prompt, start
     exp2 = ref.step(nxt, start + n_prompt)
     assert np.abs(dec.logits() - exp2).max() / np.abs(exp2).max() < LOGIT_TOL
     dec.close()
+
+
+@pytest.mark.parametrize("kv_dtype,chunk", [("f16", 64), ("f16", 17), ("i8", 64), ("i8", 40)])
+def test_prefill_in_several_passes(kv_dtype, chunk):
+    """A prompt longer than yscv_hip_decoder_set_prefill_rows runs as several passes; every pass after the first starts
+    at a position other than 0 and attends over the cache rows the earlier passes wrote (with the int8 cache: over what
+    the cache returns for them).  150 tokens in passes of 64 / 17 / 40 rows -- the row counts of the passes straddle the
+    kernel switches at 16 and 32 rows -- against the checker fed token by token, and against the one-pass result."""
+    rng = np.random.default_rng(5200)
+    cfg = dict(CFG, max_batch=1, max_ctx=256)
+    dec, ref = _build(rng, cfg, kv_dtype=kv_dtype, symmetric=True)
+    prompt = rng.integers(0, cfg["vocab"], 150).astype(np.int32)
+    for i, t in enumerate(prompt):
+        exp = ref.step(np.array([t]), i)
+    dec.prefill(prompt)
+    one_pass = dec.logits().copy()
+    dec.set_prefill_rows(chunk)
+    dec.prefill(prompt)
+    got = dec.logits()
+    assert np.abs(got - exp).max() / np.abs(exp).max() < LOGIT_TOL
+    assert np.abs(got - one_pass).max() / np.abs(one_pass).max() < LOGIT_TOL
+    for l in range(cfg["n_layers"]):
+        gk, gv = dec.get_kv(l, 1, 0, 150)
+        ek, ev = ref.kc[l][0], ref.vc[l][0]
+        assert np.abs(gk.astype(np.float32) - ek).max() <= 1e-2 * np.abs(ek).max(), l
+        assert np.abs(gv.astype(np.float32) - ev).max() <= 1e-2 * np.abs(ev).max(), l
+    with pytest.raises(Exception, match="rows per prompt pass"):
+        dec.set_prefill_rows(0)
+    dec.close()

@@ -141,6 +141,7 @@ _SIGNATURES = {
     "yscv_hip_decoder_reset": [_vp, _i32, _i32, _vp],
     "yscv_hip_decoder_run": [_vp, _i32, _i32, _vp],
     "yscv_hip_decoder_last_path": [_vp, _vp],
+    "yscv_hip_decoder_set_prefill_rows": [_vp, _i32],
     "yscv_hip_decoder_prefill": [_vp, _vp, _i32, _i32, _vp],
     "yscv_hip_decoder_set_qkv_bias": [_vp, _i32, _vp],
     "yscv_hip_rms_norm_dev": [_vp, _vp, _sz, _sz, C.c_float, _vp, _vp],

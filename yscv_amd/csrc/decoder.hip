@@ -137,6 +137,7 @@ struct yscv_hip_decoder {
   // persistent single-launch path (batch 1)
   bool persist_ok = false;     // the shape is supported and the buffers exist
   int last_path = -1;          // path of the last yscv_hip_decoder_run: 0 launches, 1 graph replays, 2 single launch
+  int prefill_rows = 4096;     // prompt rows per pass of yscv_hip_decoder_prefill: bounds its activation scratch
   PersistModel pm{};
   uint8_t *p_stream = nullptr;
   uint64_t *p_wg_off = nullptr;
@@ -1214,9 +1215,9 @@ int32_t yscv_hip_decoder_prefill(yscv_hip_decoder *d, const int32_t *tokens_host
   YSCV_TRY(toks.alloc((size_t)n_tokens * 4, s));
   DEC_HIP(hipMemcpyAsync(toks.p, tokens_host, (size_t)n_tokens * 4, hipMemcpyHostToDevice, s));
   DEC_HIP(hipStreamSynchronize(s));  // tokens_host is the caller's again
-  constexpr int kChunk = 4096;       // rows per pass: bounds the activation buffers
-  for (int32_t r0 = 0; r0 < n_tokens; r0 += kChunk) {
-    const int rows = n_tokens - r0 < kChunk ? n_tokens - r0 : kChunk;
+  const int chunk = d->prefill_rows;  // rows per pass: bounds the activation buffers
+  for (int32_t r0 = 0; r0 < n_tokens; r0 += chunk) {
+    const int rows = n_tokens - r0 < chunk ? n_tokens - r0 : chunk;
     YSCV_TRY(prefill_chunk(d, toks.as<int32_t>() + r0, rows, start_pos + r0, r0 + rows == n_tokens, s));
   }
   // as after reset(last token, start_pos + n - 1) + one decode step: the pick is the next input, position and step advance
@@ -1225,6 +1226,13 @@ int32_t yscv_hip_decoder_prefill(yscv_hip_decoder *d, const int32_t *tokens_host
   YSCV_TRY(launch_argmax(d->logits, 1, c.vocab, d->tokens, d->history, d->step, c.max_steps, s));
   YSCV_TRY(launch_advance(d->pos, d->step, s));
   d->last_path = 1;
+  return YSCV_HIP_OK;
+}
+
+int32_t yscv_hip_decoder_set_prefill_rows(yscv_hip_decoder *d, int32_t rows) {
+  YSCV_REQUIRE(d != nullptr, "null argument");
+  YSCV_REQUIRE(rows >= 1 && rows <= 65536, "rows per prompt pass must be in 1 .. 65536, got %d", rows);
+  d->prefill_rows = rows;
   return YSCV_HIP_OK;
 }
 

@@ -86,6 +86,10 @@ class Decoder:
         self.batch = 1
         lib().decoder_prefill(self._h, _p(t), int(t.size), int(start_pos), C.c_void_p(stream) if stream else None)
 
+    def set_prefill_rows(self, rows):
+        """yscv_hip_decoder_set_prefill_rows: prompt rows per pass of prefill() (default 4096)."""
+        lib().decoder_set_prefill_rows(self._h, int(rows))
+
     def run(self, n_steps, use_graph=True, stream=None, persistent=False, auto=False):
         """use_graph: replay one captured HIP graph per step; persistent: run all steps inside one
         cooperative launch (batch 1, shapes the single-launch kernel supports); auto: the fastest of the two
