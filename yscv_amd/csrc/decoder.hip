@@ -492,7 +492,10 @@ static int32_t enqueue_step(yscv_hip_decoder *d, int batch, hipStream_t s) {
     }
     const int qkv_n = (c.n_heads + 2 * c.n_kv_heads) * c.head_dim;
     if (L.qkv_bias) YSCV_TRY(launch_bias_add_f16(d->qkv, L.qkv_bias, (size_t)batch, (size_t)qkv_n, s));
-    if (d->generic_attn) {
+    if (d->generic_attn && d->fused_attn) {
+      YSCV_TRY(launch_gqa_cache(d->qkv, L.kc, L.vc, d->pos, batch, 0, c.n_heads, c.n_kv_heads, c.head_dim, c.max_ctx, d->ao, s,
+                                c.rope_theta, d->qrot));
+    } else if (d->generic_attn) {
       YSCV_TRY(launch_rope_append(d->qkv, d->pos, batch, c.n_heads, c.n_kv_heads, c.head_dim, c.rope_theta, c.max_ctx,
                                   L.kc, L.vc, s));
       YSCV_TRY(launch_gqa_cache(d->qkv, L.kc, L.vc, d->pos, batch, 0, c.n_heads, c.n_kv_heads, c.head_dim, c.max_ctx, d->ao, s));

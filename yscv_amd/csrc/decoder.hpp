@@ -53,8 +53,12 @@ int32_t launch_kv_random_fill(_Float16 *buf, size_t n, uint64_t seed, hipStream_
 // glue_ops.hip: the general attention kernel over the fp16 cache (any head width that is a multiple of 32 up to 128,
 // any number of query heads per kv head).  pos_ptr != null: `rows` batch rows at the position *pos_ptr (decode);
 // pos_ptr == null: `rows` consecutive positions start_pos .. of batch row 0, causal (prompt pass).
+// With `qrot` (decode mode only) the rotary embedding and the cache append of the new position happen inside the
+// kernel: qkv holds q, k, v unrotated, kc / vc receive the new row (they are written), qrot the rotated query heads
+// [rows][hq * hd]; without it qkv holds the rotated q and the cache already has the row.
 int32_t launch_gqa_cache(const _Float16 *qkv, const _Float16 *kc, const _Float16 *vc, const int32_t *pos_ptr, int rows,
-                         int start_pos, int hq, int hkv, int hd, int max_ctx, _Float16 *out, hipStream_t s);
+                         int start_pos, int hq, int hkv, int hd, int max_ctx, _Float16 *out, hipStream_t s,
+                         float rope_theta = 0.0f, _Float16 *qrot = nullptr);
 int32_t launch_prefill_rope_append(_Float16 *qkv, int rows, int start_pos, int hq, int hkv, int hd, float theta, int max_ctx,
                                    _Float16 *kc, _Float16 *vc, hipStream_t s);
 int32_t launch_bias_add_f16(_Float16 *x, const _Float16 *bias, size_t rows, size_t n, hipStream_t s);

@@ -26,6 +26,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <type_traits>
 
 #include "int4_common.hpp"
 #include "decoder.hpp"
@@ -45,6 +46,11 @@ struct GqaArgs {
   int causal_base;            // < 0: every query sees all Sk positions; else query s sees positions <= causal_base + s
   const int32_t *sk_minus_1;  // null, or device word holding Sk - 1 (the decoder's position counter)
   float scale;
+  // Decode with the rotary embedding and the cache append inside the kernel (FUSE): q is [B][(Hq + 2 Hkv) HD] with
+  // q, k and v of the new position unrotated; the workgroups rotate what they need themselves, the first query head
+  // of a kv group also writes the new k / v row to the cache (k, v are then written through), the rotated q goes to qrot
+  float theta;
+  _Float16 *qrot;
 };
 
 template <typename T>
@@ -72,12 +78,15 @@ __device__ __forceinline__ void store4<float>(float *p, float a, float b, float 
 
 constexpr int GQA_WAVES = 4;
 
-template <int HD, typename TQ, typename TKV, typename TO, bool V_SLAB>
+template <int HD, typename TQ, typename TKV, typename TO, bool V_SLAB, bool FUSE = false>
 __global__ void __launch_bounds__(64 * GQA_WAVES) gqa_generic_kernel(GqaArgs p) {
   static_assert(HD % 32 == 0 && HD >= 32 && HD <= 128, "head width (the merge buffer must fit the static LDS limit)");
+  static_assert(!FUSE || (V_SLAB && std::is_same<TQ, _Float16>::value && std::is_same<TKV, _Float16>::value),
+                "the fused form works on the decoder's fp16 buffers");
   constexpr int KK = HD / 32, DT = HD / 16;
   __shared__ float m_s[GQA_WAVES][16], l_s[GQA_WAVES][16];
   __shared__ float o_s[GQA_WAVES][16][HD + 4];
+  __shared__ __attribute__((aligned(16))) _Float16 q_rot[FUSE ? HD : 8], k_new[FUSE ? HD : 8], v_new[FUSE ? HD : 8];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, c = lane >> 4;
   const int q0 = blockIdx.x * 16, h = blockIdx.y, b = blockIdx.z;
@@ -90,12 +99,61 @@ __global__ void __launch_bounds__(64 * GQA_WAVES) gqa_generic_kernel(GqaArgs p) 
   const int nblocks = lim_tile / 16 + 1;
 
   const TQ *qrow = static_cast<const TQ *>(p.q) + (size_t)b * p.q_b + (size_t)qi * p.q_s + (size_t)h * HD;
-  half8_t qf[KK];
-#pragma unroll
-  for (int kk = 0; kk < KK; kk++) qf[kk] = load8<TQ>(qrow + 32 * kk + 8 * c);
-
   const TKV *kbase = static_cast<const TKV *>(p.k) + (size_t)b * p.k_b + (size_t)kvh * p.k_h;
   const TKV *vbase = static_cast<const TKV *>(p.v) + (size_t)b * p.v_b + (size_t)kvh * p.v_h;
+  half8_t qf[KK];
+  if constexpr (FUSE) {
+    // One query position per sequence (Sq = 1, the position is Sk - 1).  Wave 0 rotates this head's q, wave 1 the new
+    // k row of its kv head, waves 2 and 3 fetch the new v row: the arithmetic of the separate rope + append launch.
+    // Every workgroup of a kv group works out the same k / v row (it cannot wait for another workgroup's append) and
+    // patches it into the key block that holds the position; one of them stores it.
+    const int pos = Sk - 1, half_d = HD / 2, wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const bool writer = h % (p.Hq / p.Hkv) == 0;
+    const _Float16 *row = reinterpret_cast<const _Float16 *>(p.q) + (size_t)b * p.q_b;
+    if (wave_u < 2) {
+      const int i = lane;
+      if (i < half_d) {
+        const float inv_freq = 1.0f / powf(p.theta, (float)(2 * i) / (float)HD);
+        float sn, cs;
+        sincosf(inv_freq * (float)pos, &sn, &cs);
+        const _Float16 *src = row + (size_t)(wave_u == 0 ? h : p.Hq + kvh) * HD;
+        const float x0 = (float)src[i], x1 = (float)src[i + half_d];
+        float f0 = fmaf(x0, cs, -(x1 * sn)), f1 = fmaf(x0, sn, x1 * cs);
+        asm volatile("" : "+v"(f0), "+v"(f1));  // the f32 value exists before it is narrowed (no mixed-precision fma)
+        const _Float16 y0 = (_Float16)f0, y1 = (_Float16)f1;
+        if (wave_u == 0) {
+          q_rot[i] = y0;
+          q_rot[i + half_d] = y1;
+          _Float16 *qd = p.qrot + ((size_t)b * p.Hq + h) * HD;
+          qd[i] = y0;
+          qd[i + half_d] = y1;
+        } else {
+          k_new[i] = y0;
+          k_new[i + half_d] = y1;
+          if (writer) {
+            _Float16 *kd = const_cast<_Float16 *>(reinterpret_cast<const _Float16 *>(kbase)) + (size_t)pos * p.k_s;
+            kd[i] = y0;
+            kd[i + half_d] = y1;
+          }
+        }
+      }
+    } else {
+      const int dd = tid - 128;
+      if (dd < HD) {
+        const _Float16 v = row[(size_t)(p.Hq + p.Hkv + kvh) * HD + dd];
+        v_new[dd] = v;
+        if (writer)
+          const_cast<_Float16 *>(reinterpret_cast<const _Float16 *>(vbase))[((size_t)(pos >> 3) * HD + dd) * 8 + (pos & 7)] = v;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) qf[kk] = *reinterpret_cast<const half8_t *>(&q_rot[32 * kk + 8 * c]);
+  } else {
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) qf[kk] = load8<TQ>(qrow + 32 * kk + 8 * c);
+  }
+
   float m_run = -INFINITY, l_run = 0.0f;
   float4_t o_acc[DT];
 #pragma unroll
@@ -130,6 +188,26 @@ __global__ void __launch_bounds__(64 * GQA_WAVES) gqa_generic_kernel(GqaArgs p) 
     const int p0 = blk * 16;
     const bool more = blk + GQA_WAVES < nblocks;  // uniform in the wave
     if (more) load_block(blk + GQA_WAVES, kn, vn);
+    if constexpr (FUSE) {
+      // the row appended in this launch: the loads saw whatever the cache held before
+      const int rel = Sk - 1 - p0;
+      if (rel >= 0 && rel < 16) {  // uniform in the wave
+        if (r == rel) {
+#pragma unroll
+          for (int kk = 0; kk < KK; kk++) kf[kk] = *reinterpret_cast<const half8_t *>(&k_new[32 * kk + 8 * c]);
+        }
+        const int e_new = rel - 4 * c;
+        if (e_new >= 0 && e_new < 4) {
+#pragma unroll
+          for (int t = 0; t < DT; t++) {
+            const _Float16 nv = v_new[16 * t + r];
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+              if (e == e_new) vf[t][e] = nv;
+          }
+        }
+      }
+    }
     float4_t s = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int kk = 0; kk < KK; kk++) s = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kk], qf[kk], s, 0, 0, 0);
@@ -563,6 +641,20 @@ int32_t gqa_launch(const GqaArgs &a, int hd, hipStream_t s) {
   return YSCV_HIP_OK;
 }
 
+// decode step on the decoder's fp16 buffers with the rotary embedding and the cache append inside the kernel
+int32_t gqa_launch_fused_decode(const GqaArgs &a, int hd, hipStream_t s) {
+  const dim3 grid(1, (unsigned)a.Hq, (unsigned)a.B), block(64 * GQA_WAVES);
+  switch (hd) {
+    case 32: hipLaunchKernelGGL((gqa_generic_kernel<32, _Float16, _Float16, _Float16, true, true>), grid, block, 0, s, a); break;
+    case 64: hipLaunchKernelGGL((gqa_generic_kernel<64, _Float16, _Float16, _Float16, true, true>), grid, block, 0, s, a); break;
+    case 96: hipLaunchKernelGGL((gqa_generic_kernel<96, _Float16, _Float16, _Float16, true, true>), grid, block, 0, s, a); break;
+    case 128: hipLaunchKernelGGL((gqa_generic_kernel<128, _Float16, _Float16, _Float16, true, true>), grid, block, 0, s, a); break;
+    default: return set_error(YSCV_HIP_ERR_UNSUPPORTED, "attention: head width %d (supported: 32, 64, 96, 128)", hd);
+  }
+  YSCV_HIP_TRY(hipGetLastError());
+  return YSCV_HIP_OK;
+}
+
 // ---- RMSNorm over the last axis, f32 in and out ---------------------------------------------------------------
 __global__ void __launch_bounds__(256) rms_norm_f32_kernel(const float *__restrict__ x, const float *__restrict__ gamma, int d,
                                                            float eps, float *__restrict__ y) {
@@ -694,8 +786,11 @@ int32_t launch_bias_add_f16(_Float16 *x, const _Float16 *bias, size_t rows, size
 //   prompt ingestion (pos_ptr == null): the rows are consecutive positions start_pos .. of batch row 0, row i sees
 //   cache rows [0, start_pos + i].
 int32_t launch_gqa_cache(const _Float16 *qkv, const _Float16 *kc, const _Float16 *vc, const int32_t *pos_ptr, int rows,
-                         int start_pos, int hq, int hkv, int hd, int max_ctx, _Float16 *out, hipStream_t s) {
+                         int start_pos, int hq, int hkv, int hd, int max_ctx, _Float16 *out, hipStream_t s, float rope_theta,
+                         _Float16 *qrot) {
   GqaArgs a{};
+  a.theta = rope_theta;
+  a.qrot = qrot;
   const long long row_elems = (long long)(hq + 2 * hkv) * hd;
   a.q = qkv;
   a.k = kc;
@@ -733,6 +828,8 @@ int32_t launch_gqa_cache(const _Float16 *qkv, const _Float16 *kc, const _Float16
     a.o_b = 0;
     a.o_s = (long long)hq * hd;
   }
+  // decode mode with qrot given: q / k / v of the new position come unrotated, rope + append happen in the kernel
+  if (pos_ptr && qrot) return gqa_launch_fused_decode(a, hd, s);
   // prompt mode with enough rows: the kernel that stages K / V in LDS for four waves (its K rows must be contiguous
   // 16-byte pieces, which the cache's are)
   if (!pos_ptr && rows >= 64 && (max_ctx & 7) == 0) return gqa_launch_shared_kv(a, hd, s);
