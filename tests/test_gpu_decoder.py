@@ -237,9 +237,9 @@ def test_int8_cache_with_small_values(v_mag, use_graph):
         cur = dec.tokens(step, 1)[0].copy()
 
 
-@pytest.mark.parametrize("heads", [(4, 2, 128), (8, 1, 64), (4, 4, 32), (12, 4, 96)],
-                         ids=["4q2kv-hd128", "8q1kv-hd64", "4q4kv-hd32", "12q4kv-hd96"])
-@pytest.mark.parametrize("kv_dtype", ["f16", "i8"])
+@pytest.mark.parametrize("kv_dtype,heads", [("f16", (4, 2, 128)), ("i8", (4, 2, 128)), ("f16", (8, 1, 64)), ("f16", (4, 4, 32)),
+                                            ("f16", (12, 4, 96))],
+                         ids=["f16-4q2kv-hd128", "i8-4q2kv-hd128", "f16-8q1kv-hd64", "f16-4q4kv-hd32", "f16-12q4kv-hd96"])
 @pytest.mark.parametrize("prefill", [5, 127, 128, 133, 250])
 def test_fused_attention_equals_the_separate_rope_append(prefill, kv_dtype, heads):
     """Rotary embedding and cache append inside the attention kernel against the separate rope_append launch in front
@@ -253,8 +253,6 @@ def test_fused_attention_equals_the_separate_rope_append(prefill, kv_dtype, head
     from yscv_amd.capi import lib
 
     nh, nkv, hd = heads
-    if kv_dtype == "i8" and heads != (4, 2, 128):
-        pytest.skip("the int8 cache exists for the specialised attention kernels")
     rng = np.random.default_rng(4100 + prefill)
     cfg = dict(CFG, n_heads=nh, n_kv_heads=nkv, head_dim=hd)
     dec, _ = _build(rng, cfg, kv_dtype=kv_dtype)
