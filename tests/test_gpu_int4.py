@@ -634,7 +634,9 @@ def test_random_shapes_every_output(K, torch_cuda):
 
 
 @pytest.mark.parametrize("m,n,k,g,has_zp", [
-    (17, 4096, 4096, 32, False),    # one 32-row tile row, 32 tiles: split eight ways
+    (17, 4096, 4096, 32, False),    # 17 .. 32 rows: the register-resident kernel, one workgroup covers all of K
+    (24, 1000, 14336, 32, True),    # the same kernel with K cut into four parts (f32 partial sums + second kernel), ragged N
+    (32, 6144, 4608, 128, False),   # K not a multiple of what a workgroup covers: the last part's trailing waves idle
     (40, 1001, 2048, 64, True),     # ragged N (scalar stores of the partial sums), zero points
     (64, 6144, 4096, 32, False),    # the q/k/v projection of a 64-token prompt
     (100, 4096, 14336, 128, True),  # the down projection of a 100-token prompt: 64-row tiles, long K
@@ -644,7 +646,8 @@ def test_random_shapes_every_output(K, torch_cuda):
 ])
 def test_k_split_shapes_every_output(K, torch_cuda, m, n, k, g, has_zp):
     """Shapes with fewer output tiles than half the CUs: the LDS-ring GEMM is cut along K as well, the splits' f32
-    partial sums go through the workspace and a second kernel adds them in a fixed order and applies the epilogue.
+    partial sums go through the workspace and a second kernel adds them in a fixed order and applies the epilogue;
+    17 .. 32 rows take the kernel of int4_mid.hip, which cuts K into parts beyond 4096.
     Every output of the plain call against an fp32 product on the GPU, twice with the same bits, the same bits with a
     caller's workspace (nothing written past the announced size), and both fused epilogues against the plain result."""
     torch = torch_cuda
